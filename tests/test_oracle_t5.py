@@ -1,0 +1,417 @@
+"""Pins oracle/t5.py and oracle/models.py.
+
+Known answers and closed forms come from the reference's own tests
+(t5x/examples/t5/layers_test.py, t5x/models_test.py; lines cited per test);
+what those leave open is pinned by textbook forms (softmax attention through
+np.einsum, geometric bucket boundaries, RMS-norm invariants) and by brute force
+(full-sequence decoder forward == step-by-step cached decode).
+"""
+
+import functools
+
+import numpy as np
+import pytest
+
+from oracle import decoding
+from oracle import models
+from oracle import t5
+
+
+def tiny_cfg(dtype='float32', **kw):
+  base = dict(vocab_size=50, dtype=dtype, emb_dim=16, num_heads=4,
+              num_encoder_layers=2, num_decoder_layers=2, head_dim=8,
+              mlp_dim=32)
+  base.update(kw)
+  return t5.T5Config(**base)
+
+
+def ref_softmax(x):
+  x = np.asarray(x, np.float64)
+  e = np.exp(x - x.max(-1, keepdims=True))
+  return e / e.sum(-1, keepdims=True)
+
+
+@pytest.mark.parametrize('f', [20, 22])
+def test_multihead_attention_closed_form(f):
+  # layers_test.py:339-377
+  b, q, h, d, k = 2, 3, 4, 5, 6
+  np.random.seed(0)
+  inputs_q = np.random.randn(b, q, f)
+  inputs_kv = np.random.randn(b, k, f)
+  qk = np.random.randn(f, h, d)
+  kk = np.random.randn(f, h, d)
+  vk = np.random.randn(f, h, d)
+  ok = np.random.randn(h, d, f)
+  params = {'query': {'kernel': qk.reshape(f, -1)},
+            'key': {'kernel': kk.reshape(f, -1)},
+            'value': {'kernel': vk.reshape(f, -1)},
+            'out': {'kernel': ok.reshape(-1, f)}}
+  y, _ = t5.multi_head_attention(params, inputs_q, inputs_kv, None, None,
+                                 num_heads=h, head_dim=d, dtype='float32')
+  query = np.einsum('bqf,fhd->bqhd', inputs_q, qk)
+  key = np.einsum('bkf,fhd->bkhd', inputs_kv, kk)
+  value = np.einsum('bkf,fhd->bkhd', inputs_kv, vk)
+  w = ref_softmax(np.einsum('bqhd,bkhd->bhqk', query, key))
+  want = np.einsum('bqhd,hdf->bqf', np.einsum('bhqk,bkhd->bqhd', w, value), ok)
+  np.testing.assert_allclose(y, want, rtol=2e-4, atol=2e-4)
+
+
+def test_attention_cache_layout_and_index():
+  # layers_test.py:379-422: projections mocked to reshapes == identity kernels
+  b, h, d, k = 2, 3, 4, 5
+  f = h * d
+  eye = np.eye(f, dtype=np.float32)
+  params = {n: {'kernel': eye} for n in ('query', 'key', 'value', 'out')}
+  cache = {'cached_key': np.zeros((b, h, d, k), np.float32),
+           'cached_value': np.zeros((b, h, d, k), np.float32),
+           'cache_index': np.array(0)}
+  x = np.random.RandomState(1).randn(b, 1, f).astype(np.float32)
+  _, new = t5.multi_head_attention(params, x, x, None, None, num_heads=h,
+                                   head_dim=d, dtype='float32', decode=True,
+                                   cache=cache)
+  want = np.zeros((b, h, d, k), np.float32)
+  want[:, :, :, 0] = x.reshape(b, 1, h, d)[:, 0]
+  np.testing.assert_allclose(new['cached_key'], want)
+  np.testing.assert_allclose(new['cached_value'], want)
+  assert new['cache_index'] == 1
+
+
+def test_dot_product_attention_with_bias():
+  # layers_test.py:424-436
+  b, q, h, d, k = 2, 3, 4, 5, 6
+  np.random.seed(0)
+  query = np.random.randn(b, q, h, d)
+  key = np.random.randn(b, k, h, d)
+  value = np.random.randn(b, k, h, d)
+  bias = np.random.randn(b, h, q, k)
+  out = t5.dot_product_attention(query, key, value, bias, 'float32')
+  w = ref_softmax(np.einsum('bqhd,bkhd->bhqk', query, key) + bias)
+  np.testing.assert_allclose(out, np.einsum('bhqk,bkhd->bqhd', w, value),
+                             atol=2e-6)
+
+
+def test_dense_general_ones():
+  # layers_test.py:504-536
+  y = t5.dense_general(np.ones((1, 3)), np.ones((3, 4)), 'float32')
+  np.testing.assert_allclose(y, np.full((1, 4), 3.0))
+
+
+def test_masks():
+  # layers_test.py:121-180 (attention / causal masks; decode uses the first)
+  m = t5.make_attention_mask(np.array([[1, 1, 0]]) > 0,
+                             np.array([[1, 0, 1, 1]]) > 0)
+  assert m.shape == (1, 1, 3, 4)
+  np.testing.assert_array_equal(
+      m[0, 0], [[1, 0, 1, 1], [1, 0, 1, 1], [0, 0, 0, 0]])
+  c = t5.make_causal_mask(np.zeros((1, 3)))
+  np.testing.assert_array_equal(c[0, 0], np.tril(np.ones((3, 3))))
+  assert t5.combine_masks(None, None) is None
+  assert t5.combine_biases(None) is None
+
+
+def _bucket_from_boundaries(n, max_exact, num_buckets, max_distance):
+  # bucket b >= max_exact covers [max_exact*r^(b-max_exact), ...), with
+  # r = (max_distance/max_exact)^(1/(num_buckets-max_exact))
+  if n < max_exact:
+    return n
+  r = (max_distance / max_exact)**(1.0 / (num_buckets - max_exact))
+  b = max_exact
+  while b < num_buckets - 1 and n >= max_exact * r**(b - max_exact + 1) - 1e-9:
+    b += 1
+  return b
+
+
+def test_relative_position_bucket_unidirectional_table():
+  # layers.py:580-625 with the decoder's settings (network.py:242-251).
+  table = {}
+  ranges = [(16, 18, 16), (19, 20, 17), (21, 23, 18), (24, 26, 19),
+            (27, 30, 20), (31, 34, 21), (35, 39, 22), (40, 45, 23),
+            (46, 51, 24), (52, 58, 25), (59, 66, 26), (67, 76, 27),
+            (77, 86, 28), (87, 98, 29), (99, 112, 30), (113, 400, 31)]
+  for n in range(16):
+    table[n] = n
+  for lo, hi, b in ranges:
+    for n in range(lo, hi + 1):
+      table[n] = b
+  n = np.arange(0, 401)
+  got = t5.relative_position_bucket(-n, bidirectional=False)
+  np.testing.assert_array_equal(got, [table[i] for i in n])
+  # keys in the future (memory after query) all map to bucket 0
+  np.testing.assert_array_equal(
+      t5.relative_position_bucket(np.arange(1, 50), bidirectional=False), 0)
+  # independent derivation from the geometric bucket boundaries
+  np.testing.assert_array_equal(
+      got, [_bucket_from_boundaries(int(i), 16, 32, 128) for i in n])
+
+
+def test_relative_position_bucket_bidirectional_boundaries():
+  n = np.arange(0, 300)
+  past = t5.relative_position_bucket(-n, bidirectional=True)
+  want = np.array([_bucket_from_boundaries(int(i), 8, 16, 128) for i in n])
+  np.testing.assert_array_equal(past, want)
+  future = t5.relative_position_bucket(n[1:], bidirectional=True)
+  np.testing.assert_array_equal(future, want[1:] + 16)
+
+
+def test_relpos_bias_is_table_lookup():
+  rs = np.random.RandomState(0)
+  emb = rs.randn(3, 32).astype(np.float32)
+  bias = t5.relpos_bias(emb, 5, 5, False, 'float32')
+  assert bias.shape == (1, 3, 5, 5)
+  for q in range(5):
+    for k in range(5):
+      np.testing.assert_array_equal(bias[0, :, q, k], emb[:, max(q - k, 0)])
+
+
+def test_rms_layer_norm_closed_form_and_invariants():
+  rs = np.random.RandomState(0)
+  x = rs.randn(4, 64).astype(np.float32)
+  scale = rs.randn(64).astype(np.float32)
+  y = t5.layer_norm(x, scale, 'float32')
+  x64 = x.astype(np.float64)
+  want = x64 / np.sqrt((x64**2).mean(-1, keepdims=True) + 1e-6) * scale
+  np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-6)
+  # no mean subtraction: a constant row stays constant * scale
+  c = t5.layer_norm(np.full((1, 64), 3.0, np.float32), np.ones(64), 'float32')
+  np.testing.assert_allclose(c, 1.0, rtol=1e-5)
+  # positive rescaling of x leaves the output unchanged (up to eps)
+  np.testing.assert_allclose(t5.layer_norm(7.0 * x, scale, 'float32'), y,
+                             rtol=1e-4, atol=1e-5)
+  # linear in scale
+  np.testing.assert_allclose(t5.layer_norm(x, 2 * scale, 'float32'), 2 * y,
+                             rtol=1e-6)
+
+
+def test_bf16_round_nearest_even():
+  x = np.array([1.0, 1.00390625, 1.01171875, -2.5, 3.14159265], np.float32)
+  # 1 + 2^-8 is a tie between 1.0 and 1 + 2^-7 -> even mantissa (1.0);
+  # 1 + 3*2^-8 ties to 1 + 2^-6 (even).
+  np.testing.assert_array_equal(
+      t5.bf16_round(x), np.array([1.0, 1.0, 1.015625, -2.5, 3.140625],
+                                 np.float32))
+  import torch
+  y = np.random.RandomState(0).randn(10000).astype(np.float32) * 100
+  np.testing.assert_array_equal(
+      t5.bf16_round(y), torch.from_numpy(y).bfloat16().float().numpy())
+
+
+def test_gelu_tanh_form_values():
+  # tanh-approximate GELU; anchors from the exact erf form within 1e-3 and the
+  # identities gelu(0)=0, gelu(x)-gelu(-x)=x.
+  from scipy.special import erf
+  x = np.linspace(-4, 4, 41).astype(np.float32)
+  exact = 0.5 * x * (1 + erf(x / np.sqrt(2)))
+  np.testing.assert_allclose(t5.gelu(x), exact, atol=1e-3)
+  np.testing.assert_allclose(t5.gelu(x) - t5.gelu(-x), x, atol=1e-6)
+  assert t5.gelu(np.float32(0)) == 0
+
+
+def test_mlp_block_gated_closed_form():
+  rs = np.random.RandomState(0)
+  x = rs.randn(3, 8).astype(np.float32)
+  p = {'wi_0': {'kernel': rs.randn(8, 12).astype(np.float32)},
+       'wi_1': {'kernel': rs.randn(8, 12).astype(np.float32)},
+       'wo': {'kernel': rs.randn(12, 8).astype(np.float32)}}
+  y = t5.mlp_block(p, x, ('gelu', 'linear'), 'float32')
+  want = (t5.gelu(x @ p['wi_0']['kernel']) *
+          (x @ p['wi_1']['kernel'])) @ p['wo']['kernel']
+  np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-5)
+
+
+def test_quantize_int8_roundtrip():
+  w = np.random.RandomState(0).randn(64, 16).astype(np.float32)
+  q = t5.quantize_int8(w)
+  assert q['q'].dtype == np.int8 and np.abs(q['q']).max() == 127
+  np.testing.assert_allclose(q['q'] * q['scale'], w,
+                             atol=float(q['scale'].max()) / 2 + 1e-7)
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_stepwise_cached_decode_equals_full_sequence(dtype):
+  """Brute force: the decode=True single-step path over a cache reproduces
+  the decode=False full-sequence decoder at every position."""
+  cfg = tiny_cfg(dtype)
+  params = t5.init_params(cfg, seed=1)
+  rs = np.random.RandomState(0)
+  b, e, l = 3, 6, 5
+  enc_tokens = rs.randint(2, cfg.vocab_size, size=(b, e))
+  enc_tokens[1, 4:] = 0
+  targets = rs.randint(2, cfg.vocab_size, size=(b, l))
+  dec_in = np.concatenate([np.zeros((b, 1), int), targets[:, :-1]], axis=1)
+  encoded = t5.encode(params, cfg, enc_tokens)
+  full = t5.decode(params, cfg, encoded, enc_tokens, dec_in, targets)
+  cache = t5.init_cache(cfg, b, l)
+  for literal in (True, False):
+    cache = t5.init_cache(cfg, b, l)
+    cross_kv = None if literal else t5.project_cross_kv(params, cfg, encoded)
+    for t in range(l):
+      tok = dec_in[:, t:t + 1]
+      logits, cache = t5.decode(params, cfg, encoded, enc_tokens, tok, tok,
+                                decode=True, cache=cache, max_decode_length=l,
+                                cross_kv=cross_kv)
+      tol = 1e-4 if dtype == 'float32' else 6e-2
+      np.testing.assert_allclose(logits[:, 0], full[:, t], atol=tol, rtol=tol)
+    for lyr in cache['decoder'].values():
+      assert lyr['self_attention']['cache_index'] == l
+
+
+def test_hoisted_cross_kv_is_bit_identical():
+  cfg = tiny_cfg('bfloat16')
+  params = t5.init_params(cfg, seed=2)
+  rs = np.random.RandomState(0)
+  enc_tokens = rs.randint(2, cfg.vocab_size, size=(2, 5))
+  encoded = t5.encode(params, cfg, enc_tokens)
+  tok = np.zeros((2, 1), int)
+  a, _ = t5.decode(params, cfg, encoded, enc_tokens, tok, tok, decode=True,
+                   cache=t5.init_cache(cfg, 2, 4), max_decode_length=4)
+  b, _ = t5.decode(params, cfg, encoded, enc_tokens, tok, tok, decode=True,
+                   cache=t5.init_cache(cfg, 2, 4), max_decode_length=4,
+                   cross_kv=t5.project_cross_kv(params, cfg, encoded))
+  np.testing.assert_array_equal(a, b)
+
+
+# ---- models.py ---------------------------------------------------------------
+
+
+class _MockModule:
+  """models_test.py:640-656."""
+
+  def __init__(self, dummy_logits, batch_size=2, encoder_len=3, emb_dim=5):
+    self.dtype = 'float32'
+    self.scan_layers = False
+    self.calls = []
+    self._logits = dummy_logits
+    self._enc = np.zeros((batch_size, encoder_len, emb_dim))
+
+  def apply(self, *args, method=None, **kwargs):
+    self.calls.append({'args': args, 'kwargs': kwargs})
+    if method is None:
+      return (self._logits, {'cache': {}})
+    return method()
+
+  def encode(self):
+    return self._enc
+
+  def decode(self):
+    return (self._logits, {'cache': {}})
+
+
+@pytest.mark.parametrize('decode_fn', [
+    decoding.beam_search,
+    functools.partial(decoding.temperature_sample, topk=4)])
+def test_predict_batch_mock_module(decode_fn):
+  # models_test.py:616-675
+  batch = {'encoder_input_tokens': np.zeros((2, 3), np.int32),
+           'decoder_input_tokens': np.zeros((2, 4), np.int32)}
+  dummy = np.array([[-1e7, -1e7, 0, -1e7], [-1e7, -1e7, -1e7, 0]],
+                   np.float32)[:, None, :]
+  model = models.EncoderDecoderModel(_MockModule(dummy), decode_fn=decode_fn)
+  actual = model.predict_batch({}, batch)
+  np.testing.assert_array_equal(actual, [[2] * 4, [3] * 4])
+
+
+def test_predict_batch_rng_rules():
+  # models_test.py:677-740
+  batch = {'encoder_input_tokens': np.zeros((2, 1), np.int32),
+           'decoder_input_tokens': np.zeros((2, 2), np.int32)}
+  seen = {}
+
+  def decode_fn(**kwargs):
+    seen.clear()
+    seen.update(kwargs)
+    return np.zeros((2, 2, 3)), np.zeros((2, 2))
+
+  model = models.EncoderDecoderModel(
+      _MockModule(np.zeros((2, 1, 4), np.float32)), decode_fn=decode_fn)
+  model.predict_batch({}, batch)
+  assert 'decode_rng' not in seen
+  model.predict_batch_with_aux({}, batch)
+  assert 'decode_rng' not in seen
+  model.predict_batch_with_aux({}, batch, decoder_params={'decode_rng': 3})
+  assert seen['decode_rng'] == 3
+  model.predict_batch({}, batch, rng=4)
+  assert seen['decode_rng'] == 4
+  with pytest.raises(ValueError) as err:
+    model.predict_batch_with_aux({}, batch, rng=4,
+                                 decoder_params={'decode_rng': 3})
+  assert str(err.value) == (
+      'Got RNG both from the `rng` argument (4) and '
+      "`decoder_params['decode_rng']` (3). Please specify one or the other.")
+
+
+@pytest.mark.parametrize('dt', [np.int32, np.float32])
+def test_predict_batch_cache_init_call(dt):
+  # models_test.py:742-833
+  batch = {'encoder_input_tokens': np.zeros((2, 3), dt),
+           'decoder_input_tokens': np.zeros((2, 4), dt)}
+  module = _MockModule(np.ones((2, 1, 4), np.float32))
+  model = models.EncoderDecoderModel(module, decode_fn=decoding.beam_search)
+  model.predict_batch({}, batch)
+  call = module.calls[1]
+  assert call['args'][0] == {'params': {}}
+  kw = dict(call['kwargs'])
+  np.testing.assert_allclose(kw.pop('encoder_input_tokens'),
+                             np.ones_like(batch['encoder_input_tokens']))
+  np.testing.assert_allclose(kw.pop('decoder_input_tokens'),
+                             np.ones_like(batch['decoder_input_tokens']))
+  np.testing.assert_allclose(kw.pop('decoder_target_tokens'),
+                             np.ones_like(batch['decoder_input_tokens']))
+  assert kw == {'decode': True, 'enable_dropout': False, 'mutable': ['cache']}
+
+
+def test_forced_prompt_keeps_beam_caches_identical():
+  # models_test.py:340-468 on the restated tiny model.
+  cfg = tiny_cfg('float32')
+  params = t5.init_params(cfg, seed=3)
+  lengths = [2, 3]
+  b, k, e, l = 2, 2, 3, 7
+  dec_in = np.zeros((b, l), np.int32)
+  dec_in[0, 1:1 + lengths[0]] = np.arange(9, 9 + lengths[0])
+  dec_in[1, 1:1 + lengths[1]] = np.arange(3, 3 + lengths[1])
+  batch = {'encoder_input_tokens': np.zeros((b, e), np.int32),
+           'decoder_input_tokens': dec_in}
+  model = models.EncoderDecoderModel(
+      models.Transformer(cfg), decode_fn=decoding.beam_search,
+      output_vocabulary=models._Vocab(eos_id=cfg.vocab_size + 12))
+  calls = []
+  real = model._compute_logits_from_slice
+
+  def spy(state, **kw):
+    calls.append(state)
+    return real(state, **kw)
+
+  model._compute_logits_from_slice = spy
+  model.predict_batch_with_aux(params, batch, prompt_with_targets=True,
+                               num_decodes=k)
+  assert len(calls) == l
+  for bi in range(b):
+    for i, state in enumerate(calls):
+      if i < lengths[bi]:
+        assert state.cur_token[bi * k, 0] == dec_in[bi, i]
+        for lyr in state.cache['decoder'].values():
+          sa = lyr['self_attention']
+          for name in ('cached_key', 'cached_value'):
+            np.testing.assert_array_equal(sa[name][bi * k],
+                                          sa[name][bi * k + 1])
+
+
+def test_end_to_end_tiny_model_greedy_matches_full_forward_argmax():
+  """predict_batch (temperature 0) reproduces teacher-forced argmax of the
+  full-sequence forward on its own output."""
+  cfg = tiny_cfg('float32')
+  params = t5.init_params(cfg, seed=4)
+  rs = np.random.RandomState(0)
+  b, e, l = 2, 5, 6
+  enc = rs.randint(2, cfg.vocab_size, size=(b, e)).astype(np.int32)
+  batch = {'encoder_input_tokens': enc,
+           'decoder_input_tokens': np.zeros((b, l), np.int32)}
+  model = models.EncoderDecoderModel(
+      models.Transformer(cfg),
+      decode_fn=functools.partial(decoding.temperature_sample,
+                                  temperature=0.0),
+      output_vocabulary=models._Vocab(eos_id=cfg.vocab_size + 5))
+  out = model.predict_batch(params, batch)
+  dec_in = np.concatenate([np.zeros((b, 1), np.int32), out[:, :-1]], axis=1)
+  encoded = t5.encode(params, cfg, enc)
+  full = t5.decode(params, cfg, encoded, enc, dec_in, np.ones_like(dec_in))
+  np.testing.assert_array_equal(out, full.argmax(-1))
