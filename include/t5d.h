@@ -1,0 +1,230 @@
+/*
+ * t5d — C ABI of the MI355X (gfx950) decode-step kernels for T5.1.1
+ * encoder-decoder models.
+ *
+ * The reference (google-research/t5x) is pure Python/JAX and has no FFI of
+ * its own; every entry point below replaces a JAX expression on the decode
+ * path and cites it (paths relative to the reference checkout).  The Python
+ * host code in t5x_amd/ binds this library with ctypes and keeps the
+ * reference's call signatures (beam_search, temperature_sample,
+ * predict_batch).
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers unless the name ends in `_host`.
+ *    The library never allocates, frees or copies device memory; the caller
+ *    owns every buffer (PyTorch tensors in the Python binding).
+ *  - `stream` is a hipStream_t passed as void*.  Calls only enqueue work; none
+ *    synchronises.  A call is safe to record into a HIP graph.
+ *  - Return value: 0 on success, a negative T5D_E* code otherwise;
+ *    t5d_last_error() returns a message for the calling thread's last failure.
+ *    Shapes are validated on the host before anything is launched.
+ *  - Activation dtype: T5D_F32 or T5D_BF16.  bfloat16 values are rounded to
+ *    nearest-even at the points where the reference casts to its activation
+ *    dtype; all accumulation is float32.
+ *  - Row-major, innermost dimension contiguous, unless stated otherwise.
+ */
+#ifndef T5D_H_
+#define T5D_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { T5D_F32 = 0, T5D_BF16 = 1, T5D_I8 = 2 };
+
+enum {
+  T5D_OK = 0,
+  T5D_EINVAL = -1,   /* bad shape / dtype / alignment / null pointer */
+  T5D_EHIP = -2,     /* a HIP runtime call failed */
+  T5D_ELIMIT = -3    /* size beyond what the kernels support */
+};
+
+/* GEMM epilogues. */
+enum {
+  T5D_EPI_NONE = 0,      /* C = A·W                                    */
+  T5D_EPI_RESIDUAL = 1,  /* C = act(act(A·W) + residual)               */
+  T5D_EPI_GEGLU = 2      /* C[:, f] = act(act(gelu(act(a0))) * act(a1)) */
+};
+
+int t5d_version(void);
+const char* t5d_last_error(void);
+
+/* Number of bytes t5d_pack_weight writes for a [K, N] kernel (padded to the
+ * 32 x 16 MFMA tile grid).  w_dtype: T5D_BF16 or T5D_I8 (T5D_F32 kernels are
+ * used unpacked). */
+int64_t t5d_packed_weight_bytes(int w_dtype, int K, int N);
+
+/* Repack a row-major [K, N] kernel (already cast to w_dtype) into the tile
+ * order the bf16/int8 GEMM streams: tiles of 32(k) x 16(n), ordered
+ * [n_tile][k_tile], each tile stored lane-major so that lane l of a wavefront
+ * reads the 8 consecutive-k values W[32*kt + 8*(l/16) + j][16*nt + l%16],
+ * j = 0..7, as one 16-byte (bf16) or 8-byte (int8) load.
+ * geglu != 0: `src` is wi_0 and `src2` is wi_1 (each [K, N]); output column
+ * 16*nt + c holds wi_0[:, 8*nt + c] for c < 8 and wi_1[:, 8*nt + c - 8]
+ * otherwise, i.e. a packed [K, 2N] kernel whose tiles pair the two gates. */
+int t5d_pack_weight(void* stream, int w_dtype, const void* src,
+                    const void* src2, void* dst, int K, int N, int geglu);
+
+/* Embedding row gather.  Replaces Embed.__call__ with one_hot=True
+ * (t5x/examples/t5/layers.py:520-541): out[r, :] = table[ids[r], :]. */
+int t5d_embed(void* stream, int dtype, const void* table, const int32_t* ids,
+              void* out, int R, int d, int V);
+
+/* T5 RMS LayerNorm (t5x/examples/t5/layers.py:683-702):
+ * y = act(x * rsqrt(mean(x^2) + eps)); out = act(y * scale). */
+int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
+                void* out, int R, int d, float eps);
+
+/* Bias-free dense layer for M <= 128 rows (DenseGeneral,
+ * t5x/examples/t5/layers.py:364-414; MlpBlock gate product :460-474; the
+ * residual adds of t5x/examples/t5/network.py:146,163,177).
+ *   A [M, K] act dtype; W packed (bf16 / int8, see t5d_pack_weight) or
+ *   row-major [K, N] float32 when dtype == T5D_F32.
+ *   scales: per-output-channel float32 [N] for int8 weights, else NULL.
+ *   out_dtype: dtype of C (T5D_F32 for the logits layer,
+ *   t5x/examples/t5/network.py:286-291).
+ *   T5D_EPI_GEGLU: W is a geglu-packed [K, 2F] kernel, N = 2F, C is [M, F].
+ *   workspace/counters: float32 [split_k_max * M * N] scratch and int32
+ *   [N/16] zero-initialised counters, needed when the call splits K over
+ *   workgroups (t5d_gemm_workspace_bytes > 0); counters are left zeroed. */
+int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M, int K, int N);
+int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
+             const void* A, const void* W, const float* scales,
+             const void* residual, void* C, int M, int K, int N, int epilogue,
+             void* workspace, int32_t* counters);
+
+/* One step of cached decoder self-attention
+ * (MultiHeadDotProductAttention decode branch,
+ * t5x/examples/t5/layers.py:223-346, and dot_product_attention :52-129).
+ *   qkv [R, 3*H*64]: query | key | value projections of the current token.
+ *   cached_key / cached_value [R, H, 64, L] (the reference's cache layout,
+ *   layers.py:231-241); column t = *cache_index receives the new key/value,
+ *   then the query attends over columns 0..t.
+ *   rel_bias [H, L] act dtype: rel_bias[h, n] is the decoder's relative
+ *   position bias for distance n = t - j (RelativePositionBiases,
+ *   layers.py:560-677, bidirectional=False).
+ *   out [R, H*64].  *cache_index is read, not advanced. */
+int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
+                            void* cached_key, void* cached_value,
+                            const void* rel_bias, const int32_t* cache_index,
+                            void* out, int R, int H, int L);
+
+/* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
+ * mask :366-370).  The reference re-projects K/V from the beam-expanded
+ * encoder output every step; here they are projected once per batch item:
+ *   cross_key / cross_value [B, H, 64, E], shared by the item's `beams` rows;
+ *   enc_len [B]: number of leading valid (non-padding) encoder positions.
+ *   q [B*beams, H*64] -> out [B*beams, H*64]. */
+int t5d_cross_attention_step(void* stream, int dtype, const void* q,
+                             const void* cross_key, const void* cross_value,
+                             const int32_t* enc_len, void* out, int B,
+                             int beams, int H, int E);
+
+/* Add `delta` to n int32 values (cache_index += 1, layers.py:275). */
+int t5d_add_i32(void* stream, int32_t* x, int n, int delta);
+
+/* Beam-axis gather of cache tensors, in place
+ * (cache_gather_beams, t5x/decoding.py:808-870; call site :1449-1457).
+ *   cache: n_tensors tensors of [B, beams, inner, L] elements of elem_bytes,
+ *   spaced tensor_stride_bytes apart; new[b, e] = old[b, beam_indices[b, e]].
+ *   Only columns < *valid_len (or all L when valid_len is NULL) are moved;
+ *   batch items whose indices are the identity are skipped. */
+int t5d_cache_gather_beams(void* stream, void* cache, int64_t tensor_stride_bytes,
+                           int n_tensors, int elem_bytes, int B, int beams,
+                           int inner, int L, const int32_t* beam_indices,
+                           const int32_t* valid_len, int valid_len_offset);
+
+/* Beam-axis gather, out of place (gather_beams, t5x/decoding.py:873-915):
+ * dst[b, e, :] = src[b, beam_indices[b, e], :], rows of inner_bytes bytes. */
+int t5d_gather_beams(void* stream, const void* src, void* dst,
+                     const int32_t* beam_indices, int B, int old_beams,
+                     int new_beams, int64_t inner_bytes);
+
+/* Exact top-k along the last axis (lax.top_k as used by
+ * t5x/decoding.py:918-966,988,1426): values descending, ties toward the lower
+ * index.  x [rows, n] float32 -> vals [rows, k], idx [rows, k]. k <= 64. */
+int t5d_top_k(void* stream, const float* x, float* vals, int32_t* idx,
+              int rows, int n, int k);
+
+/* log_softmax over the vocabulary + prefix log-prob add + top-2K over
+ * beam x vocab (t5x/decoding.py:1340-1366).
+ *   logits [B*beams, V] f32, live_logprobs [B, beams] f32.
+ *   topk_vals/topk_idx [B, k]: the k largest of
+ *   (logits - max - lse) + live_logprobs over the flattened [beams*V] axis,
+ *   flat index = beam*V + token.  row_max/row_lse [B*beams] are also written
+ *   (max and log-sum-exp of the shifted row). k <= 64.
+ *   scratch: float32/int32 pairs, at least 2*B*beams*k*4 bytes. */
+int t5d_beam_topk(void* stream, const float* logits,
+                  const float* live_logprobs, float* topk_vals,
+                  int32_t* topk_idx, float* row_max, float* row_lse,
+                  void* scratch, int B, int beams, int V, int k);
+
+/* State of one beam search (t5x/decoding.py:1002-1021), device arrays. */
+typedef struct {
+  int32_t* cur_index;        /* scalar */
+  float* live_logprobs;      /* [B, K] */
+  float* finished_scores;    /* [B, K] */
+  int32_t* live_seqs;        /* [B, K, S]  S = max_decode_len + 1 */
+  int32_t* finished_seqs;    /* [B, K, S] */
+  uint8_t* finished_flags;   /* [B, K] */
+} t5d_beam_state;
+
+/* Everything in the beam_search loop body after the top-2K
+ * (t5x/decoding.py:1366-1506): prompt forcing, sequence gather + token write,
+ * EOS handling, second top-K with flip, brevity-penalised finished pool merge.
+ *   in/out: `cur` is read, `next` is written (distinct buffers);
+ *   next.cur_index = cur.cur_index + 1.
+ *   inputs [B, Lin] prompt tokens; initial_index [B];
+ *   brevity [S + max(initial_index) + 1] f32: ((5+len)/6)^alpha by length.
+ *   top_alive_indices [B, K] (out): source beam of each surviving beam, the
+ *   argument of cache_gather_beams. */
+int t5d_beam_update(void* stream, const t5d_beam_state* cur,
+                    const t5d_beam_state* next, const float* topk_vals,
+                    const int32_t* topk_idx, const int32_t* inputs,
+                    const int32_t* initial_index, const float* brevity,
+                    int32_t* top_alive_indices, int B, int K, int S, int Lin,
+                    int V, int eos_id);
+
+/* Loop condition of beam_search (t5x/decoding.py:1250-1300) evaluated on
+ * `state`; writes 1 (continue) or 0 to *keep_going.
+ *   min_brevity: ((5 + S)/6)^alpha; min_initial_index: min(initial_index). */
+int t5d_beam_cond(void* stream, const t5d_beam_state* state, int B, int K,
+                  int S, float min_brevity, float min_log_prob,
+                  int max_decode_step, int min_initial_index,
+                  int32_t* keep_going);
+
+/* Token choice of one temperature_sample step (t5x/decoding.py:541-621 and
+ * t5x/binary_search.py:167-227):
+ *   temperature[r] <= 1e-4: argmax(logits[r]) (first occurrence);
+ *   else scaled = logits / max(T, 1e-4); top-k mask (keep scaled >= k-th
+ *   largest, others = -1e7) when topk > 0, or top-p mask (smallest set with
+ *   probability mass >= topp, t5x/binary_search.py:230-299) when topp > 0;
+ *   token = argmax(scaled + gumbel[r]);
+ *   log-prob = log_softmax(rescale ? scaled : logits)[token]
+ *   (0 for the greedy branch when rescale).
+ *   logits, gumbel [R, V] f32 (gumbel may be NULL when every T <= 1e-4);
+ *   temperature [R] f32; tokens [R] i32, logprobs [R] f32 (out). */
+int t5d_sample_tokens(void* stream, const float* logits, const float* gumbel,
+                      const float* temperature, int32_t* tokens,
+                      float* logprobs, int R, int V, int topk, float topp,
+                      int rescale);
+
+/* Bookkeeping of one temperature_sample step (t5x/decoding.py:631-700):
+ * prompt teacher forcing, log-prob accumulation, sequence write at i+1, EOS
+ * counting, `ended` update.  All arrays are updated in place.
+ *   sequences [R, S] (S = L + 2); cur_index [R]; cur_token [R];
+ *   ended [R] u8; log_prob [R]; max_decode_len [R]; initial_eos_count [R];
+ *   *all_ended (out) = every row ended. */
+int t5d_sample_update(void* stream, const int32_t* tokens,
+                      const float* token_logprobs, int32_t* sequences,
+                      int32_t* cur_index, int32_t* cur_token, uint8_t* ended,
+                      float* log_prob, const int32_t* max_decode_len,
+                      const int32_t* initial_eos_count, int32_t* all_ended,
+                      int R, int S, int eos_id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* T5D_H_ */

@@ -1,0 +1,123 @@
+"""ctypes binding of libt5d.so (the HIP kernels behind include/t5d.h).
+
+There is no fallback: if the shared library has not been built, anything that
+needs a kernel raises.  Pointers are passed as plain integers
+(`tensor.data_ptr()`), the stream as the current torch stream's handle.
+"""
+
+import ctypes
+import os
+from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int32,
+                    c_int64, c_uint8, c_void_p)
+
+F32, BF16, I8 = 0, 1, 2
+EPI_NONE, EPI_RESIDUAL, EPI_GEGLU = 0, 1, 2
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'csrc', 'libt5d.so')
+
+
+class BeamStatePtrs(Structure):
+  """t5d_beam_state."""
+  _fields_ = [('cur_index', c_void_p), ('live_logprobs', c_void_p),
+              ('finished_scores', c_void_p), ('live_seqs', c_void_p),
+              ('finished_seqs', c_void_p), ('finished_flags', c_void_p)]
+
+
+_P = c_void_p
+_SIGNATURES = {
+    't5d_version': (c_int, []),
+    't5d_last_error': (c_char_p, []),
+    't5d_packed_weight_bytes': (c_int64, [c_int, c_int, c_int]),
+    't5d_pack_weight': (c_int, [_P, c_int, _P, _P, _P, c_int, c_int, c_int]),
+    't5d_embed': (c_int, [_P, c_int, _P, _P, _P, c_int, c_int, c_int]),
+    't5d_rmsnorm': (c_int, [_P, c_int, _P, _P, _P, c_int, c_int, c_float]),
+    't5d_gemm_workspace_bytes': (c_int64, [c_int] * 5),
+    't5d_gemm': (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
+                         c_int, c_int, c_int, _P, _P]),
+    't5d_self_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P,
+                                        c_int, c_int, c_int]),
+    't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
+                                         c_int, c_int, c_int]),
+    't5d_add_i32': (c_int, [_P, _P, c_int, c_int]),
+    't5d_cache_gather_beams': (c_int, [_P, _P, c_int64, c_int, c_int, c_int,
+                                       c_int, c_int, c_int, _P, _P, c_int]),
+    't5d_gather_beams': (c_int, [_P, _P, _P, _P, c_int, c_int, c_int,
+                                 c_int64]),
+    't5d_top_k': (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
+    't5d_beam_topk': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int,
+                              c_int, c_int]),
+    't5d_beam_update': (c_int, [_P, POINTER(BeamStatePtrs),
+                                POINTER(BeamStatePtrs), _P, _P, _P, _P, _P, _P,
+                                c_int, c_int, c_int, c_int, c_int, c_int]),
+    't5d_beam_cond': (c_int, [_P, POINTER(BeamStatePtrs), c_int, c_int, c_int,
+                              c_float, c_float, c_int, c_int, _P]),
+    't5d_sample_tokens': (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int,
+                                  c_float, c_int]),
+    't5d_sample_update': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
+                                  c_int, c_int, c_int]),
+}
+
+_lib = None
+
+
+class T5DError(RuntimeError):
+  pass
+
+
+def load():
+  """Loads libt5d.so once and declares every entry point's signature."""
+  global _lib
+  if _lib is not None:
+    return _lib
+  if not os.path.exists(LIB_PATH):
+    raise T5DError(
+        f'{LIB_PATH} is missing: build the HIP kernels first '
+        '(python -c "import __graft_entry__ as g; g.build()" or '
+        '`make -C t5x_amd/csrc`). There is no CPU fallback.')
+  lib = ctypes.CDLL(LIB_PATH)
+  for name, (restype, argtypes) in _SIGNATURES.items():
+    fn = getattr(lib, name)
+    fn.restype = restype
+    fn.argtypes = argtypes
+  _lib = lib
+  return lib
+
+
+def exported_names():
+  return sorted(_SIGNATURES)
+
+
+def last_error() -> str:
+  return load().t5d_last_error().decode('utf-8', 'replace')
+
+
+def call(name, *args):
+  """Calls entry point `name`; raises on a non-zero status."""
+  rc = getattr(load(), name)(*args)
+  if rc != 0:
+    msg = last_error()
+    if rc == -1:
+      raise ValueError(msg)
+    raise T5DError(f'{name} failed ({rc}): {msg}')
+
+
+def stream_handle():
+  import torch
+  return torch.cuda.current_stream().cuda_stream
+
+
+def ptr(t):
+  """Device pointer of a torch tensor (None -> NULL)."""
+  return None if t is None else t.data_ptr()
+
+
+def dtype_code(torch_dtype):
+  import torch
+  if torch_dtype == torch.float32:
+    return F32
+  if torch_dtype == torch.bfloat16:
+    return BF16
+  if torch_dtype == torch.int8:
+    return I8
+  raise ValueError(f'unsupported dtype {torch_dtype}')

@@ -1,0 +1,107 @@
+// Shared helpers for the t5d HIP kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/t5d.h"
+
+namespace t5d {
+
+// ---- error reporting --------------------------------------------------------
+void set_error(const char* fmt, ...);
+
+#define T5D_REQUIRE(cond, code, ...)      \
+  do {                                    \
+    if (!(cond)) {                        \
+      ::t5d::set_error(__VA_ARGS__);      \
+      return (code);                      \
+    }                                     \
+  } while (0)
+
+#define T5D_CHECK_LAUNCH(name)                                            \
+  do {                                                                    \
+    hipError_t e_ = hipGetLastError();                                    \
+    if (e_ != hipSuccess) {                                               \
+      ::t5d::set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return T5D_EHIP;                                                    \
+    }                                                                     \
+  } while (0)
+
+// ---- bfloat16 <-> float32 ---------------------------------------------------
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t packed) {
+  return __uint_as_float(packed << 16);
+}
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t packed) {
+  return __uint_as_float(packed & 0xFFFF0000u);
+}
+// Round to nearest even (inputs are finite on this path).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float round_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return __uint_as_float(u & 0xFFFF0000u);
+}
+
+// Activation-dtype traits: how a value is rounded / loaded / stored.
+template <typename T> struct Act;
+template <> struct Act<float> {
+  static constexpr int kElemsPer16B = 4;
+  __device__ static __forceinline__ float round(float v) { return v; }
+  __device__ static __forceinline__ float load(const float* p) { return *p; }
+  __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Act<bf16_t> {
+  static constexpr int kElemsPer16B = 8;
+  __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
+  __device__ static __forceinline__ float load(const bf16_t* p) {
+    return bf16_to_f32(*p);
+  }
+  __device__ static __forceinline__ void store(bf16_t* p, float v) {
+    *p = f32_to_bf16(v);
+  }
+};
+
+// Unpack a 16-byte vector of activations into floats.
+__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[8]) {
+  f[0] = bf16lo_to_f32(v.x); f[1] = bf16hi_to_f32(v.x);
+  f[2] = bf16lo_to_f32(v.y); f[3] = bf16hi_to_f32(v.y);
+  f[4] = bf16lo_to_f32(v.z); f[5] = bf16hi_to_f32(v.z);
+  f[6] = bf16lo_to_f32(v.w); f[7] = bf16hi_to_f32(v.w);
+}
+__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[4]) {
+  f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+  f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+
+// ---- wavefront (64 lanes) reductions ---------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// T5 tanh-approximate GELU in float32.
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;  // sqrt(2/pi)
+  return x * (0.5f * (1.0f + tanhf(c * (x + 0.044715f * (x * x * x)))));
+}
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+}  // namespace t5d

@@ -1,0 +1,480 @@
+// Weight-streaming dense layers for M <= 128 activation rows.
+//
+// At these row counts every GEMM of the decode step is bound by reading the
+// weight matrix once, so the kernels are organised around the weight stream:
+//   * bf16 / int8 weights are pre-packed into 32(k) x 16(n) MFMA B-operand
+//     tiles stored lane-major, so one wavefront load instruction fetches one
+//     whole tile as a single contiguous 1 KB (bf16) / 512 B (int8) burst
+//     straight into the registers v_mfma_f32_16x16x32_bf16 consumes;
+//   * a workgroup owns N_TILES adjacent 16-column tiles and all M rows; its 4
+//     wavefronts split the K range (k-tile kt goes to wave kt % 4) so that
+//     every byte of the workgroup's weight slice is requested exactly once and
+//     as early as possible, then the 4 partial accumulators are summed through
+//     LDS in a fixed order (bitwise deterministic);
+//   * small-N layers additionally split K across workgroups; partial tiles go
+//     to a float32 workspace and the last workgroup to arrive (per column
+//     group) sums them in split order and applies the epilogue.
+// The activation operand (<= 128 x K) is re-read by every workgroup from L2.
+#include "common.h"
+
+namespace t5d {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_v;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_v;
+
+union Frag {
+  uint4 u;
+  bf16x8_v v;
+};
+
+__device__ __forceinline__ uint32_t pack_i8x2_to_bf16x2(int a, int b) {
+  // int8 values are exactly representable in bfloat16.
+  uint32_t fa = __float_as_uint((float)a) >> 16;
+  uint32_t fb = __float_as_uint((float)b) & 0xFFFF0000u;
+  return fa | fb;
+}
+
+template <typename WT> struct WeightTile;
+template <> struct WeightTile<bf16_t> {
+  static constexpr int kTileBytes = 1024;
+  __device__ static __forceinline__ Frag load(const void* tile, int lane) {
+    Frag f;
+    f.u = reinterpret_cast<const uint4*>(tile)[lane];
+    return f;
+  }
+};
+template <> struct WeightTile<int8_t> {
+  static constexpr int kTileBytes = 512;
+  __device__ static __forceinline__ Frag load(const void* tile, int lane) {
+    uint2 q = reinterpret_cast<const uint2*>(tile)[lane];
+    Frag f;
+    f.u.x = pack_i8x2_to_bf16x2((int8_t)(q.x), (int8_t)(q.x >> 8));
+    f.u.y = pack_i8x2_to_bf16x2((int8_t)(q.x >> 16), (int8_t)(q.x >> 24));
+    f.u.z = pack_i8x2_to_bf16x2((int8_t)(q.y), (int8_t)(q.y >> 8));
+    f.u.w = pack_i8x2_to_bf16x2((int8_t)(q.y >> 16), (int8_t)(q.y >> 24));
+    return f;
+  }
+};
+
+struct GemmArgs {
+  const bf16_t* A;      // [M, K]
+  const void* W;        // packed tiles
+  const float* scales;  // [N] or null
+  const void* residual; // [M, Nout] act dtype or null
+  void* C;              // [M, Nout]
+  float* workspace;     // [split_k, M_pad, N] f32
+  int32_t* counters;    // [gridDim.x]
+  int M, K, N;          // N = number of weight columns
+  int epilogue;
+  int out_f32;
+};
+
+// Apply scale + epilogue to one finished column (pair) of row m.
+__device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
+                                             float v, float v_gate) {
+  if (g.epilogue == T5D_EPI_GEGLU) {
+    const int f = (n >> 4) * 8 + (n & 7);
+    const int F = g.N >> 1;
+    float a0 = round_bf16(v), a1 = round_bf16(v_gate);
+    float h = round_bf16(round_bf16(gelu_tanh(a0)) * a1);
+    reinterpret_cast<bf16_t*>(g.C)[(size_t)m * F + f] = f32_to_bf16(h);
+    return;
+  }
+  const size_t o = (size_t)m * g.N + n;
+  if (g.out_f32) {
+    reinterpret_cast<float*>(g.C)[o] = v;
+    return;
+  }
+  if (g.epilogue == T5D_EPI_RESIDUAL) {
+    float r = bf16_to_f32(reinterpret_cast<const bf16_t*>(g.residual)[o]);
+    v = round_bf16(v) + r;
+  }
+  reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(v);
+}
+
+template <int M_TILES, int N_TILES, typename WT>
+__global__ void __launch_bounds__(256)
+gemm_mfma_kernel(GemmArgs g) {
+  constexpr int ACC = M_TILES * N_TILES;
+  constexpr int TN = N_TILES * 16;
+  static_assert(ACC <= 16, "accumulator tile budget");
+  __shared__ float red[2][ACC * 4][64];
+  __shared__ int is_last;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int KT = g.K >> 5;
+  const int n_tiles_total = g.N >> 4;
+  const int nt0 = blockIdx.x * N_TILES;
+  const int split = gridDim.y;
+  const int kt_begin = (int)(((long)KT * blockIdx.y) / split);
+  const int kt_end = (int)(((long)KT * (blockIdx.y + 1)) / split);
+
+  f32x4_v acc[ACC];
+#pragma unroll
+  for (int i = 0; i < ACC; ++i) acc[i] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+
+  const int arow = lane & 15;
+  const int akoff = (lane >> 4) * 8;
+  const char* wbase = reinterpret_cast<const char*>(g.W);
+
+  for (int kt = kt_begin + wave; kt < kt_end; kt += 4) {
+    Frag b[N_TILES];
+#pragma unroll
+    for (int nn = 0; nn < N_TILES; ++nn) {
+      const int nt = nt0 + nn;
+      if (nt < n_tiles_total) {
+        b[nn] = WeightTile<WT>::load(
+            wbase + ((size_t)nt * KT + kt) * WeightTile<WT>::kTileBytes, lane);
+      } else {
+        b[nn].u = make_uint4(0, 0, 0, 0);
+      }
+    }
+    Frag a[M_TILES];
+#pragma unroll
+    for (int mt = 0; mt < M_TILES; ++mt) {
+      const int row = mt * 16 + arow;
+      if (row < g.M) {
+        a[mt].u = *reinterpret_cast<const uint4*>(g.A + (size_t)row * g.K +
+                                                  kt * 32 + akoff);
+      } else {
+        a[mt].u = make_uint4(0, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < M_TILES; ++mt)
+#pragma unroll
+      for (int nn = 0; nn < N_TILES; ++nn)
+        acc[mt * N_TILES + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            a[mt].v, b[nn].v, acc[mt * N_TILES + nn], 0, 0, 0);
+  }
+
+  // Cross-wave reduction in a fixed order: (w0 + w2) + (w1 + w3).
+  // Accumulator element i of tile (mt, nn) in lane l is
+  // C[16*mt + 4*(l/16) + i][16*nn + l%16].
+  if (wave >= 2) {
+#pragma unroll
+    for (int t = 0; t < ACC; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave - 2][t * 4 + i][lane] = acc[t][i];
+  }
+  __syncthreads();
+  if (wave < 2) {
+#pragma unroll
+    for (int t = 0; t < ACC; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[t][i] += red[wave][t * 4 + i][lane];
+  }
+  __syncthreads();
+  if (wave == 1) {
+#pragma unroll
+    for (int t = 0; t < ACC; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[0][t * 4 + i][lane] = acc[t][i];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < ACC; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        red[1][t * 4 + i][lane] = acc[t][i] + red[0][t * 4 + i][lane];
+  }
+  __syncthreads();
+
+  const int m_rows = M_TILES * 16;
+  const bool geglu = g.epilogue == T5D_EPI_GEGLU;
+
+  auto tile_sum = [&](int m, int nl) -> float {
+    const int mt = m >> 4, i = m & 3, c = (m & 15) >> 2;
+    const int nn = nl >> 4, l = c * 16 + (nl & 15);
+    return red[1][(mt * N_TILES + nn) * 4 + i][l];
+  };
+
+  if (split == 1) {
+    for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
+      const int m = e / TN, nl = e % TN;
+      const int n = nt0 * 16 + nl;
+      if (m >= g.M || n >= g.N) continue;
+      if (geglu && (nl & 8)) continue;
+      float v = tile_sum(m, nl);
+      float vg = geglu ? tile_sum(m, nl + 8) : 0.f;
+      if (g.scales) {
+        v *= g.scales[n];
+        if (geglu) vg *= g.scales[n + 8];
+      }
+      store_result(g, m, n, v, vg);
+    }
+    return;
+  }
+
+  // Split-K: publish this workgroup's partial tile, last arrival finishes.
+  const size_t ws_stride = (size_t)m_rows * g.N;
+  float* ws = g.workspace + (size_t)blockIdx.y * ws_stride;
+  for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
+    const int m = e / TN, nl = e % TN;
+    const int n = nt0 * 16 + nl;
+    if (n < g.N) ws[(size_t)m * g.N + n] = tile_sum(m, nl);
+  }
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int prev = atomicAdd(&g.counters[blockIdx.x], 1);
+    is_last = (prev == split - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
+    const int m = e / TN, nl = e % TN;
+    const int n = nt0 * 16 + nl;
+    if (m >= g.M || n >= g.N) continue;
+    if (geglu && (nl & 8)) continue;
+    float v = 0.f, vg = 0.f;
+    for (int s = 0; s < split; ++s) {
+      const float* p = g.workspace + (size_t)s * ws_stride + (size_t)m * g.N;
+      v += p[n];
+      if (geglu) vg += p[n + 8];
+    }
+    if (g.scales) {
+      v *= g.scales[n];
+      if (geglu) vg *= g.scales[n + 8];
+    }
+    store_result(g, m, n, v, vg);
+  }
+  if (threadIdx.x == 0) g.counters[blockIdx.x] = 0;
+}
+
+// ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
+// Lane = output column, the 4 wavefronts split K, MB rows per pass.
+template <int MB>
+__global__ void __launch_bounds__(256)
+gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
+                const float* __restrict__ residual, float* __restrict__ C,
+                int M, int K, int N, int epilogue) {
+  __shared__ float red[4][2 * MB][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool geglu = epilogue == T5D_EPI_GEGLU;
+  const int F = N >> 1;
+  const int ncols = geglu ? F : N;  // columns of work
+  const int n = blockIdx.x * 64 + lane;
+  const int m0 = blockIdx.y * MB;
+  const bool active = n < ncols;
+  float acc0[MB], acc1[MB];
+#pragma unroll
+  for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
+  const int kq = (K + 3) / 4;
+  const int kb = wave * kq, ke = min(K, kb + kq);
+  for (int k = kb; k < ke; ++k) {
+    const float w0 = active ? W[(size_t)k * N + n] : 0.f;
+    const float w1 = (active && geglu) ? W[(size_t)k * N + F + n] : 0.f;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const int row = m0 + m;
+      const float a = row < M ? A[(size_t)row * K + k] : 0.f;
+      acc0[m] = fmaf(a, w0, acc0[m]);
+      acc1[m] = fmaf(a, w1, acc1[m]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    red[wave][m][lane] = acc0[m];
+    red[wave][MB + m][lane] = acc1[m];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < MB * 64; e += 256) {
+    const int m = e >> 6, l = e & 63;
+    const int col = blockIdx.x * 64 + l;
+    const int row = m0 + m;
+    if (row >= M || col >= ncols) continue;
+    float v = (red[0][m][l] + red[1][m][l]) + (red[2][m][l] + red[3][m][l]);
+    if (geglu) {
+      float vg = (red[0][MB + m][l] + red[1][MB + m][l]) +
+                 (red[2][MB + m][l] + red[3][MB + m][l]);
+      C[(size_t)row * F + col] = gelu_tanh(v) * vg;
+    } else {
+      if (epilogue == T5D_EPI_RESIDUAL) v += residual[(size_t)row * N + col];
+      C[(size_t)row * N + col] = v;
+    }
+  }
+}
+
+// ---- weight packing -----------------------------------------------------------
+template <typename WT>
+__global__ void pack_weight_kernel(const WT* __restrict__ src,
+                                   const WT* __restrict__ src2,
+                                   WT* __restrict__ dst, int K, int N,
+                                   int geglu) {
+  // One thread per packed element; N here is the packed column count.
+  const int KT = K >> 5;
+  const size_t total = (size_t)K * N;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int j = idx & 7;
+  const int lane = (idx >> 3) & 63;
+  const size_t tile = idx >> 9;
+  const int kt = tile % KT;
+  const int nt = tile / KT;
+  const int k = kt * 32 + (lane >> 4) * 8 + j;
+  const int c = lane & 15;
+  WT v;
+  if (geglu) {
+    const int Nsrc = N >> 1;
+    const int f = nt * 8 + (c & 7);
+    v = (c < 8) ? src[(size_t)k * Nsrc + f] : src2[(size_t)k * Nsrc + f];
+  } else {
+    v = src[(size_t)k * N + nt * 16 + c];
+  }
+  dst[idx] = v;
+}
+
+struct GemmPlan {
+  int m_tiles, n_tiles, split_k;
+};
+
+static GemmPlan plan_gemm(int M, int K, int N) {
+  GemmPlan p;
+  p.m_tiles = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
+  const int nt = N / 16;
+  const int kt = K / 32;
+  // Wider column groups amortise the activation re-read; keep at least ~256
+  // workgroups so every CU has work.
+  int n_tiles = 16 / p.m_tiles;       // accumulator budget: m_tiles*n_tiles<=16
+  if (n_tiles > 4) n_tiles = 4;
+  while (n_tiles > 1 && nt / n_tiles < 256) n_tiles >>= 1;
+  p.n_tiles = n_tiles;
+  const int groups = (nt + n_tiles - 1) / n_tiles;
+  int split = 1;
+  while (groups * split < 192 && kt / (split * 2) >= 4 && split < 16) split *= 2;
+  p.split_k = split;
+  return p;
+}
+
+template <typename WT>
+static void launch_mfma(const GemmPlan& p, const GemmArgs& g, hipStream_t s) {
+  const int groups = (g.N / 16 + p.n_tiles - 1) / p.n_tiles;
+  dim3 grid(groups, p.split_k), block(256);
+#define T5D_GEMM_CASE(MT, NT)                                              \
+  if (p.m_tiles == MT && p.n_tiles == NT) {                                \
+    hipLaunchKernelGGL((gemm_mfma_kernel<MT, NT, WT>), grid, block, 0, s, g); \
+    return;                                                                \
+  }
+  T5D_GEMM_CASE(1, 1) T5D_GEMM_CASE(1, 2) T5D_GEMM_CASE(1, 4)
+  T5D_GEMM_CASE(2, 1) T5D_GEMM_CASE(2, 2) T5D_GEMM_CASE(2, 4)
+  T5D_GEMM_CASE(4, 1) T5D_GEMM_CASE(4, 2) T5D_GEMM_CASE(4, 4)
+  T5D_GEMM_CASE(8, 1) T5D_GEMM_CASE(8, 2)
+#undef T5D_GEMM_CASE
+}
+
+}  // namespace t5d
+
+using namespace t5d;
+
+extern "C" int64_t t5d_packed_weight_bytes(int w_dtype, int K, int N) {
+  if (K <= 0 || N <= 0 || K % 32 || N % 16) return -1;
+  if (w_dtype == T5D_BF16) return (int64_t)K * N * 2;
+  if (w_dtype == T5D_I8) return (int64_t)K * N;
+  return -1;
+}
+
+extern "C" int t5d_pack_weight(void* stream, int w_dtype, const void* src,
+                               const void* src2, void* dst, int K, int N,
+                               int geglu) {
+  T5D_REQUIRE(w_dtype == T5D_BF16 || w_dtype == T5D_I8, T5D_EINVAL,
+              "t5d_pack_weight: w_dtype %d", w_dtype);
+  T5D_REQUIRE(src && dst && (!geglu || src2), T5D_EINVAL,
+              "t5d_pack_weight: null pointer");
+  const int Np = geglu ? 2 * N : N;
+  T5D_REQUIRE(K > 0 && N > 0 && K % 32 == 0 && Np % 16 == 0 &&
+                  (!geglu || N % 8 == 0),
+              T5D_EINVAL, "t5d_pack_weight: K=%d N=%d must tile 32x16", K, N);
+  const size_t total = (size_t)K * Np;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((total + threads - 1) / threads);
+  if (w_dtype == T5D_BF16)
+    hipLaunchKernelGGL(pack_weight_kernel<bf16_t>, dim3(blocks), dim3(threads),
+                       0, as_stream(stream), (const bf16_t*)src,
+                       (const bf16_t*)src2, (bf16_t*)dst, K, Np, geglu);
+  else
+    hipLaunchKernelGGL(pack_weight_kernel<int8_t>, dim3(blocks), dim3(threads),
+                       0, as_stream(stream), (const int8_t*)src,
+                       (const int8_t*)src2, (int8_t*)dst, K, Np, geglu);
+  T5D_CHECK_LAUNCH("t5d_pack_weight");
+  return T5D_OK;
+}
+
+extern "C" int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M,
+                                            int K, int N) {
+  (void)w_dtype;
+  if (dtype != T5D_BF16 || M <= 0 || M > 128 || K % 32 || N % 16) return 0;
+  GemmPlan p = plan_gemm(M, K, N);
+  if (p.split_k == 1) return 0;
+  return (int64_t)p.split_k * p.m_tiles * 16 * N * 4;
+}
+
+extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
+                        const void* A, const void* W, const float* scales,
+                        const void* residual, void* C, int M, int K, int N,
+                        int epilogue, void* workspace, int32_t* counters) {
+  T5D_REQUIRE(A && W && C, T5D_EINVAL, "t5d_gemm: null pointer");
+  T5D_REQUIRE(M > 0 && K > 0 && N > 0, T5D_EINVAL, "t5d_gemm: M=%d K=%d N=%d",
+              M, K, N);
+  T5D_REQUIRE(epilogue >= T5D_EPI_NONE && epilogue <= T5D_EPI_GEGLU,
+              T5D_EINVAL, "t5d_gemm: epilogue %d", epilogue);
+  T5D_REQUIRE(epilogue != T5D_EPI_RESIDUAL || residual, T5D_EINVAL,
+              "t5d_gemm: residual epilogue without residual");
+  T5D_REQUIRE(epilogue != T5D_EPI_GEGLU || N % 2 == 0, T5D_EINVAL,
+              "t5d_gemm: geglu needs even N");
+  hipStream_t s = as_stream(stream);
+  if (dtype == T5D_F32) {
+    T5D_REQUIRE(w_dtype == T5D_F32 && out_dtype == T5D_F32, T5D_EINVAL,
+                "t5d_gemm: float32 activations need float32 weights/outputs");
+    const int ncols = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
+    if (M <= 8) {
+      dim3 grid((ncols + 63) / 64, 1);
+      hipLaunchKernelGGL(gemm_f32_kernel<8>, grid, dim3(256), 0, s,
+                         (const float*)A, (const float*)W,
+                         (const float*)residual, (float*)C, M, K, N, epilogue);
+    } else {
+      dim3 grid((ncols + 63) / 64, (M + 15) / 16);
+      hipLaunchKernelGGL(gemm_f32_kernel<16>, grid, dim3(256), 0, s,
+                         (const float*)A, (const float*)W,
+                         (const float*)residual, (float*)C, M, K, N, epilogue);
+    }
+    T5D_CHECK_LAUNCH("t5d_gemm(f32)");
+    return T5D_OK;
+  }
+  T5D_REQUIRE(dtype == T5D_BF16, T5D_EINVAL, "t5d_gemm: dtype %d", dtype);
+  T5D_REQUIRE(w_dtype == T5D_BF16 || w_dtype == T5D_I8, T5D_EINVAL,
+              "t5d_gemm: w_dtype %d", w_dtype);
+  T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
+              "t5d_gemm: int8 weights need scales");
+  T5D_REQUIRE(out_dtype == T5D_BF16 ||
+                  (out_dtype == T5D_F32 && epilogue == T5D_EPI_NONE),
+              T5D_EINVAL, "t5d_gemm: out_dtype %d with epilogue %d", out_dtype,
+              epilogue);
+  T5D_REQUIRE(M <= 128, T5D_ELIMIT, "t5d_gemm: M=%d > 128 rows", M);
+  T5D_REQUIRE(K % 32 == 0 && N % 16 == 0, T5D_EINVAL,
+              "t5d_gemm: K=%d N=%d must tile 32x16", K, N);
+  T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
+              "t5d_gemm: A/W must be 16-byte aligned");
+  GemmPlan p = plan_gemm(M, K, N);
+  T5D_REQUIRE(p.split_k == 1 || (workspace && counters), T5D_EINVAL,
+              "t5d_gemm: split-K plan needs workspace and counters");
+  GemmArgs g;
+  g.A = (const bf16_t*)A;
+  g.W = W;
+  g.scales = w_dtype == T5D_I8 ? scales : nullptr;
+  g.residual = residual;
+  g.C = C;
+  g.workspace = (float*)workspace;
+  g.counters = counters;
+  g.M = M; g.K = K; g.N = N;
+  g.epilogue = epilogue;
+  g.out_f32 = out_dtype == T5D_F32;
+  if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);
+  else launch_mfma<int8_t>(p, g, s);
+  T5D_CHECK_LAUNCH("t5d_gemm");
+  return T5D_OK;
+}

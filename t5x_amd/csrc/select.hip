@@ -1,0 +1,761 @@
+// Selection kernels of the decode loops: exact top-k, fused
+// log_softmax + prefix add + top-2K over beam x vocab, beam bookkeeping, the
+// loop condition, and the sampling step (greedy / top-k / top-p + Gumbel).
+//
+// All orderings are total: candidates compare by (value descending, index
+// ascending), which is lax.top_k's tie rule and jnp.argmax's first-occurrence
+// rule, so results do not depend on how the work is split over lanes.
+#include <math.h>
+
+#include "common.h"
+
+namespace t5d {
+
+constexpr float kNegInf = -1.0e7f;  // t5x/decoding.py:33
+
+struct Cand {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {
+  return va > vb || (va == vb && ia < ib);
+}
+
+__device__ __forceinline__ Cand wave_best(Cand c) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    float v = __shfl_xor(c.v, o, 64);
+    int i = __shfl_xor(c.i, o, 64);
+    if (better(v, i, c.v, c.i)) { c.v = v; c.i = i; }
+  }
+  return c;
+}
+
+// Best candidate of a workgroup (blockDim.x a multiple of 64, <= 1024).
+// `scratch` holds one Cand per wavefront.  Result is returned to all threads.
+__device__ __forceinline__ Cand block_best(Cand c, Cand* scratch) {
+  c = wave_best(c);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[wave] = c;
+  __syncthreads();
+  Cand r = scratch[0];
+  for (int w = 1; w < nw; ++w) {
+    Cand o = scratch[w];
+    if (better(o.v, o.i, r.v, r.i)) r = o;
+  }
+  return r;
+}
+
+__device__ __forceinline__ double block_sum_f64(double v, double* scratch) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  double r = 0.0;
+  for (int w = 0; w < nw; ++w) r += scratch[w];
+  return r;
+}
+
+__device__ __forceinline__ float block_max_f32(float v, float* scratch) {
+  v = wave_max(v);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float r = scratch[0];
+  for (int w = 1; w < nw; ++w) r = fmaxf(r, scratch[w]);
+  return r;
+}
+
+__device__ __forceinline__ int block_sum_i32(int v, int* scratch) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  int r = 0;
+  for (int w = 0; w < nw; ++w) r += scratch[w];
+  return r;
+}
+
+// ---- generic exact top-k -----------------------------------------------------
+// One workgroup per row; k rounds, each finds the best element strictly after
+// the previously selected one in the total order.
+__global__ void __launch_bounds__(256)
+top_k_kernel(const float* __restrict__ x, float* __restrict__ vals,
+             int32_t* __restrict__ idx, int n, int k) {
+  __shared__ Cand scratch[4];
+  const float* row = x + (size_t)blockIdx.x * n;
+  float pv = INFINITY;
+  int pi = -1;
+  for (int r = 0; r < k; ++r) {
+    Cand best = {-INFINITY, 0x7FFFFFFF};
+    for (int j = threadIdx.x; j < n; j += 256) {
+      const float v = row[j];
+      const bool after = better(pv, pi, v, j);  // (pv,pi) ranks before (v,j)
+      if (after && better(v, j, best.v, best.i)) { best.v = v; best.i = j; }
+    }
+    best = block_best(best, scratch);
+    if (threadIdx.x == 0) {
+      vals[(size_t)blockIdx.x * k + r] = best.v;
+      idx[(size_t)blockIdx.x * k + r] = best.i;
+    }
+    pv = best.v;
+    pi = best.i;
+  }
+}
+
+// ---- log_softmax + prefix add + per-row top-k --------------------------------
+// One workgroup per (batch, beam) row.  max and log-sum-exp first (the sum is
+// carried in double so the result does not depend on the reduction shape),
+// then every thread keeps the best KMAX of its strided share of
+//   f(j) = ((x[j] - max) - lse) + live_logprob
+// and the workgroup merges the lists by k rounds of arg-best.
+template <int KMAX>
+__global__ void __launch_bounds__(256)
+beam_row_topk_kernel(const float* __restrict__ logits,
+                     const float* __restrict__ live_logprobs,
+                     float* __restrict__ row_max, float* __restrict__ row_lse,
+                     float* __restrict__ cand_vals, int32_t* __restrict__ cand_idx,
+                     int V, int beams, int k) {
+  __shared__ Cand scratch[4];
+  __shared__ float fscratch[4];
+  __shared__ double dscratch[4];
+  const int r = blockIdx.x;
+  const float* x = logits + (size_t)r * V;
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < V; j += 256) m = fmaxf(m, x[j]);
+  m = block_max_f32(m, fscratch);
+  double sum = 0.0;
+  for (int j = threadIdx.x; j < V; j += 256) sum += (double)expf(x[j] - m);
+  sum = block_sum_f64(sum, dscratch);
+  const float lse = (float)log(sum);
+  const float lp = live_logprobs[r];
+  if (threadIdx.x == 0) {
+    row_max[r] = m;
+    row_lse[r] = lse;
+  }
+  const int base = (r % beams) * V;
+
+  float lv[KMAX];
+  int li[KMAX];
+#pragma unroll
+  for (int q = 0; q < KMAX; ++q) { lv[q] = -INFINITY; li[q] = 0x7FFFFFFF; }
+  for (int j = threadIdx.x; j < V; j += 256) {
+    const float f = ((x[j] - m) - lse) + lp;
+    const int fi = base + j;
+    if (better(f, fi, lv[KMAX - 1], li[KMAX - 1])) {
+      // insertion keeping the list sorted best-first
+      float cv = f;
+      int ci = fi;
+#pragma unroll
+      for (int q = 0; q < KMAX; ++q) {
+        if (better(cv, ci, lv[q], li[q])) {
+          const float tv = lv[q]; const int ti = li[q];
+          lv[q] = cv; li[q] = ci;
+          cv = tv; ci = ti;
+        }
+      }
+    }
+  }
+  for (int out = 0; out < k; ++out) {
+    Cand head = {lv[0], li[0]};
+    Cand best = block_best(head, scratch);
+    if (head.i == best.i && head.v == best.v && best.i != 0x7FFFFFFF) {
+      // pop (indices are unique, so exactly one thread matches)
+#pragma unroll
+      for (int q = 0; q + 1 < KMAX; ++q) { lv[q] = lv[q + 1]; li[q] = li[q + 1]; }
+      lv[KMAX - 1] = -INFINITY; li[KMAX - 1] = 0x7FFFFFFF;
+    }
+    if (threadIdx.x == 0) {
+      cand_vals[(size_t)r * k + out] = best.v;
+      cand_idx[(size_t)r * k + out] = best.i;
+    }
+  }
+}
+
+// Merge the beams' per-row candidates of one batch item: one wavefront, one
+// candidate per lane (beams*k <= 64), rank by counting better candidates.
+__global__ void __launch_bounds__(64)
+beam_merge_kernel(const float* __restrict__ cand_vals,
+                  const int32_t* __restrict__ cand_idx,
+                  float* __restrict__ topk_vals, int32_t* __restrict__ topk_idx,
+                  int beams, int k) {
+  const int b = blockIdx.x, lane = threadIdx.x;
+  const int n = beams * k;
+  float v = -INFINITY;
+  int i = 0x7FFFFFFF;
+  if (lane < n) {
+    v = cand_vals[(size_t)b * n + lane];
+    i = cand_idx[(size_t)b * n + lane];
+  }
+  int rank = 0;
+  for (int o = 0; o < 64; ++o) {
+    const float ov = __shfl(v, o, 64);
+    const int oi = __shfl(i, o, 64);
+    if (better(ov, oi, v, i)) ++rank;
+  }
+  if (lane < n && rank < k) {
+    topk_vals[(size_t)b * k + rank] = v;
+    topk_idx[(size_t)b * k + rank] = i;
+  }
+}
+
+// ---- beam bookkeeping -------------------------------------------------------
+constexpr int kMaxBeams = 8;
+
+struct BeamUpdateArgs {
+  t5d_beam_state cur, next;
+  const float* topk_vals;
+  const int32_t* topk_idx;
+  const int32_t* inputs;
+  const int32_t* initial_index;
+  const float* brevity;
+  int32_t* top_alive_indices;
+  int B, K, S, Lin, V, eos_id;
+};
+
+// Stable descending order of n values (ties keep index order).
+__device__ __forceinline__ void stable_order_desc(const float* v, int n,
+                                                  int* order) {
+  for (int a = 0; a < n; ++a) {
+    int rank = 0;
+    for (int c = 0; c < n; ++c)
+      if (better(v[c], c, v[a], a)) ++rank;
+    order[rank] = a;
+  }
+}
+
+__global__ void __launch_bounds__(64)
+beam_update_kernel(BeamUpdateArgs a) {
+  __shared__ int s_src_live[kMaxBeams];       // source live beam of new live e
+  __shared__ int s_tok_live[kMaxBeams];
+  __shared__ int s_fin_from[kMaxBeams];       // <K: old finished; else K+cand
+  __shared__ int s_cand_beam[2 * kMaxBeams];
+  __shared__ int s_cand_tok[2 * kMaxBeams];
+  const int b = blockIdx.x;
+  const int K = a.K, K2 = 2 * a.K, S = a.S;
+  const int cur = *a.cur.cur_index;
+
+  if (threadIdx.x == 0) {
+    float lp[2 * kMaxBeams], new_lp[2 * kMaxBeams];
+    float pool[3 * kMaxBeams];
+    int id[2 * kMaxBeams], beam[2 * kMaxBeams];
+    bool fin[2 * kMaxBeams];
+    int order[3 * kMaxBeams];
+    const int col = min(cur + 1, a.Lin - 1);
+    const int nxt = a.inputs[(size_t)b * a.Lin + col];
+    const bool oop = nxt == 0;
+    for (int c = 0; c < K2; ++c) {
+      const float raw = a.topk_vals[(size_t)b * K2 + c];
+      const int fi = a.topk_idx[(size_t)b * K2 + c];
+      beam[c] = fi / a.V;
+      id[c] = oop ? fi % a.V : nxt;
+      lp[c] = oop ? raw : (c == 0 ? 0.f : kNegInf);
+      fin[c] = id[c] == a.eos_id;
+      new_lp[c] = lp[c] + (fin[c] ? kNegInf : 0.f);
+      s_cand_beam[c] = beam[c];
+      s_cand_tok[c] = id[c];
+    }
+    // live beams: top K of the 2K, ascending (lax.top_k then flip)
+    stable_order_desc(new_lp, K2, order);
+    for (int e = 0; e < K; ++e) {
+      const int c = order[K - 1 - e];
+      a.next.live_logprobs[(size_t)b * K + e] = new_lp[c];
+      a.top_alive_indices[(size_t)b * K + e] = beam[c];
+      s_src_live[e] = beam[c];
+      s_tok_live[e] = id[c];
+    }
+    // finished pool: K old + 2K new, brevity-penalised
+    const int len = a.initial_index[b] + cur + 1;
+    const float bp = a.brevity[len];
+    for (int e = 0; e < K; ++e) pool[e] = a.cur.finished_scores[(size_t)b * K + e];
+    for (int c = 0; c < K2; ++c)
+      pool[K + c] = lp[c] / bp + (fin[c] ? 0.f : kNegInf);
+    stable_order_desc(pool, 3 * K, order);
+    for (int e = 0; e < K; ++e) {
+      const int src = order[K - 1 - e];
+      s_fin_from[e] = src;
+      a.next.finished_scores[(size_t)b * K + e] = pool[src];
+      a.next.finished_flags[(size_t)b * K + e] =
+          src < K ? a.cur.finished_flags[(size_t)b * K + src]
+                  : (uint8_t)fin[src - K];
+    }
+    if (b == 0) *a.next.cur_index = cur + 1;
+  }
+  __syncthreads();
+
+  const int32_t* live = a.cur.live_seqs + (size_t)b * K * S;
+  for (int e = 0; e < K; ++e) {
+    int32_t* dst = a.next.live_seqs + ((size_t)b * K + e) * S;
+    const int32_t* src = live + (size_t)s_src_live[e] * S;
+    for (int j = threadIdx.x; j < S; j += 64)
+      dst[j] = (j == cur + 1) ? s_tok_live[e] : src[j];
+    int32_t* fdst = a.next.finished_seqs + ((size_t)b * K + e) * S;
+    const int from = s_fin_from[e];
+    if (from < K) {
+      const int32_t* fsrc = a.cur.finished_seqs + ((size_t)b * K + from) * S;
+      for (int j = threadIdx.x; j < S; j += 64) fdst[j] = fsrc[j];
+    } else {
+      const int c = from - K;
+      const int32_t* fsrc = live + (size_t)s_cand_beam[c] * S;
+      const int tok = s_cand_tok[c];
+      for (int j = threadIdx.x; j < S; j += 64)
+        fdst[j] = (j == cur + 1) ? tok : fsrc[j];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+beam_cond_kernel(t5d_beam_state st, int B, int K, int S, float min_brevity,
+                 float min_log_prob, int max_decode_step, int min_initial_index,
+                 int32_t* keep_going) {
+  __shared__ int iscratch[4];
+  const int cur = *st.cur_index;
+  const float raw_min = min_log_prob / min_brevity;
+  int not_terminated = 0, passes_min = 0;
+  for (int b = threadIdx.x; b < B; b += 256) {
+    const float best_live = st.live_logprobs[(size_t)b * K + K - 1] / min_brevity;
+    float worst = INFINITY;
+    for (int e = 0; e < K; ++e)
+      worst = fminf(worst, st.finished_scores[(size_t)b * K + e]);
+    bool term = true;
+    for (int e = 0; e < K; ++e) {
+      const float w = st.finished_flags[(size_t)b * K + e] ? worst : kNegInf;
+      term = term && (w > best_live);
+    }
+    if (!term) ++not_terminated;
+    if (!(best_live < raw_min)) ++passes_min;
+  }
+  not_terminated = block_sum_i32(not_terminated, iscratch);
+  passes_min = block_sum_i32(passes_min, iscratch);
+  if (threadIdx.x == 0) {
+    const bool not_at_end = (cur + min_initial_index) < S - 1;
+    const bool exceed = (max_decode_step > 0) && (cur >= max_decode_step);
+    const bool search_terminated = not_terminated == 0;
+    const bool none_pass = (passes_min == 0) && (cur > 0);
+    *keep_going = (not_at_end && !search_terminated && !none_pass && !exceed) ? 1 : 0;
+  }
+}
+
+// ---- sampling -----------------------------------------------------------------
+__device__ __forceinline__ uint32_t order_key(float f) {
+  // Monotone map float -> uint32 (t5x/binary_search.py:74-101 does the same
+  // through int32).
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+  const uint32_t u = (k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k;
+  return __uint_as_float(u);
+}
+
+struct SampleArgs {
+  const float* logits;
+  const float* gumbel;
+  const float* temperature;
+  int32_t* tokens;
+  float* logprobs;
+  int V, topk, rescale;
+  float topp;
+};
+
+// One workgroup per row.
+__global__ void __launch_bounds__(256)
+sample_tokens_kernel(SampleArgs a) {
+  __shared__ Cand cscratch[4];
+  __shared__ float fscratch[4];
+  __shared__ double dscratch[4];
+  __shared__ int iscratch[4];
+  __shared__ unsigned hist[256];
+  const int r = blockIdx.x;
+  const int V = a.V;
+  const float* x = a.logits + (size_t)r * V;
+  const float T = a.temperature[r];
+  const float kMinT = 1e-4f;
+
+  if (!(T > kMinT)) {  // greedy (t5x/decoding.py:575-592)
+    Cand best = {-INFINITY, 0x7FFFFFFF};
+    for (int j = threadIdx.x; j < V; j += 256)
+      if (better(x[j], j, best.v, best.i)) { best.v = x[j]; best.i = j; }
+    best = block_best(best, cscratch);
+    float lp = 0.f;
+    if (!a.rescale) {
+      double sum = 0.0;
+      for (int j = threadIdx.x; j < V; j += 256) sum += (double)expf(x[j] - best.v);
+      sum = block_sum_f64(sum, dscratch);
+      lp = (best.v - best.v) - (float)log(sum);
+    }
+    if (threadIdx.x == 0) { a.tokens[r] = best.i; a.logprobs[r] = lp; }
+    return;
+  }
+
+  const float Tm = fmaxf(T, kMinT);
+  float cutoff = -INFINITY;  // keep scaled >= cutoff
+
+  if (a.topk > 0 && a.topk < V) {
+    // k-th largest of scaled logits by radix select on the order-preserving
+    // key, most significant byte first.
+    uint32_t prefix = 0, mask = 0;
+    int want = a.topk;  // rank (1-based, from the top) within the current set
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hist[threadIdx.x] = 0;
+      __syncthreads();
+      for (int j = threadIdx.x; j < V; j += 256) {
+        const uint32_t key = order_key(x[j] / Tm);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xFF], 1u);
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        int digit = 255, acc = 0;
+        for (; digit > 0; --digit) {
+          if (acc + (int)hist[digit] >= want) break;
+          acc += hist[digit];
+        }
+        iscratch[0] = digit;
+        iscratch[1] = want - acc;
+      }
+      __syncthreads();
+      prefix |= ((uint32_t)iscratch[0]) << shift;
+      mask |= 0xFFu << shift;
+      want = iscratch[1];
+      __syncthreads();
+    }
+    cutoff = key_to_float(prefix);
+  }
+
+  float pcut = -INFINITY;  // top-p: keep prob >= pcut
+  float smax = 0.f, ssum = 1.f;
+  if (a.topp > 0.f) {
+    // t5x/binary_search.py:230-299 — largest threshold whose kept mass >= p,
+    // found by the same 32-step search over float bit patterns.
+    float m = -INFINITY;
+    for (int j = threadIdx.x; j < V; j += 256) {
+      float y = x[j] / Tm;
+      y = (y >= cutoff) ? y : kNegInf;
+      m = fmaxf(m, y);
+    }
+    m = block_max_f32(m, fscratch);
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < V; j += 256) {
+      float y = x[j] / Tm;
+      y = (y >= cutoff) ? y : kNegInf;
+      sum += (double)expf(y - m);
+    }
+    sum = block_sum_f64(sum, dscratch);
+    smax = m;
+    ssum = (float)sum;
+    int32_t bits = 0;
+    for (int it = 0; it < 32; ++it) {
+      int32_t mid = it == 0 ? bits : (bits | (int32_t)(1u << (31 - it)));
+      int32_t pat = mid ^ (mid < 0 ? 0x7FFFFFFF : 0);
+      const bool finite = (pat & 0x7F800000) != 0x7F800000;
+      bool pred;
+      if (finite) {
+        const float thr = __int_as_float(pat);
+        double mass = 0.0;
+        for (int j = threadIdx.x; j < V; j += 256) {
+          float y = x[j] / Tm;
+          y = (y >= cutoff) ? y : kNegInf;
+          const float pr = expf(y - smax) / ssum;
+          if (pr >= thr) mass += (double)pr;
+        }
+        mass = block_sum_f64(mass, dscratch);
+        pred = (float)mass < a.topp;
+      } else {
+        pred = pat >= 0;
+      }
+      if (it == 0) {
+        if (pred) bits |= (int32_t)0x80000000u;
+      } else if (!pred) {
+        bits |= (int32_t)(1u << (31 - it));
+      }
+    }
+    const int32_t pat = bits ^ (bits < 0 ? 0x7FFFFFFF : 0);
+    pcut = __int_as_float(pat);
+  }
+
+  // argmax(masked + gumbel), and log-softmax statistics of the masked row.
+  Cand best = {-INFINITY, 0x7FFFFFFF};
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < V; j += 256) {
+    float y = x[j] / Tm;
+    y = (y >= cutoff) ? y : kNegInf;
+    if (a.topp > 0.f) {
+      const float pr = expf(y - smax) / ssum;
+      y = (pr >= pcut) ? y : kNegInf;
+    }
+    const float z = y + a.gumbel[(size_t)r * V + j];
+    if (better(z, j, best.v, best.i)) { best.v = z; best.i = j; }
+    m = fmaxf(m, a.rescale ? y : x[j]);
+  }
+  best = block_best(best, cscratch);
+  m = block_max_f32(m, fscratch);
+  double sum = 0.0;
+  float ytok = 0.f;
+  for (int j = threadIdx.x; j < V; j += 256) {
+    float y = x[j] / Tm;
+    y = (y >= cutoff) ? y : kNegInf;
+    if (a.topp > 0.f) {
+      const float pr = expf(y - smax) / ssum;
+      y = (pr >= pcut) ? y : kNegInf;
+    }
+    const float w = a.rescale ? y : x[j];
+    sum += (double)expf(w - m);
+    if (j == best.i) ytok = w;
+  }
+  sum = block_sum_f64(sum, dscratch);
+  // ytok lives in exactly one thread; broadcast through the float scratch.
+  __syncthreads();
+  if ((best.i & 255) == (int)threadIdx.x) fscratch[0] = ytok;
+  __syncthreads();
+  ytok = fscratch[0];
+  if (threadIdx.x == 0) {
+    a.tokens[r] = best.i;
+    a.logprobs[r] = (ytok - m) - (float)log(sum);
+  }
+}
+
+struct SampleUpdateArgs {
+  const int32_t* tokens;
+  const float* token_logprobs;
+  int32_t* sequences;
+  int32_t* cur_index;
+  int32_t* cur_token;
+  uint8_t* ended;
+  float* log_prob;
+  const int32_t* max_decode_len;
+  const int32_t* initial_eos_count;
+  int32_t* all_ended;
+  int R, S, eos_id;
+};
+
+__global__ void __launch_bounds__(256)
+sample_update_kernel(SampleUpdateArgs a) {
+  __shared__ int iscratch[4];
+  int not_ended = 0;
+  for (int r = threadIdx.x; r < a.R; r += 256) {
+    int32_t* seq = a.sequences + (size_t)r * a.S;
+    const int mdl = a.max_decode_len[r];
+    const int i = min(a.cur_index[r], mdl);
+    const int next_input = seq[i + 1];
+    const bool oop = next_input == 0;
+    const bool was_ended = a.ended[r] != 0;
+    const int tok = oop ? a.tokens[r] : next_input;
+    if (oop && !was_ended) a.log_prob[r] = a.log_prob[r] + a.token_logprobs[r];
+    const int out_tok = was_ended ? 0 : tok;
+    seq[i + 1] = out_tok;
+    int eos = 0;
+    for (int j = 0; j < a.S; ++j) eos += (seq[j] == a.eos_id);
+    const bool ended = was_ended || (eos > a.initial_eos_count[r]) ||
+                       (i >= mdl - 1);
+    a.ended[r] = ended ? 1 : 0;
+    a.cur_index[r] = i + 1;
+    a.cur_token[r] = out_tok;
+    if (!ended) ++not_ended;
+  }
+  not_ended = block_sum_i32(not_ended, iscratch);
+  if (threadIdx.x == 0) *a.all_ended = not_ended == 0 ? 1 : 0;
+}
+
+// ---- generic beam-axis gather (out of place) -----------------------------------
+__global__ void gather_beams_kernel(const char* __restrict__ src,
+                                    char* __restrict__ dst,
+                                    const int32_t* __restrict__ idx,
+                                    int old_beams, int new_beams,
+                                    size_t inner_bytes) {
+  const int be = blockIdx.x;  // b * new_beams + e
+  const int b = be / new_beams;
+  int s = idx[be];
+  s = s < 0 ? 0 : (s >= old_beams ? old_beams - 1 : s);
+  const char* p = src + ((size_t)b * old_beams + s) * inner_bytes;
+  char* q = dst + (size_t)be * inner_bytes;
+  if ((inner_bytes % 16) == 0 && (((uintptr_t)p | (uintptr_t)q) % 16) == 0) {
+    const size_t n = inner_bytes / 16;
+    for (size_t i = (size_t)blockIdx.y * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.y * blockDim.x)
+      reinterpret_cast<uint4*>(q)[i] = reinterpret_cast<const uint4*>(p)[i];
+  } else {
+    for (size_t i = (size_t)blockIdx.y * blockDim.x + threadIdx.x;
+         i < inner_bytes; i += (size_t)gridDim.y * blockDim.x)
+      q[i] = p[i];
+  }
+}
+
+}  // namespace t5d
+
+using namespace t5d;
+
+extern "C" int t5d_top_k(void* stream, const float* x, float* vals,
+                         int32_t* idx, int rows, int n, int k) {
+  T5D_REQUIRE(x && vals && idx, T5D_EINVAL, "t5d_top_k: null pointer");
+  T5D_REQUIRE(rows > 0 && n > 0 && k > 0 && k <= n, T5D_EINVAL,
+              "t5d_top_k: rows=%d n=%d k=%d", rows, n, k);
+  T5D_REQUIRE(k <= 64, T5D_ELIMIT, "t5d_top_k: k=%d > 64", k);
+  hipLaunchKernelGGL(top_k_kernel, dim3(rows), dim3(256), 0, as_stream(stream),
+                     x, vals, idx, n, k);
+  T5D_CHECK_LAUNCH("t5d_top_k");
+  return T5D_OK;
+}
+
+extern "C" int t5d_beam_topk(void* stream, const float* logits,
+                             const float* live_logprobs, float* topk_vals,
+                             int32_t* topk_idx, float* row_max, float* row_lse,
+                             void* scratch, int B, int beams, int V, int k) {
+  T5D_REQUIRE(logits && live_logprobs && topk_vals && topk_idx && row_max &&
+                  row_lse && scratch,
+              T5D_EINVAL, "t5d_beam_topk: null pointer");
+  T5D_REQUIRE(B > 0 && beams > 0 && V > 0 && k > 0, T5D_EINVAL,
+              "t5d_beam_topk: B=%d beams=%d V=%d k=%d", B, beams, V, k);
+  T5D_REQUIRE(k <= 16 && beams * k <= 64, T5D_ELIMIT,
+              "t5d_beam_topk: k=%d beams=%d (need k<=16, beams*k<=64)", k,
+              beams);
+  T5D_REQUIRE((long)beams * V < 0x7FFFFFFFL && k <= beams * V, T5D_EINVAL,
+              "t5d_beam_topk: beams*V out of range");
+  const int R = B * beams;
+  float* cand_vals = (float*)scratch;
+  int32_t* cand_idx = (int32_t*)((char*)scratch + (size_t)R * k * 4);
+  hipStream_t s = as_stream(stream);
+  if (k <= 4)
+    hipLaunchKernelGGL(beam_row_topk_kernel<4>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k);
+  else if (k <= 8)
+    hipLaunchKernelGGL(beam_row_topk_kernel<8>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k);
+  else
+    hipLaunchKernelGGL(beam_row_topk_kernel<16>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k);
+  T5D_CHECK_LAUNCH("t5d_beam_topk(rows)");
+  hipLaunchKernelGGL(beam_merge_kernel, dim3(B), dim3(64), 0, s, cand_vals,
+                     cand_idx, topk_vals, topk_idx, beams, k);
+  T5D_CHECK_LAUNCH("t5d_beam_topk(merge)");
+  return T5D_OK;
+}
+
+static int check_state(const char* name, const t5d_beam_state* st) {
+  T5D_REQUIRE(st && st->cur_index && st->live_logprobs && st->finished_scores &&
+                  st->live_seqs && st->finished_seqs && st->finished_flags,
+              T5D_EINVAL, "%s: null beam state pointer", name);
+  return T5D_OK;
+}
+
+extern "C" int t5d_beam_update(void* stream, const t5d_beam_state* cur,
+                               const t5d_beam_state* next,
+                               const float* topk_vals, const int32_t* topk_idx,
+                               const int32_t* inputs,
+                               const int32_t* initial_index,
+                               const float* brevity,
+                               int32_t* top_alive_indices, int B, int K, int S,
+                               int Lin, int V, int eos_id) {
+  int rc = check_state("t5d_beam_update", cur);
+  if (rc) return rc;
+  rc = check_state("t5d_beam_update", next);
+  if (rc) return rc;
+  T5D_REQUIRE(topk_vals && topk_idx && inputs && initial_index && brevity &&
+                  top_alive_indices,
+              T5D_EINVAL, "t5d_beam_update: null pointer");
+  T5D_REQUIRE(B > 0 && K > 0 && S > 1 && Lin > 0 && V > 0, T5D_EINVAL,
+              "t5d_beam_update: B=%d K=%d S=%d Lin=%d V=%d", B, K, S, Lin, V);
+  T5D_REQUIRE(K <= kMaxBeams, T5D_ELIMIT, "t5d_beam_update: K=%d > %d", K,
+              kMaxBeams);
+  T5D_REQUIRE(cur->live_seqs != next->live_seqs &&
+                  cur->finished_seqs != next->finished_seqs,
+              T5D_EINVAL, "t5d_beam_update: cur and next must be distinct");
+  BeamUpdateArgs a;
+  a.cur = *cur; a.next = *next;
+  a.topk_vals = topk_vals; a.topk_idx = topk_idx; a.inputs = inputs;
+  a.initial_index = initial_index; a.brevity = brevity;
+  a.top_alive_indices = top_alive_indices;
+  a.B = B; a.K = K; a.S = S; a.Lin = Lin; a.V = V; a.eos_id = eos_id;
+  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0,
+                     as_stream(stream), a);
+  T5D_CHECK_LAUNCH("t5d_beam_update");
+  return T5D_OK;
+}
+
+extern "C" int t5d_beam_cond(void* stream, const t5d_beam_state* state, int B,
+                             int K, int S, float min_brevity,
+                             float min_log_prob, int max_decode_step,
+                             int min_initial_index, int32_t* keep_going) {
+  int rc = check_state("t5d_beam_cond", state);
+  if (rc) return rc;
+  T5D_REQUIRE(keep_going && B > 0 && K > 0 && S > 1, T5D_EINVAL,
+              "t5d_beam_cond: B=%d K=%d S=%d", B, K, S);
+  hipLaunchKernelGGL(beam_cond_kernel, dim3(1), dim3(256), 0,
+                     as_stream(stream), *state, B, K, S, min_brevity,
+                     min_log_prob, max_decode_step, min_initial_index,
+                     keep_going);
+  T5D_CHECK_LAUNCH("t5d_beam_cond");
+  return T5D_OK;
+}
+
+extern "C" int t5d_sample_tokens(void* stream, const float* logits,
+                                 const float* gumbel, const float* temperature,
+                                 int32_t* tokens, float* logprobs, int R,
+                                 int V, int topk, float topp, int rescale) {
+  T5D_REQUIRE(logits && temperature && tokens && logprobs, T5D_EINVAL,
+              "t5d_sample_tokens: null pointer");
+  T5D_REQUIRE(R > 0 && V > 0 && topk >= 0 && topp >= 0.f, T5D_EINVAL,
+              "t5d_sample_tokens: R=%d V=%d topk=%d topp=%f", R, V, topk,
+              (double)topp);
+  T5D_REQUIRE(!(topk > 0 && topp > 0.f), T5D_EINVAL,
+              "At most one of `topp` or `topk` may be non-zero.");
+  SampleArgs a;
+  a.logits = logits; a.gumbel = gumbel; a.temperature = temperature;
+  a.tokens = tokens; a.logprobs = logprobs;
+  a.V = V; a.topk = topk; a.rescale = rescale; a.topp = topp;
+  hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0,
+                     as_stream(stream), a);
+  T5D_CHECK_LAUNCH("t5d_sample_tokens");
+  return T5D_OK;
+}
+
+extern "C" int t5d_sample_update(void* stream, const int32_t* tokens,
+                                 const float* token_logprobs,
+                                 int32_t* sequences, int32_t* cur_index,
+                                 int32_t* cur_token, uint8_t* ended,
+                                 float* log_prob, const int32_t* max_decode_len,
+                                 const int32_t* initial_eos_count,
+                                 int32_t* all_ended, int R, int S, int eos_id) {
+  T5D_REQUIRE(tokens && token_logprobs && sequences && cur_index && cur_token &&
+                  ended && log_prob && max_decode_len && initial_eos_count &&
+                  all_ended,
+              T5D_EINVAL, "t5d_sample_update: null pointer");
+  T5D_REQUIRE(R > 0 && S > 2, T5D_EINVAL, "t5d_sample_update: R=%d S=%d", R, S);
+  SampleUpdateArgs a;
+  a.tokens = tokens; a.token_logprobs = token_logprobs; a.sequences = sequences;
+  a.cur_index = cur_index; a.cur_token = cur_token; a.ended = ended;
+  a.log_prob = log_prob; a.max_decode_len = max_decode_len;
+  a.initial_eos_count = initial_eos_count; a.all_ended = all_ended;
+  a.R = R; a.S = S; a.eos_id = eos_id;
+  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(256), 0,
+                     as_stream(stream), a);
+  T5D_CHECK_LAUNCH("t5d_sample_update");
+  return T5D_OK;
+}
+
+extern "C" int t5d_gather_beams(void* stream, const void* src, void* dst,
+                                const int32_t* beam_indices, int B,
+                                int old_beams, int new_beams,
+                                int64_t inner_bytes) {
+  T5D_REQUIRE(src && dst && beam_indices && src != dst, T5D_EINVAL,
+              "t5d_gather_beams: null or aliased pointer");
+  T5D_REQUIRE(B > 0 && old_beams > 0 && new_beams > 0 && inner_bytes > 0,
+              T5D_EINVAL, "t5d_gather_beams: B=%d old=%d new=%d inner=%ld", B,
+              old_beams, new_beams, (long)inner_bytes);
+  int gy = (int)((inner_bytes / 16 + 255) / 256);
+  gy = gy < 1 ? 1 : (gy > 64 ? 64 : gy);
+  hipLaunchKernelGGL(gather_beams_kernel, dim3(B * new_beams, gy), dim3(256), 0,
+                     as_stream(stream), (const char*)src, (char*)dst,
+                     beam_indices, old_beams, new_beams, (size_t)inner_bytes);
+  T5D_CHECK_LAUNCH("t5d_gather_beams");
+  return T5D_OK;
+}

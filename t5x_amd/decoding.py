@@ -1,0 +1,585 @@
+"""Decode loops with the reference's call signatures, driven from Python over
+the HIP kernels (t5x/decoding.py is the interface being mirrored; line numbers
+below refer to it).
+
+Arrays are torch tensors on the GPU.  `tokens_to_logits` is any callable
+`DecodingState -> (logits [rows, vocab], new_cache)`; NumPy results are
+uploaded.  The per-step selection work — log_softmax, prefix add, top-2K over
+beam x vocab, beam bookkeeping, cache reorder, sampling — runs in the kernels
+declared in include/t5d.h; torch is used for allocation, views and the handful
+of tiny prologue/epilogue array edits outside the step loop.
+
+Contract differences from the functional reference, both invisible to a
+caller that follows the protocol:
+  * caches are updated IN PLACE: `tokens_to_logits` may mutate and return the
+    cache it was given, and `cache_gather_beams` permutes beam slices in place;
+  * `decode_rng` is an integer seed, a torch.Generator, or an object with a
+    `noise(step, shape)` method returning that step's Gumbel tensor
+    (jax.random.categorical(key, x) == argmax(x + gumbel)).
+"""
+
+import dataclasses
+import functools
+from typing import Any, Callable, Mapping, Optional, Tuple, Union
+
+import numpy as np
+import torch
+
+from t5x_amd import ops
+
+NEG_INF = np.array(-1.0e7)  # :33
+NEG_INF_VALUE = -1.0e7
+MIN_TEMPERATURE = np.array(1e-4)  # :39
+
+
+def _device():
+  if not torch.cuda.is_available():
+    raise RuntimeError('t5x_amd.decoding needs a GPU: the decode loops run on '
+                       'HIP kernels and have no CPU fallback')
+  return torch.device('cuda')
+
+
+def _dev(x, dtype=None):
+  """Uploads array-likes; passes GPU tensors through."""
+  if isinstance(x, torch.Tensor):
+    t = x if x.is_cuda else x.to(_device())
+  else:
+    t = torch.as_tensor(np.asarray(x), device=_device())
+  if dtype is not None and t.dtype != dtype:
+    t = t.to(dtype)
+  return t
+
+
+@dataclasses.dataclass
+class DecodingState:
+  """:42-66."""
+  cur_index: torch.Tensor
+  sequences: torch.Tensor
+  cur_token: torch.Tensor
+  cache: Mapping[str, Any]
+
+
+@dataclasses.dataclass
+class SamplingLoopState:
+  """:74-99."""
+  step: torch.Tensor
+  cur_index: torch.Tensor
+  sequences: torch.Tensor
+  cache: Mapping[str, Any]
+  cur_token: torch.Tensor
+  ended: torch.Tensor
+  rng: Any
+  log_prob: torch.Tensor
+
+  def replace(self, **kw):
+    return dataclasses.replace(self, **kw)
+
+
+# ------------------------------------------------------------------------------
+# cache / beam helpers (:739-915)
+# ------------------------------------------------------------------------------
+
+
+def _flatten_dict(d, prefix=()):
+  out = {}
+  for k, v in d.items():
+    if isinstance(v, Mapping) and v:
+      out.update(_flatten_dict(v, prefix + (k,)))
+    else:
+      out[prefix + (k,)] = v
+  return out
+
+
+def _unflatten_dict(flat):
+  out = {}
+  for path, v in flat.items():
+    cur = out
+    for k in path[:-1]:
+      cur = cur.setdefault(k, {})
+    cur[path[-1]] = v
+  return out
+
+
+_NEVER_MAPPED = ('cached_bias', 'position_embedder_index')
+
+
+def cache_map(fn, cache, apply_to_index: bool = False):
+  """:739-770 — `cache_index` leaves are skipped unless apply_to_index; leaves
+  named cached_bias / position_embedder_index always are."""
+  flat_cache = _flatten_dict(cache)
+  keyvals = {
+      k: v for k, v in flat_cache.items()
+      if (apply_to_index or k[-1] != 'cache_index') and
+      k[-1] not in _NEVER_MAPPED
+  }
+  flat_cache.update({k: fn(v) for k, v in keyvals.items()})
+  return _unflatten_dict(flat_cache)
+
+
+def add_beam_dim(x, beam_size: int, offset: int = 0):
+  """:773-780."""
+  x = _dev(x).unsqueeze(offset + 1)
+  reps = [1] * x.dim()
+  reps[offset + 1] = beam_size
+  return x.repeat(*reps)
+
+
+def flatten_beam_dim(x, offset: int = 0):
+  """:783-788."""
+  x = _dev(x)
+  shape = list(x.shape)
+  b = shape.pop(offset)
+  shape[offset] *= b
+  return x.reshape(shape)
+
+
+def unflatten_beam_dim(x, batch_size: int, beam_size: int, offset: int = 0):
+  """:791-798."""
+  x = _dev(x)
+  assert batch_size * beam_size == x.shape[offset]
+  shape = list(x.shape)
+  return x.reshape(shape[:offset] + [batch_size, beam_size] +
+                   shape[offset + 1:])
+
+
+def flat_batch_beam_expand(x, beam_size: int, offset: int = 0):
+  """:801-805."""
+  return flatten_beam_dim(add_beam_dim(x, beam_size, offset), offset)
+
+
+def _gather_leaf(x, beam_indices):
+  x = _dev(x)
+  if x.dtype == torch.bool:
+    return ops.gather_beams(x.to(torch.uint8).contiguous(),
+                            beam_indices).to(torch.bool)
+  return ops.gather_beams(x.contiguous(), beam_indices)
+
+
+def gather_beams(nested, beam_indices, batch_size, old_beam_size,
+                 new_beam_size, one_hot: bool = True):
+  """:873-915 (the one-hot contraction is an exact row pick)."""
+  del batch_size, old_beam_size, new_beam_size, one_hot
+  beam_indices = _dev(beam_indices, torch.int32).contiguous()
+
+  def walk(node):
+    if isinstance(node, (list, tuple)):
+      return type(node)(walk(n) for n in node)
+    if isinstance(node, Mapping):
+      return {k: walk(v) for k, v in node.items()}
+    return _gather_leaf(node, beam_indices)
+
+  return walk(nested)
+
+
+def cache_gather_beams(nested, beam_indices, batch_size, old_beam_size,
+                       new_beam_size, one_hot: bool = True, offset: int = 0,
+                       valid_len: Optional[torch.Tensor] = None):
+  """:808-870.  Same-size gathers of [B, beams, ..., L] leaves whose rows are
+  16-byte multiples are done in place (valid prefix only when `valid_len`, a
+  device int32 scalar, is given); anything else goes out of place."""
+  del batch_size, one_hot
+  assert offset in (0, 1), 'general offsets not supported'
+  beam_indices = _dev(beam_indices, torch.int32).contiguous()
+
+  def gather_fn(x):
+    x = _dev(x)
+    in_place = (old_beam_size == new_beam_size and x.dim() >= 3 + offset and
+                x.is_contiguous() and x.element_size() in (2, 4) and
+                (x.shape[-1] * x.element_size()) % 16 == 0 and
+                new_beam_size <= 8 and x.data_ptr() % 16 == 0)
+    if offset == 0:
+      if in_place:
+        return ops.cache_gather_beams(x, beam_indices, valid_len=valid_len)
+      return _gather_leaf(x, beam_indices)
+    if in_place:
+      per_layer = x[0].numel() * x.element_size()
+      ops.cache_gather_beams(x[0], beam_indices, valid_len=valid_len,
+                             n_tensors=x.shape[0],
+                             tensor_stride_bytes=per_layer)
+      return x
+    return torch.stack([_gather_leaf(x[l], beam_indices)
+                        for l in range(x.shape[0])])
+
+  return cache_map(gather_fn, nested)
+
+
+def top_k_two_stage(x, k):
+  """:918-966.  The reference's two-stage form is a TPU layout optimisation
+  whose result equals lax.top_k; one exact kernel serves both."""
+  return ops.top_k(_dev(x, torch.float32).contiguous(), k)
+
+
+def gather_topk_beams(nested, score_or_log_prob, batch_size, new_beam_size):
+  """:969-996."""
+  _, topk_indices = ops.top_k(
+      _dev(score_or_log_prob, torch.float32).contiguous(), new_beam_size)
+  topk_indices = torch.flip(topk_indices, dims=[1]).contiguous()
+  return gather_beams(nested, topk_indices, batch_size,
+                      score_or_log_prob.shape[1], new_beam_size)
+
+
+def brevity_penalty(alpha: float, length):
+  """:723-733, float32.  A Python int keeps the base in double until the
+  power; an int32 array promotes to float32 first."""
+  if isinstance(length, (int, np.integer)):
+    base = np.float32((5.0 + float(length)) / 6.0)
+  else:
+    if isinstance(length, torch.Tensor):
+      length = length.cpu().numpy()
+    base = ((np.float32(5.0) + np.asarray(length).astype(np.float32)) /
+            np.float32(6.0))
+  return np.power(base, np.float32(alpha), dtype=np.float32)
+
+
+# ------------------------------------------------------------------------------
+# Sampling noise
+# ------------------------------------------------------------------------------
+
+
+class _Key:
+  """Stand-in for a PRNG key: which loop step's noise to draw."""
+
+  def __init__(self, source, step):
+    self.source, self.step = source, step
+
+
+class _SeededNoise:
+  """Gumbel noise from a torch generator (seeded per step)."""
+
+  def __init__(self, seed):
+    self.seed = int(seed)
+
+  def noise(self, step, shape):
+    gen = torch.Generator(device=_device())
+    gen.manual_seed(self.seed * 1000003 + int(step))
+    u = torch.rand(shape, generator=gen, device=_device(),
+                   dtype=torch.float32)
+    tiny = float(np.finfo(np.float32).tiny)
+    return -torch.log(-torch.log(u.clamp_min(tiny)))
+
+
+def _noise_source(decode_rng):
+  if decode_rng is None:
+    return _SeededNoise(0)  # :345-346
+  if hasattr(decode_rng, 'noise'):
+    return decode_rng
+  if isinstance(decode_rng, torch.Generator):
+    return _SeededNoise(decode_rng.initial_seed())
+  return _SeededNoise(int(np.asarray(decode_rng).reshape(-1)[-1]))
+
+
+# ------------------------------------------------------------------------------
+# Temperature sampling (:115-715)
+# ------------------------------------------------------------------------------
+
+
+def temperature_sample(
+    inputs, cache, tokens_to_logits, eos_id: int, decode_rng=None,
+    num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
+    topk: int = 1, topp: float = 0.0, cache_offset: int = 0,
+    initial_index=None, max_decode_steps=None,
+    max_decode_steps_hard_limit: Optional[int] = None,
+    rescale_log_probs: bool = True,
+    state_callback_fn: Optional[Callable] = None,
+    logit_callback_fn: Optional[Callable] = None,
+):
+  """:115-409 -> (decodes [B, num_decodes, L] i32, log_prob [B, num_decodes])
+  sorted ascending by log-prob."""
+  if (max_decode_steps_hard_limit is not None and
+      max_decode_steps_hard_limit > 0 and max_decode_steps is not None):
+    max_decode_steps = np.minimum(max_decode_steps,
+                                  max_decode_steps_hard_limit)
+  inputs = _dev(inputs, torch.int32)
+  if num_decodes > 1:
+    expanded_inputs = flat_batch_beam_expand(inputs, num_decodes)
+    expanded_cache = cache_map(
+        functools.partial(flat_batch_beam_expand, beam_size=num_decodes,
+                          offset=cache_offset),
+        cache, apply_to_index=initial_index is not None)
+    if initial_index is not None:
+      initial_index = flat_batch_beam_expand(
+          _dev(initial_index, torch.int32), num_decodes)
+  else:
+    expanded_inputs, expanded_cache = inputs, cache
+
+  expanded_decodes, expanded_log_prob = _temperature_sample_single_trial(
+      expanded_inputs, expanded_cache, tokens_to_logits, eos_id, decode_rng,
+      num_decodes, temperature, topk, topp, initial_index=initial_index,
+      max_decode_steps=max_decode_steps, rescale_log_probs=rescale_log_probs,
+      state_callback_fn=state_callback_fn, logit_callback_fn=logit_callback_fn)
+
+  batch_size = inputs.shape[0]
+  decodes = unflatten_beam_dim(expanded_decodes, batch_size, num_decodes)
+  log_prob = unflatten_beam_dim(expanded_log_prob, batch_size, num_decodes)
+  # :401-409 ascending, stable.  top_k of the negated scores is a stable
+  # descending order of -log_prob, i.e. a stable ascending order of log_prob.
+  if num_decodes > 1:
+    _, idxs = ops.top_k((-log_prob).contiguous(), num_decodes)
+    decodes = ops.gather_beams(decodes.contiguous(), idxs)
+    log_prob = ops.gather_beams(log_prob.contiguous(), idxs)
+  return decodes, log_prob
+
+
+def _temperature_sample_single_trial(
+    inputs, cache, tokens_to_logits, eos_id: int, prng_key,
+    num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
+    topk: int = 20, topp: float = 0.0, initial_index=None,
+    max_decode_steps=None, rescale_log_probs: bool = True,
+    state_callback_fn: Optional[Callable] = None,
+    logit_callback_fn: Optional[Callable] = None,
+):
+  """:412-715."""
+  if topp and topk:
+    raise ValueError('At most one of `topp` or `topk` may be non-zero.')
+  dev = _device()
+  inputs = _dev(inputs, torch.int32)
+  batch_size, length = inputs.shape
+  inputs_np = inputs.cpu().numpy()
+
+  max_decode_len = np.full((batch_size,), length, np.int32)
+  if max_decode_steps is not None:  # :438-455
+    if np.ndim(max_decode_steps) == 0 and max_decode_steps > length:
+      raise ValueError('Cannot decode more steps than the sequence length.')
+    max_decode_len = np.minimum(
+        length, np.sum(inputs_np != 0, axis=1) + max_decode_steps).astype(
+            np.int32)
+
+  sequences_np = np.concatenate(
+      [inputs_np, np.zeros((batch_size, 2), np.int32)], axis=1)  # :465-470
+  if initial_index is None:
+    i0 = np.zeros((batch_size,), np.int32)
+    token0 = np.zeros((batch_size,), np.int32)
+  else:
+    i0 = _dev(initial_index).cpu().numpy().astype(np.int32)
+    token0 = np.take_along_axis(sequences_np, i0[:, None], axis=1)[:, 0]
+  initial_eos = np.sum(sequences_np == eos_id, axis=-1).astype(np.int32)
+
+  temps = np.asarray(temperature, dtype=np.float32)
+  if temps.ndim == 1:  # per-item temperatures (:595-612)
+    temps = np.repeat(temps, num_decodes)
+  else:
+    temps = np.full((batch_size,), float(temps), np.float32)
+  any_sampling = bool(np.any(temps > np.float32(MIN_TEMPERATURE)))
+
+  sequences = torch.as_tensor(sequences_np, device=dev).contiguous()
+  cur_index = torch.as_tensor(i0, device=dev)
+  cur_token = torch.as_tensor(token0.astype(np.int32), device=dev)
+  ended = torch.zeros((batch_size,), dtype=torch.uint8, device=dev)
+  log_prob = torch.zeros((batch_size,), dtype=torch.float32, device=dev)
+  mdl = torch.as_tensor(max_decode_len, device=dev)
+  eos0 = torch.as_tensor(initial_eos, device=dev)
+  temps_dev = torch.as_tensor(temps, device=dev)
+  all_ended = torch.zeros((), dtype=torch.int32, device=dev)
+  tokens = torch.empty((batch_size,), dtype=torch.int32, device=dev)
+  tok_lp = torch.empty((batch_size,), dtype=torch.float32, device=dev)
+  source = _noise_source(prng_key)
+  step = 0
+
+  def loop_state():
+    return SamplingLoopState(
+        torch.tensor(step, dtype=torch.int32), cur_index, sequences, cache,
+        cur_token[:, None], ended.bool()[:, None], _Key(source, step),
+        log_prob)
+
+  while True:  # cond: not all ended (:509-515); nothing has ended at step 0
+    if state_callback_fn is not None:
+      st = state_callback_fn(loop_state())
+      sequences = _dev(st.sequences, torch.int32).contiguous()
+      cur_index = _dev(st.cur_index, torch.int32).contiguous()
+      cache = st.cache
+    decoding_state = DecodingState(cur_index=cur_index,
+                                   sequences=sequences[:, :-2],
+                                   cur_token=cur_token[:, None], cache=cache)
+    logits, cache = tokens_to_logits(decoding_state)
+    if logit_callback_fn is not None:
+      if not isinstance(logits, torch.Tensor):
+        logits = np.array(logits, dtype=np.float32)
+      logits = logit_callback_fn(logits, loop_state())
+    logits = _dev(logits, torch.float32).contiguous()
+    gumbel = None
+    if any_sampling:
+      gumbel = _dev(source.noise(step, tuple(logits.shape)),
+                    torch.float32).contiguous()
+    ops.sample_tokens(logits, gumbel, temps_dev, topk, topp,
+                      rescale_log_probs, tokens, tok_lp)
+    ops.sample_update(tokens, tok_lp, sequences, cur_index, cur_token, ended,
+                      log_prob, mdl, eos0, all_ended, eos_id)
+    step += 1
+    if int(all_ended.item()):
+      break
+
+  if state_callback_fn is not None:
+    st = state_callback_fn(loop_state())
+    sequences = _dev(st.sequences, torch.int32)
+  return sequences[:, 1:-1], log_prob
+
+
+# ------------------------------------------------------------------------------
+# Beam search (:999-1569)
+# ------------------------------------------------------------------------------
+
+
+def _right_align_prompts(prompts):
+  """:1069-1095 (host side; prompts are small int arrays)."""
+  prompts = np.asarray(prompts)
+  max_len = prompts.shape[1]
+  nbits = np.ceil(np.log2(max_len)).astype(np.int32)
+  indices = np.arange(max_len)
+  prompt_max_index = np.argmax((prompts != 0) * indices[None, :], axis=1)
+  shifts = max_len - prompt_max_index - 1
+  for i in range(0, nbits + 1):
+    bitmask = 2**i
+    prompts = np.where((shifts & bitmask)[:, None] != 0,
+                       np.pad(prompts, ((0, 0), (bitmask, 0)))[:, :-bitmask],
+                       prompts)
+  return prompts
+
+
+def _left_align_prompts(prompts):
+  """:1098-1120."""
+  prompts = np.asarray(prompts)
+  max_len = prompts.shape[1]
+  indices = np.arange(max_len)
+  non_padding_positions = (prompts != 0) * (indices[None, :] + 1)
+  m = np.where(non_padding_positions != 0, non_padding_positions, max_len + 1)
+  shifts = np.argmin(m, axis=1)
+  temp = prompts
+  nbits = np.ceil(np.log2(max_len)).astype(np.int32)
+  for i in range(0, nbits + 1):
+    bitmask = 2**i
+    temp = np.where((shifts & bitmask)[:, None] != 0,
+                    np.pad(temp, ((0, 0), (0, bitmask)))[:, bitmask:], temp)
+  return temp
+
+
+def _pick_last_prompt_token(prompts):
+  """:1123-1127."""
+  prompts = np.asarray(prompts)
+  return prompts[np.arange(prompts.shape[0]), np.sum(prompts != 0, axis=1)]
+
+
+def beam_init(batch_size, beam_size, max_decode_len, cache, offset=0,
+              live_seqs=None, initial_index=None):
+  """:1024-1066 -> (BeamBuffers, beam-expanded cache)."""
+  dev = _device()
+  st = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
+  st.live_logprobs.copy_(torch.tensor(
+      [0.0] + [NEG_INF_VALUE] * (beam_size - 1), dtype=torch.float32,
+      device=dev).expand(batch_size, beam_size))
+  st.finished_scores.fill_(NEG_INF_VALUE)
+  if live_seqs is not None:
+    st.live_seqs.copy_(_dev(live_seqs, torch.int32))
+  beam_cache = cache_map(lambda x: add_beam_dim(x, beam_size, offset), cache,
+                         apply_to_index=live_seqs is not None)
+  return st, beam_cache
+
+
+def beam_search(
+    inputs, cache, tokens_to_logits, eos_id: int, num_decodes: int = 4,
+    alpha: float = 0.6, max_decode_len: Optional[int] = None,
+    max_decode_step: int = -1, min_log_prob: float = NEG_INF_VALUE,
+    decode_rng=None, cache_offset: int = 0, initial_index=None,
+):
+  """:1131-1569 -> (sequences [B, K, L] i32, scores [B, K] f32), the beam axis
+  sorted ascending by score."""
+  del decode_rng
+  dev = _device()
+  inputs_np = _dev(inputs).cpu().numpy().astype(np.int32)
+  beam_size = num_decodes
+  batch_size = inputs_np.shape[0]
+  if max_decode_len is None:
+    max_decode_len = inputs_np.shape[1]
+  max_decode_len += 1  # :1208
+
+  right_aligned_input = None
+  live_seqs = None
+  if initial_index is not None:  # :1212-1235
+    initial_index_np = _dev(initial_index).cpu().numpy().astype(np.int32)
+    right_aligned_input = _right_align_prompts(inputs_np)
+    length = inputs_np.shape[1]
+    last = right_aligned_input[:, -1][:, None]
+    inputs_np = np.pad(last, ((0, 0), (0, length - 1)), constant_values=0)
+    live_seqs = np.pad(last, ((0, 0), (0, max_decode_len - 1)),
+                       constant_values=0)
+    live_seqs = np.ascontiguousarray(np.broadcast_to(
+        live_seqs[:, None, :], (batch_size, beam_size, max_decode_len)))
+  else:
+    initial_index_np = np.zeros((batch_size,), np.int32)
+
+  cur, beam_cache = beam_init(batch_size, beam_size, max_decode_len, cache,
+                              cache_offset, live_seqs=live_seqs,
+                              initial_index=initial_index_np)
+  nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
+  inputs_dev = torch.as_tensor(np.ascontiguousarray(inputs_np), device=dev)
+  init_idx_dev = torch.as_tensor(initial_index_np, device=dev)
+  max_len_for_bp = max_decode_len + int(initial_index_np.max()) + 2
+  brevity = torch.as_tensor(
+      brevity_penalty(alpha, np.arange(max_len_for_bp, dtype=np.int32)),
+      device=dev).contiguous()
+  min_brevity = float(brevity_penalty(alpha, max_decode_len))  # :1268
+  min_initial = int(initial_index_np.min())
+  keep_going = torch.zeros((), dtype=torch.int32, device=dev)
+  top_alive = torch.empty((batch_size, beam_size), dtype=torch.int32,
+                          device=dev)
+  topk_bufs = None
+  vocab_size = None
+
+  def cond(state):  # :1250-1300
+    ops.beam_cond(state, min_brevity, min_log_prob, max_decode_step,
+                  min_initial, keep_going)
+    return bool(keep_going.item())
+
+  step = 0
+  while cond(cur):  # :1509
+    flat_ids = flatten_beam_dim(cur.live_seqs[:, :, step:step + 1])
+    flat_cache = cache_map(
+        functools.partial(flatten_beam_dim, offset=cache_offset), beam_cache)
+    decoding_state = DecodingState(
+        cur_index=cur.cur_index, sequences=flatten_beam_dim(cur.live_seqs),
+        cur_token=flat_ids, cache=flat_cache)
+    flat_logits, new_flat_cache = tokens_to_logits(decoding_state)
+    flat_logits = _dev(flat_logits, torch.float32).contiguous()
+    if vocab_size is None:
+      vocab_size = flat_logits.shape[-1]
+      R, k2 = batch_size * beam_size, 2 * beam_size
+      topk_bufs = (torch.empty((batch_size, k2), dtype=torch.float32,
+                               device=dev),
+                   torch.empty((batch_size, k2), dtype=torch.int32,
+                               device=dev),
+                   torch.empty((R,), dtype=torch.float32, device=dev),
+                   torch.empty((R,), dtype=torch.float32, device=dev),
+                   torch.empty((2 * R * k2,), dtype=torch.int32, device=dev))
+    new_cache = cache_map(
+        lambda x: unflatten_beam_dim(x, batch_size, beam_size, cache_offset),
+        new_flat_cache)
+    # :1340-1366 log_softmax + prefix add + top-2K over beam x vocab
+    topk_vals, topk_idx, _, _ = ops.beam_topk(flat_logits, cur.live_logprobs,
+                                              2 * beam_size, topk_bufs)
+    # :1366-1506 everything after the top-k
+    ops.beam_update(cur, nxt, topk_vals, topk_idx, inputs_dev, init_idx_dev,
+                    brevity, top_alive, vocab_size, eos_id)
+    # :1449-1457
+    beam_cache = cache_gather_beams(new_cache, top_alive, batch_size,
+                                    beam_size, beam_size, True, cache_offset)
+    cur, nxt = nxt, cur
+    step += 1
+
+  # :1516-1528 batch items with no finished sequence fall back to live ones
+  any_finished = cur.finished_flags.bool().any(dim=1)
+  finished_seqs = torch.where(any_finished[:, None, None], cur.finished_seqs,
+                              cur.live_seqs)
+  finished_scores = torch.where(any_finished[:, None], cur.finished_scores,
+                                cur.live_logprobs)
+
+  if right_aligned_input is not None:  # :1532-1564
+    seqs = finished_seqs.cpu().numpy()[:, :, 1:]
+    prompt = np.broadcast_to(
+        right_aligned_input[:, None, :],
+        (batch_size, seqs.shape[1], right_aligned_input.shape[-1]))
+    seqs = np.concatenate([prompt, seqs], axis=-1)
+    flat = _left_align_prompts(seqs.reshape(-1, seqs.shape[-1]))
+    seqs = flat.reshape(seqs.shape)[:, :, :max_decode_len - 1]
+    finished_seqs = torch.as_tensor(np.ascontiguousarray(seqs), device=dev)
+  else:
+    finished_seqs = finished_seqs[:, :, 1:]  # :1567
+  return finished_seqs, finished_scores

@@ -1,0 +1,170 @@
+"""Inference slice of t5x/models.py with the same call signatures:
+`EncoderDecoderModel.predict_batch` / `predict_batch_with_aux`,
+`_compute_logits_from_slice`, `_compute_kv_cache` (t5x/models.py:364-758).
+Arrays are torch tensors on the GPU; NumPy inputs are uploaded.
+"""
+
+import dataclasses
+import functools
+import inspect
+from typing import Any, Callable, Mapping, MutableMapping, Optional, Tuple
+
+import numpy as np
+import torch
+
+from t5x_amd import decoding
+from t5x_amd import network
+
+
+@dataclasses.dataclass
+class DecoderParams:
+  """t5x/models.py:358-361."""
+  return_all_decodes: bool = False
+  num_decodes: int = 1
+
+
+@dataclasses.dataclass
+class Vocabulary:
+  """Only `eos_id` is read on this path (t5x/models.py:741-742)."""
+  eos_id: int = 1
+
+
+def _is_array(x):
+  return isinstance(x, (np.ndarray, torch.Tensor))
+
+
+class EncoderDecoderModel:
+  """t5x/models.py:364-758, inference methods only."""
+
+  def __init__(self, module, input_vocabulary: Any = None,
+               output_vocabulary: Any = None, optimizer_def: Any = None,
+               decode_fn: Callable = decoding.beam_search,
+               default_decoder_params: Optional[DecoderParams] = None,
+               **unused_training_kwargs):
+    del optimizer_def, unused_training_kwargs
+    self.module = module
+    self._input_vocabulary = input_vocabulary or Vocabulary()
+    self._output_vocabulary = output_vocabulary or Vocabulary()
+    self._decode_fn = decode_fn
+    self._default_decoder_params = default_decoder_params or DecoderParams()
+
+  @property
+  def decode_fn(self):
+    return self._decode_fn
+
+  @property
+  def output_vocabulary(self):
+    return self._output_vocabulary
+
+  def _compute_logits_from_slice(self, decoding_state, params, encoded_inputs,
+                                 raw_inputs, max_decode_length):
+    """t5x/models.py:484-515."""
+    flat_ids = decoding_state.cur_token
+    flat_cache = decoding_state.cache
+    flat_logits, new_vars = self.module.apply(
+        {'params': params, 'cache': flat_cache}, encoded_inputs, raw_inputs,
+        flat_ids, flat_ids, enable_dropout=False, decode=True,
+        max_decode_length=max_decode_length, mutable=['cache'],
+        method=self.module.decode)
+    if isinstance(flat_logits, torch.Tensor):
+      flat_logits = flat_logits.squeeze(1)
+    else:
+      flat_logits = np.squeeze(flat_logits, axis=1)
+    return flat_logits, new_vars['cache']
+
+  def _compute_kv_cache(self, params, encoded_inputs, encoder_input_tokens,
+                        decoder_input_tokens,
+                        prefill_decoder_prompt: bool = False):
+    """t5x/models.py:517-582 (the examples/t5 module has no prefill)."""
+    del encoded_inputs
+    ones_like = (torch.ones_like if isinstance(encoder_input_tokens,
+                                               torch.Tensor) else np.ones_like)
+    ones_like_d = (torch.ones_like if isinstance(decoder_input_tokens,
+                                                 torch.Tensor) else
+                   np.ones_like)
+    _, initial_variables = self.module.apply(
+        {'params': params},
+        encoder_input_tokens=ones_like(encoder_input_tokens),
+        decoder_input_tokens=ones_like_d(decoder_input_tokens),
+        decoder_target_tokens=ones_like_d(decoder_input_tokens),
+        mutable=['cache'], decode=True, enable_dropout=False)
+    cache = initial_variables['cache']
+    if prefill_decoder_prompt:
+      raise NotImplementedError('module.decode has no `prefill` argument')
+    return cache, None
+
+  def predict_batch(self, params, batch, rng=None):
+    """t5x/models.py:177-193."""
+    return self.predict_batch_with_aux(params=params, batch=batch, rng=rng)[0]
+
+  def predict_batch_with_aux(
+      self, params, batch, rng=None,
+      decoder_params: Optional[MutableMapping[str, Any]] = None,
+      return_all_decodes: bool = None, num_decodes: int = None,
+      prompt_with_targets: bool = False):
+    """t5x/models.py:584-758."""
+    if return_all_decodes is None:
+      return_all_decodes = self._default_decoder_params.return_all_decodes
+    if num_decodes is None:
+      num_decodes = self._default_decoder_params.num_decodes
+
+    encoder_input_tokens = batch['encoder_input_tokens']
+    decoder_input_tokens = batch['decoder_input_tokens']
+    if prompt_with_targets:
+      decoder_prompt_inputs = decoder_input_tokens * (
+          decoder_input_tokens != self.output_vocabulary.eos_id)
+    elif isinstance(decoder_input_tokens, torch.Tensor):
+      decoder_prompt_inputs = torch.zeros_like(decoder_input_tokens)
+    else:
+      decoder_prompt_inputs = np.zeros_like(decoder_input_tokens)
+
+    encoded_inputs = self.module.apply(
+        {'params': params}, encoder_input_tokens, enable_dropout=False,
+        method=self.module.encode)
+
+    prefill_decoder_prompt = (
+        'initial_index' in inspect.signature(self.decode_fn).parameters and
+        'prefill' in inspect.signature(self.module.decode).parameters)
+    cache, initial_index = self._compute_kv_cache(
+        params, encoded_inputs=encoded_inputs,
+        encoder_input_tokens=encoder_input_tokens,
+        decoder_input_tokens=decoder_prompt_inputs,
+        prefill_decoder_prompt=prefill_decoder_prompt)
+
+    # :696-715.  The reference expands the encoder output per beam; when the
+    # module understands it, the expansion stays logical (BeamShared) so the
+    # cross-attention K/V are held once per batch item.
+    if isinstance(self.module, network.Transformer):
+      expand = lambda x: network.BeamShared(x, num_decodes)
+    else:
+      expand = lambda x: decoding.flat_batch_beam_expand(x, num_decodes)
+    tokens_ids_to_logits = functools.partial(
+        self._compute_logits_from_slice, params=params,
+        encoded_inputs=expand(encoded_inputs),
+        raw_inputs=expand(encoder_input_tokens),
+        max_decode_length=decoder_input_tokens.shape[1])
+
+    if decoder_params is None:
+      decoder_params = {}
+    if initial_index is not None:
+      decoder_params['initial_index'] = initial_index
+    if rng is not None:
+      if decoder_params.get('decode_rng') is not None:
+        raise ValueError(
+            f'Got RNG both from the `rng` argument ({rng}) and'
+            " `decoder_params['decode_rng']`"
+            f' ({decoder_params["decode_rng"]}). Please specify one or the'
+            ' other.')
+      decoder_params['decode_rng'] = rng
+
+    scanned = hasattr(self.module, 'scan_layers') and self.module.scan_layers
+    if 'eos_id' not in decoder_params:
+      decoder_params['eos_id'] = self.output_vocabulary.eos_id or 1
+    decodes, scores = self._decode_fn(
+        inputs=decoder_prompt_inputs, cache=cache,
+        tokens_to_logits=tokens_ids_to_logits, num_decodes=num_decodes,
+        cache_offset=1 if scanned else 0, **decoder_params)
+
+    if return_all_decodes:
+      return decodes, {'scores': scores}
+    return decodes[:, -1, :], {'scores': scores[:, -1]}

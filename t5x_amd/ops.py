@@ -1,0 +1,435 @@
+"""Tensor-level wrappers over the t5d C ABI.
+
+Each function takes torch device tensors, checks what the kernel assumes
+(shape, dtype, contiguity, device) and enqueues the kernel on the current
+torch stream.  No function here computes anything in torch.
+"""
+
+import ctypes
+
+import torch
+
+from t5x_amd import _lib
+from t5x_amd._lib import BF16, EPI_GEGLU, EPI_NONE, EPI_RESIDUAL, F32, I8
+
+__all__ = [
+    'PackedWeight', 'pack_weight', 'embed', 'rmsnorm', 'gemm',
+    'self_attention_step', 'cross_attention_step', 'add_i32',
+    'cache_gather_beams', 'gather_beams', 'top_k', 'beam_topk', 'BeamBuffers',
+    'beam_update', 'beam_cond', 'sample_tokens', 'sample_update',
+]
+
+
+def _chk(t, name, dtype=None, ndim=None):
+  if not isinstance(t, torch.Tensor):
+    raise TypeError(f'{name}: expected a torch tensor, got {type(t)}')
+  if not t.is_cuda:
+    raise ValueError(f'{name}: tensor must live on the GPU')
+  if not t.is_contiguous():
+    raise ValueError(f'{name}: tensor must be contiguous')
+  if dtype is not None and t.dtype != dtype:
+    raise ValueError(f'{name}: dtype {t.dtype}, expected {dtype}')
+  if ndim is not None and t.dim() != ndim:
+    raise ValueError(f'{name}: rank {t.dim()}, expected {ndim}')
+  return t
+
+
+def _s():
+  return _lib.stream_handle()
+
+
+class PackedWeight:
+  """A dense kernel in the layout t5d_gemm streams.
+
+  dtype float32: row-major [K, N] (or [K, 2F] = wi_0 | wi_1 for geglu).
+  dtype bfloat16 / int8: 32x16 MFMA tiles (see include/t5d.h), `scales` holds
+  the per-output-channel float32 scales of int8 weights in packed column order.
+  """
+
+  def __init__(self, data, K, N, w_dtype, geglu=False, scales=None):
+    self.data, self.K, self.N = data, K, N
+    self.w_dtype, self.geglu, self.scales = w_dtype, geglu, scales
+
+  @property
+  def out_features(self):
+    return self.N // 2 if self.geglu else self.N
+
+  def nbytes(self):
+    n = self.data.numel() * self.data.element_size()
+    if self.scales is not None:
+      n += self.scales.numel() * 4
+    return n
+
+
+def _quantize(w):
+  """Per-output-channel symmetric int8 (scale = max|w| / 127)."""
+  scale = w.abs().amax(dim=0).clamp_min(1e-30) / 127.0
+  q = torch.clamp(torch.round(w / scale), -127, 127).to(torch.int8)
+  return q, scale.to(torch.float32)
+
+
+def pack_weight(kernel, act_dtype, weight_dtype=None, gate_kernel=None):
+  """kernel: float32 [K, N] device tensor (reference layout).  `gate_kernel`
+  (wi_1) makes a geglu-packed pair with `kernel` as wi_0."""
+  _chk(kernel, 'kernel', torch.float32, 2)
+  K, N = kernel.shape
+  geglu = gate_kernel is not None
+  if geglu:
+    _chk(gate_kernel, 'gate_kernel', torch.float32, 2)
+    if gate_kernel.shape != kernel.shape:
+      raise ValueError('wi_0 / wi_1 shapes differ')
+  weight_dtype = weight_dtype or act_dtype
+  if act_dtype == torch.float32:
+    if weight_dtype != torch.float32:
+      raise ValueError('float32 activations need float32 weights')
+    data = torch.cat([kernel, gate_kernel], dim=1) if geglu else kernel.clone()
+    return PackedWeight(data.contiguous(), K, data.shape[1], F32, geglu)
+  if act_dtype != torch.bfloat16:
+    raise ValueError(f'unsupported activation dtype {act_dtype}')
+  Np = 2 * N if geglu else N
+  scales = None
+  if weight_dtype == torch.bfloat16:
+    src = kernel.to(torch.bfloat16).contiguous()
+    src2 = gate_kernel.to(torch.bfloat16).contiguous() if geglu else None
+    code = BF16
+  elif weight_dtype == torch.int8:
+    src, s0 = _quantize(kernel)
+    src = src.contiguous()
+    if geglu:
+      src2, s1 = _quantize(gate_kernel)
+      src2 = src2.contiguous()
+      # packed column 16*nt + c <- wi_0[8*nt + c] (c < 8) | wi_1[8*nt + c - 8]
+      scales = torch.stack([s0.view(-1, 8), s1.view(-1, 8)], dim=1).reshape(-1)
+    else:
+      src2, scales = None, s0
+    scales = scales.contiguous()
+    code = I8
+  else:
+    raise ValueError(f'unsupported weight dtype {weight_dtype}')
+  nbytes = _lib.load().t5d_packed_weight_bytes(code, K, Np)
+  if nbytes < 0:
+    raise ValueError(f'kernel [{K}, {Np}] does not tile 32x16')
+  dst = torch.empty(nbytes, dtype=torch.uint8, device=kernel.device)
+  _lib.call('t5d_pack_weight', _s(), code, src.data_ptr(), _lib.ptr(src2),
+            dst.data_ptr(), K, N, int(geglu))
+  return PackedWeight(dst, K, Np, code, geglu, scales)
+
+
+def embed(table, ids, out=None):
+  _chk(table, 'table', ndim=2)
+  _chk(ids, 'ids', torch.int32)
+  V, d = table.shape
+  R = ids.numel()
+  if out is None:
+    out = torch.empty((R, d), dtype=table.dtype, device=table.device)
+  _chk(out, 'out', table.dtype)
+  _lib.call('t5d_embed', _s(), _lib.dtype_code(table.dtype), table.data_ptr(),
+            ids.data_ptr(), out.data_ptr(), R, d, V)
+  return out
+
+
+def rmsnorm(x, scale, out=None, eps=1e-6):
+  _chk(x, 'x', ndim=2)
+  _chk(scale, 'scale', x.dtype, 1)
+  R, d = x.shape
+  if scale.shape[0] != d:
+    raise ValueError('scale length mismatch')
+  if out is None:
+    out = torch.empty_like(x)
+  _chk(out, 'out', x.dtype)
+  _lib.call('t5d_rmsnorm', _s(), _lib.dtype_code(x.dtype), x.data_ptr(),
+            scale.data_ptr(), out.data_ptr(), R, d, float(eps))
+  return out
+
+
+class GemmScratch:
+  """Split-K workspace + counters, grown on demand and reused."""
+
+  def __init__(self, device):
+    self.device = device
+    self.workspace = None
+    self.counters = torch.zeros(4096, dtype=torch.int32, device=device)
+
+  def get(self, nbytes):
+    if nbytes and (self.workspace is None or
+                   self.workspace.numel() < nbytes):
+      self.workspace = torch.empty(nbytes, dtype=torch.uint8,
+                                   device=self.device)
+    return self.workspace
+
+
+_scratch = {}
+
+
+def _default_scratch(device):
+  key = (device.type, device.index)
+  if key not in _scratch:
+    _scratch[key] = GemmScratch(device)
+  return _scratch[key]
+
+
+def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
+         scratch=None):
+  """C = epilogue(a @ W).  a [M, K]; geglu weights give [M, F]."""
+  _chk(a, 'a', ndim=2)
+  M, K = a.shape
+  if K != w.K:
+    raise ValueError(f'a is [{M}, {K}] but the kernel has K={w.K}')
+  epi = EPI_GEGLU if w.geglu else (EPI_RESIDUAL if residual is not None
+                                   else EPI_NONE)
+  out_dtype = out_dtype or a.dtype
+  n_out = w.out_features
+  if out is None:
+    out = torch.empty((M, n_out), dtype=out_dtype, device=a.device)
+  _chk(out, 'out', out_dtype, 2)
+  if tuple(out.shape) != (M, n_out):
+    raise ValueError(f'out shape {tuple(out.shape)} != {(M, n_out)}')
+  if residual is not None:
+    _chk(residual, 'residual', a.dtype, 2)
+    if tuple(residual.shape) != (M, n_out):
+      raise ValueError('residual shape mismatch')
+  dt = _lib.dtype_code(a.dtype)
+  ws_bytes = _lib.load().t5d_gemm_workspace_bytes(dt, w.w_dtype, M, K, w.N)
+  ws = cnt = None
+  if ws_bytes:
+    scratch = scratch or _default_scratch(a.device)
+    ws = scratch.get(ws_bytes)
+    cnt = scratch.counters
+    if w.N // 16 > cnt.numel():
+      raise ValueError('too many column tiles for the counter buffer')
+  _lib.call('t5d_gemm', _s(), dt, w.w_dtype, _lib.dtype_code(out_dtype),
+            a.data_ptr(), w.data.data_ptr(), _lib.ptr(w.scales),
+            _lib.ptr(residual), out.data_ptr(), M, K, w.N, epi, _lib.ptr(ws),
+            _lib.ptr(cnt))
+  return out
+
+
+def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
+                        out=None):
+  _chk(qkv, 'qkv', ndim=2)
+  _chk(cached_key, 'cached_key', qkv.dtype, 4)
+  _chk(cached_value, 'cached_value', qkv.dtype, 4)
+  _chk(rel_bias, 'rel_bias', qkv.dtype, 2)
+  _chk(cache_index, 'cache_index', torch.int32)
+  R, H, D, L = cached_key.shape
+  if D != 64:
+    raise ValueError('head_dim must be 64')
+  if cached_value.shape != cached_key.shape:
+    raise ValueError('cached_key / cached_value shapes differ')
+  if tuple(qkv.shape) != (R, 3 * H * D):
+    raise ValueError(f'qkv shape {tuple(qkv.shape)} != {(R, 3 * H * D)}')
+  if tuple(rel_bias.shape) != (H, L):
+    raise ValueError(f'rel_bias shape {tuple(rel_bias.shape)} != {(H, L)}')
+  if cache_index.numel() != 1:
+    raise ValueError('cache_index must be a scalar')
+  if out is None:
+    out = torch.empty((R, H * D), dtype=qkv.dtype, device=qkv.device)
+  _chk(out, 'out', qkv.dtype, 2)
+  _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
+            qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),
+            rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), R, H,
+            L)
+  return out
+
+
+def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
+  _chk(q, 'q', ndim=2)
+  _chk(cross_key, 'cross_key', q.dtype, 4)
+  _chk(cross_value, 'cross_value', q.dtype, 4)
+  _chk(enc_len, 'enc_len', torch.int32, 1)
+  B, H, D, E = cross_key.shape
+  if D != 64:
+    raise ValueError('head_dim must be 64')
+  if cross_value.shape != cross_key.shape:
+    raise ValueError('cross_key / cross_value shapes differ')
+  if tuple(q.shape) != (B * beams, H * D):
+    raise ValueError(f'q shape {tuple(q.shape)} != {(B * beams, H * D)}')
+  if enc_len.shape[0] != B:
+    raise ValueError('enc_len length mismatch')
+  if out is None:
+    out = torch.empty_like(q)
+  _chk(out, 'out', q.dtype, 2)
+  _lib.call('t5d_cross_attention_step', _s(), _lib.dtype_code(q.dtype),
+            q.data_ptr(), cross_key.data_ptr(), cross_value.data_ptr(),
+            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E)
+  return out
+
+
+def add_i32(x, delta):
+  _chk(x, 'x', torch.int32)
+  _lib.call('t5d_add_i32', _s(), x.data_ptr(), x.numel(), int(delta))
+  return x
+
+
+def cache_gather_beams(cache, beam_indices, valid_len=None, valid_offset=0,
+                       n_tensors=1, tensor_stride_bytes=0):
+  """In-place gather of [.., B, beams, inner.., L] cache tensors.
+
+  `cache` is [B, beams, ..., L] (n_tensors == 1) or the first of n_tensors
+  such tensors spaced tensor_stride_bytes apart."""
+  _chk(cache, 'cache')
+  _chk(beam_indices, 'beam_indices', torch.int32, 2)
+  B, beams = beam_indices.shape
+  if cache.shape[0] != B or cache.shape[1] != beams:
+    raise ValueError(f'cache {tuple(cache.shape)} vs indices {(B, beams)}')
+  L = cache.shape[-1]
+  inner = 1
+  for s in cache.shape[2:-1]:
+    inner *= s
+  if valid_len is not None:
+    _chk(valid_len, 'valid_len', torch.int32)
+  _lib.call('t5d_cache_gather_beams', _s(), cache.data_ptr(),
+            int(tensor_stride_bytes), int(n_tensors), cache.element_size(), B,
+            beams, inner, L, beam_indices.data_ptr(), _lib.ptr(valid_len),
+            int(valid_offset))
+  return cache
+
+
+def gather_beams(x, beam_indices, out=None):
+  """out[b, e] = x[b, beam_indices[b, e]] (out of place)."""
+  _chk(x, 'x')
+  _chk(beam_indices, 'beam_indices', torch.int32, 2)
+  B, new_beams = beam_indices.shape
+  if x.dim() < 2 or x.shape[0] != B:
+    raise ValueError(f'x {tuple(x.shape)} vs indices {(B, new_beams)}')
+  old_beams = x.shape[1]
+  inner = x[0, 0].numel() * x.element_size()
+  if out is None:
+    out = torch.empty((B, new_beams) + tuple(x.shape[2:]), dtype=x.dtype,
+                      device=x.device)
+  if inner == 0 or B == 0:
+    return out
+  _lib.call('t5d_gather_beams', _s(), x.data_ptr(), out.data_ptr(),
+            beam_indices.data_ptr(), B, old_beams, new_beams, inner)
+  return out
+
+
+def top_k(x, k):
+  _chk(x, 'x', torch.float32, 2)
+  rows, n = x.shape
+  vals = torch.empty((rows, k), dtype=torch.float32, device=x.device)
+  idx = torch.empty((rows, k), dtype=torch.int32, device=x.device)
+  _lib.call('t5d_top_k', _s(), x.data_ptr(), vals.data_ptr(), idx.data_ptr(),
+            rows, n, k)
+  return vals, idx
+
+
+def beam_topk(logits, live_logprobs, k, bufs=None):
+  """-> (topk_vals [B, k], topk_idx [B, k], row_max [R], row_lse [R])."""
+  _chk(logits, 'logits', torch.float32, 2)
+  _chk(live_logprobs, 'live_logprobs', torch.float32, 2)
+  B, beams = live_logprobs.shape
+  R, V = logits.shape
+  if R != B * beams:
+    raise ValueError(f'logits rows {R} != {B}*{beams}')
+  dev = logits.device
+  if bufs is None:
+    bufs = (torch.empty((B, k), dtype=torch.float32, device=dev),
+            torch.empty((B, k), dtype=torch.int32, device=dev),
+            torch.empty((R,), dtype=torch.float32, device=dev),
+            torch.empty((R,), dtype=torch.float32, device=dev),
+            torch.empty((2 * R * k,), dtype=torch.int32, device=dev))
+  vals, idx, row_max, row_lse, scratch = bufs
+  _lib.call('t5d_beam_topk', _s(), logits.data_ptr(), live_logprobs.data_ptr(),
+            vals.data_ptr(), idx.data_ptr(), row_max.data_ptr(),
+            row_lse.data_ptr(), scratch.data_ptr(), B, beams, V, k)
+  return vals, idx, row_max, row_lse
+
+
+class BeamBuffers:
+  """Device arrays of one BeamState (t5x/decoding.py:1002-1021)."""
+
+  def __init__(self, B, K, S, device):
+    self.B, self.K, self.S = B, K, S
+    self.cur_index = torch.zeros((), dtype=torch.int32, device=device)
+    self.live_logprobs = torch.zeros((B, K), dtype=torch.float32,
+                                     device=device)
+    self.finished_scores = torch.zeros((B, K), dtype=torch.float32,
+                                       device=device)
+    self.live_seqs = torch.zeros((B, K, S), dtype=torch.int32, device=device)
+    self.finished_seqs = torch.zeros((B, K, S), dtype=torch.int32,
+                                     device=device)
+    self.finished_flags = torch.zeros((B, K), dtype=torch.uint8, device=device)
+    self._ptrs = _lib.BeamStatePtrs(
+        self.cur_index.data_ptr(), self.live_logprobs.data_ptr(),
+        self.finished_scores.data_ptr(), self.live_seqs.data_ptr(),
+        self.finished_seqs.data_ptr(), self.finished_flags.data_ptr())
+
+  def ptrs(self):
+    return ctypes.byref(self._ptrs)
+
+
+def beam_update(cur: BeamBuffers, nxt: BeamBuffers, topk_vals, topk_idx,
+                inputs, initial_index, brevity, top_alive_indices, V, eos_id):
+  _chk(topk_vals, 'topk_vals', torch.float32, 2)
+  _chk(topk_idx, 'topk_idx', torch.int32, 2)
+  _chk(inputs, 'inputs', torch.int32, 2)
+  _chk(initial_index, 'initial_index', torch.int32, 1)
+  _chk(brevity, 'brevity', torch.float32, 1)
+  _chk(top_alive_indices, 'top_alive_indices', torch.int32, 2)
+  B, K, S = cur.B, cur.K, cur.S
+  if tuple(topk_vals.shape) != (B, 2 * K) or topk_idx.shape != topk_vals.shape:
+    raise ValueError('top-k buffers must be [B, 2K]')
+  if inputs.shape[0] != B or initial_index.shape[0] != B:
+    raise ValueError('inputs / initial_index batch mismatch')
+  if tuple(top_alive_indices.shape) != (B, K):
+    raise ValueError('top_alive_indices must be [B, K]')
+  _lib.call('t5d_beam_update', _s(), cur.ptrs(), nxt.ptrs(),
+            topk_vals.data_ptr(), topk_idx.data_ptr(), inputs.data_ptr(),
+            initial_index.data_ptr(), brevity.data_ptr(),
+            top_alive_indices.data_ptr(), B, K, S, inputs.shape[1], V,
+            int(eos_id))
+
+
+def beam_cond(state: BeamBuffers, min_brevity, min_log_prob, max_decode_step,
+              min_initial_index, keep_going):
+  _chk(keep_going, 'keep_going', torch.int32)
+  _lib.call('t5d_beam_cond', _s(), state.ptrs(), state.B, state.K, state.S,
+            float(min_brevity), float(min_log_prob), int(max_decode_step),
+            int(min_initial_index), keep_going.data_ptr())
+
+
+def sample_tokens(logits, gumbel, temperature, topk, topp, rescale, tokens=None,
+                  logprobs=None):
+  _chk(logits, 'logits', torch.float32, 2)
+  _chk(temperature, 'temperature', torch.float32, 1)
+  R, V = logits.shape
+  if temperature.shape[0] != R:
+    raise ValueError('temperature must be [R]')
+  if gumbel is not None:
+    _chk(gumbel, 'gumbel', torch.float32, 2)
+    if gumbel.shape != logits.shape:
+      raise ValueError('gumbel shape mismatch')
+  if tokens is None:
+    tokens = torch.empty((R,), dtype=torch.int32, device=logits.device)
+  if logprobs is None:
+    logprobs = torch.empty((R,), dtype=torch.float32, device=logits.device)
+  _lib.call('t5d_sample_tokens', _s(), logits.data_ptr(), _lib.ptr(gumbel),
+            temperature.data_ptr(), tokens.data_ptr(), logprobs.data_ptr(), R,
+            V, int(topk), float(topp), int(bool(rescale)))
+  return tokens, logprobs
+
+
+def sample_update(tokens, token_logprobs, sequences, cur_index, cur_token,
+                  ended, log_prob, max_decode_len, initial_eos_count,
+                  all_ended, eos_id):
+  R, S = sequences.shape
+  for t, name, dt in ((tokens, 'tokens', torch.int32),
+                      (token_logprobs, 'token_logprobs', torch.float32),
+                      (sequences, 'sequences', torch.int32),
+                      (cur_index, 'cur_index', torch.int32),
+                      (cur_token, 'cur_token', torch.int32),
+                      (ended, 'ended', torch.uint8),
+                      (log_prob, 'log_prob', torch.float32),
+                      (max_decode_len, 'max_decode_len', torch.int32),
+                      (initial_eos_count, 'initial_eos_count', torch.int32),
+                      (all_ended, 'all_ended', torch.int32)):
+    _chk(t, name, dt)
+    if name not in ('sequences', 'all_ended') and t.numel() != R:
+      raise ValueError(f'{name} must have {R} elements')
+  _lib.call('t5d_sample_update', _s(), tokens.data_ptr(),
+            token_logprobs.data_ptr(), sequences.data_ptr(),
+            cur_index.data_ptr(), cur_token.data_ptr(), ended.data_ptr(),
+            log_prob.data_ptr(), max_decode_len.data_ptr(),
+            initial_eos_count.data_ptr(), all_ended.data_ptr(), R, S,
+            int(eos_id))

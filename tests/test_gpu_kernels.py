@@ -1,0 +1,371 @@
+"""Per-kernel parity of the HIP path against the CPU oracle, through the C ABI.
+
+Integer / index results (token ids, beam indices, top-k selections, cache
+contents) must be bit-exact.  Floating point: float32 activations within 1e-4,
+bfloat16 activations within 2e-2 absolute (one bf16 rounding of an O(1) value
+is 4e-3), as stated by the parity rule for this path.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decoding as odec
+from oracle import binary_search as obs
+from oracle import t5 as ot5
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+
+
+def dev(x, dtype=None):
+  t = torch.as_tensor(np.ascontiguousarray(x), device='cuda')
+  return t.to(dtype) if dtype is not None else t
+
+
+def host(t):
+  return t.detach().float().cpu().numpy() if t.is_floating_point() else \
+      t.detach().cpu().numpy()
+
+
+def oracle_dtype(dt):
+  return 'bfloat16' if dt == torch.bfloat16 else 'float32'
+
+
+@pytest.fixture(scope='module')
+def ops():
+  from t5x_amd import ops as _ops
+  return _ops
+
+
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+def test_embed_exact(ops, dt):
+  rs = np.random.RandomState(0)
+  table = dev(rs.randn(100, 64).astype(np.float32), dt)
+  ids = dev(rs.randint(0, 100, size=(17,)).astype(np.int32))
+  out = ops.embed(table, ids)
+  np.testing.assert_array_equal(host(out), host(table)[host(ids)])
+
+
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('R,d', [(1, 64), (8, 512), (128, 768), (5, 4096)])
+def test_rmsnorm(ops, dt, R, d):
+  rs = np.random.RandomState(R + d)
+  x = dev(3 * rs.randn(R, d).astype(np.float32), dt)
+  scale = dev(1 + 0.1 * rs.randn(d).astype(np.float32), dt)
+  out = ops.rmsnorm(x, scale)
+  want = ot5.layer_norm(host(x), host(scale), oracle_dtype(dt))
+  # two roundings to bf16: allow one bf16 ulp (2^-8 relative) of slack
+  np.testing.assert_allclose(host(out), want, atol=TOL[dt], rtol=2**-7 if
+                             dt == torch.bfloat16 else 1e-5)
+
+
+GEMM_SHAPES = [(1, 64, 32), (8, 96, 48), (16, 768, 768), (20, 768, 2304),
+               (64, 1024, 1024), (128, 768, 768), (128, 2048, 768),
+               (128, 768, 4096)]
+
+
+@pytest.mark.parametrize('M,K,N', GEMM_SHAPES)
+@pytest.mark.parametrize('epi', ['none', 'residual', 'geglu'])
+def test_gemm_bf16(ops, M, K, N, epi):
+  rs = np.random.RandomState(M * 7 + K + N)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  a_np = host(a)
+  if epi == 'geglu':
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, gate_kernel=dev(w1))
+    out = ops.gemm(a, pw)
+    want = ot5.mlp_block(
+        {'wi_0': {'kernel': w0}, 'wi_1': {'kernel': w1},
+         'wo': {'kernel': np.eye(N, dtype=np.float32)}}, a_np,
+        ('gelu', 'linear'), 'bfloat16')
+  else:
+    pw = ops.pack_weight(dev(w0), torch.bfloat16)
+    res = None
+    want = ot5.dense_general(a_np, w0, 'bfloat16')
+    if epi == 'residual':
+      res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+      want = ot5.bf16_round(want + host(res))
+    out = ops.gemm(a, pw, residual=res)
+  assert out.shape == want.shape
+  np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
+
+
+@pytest.mark.parametrize('M', [8, 128])
+def test_gemm_logits_f32_out(ops, M):
+  K, N = 768, 32128
+  rs = np.random.RandomState(M)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  pw = ops.pack_weight(dev(w), torch.bfloat16)
+  out = ops.gemm(a, pw, out_dtype=torch.float32)
+  want = host(a) @ ot5.bf16_round(w)
+  np.testing.assert_allclose(host(out), want, atol=1e-3, rtol=1e-4)
+  # bitwise deterministic across launches
+  out2 = ops.gemm(a, pw, out_dtype=torch.float32)
+  assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize('M,K,N', [(16, 768, 768), (64, 2048, 5120),
+                                   (128, 768, 2304)])
+@pytest.mark.parametrize('geglu', [False, True])
+def test_gemm_int8_weights(ops, M, K, N, geglu):
+  rs = np.random.RandomState(K + N + M)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  q0 = ot5.quantize_int8(w0)
+  if geglu:
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    q1 = ot5.quantize_int8(w1)
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, torch.int8,
+                         gate_kernel=dev(w1))
+    want = ot5.mlp_block({'wi_0': {'kernel': q0}, 'wi_1': {'kernel': q1},
+                          'wo': {'kernel': np.eye(N, dtype=np.float32)}},
+                         host(a), ('gelu', 'linear'), 'bfloat16')
+  else:
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, torch.int8)
+    want = ot5.dense_general(host(a), q0, 'bfloat16')
+  out = ops.gemm(a, pw)
+  np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
+
+
+@pytest.mark.parametrize('M,K,N', [(8, 512, 384), (8, 512, 32128),
+                                   (3, 100, 70), (20, 64, 128)])
+@pytest.mark.parametrize('epi', ['none', 'residual', 'geglu'])
+def test_gemm_f32(ops, M, K, N, epi):
+  rs = np.random.RandomState(M + K + N)
+  a = rs.randn(M, K).astype(np.float32)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  if epi == 'geglu':
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    pw = ops.pack_weight(dev(w0), torch.float32, gate_kernel=dev(w1))
+    out = ops.gemm(dev(a), pw)
+    want = ot5.gelu(a @ w0) * (a @ w1)
+  else:
+    pw = ops.pack_weight(dev(w0), torch.float32)
+    res = rs.randn(M, N).astype(np.float32) if epi == 'residual' else None
+    out = ops.gemm(dev(a), pw, residual=None if res is None else dev(res))
+    want = a @ w0 + (0 if res is None else res)
+  np.testing.assert_allclose(host(out), want, atol=1e-4, rtol=1e-4)
+
+
+def test_gemm_rejects_bad_shapes(ops):
+  a = dev(np.zeros((200, 64), np.float32), torch.bfloat16)
+  pw = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.bfloat16)
+  with pytest.raises(Exception, match='128'):
+    ops.gemm(a, pw)
+  with pytest.raises(ValueError, match='tile'):
+    ops.pack_weight(dev(np.zeros((40, 32), np.float32)), torch.bfloat16)
+
+
+def _self_attn_oracle(qkv, ck, cv, rel_emb, t, dtype):
+  """Oracle decode-branch attention with selection 'projections'."""
+  R, H, D, L = ck.shape
+  HD = H * D
+  sel = lambda o: np.eye(3 * HD, dtype=np.float32)[:, o * HD:(o + 1) * HD]
+  params = {'query': {'kernel': sel(0)}, 'key': {'kernel': sel(1)},
+            'value': {'kernel': sel(2)},
+            'out': {'kernel': np.eye(HD, dtype=np.float32)}}
+  bias = ot5.relpos_bias(rel_emb, L, L, False, dtype)
+  x = qkv[:, None, :]
+  cache = {'cached_key': ck, 'cached_value': cv, 'cache_index': np.array(t)}
+  out, new = ot5.multi_head_attention(params, x, x, None, bias, num_heads=H,
+                                      head_dim=D, dtype=dtype, decode=True,
+                                      cache=cache)
+  return out[:, 0], new
+
+
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('R,H,L,t', [(2, 3, 32, 0), (2, 3, 32, 5),
+                                     (4, 6, 32, 31), (3, 2, 128, 77),
+                                     (2, 2, 256, 130), (2, 2, 256, 255),
+                                     (8, 12, 128, 127)])
+def test_self_attention_step(ops, dt, R, H, L, t):
+  from t5x_amd import network
+  rs = np.random.RandomState(R * 1000 + L + t)
+  D = 64
+  od = oracle_dtype(dt)
+  ck = np.zeros((R, H, D, L), np.float32)
+  cv = np.zeros((R, H, D, L), np.float32)
+  ck[..., :t] = rs.randn(R, H, D, t)
+  cv[..., :t] = rs.randn(R, H, D, t)
+  ck, cv = ot5.cast(ck, od), ot5.cast(cv, od)
+  qkv = ot5.cast(rs.randn(R, 3 * H * D).astype(np.float32) *
+                 np.concatenate([np.full(H * D, 0.125), np.ones(2 * H * D)]),
+                 od)
+  rel_emb = rs.randn(H, 32).astype(np.float32)
+  want, new = _self_attn_oracle(qkv, ck, cv, rel_emb, t, od)
+
+  bucket = network.relative_position_bucket(-np.arange(L), bidirectional=False)
+  rel_bias = dev(ot5.cast(rel_emb, od)[:, bucket], dt)
+  ck_d, cv_d = dev(ck, dt), dev(cv, dt)
+  out = ops.self_attention_step(dev(qkv, dt), ck_d, cv_d, rel_bias,
+                                dev(np.array(t, np.int32)))
+  np.testing.assert_array_equal(host(ck_d), new['cached_key'])
+  np.testing.assert_array_equal(host(cv_d), new['cached_value'])
+  np.testing.assert_allclose(host(out), want, atol=TOL[dt], rtol=TOL[dt])
+
+
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('B,beams,H,E', [(2, 1, 3, 64), (3, 4, 2, 512),
+                                         (2, 2, 2, 128), (1, 8, 2, 264),
+                                         (2, 3, 2, 1024), (1, 1, 2, 2048)])
+def test_cross_attention_step(ops, dt, B, beams, H, E):
+  rs = np.random.RandomState(B * 100 + beams * 10 + E)
+  D = 64
+  od = oracle_dtype(dt)
+  if dt == torch.float32 and E > 1024:
+    pytest.skip('float32 rows cover at most 1024 positions per workgroup')
+  lens = rs.randint(1, E + 1, size=(B,)).astype(np.int32)
+  lens[0] = E
+  k = ot5.cast(rs.randn(B, E, H, D).astype(np.float32), od)
+  v = ot5.cast(rs.randn(B, E, H, D).astype(np.float32), od)
+  R = B * beams
+  q = ot5.cast(0.125 * rs.randn(R, H * D).astype(np.float32), od)
+  eye = np.eye(H * D, dtype=np.float32)
+  params = {'query': {'kernel': eye}, 'out': {'kernel': eye}}
+  tokens = (np.arange(E)[None, :] < lens[:, None]).astype(np.int32)
+  mask = ot5.make_attention_mask(np.ones((R, 1)),
+                                 np.repeat(tokens, beams, axis=0) > 0)
+  want, _ = ot5.multi_head_attention(
+      params, q[:, None, :], None, mask, None, num_heads=H, head_dim=D,
+      dtype=od, projected_kv=(np.repeat(k, beams, axis=0),
+                              np.repeat(v, beams, axis=0)))
+  kd = dev(np.ascontiguousarray(k.transpose(0, 2, 3, 1)), dt)
+  vd = dev(np.ascontiguousarray(v.transpose(0, 2, 3, 1)), dt)
+  out = ops.cross_attention_step(dev(q, dt), kd, vd, dev(lens), beams)
+  np.testing.assert_allclose(host(out), want[:, 0], atol=TOL[dt],
+                             rtol=TOL[dt])
+
+
+@pytest.mark.parametrize('rows,n,k', [(1, 10, 3), (4, 1000, 8), (3, 128512, 8),
+                                      (2, 24, 24), (5, 77, 64)])
+def test_top_k_exact_with_ties(ops, rows, n, k):
+  rs = np.random.RandomState(n + k)
+  x = rs.randint(0, max(2, n // 3), size=(rows, n)).astype(np.float32)
+  x[:, ::5] = -1e7
+  vals, idx = ops.top_k(dev(x), k)
+  wv, wi = odec.top_k(x, k)
+  np.testing.assert_array_equal(host(idx), wi)
+  np.testing.assert_array_equal(host(vals), wv)
+
+
+@pytest.mark.parametrize('B,beams,V', [(2, 2, 4), (2, 2, 8), (3, 4, 1000),
+                                       (32, 4, 32128), (2, 8, 5000),
+                                       (1, 1, 32128)])
+def test_beam_topk(ops, B, beams, V):
+  rs = np.random.RandomState(B + beams + V)
+  logits = (3 * rs.randn(B * beams, V)).astype(np.float32)
+  logits[:, 1] = -1e10
+  live = np.sort(-np.abs(rs.randn(B, beams)).astype(np.float32), axis=1)
+  live[0, 0] = -1e7  # a dead beam: candidates collapse into exact ties
+  if B > 1:
+    logits[beams:2 * beams] = logits[beams]  # identical rows: cross-beam ties
+    live[1, :] = live[1, 0]
+  k = 2 * beams
+  vals, idx, row_max, row_lse = ops.beam_topk(dev(logits), dev(live), k)
+  # log-softmax statistics to tolerance ...
+  lp = odec.log_softmax(logits)
+  want_lse = -(lp - (logits - logits.max(-1, keepdims=True)))[:, 0]
+  np.testing.assert_allclose(host(row_lse), want_lse, atol=1e-5, rtol=1e-6)
+  np.testing.assert_array_equal(host(row_max), logits.max(-1))
+  # ... and the selection bit-exact given the same log-probs.
+  cand = ((logits - host(row_max)[:, None]) - host(row_lse)[:, None]).astype(
+      np.float32)
+  flat = (cand.reshape(B, beams, V) + live[:, :, None]).astype(
+      np.float32).reshape(B, beams * V)
+  wv, wi = odec.top_k(flat, k)
+  np.testing.assert_array_equal(host(idx), wi)
+  np.testing.assert_array_equal(host(vals), wv)
+
+
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('B,beams,H,L,valid', [(2, 2, 2, 32, None),
+                                               (3, 4, 3, 128, 57),
+                                               (2, 8, 1, 64, 64),
+                                               (4, 3, 2, 40, 1)])
+def test_cache_gather_beams(ops, dt, B, beams, H, L, valid):
+  rs = np.random.RandomState(B + beams + L)
+  layers = 3
+  x = rs.randn(layers, 2, B, beams, H, 64, L).astype(np.float32)
+  idx = rs.randint(0, beams, size=(B, beams)).astype(np.int32)
+  idx[0] = np.arange(beams)  # identity item is skipped
+  t = dev(x, dt)
+  before = host(t).copy()
+  want = before.copy()
+  b = np.arange(B)[:, None]
+  nv = L if valid is None else valid
+  want[:, :, :, :, :, :, :nv] = before[:, :, b, idx][..., :nv]
+  vl = None if valid is None else dev(np.array(valid - 1, np.int32))
+  stride = t[0, 0].numel() * t.element_size()
+  ops.cache_gather_beams(t[0, 0], dev(idx), valid_len=vl, valid_offset=1,
+                         n_tensors=layers * 2, tensor_stride_bytes=stride)
+  got = host(t)
+  el = 16 // t.element_size()
+  nv_pad = min(L, (nv + el - 1) // el * el)
+  np.testing.assert_array_equal(got[..., :nv], want[..., :nv])
+  # columns past the 16-byte chunk holding the last valid one are untouched
+  np.testing.assert_array_equal(got[..., nv_pad:], before[..., nv_pad:])
+
+
+def test_gather_beams_out_of_place(ops):
+  rs = np.random.RandomState(0)
+  x = rs.randint(0, 100, size=(3, 4, 129)).astype(np.int32)
+  idx = rs.randint(0, 4, size=(3, 8)).astype(np.int32)
+  out = ops.gather_beams(dev(x), dev(idx))
+  np.testing.assert_array_equal(host(out), x[np.arange(3)[:, None], idx])
+  y = rs.randn(3, 4).astype(np.float32)
+  out = ops.gather_beams(dev(y), dev(idx))
+  np.testing.assert_array_equal(host(out), y[np.arange(3)[:, None], idx])
+
+
+@pytest.mark.parametrize('V,topk', [(7, 3), (1000, 40), (32128, 40),
+                                    (32128, 1), (50, 0)])
+@pytest.mark.parametrize('temp', [0.0, 0.7, 1.0])
+@pytest.mark.parametrize('rescale', [True, False])
+def test_sample_tokens_topk(ops, V, topk, temp, rescale):
+  rs = np.random.RandomState(V + topk)
+  R = 6
+  logits = (2 * rs.randn(R, V)).astype(np.float32)
+  logits[:, ::4] = logits[:, 1:2]  # ties, also at the cutoff for small k
+  g = odec.GumbelNoise(seed=3).noise(0, (R, V))
+  temps = np.full((R,), temp, np.float32)
+  tok, lp = ops.sample_tokens(dev(logits), dev(g), dev(temps), topk, 0.0,
+                              rescale)
+  if temp > 1e-4:
+    scaled = (logits / np.maximum(np.float32(temp), np.float32(1e-4))).astype(
+        np.float32)
+    if topk:
+      scaled = obs.topk_mask(scaled, topk, np.float32(-1e7))
+    want_tok = np.argmax(scaled + g, axis=-1)
+    src = scaled if rescale else logits
+    want_lp = odec.log_softmax(src)[np.arange(R), want_tok]
+  else:
+    want_tok = np.argmax(logits, axis=-1)
+    want_lp = (np.zeros(R, np.float32) if rescale else
+               odec.log_softmax(logits)[np.arange(R), want_tok])
+  np.testing.assert_array_equal(host(tok), want_tok)
+  np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
+
+
+def test_sample_tokens_topp_table(ops):
+  # t5x/binary_search_test.py:143-209 through the kernel: with a huge Gumbel
+  # bonus on one index the sampled token reveals whether it survived the mask.
+  probs = np.asarray([[0.0, 0.7, 0.04, 0.06, 0.2, 0.0],
+                      [0.0, 0.2, 0.2, 0.2, 0.3, 0.1]])
+  with np.errstate(divide='ignore'):
+    logits = np.maximum(np.log(probs), -1e10).astype(np.float32)
+  keep_table = {0.1: [[1], [4]], 0.3: [[1], [4]], 0.4: [[1], [1, 2, 3, 4]],
+                0.8: [[1, 4], [1, 2, 3, 4]],
+                0.95: [[1, 3, 4], [1, 2, 3, 4, 5]]}
+  temps = dev(np.ones(2, np.float32))
+  for p, keep in keep_table.items():
+    for j in range(6):
+      g = np.zeros((2, 6), np.float32)
+      g[:, j] = 1000.0
+      tok, _ = ops.sample_tokens(dev(logits), dev(g), temps, 0, p, True)
+      for r in range(2):
+        survived = int(host(tok)[r]) == j
+        assert survived == (j in keep[r]), (p, r, j)
