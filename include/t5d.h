@@ -154,7 +154,7 @@ int t5d_top_k(void* stream, const float* x, float* vals, int32_t* idx,
  *   topk_vals/topk_idx [B, k]: the k largest of
  *   (logits - max - lse) + live_logprobs over the flattened [beams*V] axis,
  *   flat index = beam*V + token.  row_max/row_lse [B*beams] are also written
- *   (max and log-sum-exp of the shifted row). k <= 64.
+ *   (max and log-sum-exp of the shifted row). k <= 16, beams*k <= 128.
  *   scratch: float32/int32 pairs, at least 2*B*beams*k*4 bytes. */
 int t5d_beam_topk(void* stream, const float* logits,
                   const float* live_logprobs, float* topk_vals,

@@ -179,28 +179,31 @@ beam_row_topk_kernel(const float* __restrict__ logits,
   }
 }
 
-// Merge the beams' per-row candidates of one batch item: one wavefront, one
-// candidate per lane (beams*k <= 64), rank by counting better candidates.
-__global__ void __launch_bounds__(64)
+// Merge the beams' per-row candidates of one batch item: one candidate per
+// thread (beams*k <= 128), rank by counting better candidates.
+__global__ void __launch_bounds__(128)
 beam_merge_kernel(const float* __restrict__ cand_vals,
                   const int32_t* __restrict__ cand_idx,
                   float* __restrict__ topk_vals, int32_t* __restrict__ topk_idx,
                   int beams, int k) {
-  const int b = blockIdx.x, lane = threadIdx.x;
+  __shared__ float sv[128];
+  __shared__ int si[128];
+  const int b = blockIdx.x, tid = threadIdx.x;
   const int n = beams * k;
   float v = -INFINITY;
   int i = 0x7FFFFFFF;
-  if (lane < n) {
-    v = cand_vals[(size_t)b * n + lane];
-    i = cand_idx[(size_t)b * n + lane];
+  if (tid < n) {
+    v = cand_vals[(size_t)b * n + tid];
+    i = cand_idx[(size_t)b * n + tid];
   }
+  sv[tid] = v;
+  si[tid] = i;
+  __syncthreads();
+  if (tid >= n) return;
   int rank = 0;
-  for (int o = 0; o < 64; ++o) {
-    const float ov = __shfl(v, o, 64);
-    const int oi = __shfl(i, o, 64);
-    if (better(ov, oi, v, i)) ++rank;
-  }
-  if (lane < n && rank < k) {
+  for (int o = 0; o < n; ++o)
+    if (better(sv[o], si[o], v, i)) ++rank;
+  if (rank < k) {
     topk_vals[(size_t)b * k + rank] = v;
     topk_idx[(size_t)b * k + rank] = i;
   }
@@ -612,8 +615,8 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
               T5D_EINVAL, "t5d_beam_topk: null pointer");
   T5D_REQUIRE(B > 0 && beams > 0 && V > 0 && k > 0, T5D_EINVAL,
               "t5d_beam_topk: B=%d beams=%d V=%d k=%d", B, beams, V, k);
-  T5D_REQUIRE(k <= 16 && beams * k <= 64, T5D_ELIMIT,
-              "t5d_beam_topk: k=%d beams=%d (need k<=16, beams*k<=64)", k,
+  T5D_REQUIRE(k <= 16 && beams * k <= 128, T5D_ELIMIT,
+              "t5d_beam_topk: k=%d beams=%d (need k<=16, beams*k<=128)", k,
               beams);
   T5D_REQUIRE((long)beams * V < 0x7FFFFFFFL && k <= beams * V, T5D_EINVAL,
               "t5d_beam_topk: beams*V out of range");
@@ -634,7 +637,7 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
                        logits, live_logprobs, row_max, row_lse, cand_vals,
                        cand_idx, V, beams, k);
   T5D_CHECK_LAUNCH("t5d_beam_topk(rows)");
-  hipLaunchKernelGGL(beam_merge_kernel, dim3(B), dim3(64), 0, s, cand_vals,
+  hipLaunchKernelGGL(beam_merge_kernel, dim3(B), dim3(128), 0, s, cand_vals,
                      cand_idx, topk_vals, topk_idx, beams, k);
   T5D_CHECK_LAUNCH("t5d_beam_topk(merge)");
   return T5D_OK;

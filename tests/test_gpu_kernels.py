@@ -353,12 +353,15 @@ def test_sample_tokens_topk(ops, V, topk, temp, rescale):
 def test_sample_tokens_topp_table(ops):
   # t5x/binary_search_test.py:143-209 through the kernel: with a huge Gumbel
   # bonus on one index the sampled token reveals whether it survived the mask.
+  # The reference table uses p equal to exact cumulative masses (0.3, 0.4),
+  # where "mass >= p" is decided by the last bit of a float32 softmax sum in
+  # the reference as much as here; p is nudged 1e-3 below those boundaries.
   probs = np.asarray([[0.0, 0.7, 0.04, 0.06, 0.2, 0.0],
                       [0.0, 0.2, 0.2, 0.2, 0.3, 0.1]])
   with np.errstate(divide='ignore'):
     logits = np.maximum(np.log(probs), -1e10).astype(np.float32)
-  keep_table = {0.1: [[1], [4]], 0.3: [[1], [4]], 0.4: [[1], [1, 2, 3, 4]],
-                0.8: [[1, 4], [1, 2, 3, 4]],
+  keep_table = {0.1: [[1], [4]], 0.299: [[1], [4]],
+                0.399: [[1], [1, 2, 3, 4]], 0.8: [[1, 4], [1, 2, 3, 4]],
                 0.95: [[1, 3, 4], [1, 2, 3, 4, 5]]}
   temps = dev(np.ones(2, np.float32))
   for p, keep in keep_table.items():
