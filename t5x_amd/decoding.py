@@ -474,6 +474,132 @@ def beam_init(batch_size, beam_size, max_decode_len, cache, offset=0,
   return st, beam_cache
 
 
+class BeamLoop:
+  """The beam_search loop (:1131-1569) as an object: `cond()` / `body()` are
+  the while-loop's condition and body, `finish()` the epilogue.  beam_search()
+  below is `while loop.cond(): loop.body()`; exposing the pieces lets a caller
+  time or single-step the loop without re-implementing it."""
+
+  def __init__(self, inputs, cache, tokens_to_logits, eos_id: int,
+               num_decodes: int = 4, alpha: float = 0.6,
+               max_decode_len: Optional[int] = None, max_decode_step: int = -1,
+               min_log_prob: float = NEG_INF_VALUE, cache_offset: int = 0,
+               initial_index=None):
+    dev = _device()
+    self.tokens_to_logits = tokens_to_logits
+    self.eos_id = eos_id
+    self.cache_offset = cache_offset
+    self.max_decode_step = max_decode_step
+    self.min_log_prob = min_log_prob
+    inputs_np = _dev(inputs).cpu().numpy().astype(np.int32)
+    self.beam_size = beam_size = num_decodes
+    self.batch_size = batch_size = inputs_np.shape[0]
+    if max_decode_len is None:
+      max_decode_len = inputs_np.shape[1]
+    max_decode_len += 1  # :1208
+    self.max_decode_len = max_decode_len
+
+    self.right_aligned_input = None
+    live_seqs = None
+    if initial_index is not None:  # :1212-1235
+      initial_index_np = _dev(initial_index).cpu().numpy().astype(np.int32)
+      self.right_aligned_input = _right_align_prompts(inputs_np)
+      length = inputs_np.shape[1]
+      last = self.right_aligned_input[:, -1][:, None]
+      inputs_np = np.pad(last, ((0, 0), (0, length - 1)), constant_values=0)
+      live_seqs = np.pad(last, ((0, 0), (0, max_decode_len - 1)),
+                         constant_values=0)
+      live_seqs = np.ascontiguousarray(np.broadcast_to(
+          live_seqs[:, None, :], (batch_size, beam_size, max_decode_len)))
+    else:
+      initial_index_np = np.zeros((batch_size,), np.int32)
+
+    self.cur, self.beam_cache = beam_init(
+        batch_size, beam_size, max_decode_len, cache, cache_offset,
+        live_seqs=live_seqs, initial_index=initial_index_np)
+    self.nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
+    self.inputs_dev = torch.as_tensor(np.ascontiguousarray(inputs_np),
+                                      device=dev)
+    self.init_idx_dev = torch.as_tensor(initial_index_np, device=dev)
+    max_len_for_bp = max_decode_len + int(initial_index_np.max()) + 2
+    self.brevity = torch.as_tensor(
+        brevity_penalty(alpha, np.arange(max_len_for_bp, dtype=np.int32)),
+        device=dev).contiguous()
+    self.min_brevity = float(brevity_penalty(alpha, max_decode_len))  # :1268
+    self.min_initial = int(initial_index_np.min())
+    self.keep_going = torch.zeros((), dtype=torch.int32, device=dev)
+    self.top_alive = torch.empty((batch_size, beam_size), dtype=torch.int32,
+                                 device=dev)
+    self.topk_bufs = None
+    self.vocab_size = None
+    self.step = 0
+
+  def cond(self) -> bool:
+    """:1250-1300 (reads one flag back from the device)."""
+    ops.beam_cond(self.cur, self.min_brevity, self.min_log_prob,
+                  self.max_decode_step, self.min_initial, self.keep_going)
+    return bool(self.keep_going.item())
+
+  def body(self):
+    """:1302-1506."""
+    cur, nxt = self.cur, self.nxt
+    B, K, dev = self.batch_size, self.beam_size, cur.live_seqs.device
+    step, off = self.step, self.cache_offset
+    flat_ids = flatten_beam_dim(cur.live_seqs[:, :, step:step + 1])
+    flat_cache = cache_map(functools.partial(flatten_beam_dim, offset=off),
+                           self.beam_cache)
+    decoding_state = DecodingState(
+        cur_index=cur.cur_index, sequences=flatten_beam_dim(cur.live_seqs),
+        cur_token=flat_ids, cache=flat_cache)
+    flat_logits, new_flat_cache = self.tokens_to_logits(decoding_state)
+    flat_logits = _dev(flat_logits, torch.float32).contiguous()
+    if self.vocab_size is None:
+      self.vocab_size = flat_logits.shape[-1]
+      R, k2 = B * K, 2 * K
+      self.topk_bufs = (
+          torch.empty((B, k2), dtype=torch.float32, device=dev),
+          torch.empty((B, k2), dtype=torch.int32, device=dev),
+          torch.empty((R,), dtype=torch.float32, device=dev),
+          torch.empty((R,), dtype=torch.float32, device=dev),
+          torch.empty((2 * R * k2,), dtype=torch.int32, device=dev))
+    new_cache = cache_map(lambda x: unflatten_beam_dim(x, B, K, off),
+                          new_flat_cache)
+    # :1340-1366 log_softmax + prefix add + top-2K over beam x vocab
+    topk_vals, topk_idx, _, _ = ops.beam_topk(flat_logits, cur.live_logprobs,
+                                              2 * K, self.topk_bufs)
+    # :1366-1506 everything after the top-k
+    ops.beam_update(cur, nxt, topk_vals, topk_idx, self.inputs_dev,
+                    self.init_idx_dev, self.brevity, self.top_alive,
+                    self.vocab_size, self.eos_id)
+    # :1449-1457.  After this step the caches hold step + 1 valid columns.
+    self.beam_cache = cache_gather_beams(new_cache, self.top_alive, B, K, K,
+                                         True, off)
+    self.cur, self.nxt = nxt, cur
+    self.step += 1
+
+  def finish(self):
+    """:1513-1569."""
+    cur, dev = self.cur, self.cur.live_seqs.device
+    # batch items with no finished sequence fall back to the live ones
+    any_finished = cur.finished_flags.bool().any(dim=1)
+    finished_seqs = torch.where(any_finished[:, None, None], cur.finished_seqs,
+                                cur.live_seqs)
+    finished_scores = torch.where(any_finished[:, None], cur.finished_scores,
+                                  cur.live_logprobs)
+    if self.right_aligned_input is not None:  # :1532-1564
+      seqs = finished_seqs.cpu().numpy()[:, :, 1:]
+      prompt = np.broadcast_to(
+          self.right_aligned_input[:, None, :],
+          (self.batch_size, seqs.shape[1], self.right_aligned_input.shape[-1]))
+      seqs = np.concatenate([prompt, seqs], axis=-1)
+      flat = _left_align_prompts(seqs.reshape(-1, seqs.shape[-1]))
+      seqs = flat.reshape(seqs.shape)[:, :, :self.max_decode_len - 1]
+      finished_seqs = torch.as_tensor(np.ascontiguousarray(seqs), device=dev)
+    else:
+      finished_seqs = finished_seqs[:, :, 1:]  # :1567
+    return finished_seqs, finished_scores
+
+
 def beam_search(
     inputs, cache, tokens_to_logits, eos_id: int, num_decodes: int = 4,
     alpha: float = 0.6, max_decode_len: Optional[int] = None,
@@ -483,103 +609,9 @@ def beam_search(
   """:1131-1569 -> (sequences [B, K, L] i32, scores [B, K] f32), the beam axis
   sorted ascending by score."""
   del decode_rng
-  dev = _device()
-  inputs_np = _dev(inputs).cpu().numpy().astype(np.int32)
-  beam_size = num_decodes
-  batch_size = inputs_np.shape[0]
-  if max_decode_len is None:
-    max_decode_len = inputs_np.shape[1]
-  max_decode_len += 1  # :1208
-
-  right_aligned_input = None
-  live_seqs = None
-  if initial_index is not None:  # :1212-1235
-    initial_index_np = _dev(initial_index).cpu().numpy().astype(np.int32)
-    right_aligned_input = _right_align_prompts(inputs_np)
-    length = inputs_np.shape[1]
-    last = right_aligned_input[:, -1][:, None]
-    inputs_np = np.pad(last, ((0, 0), (0, length - 1)), constant_values=0)
-    live_seqs = np.pad(last, ((0, 0), (0, max_decode_len - 1)),
-                       constant_values=0)
-    live_seqs = np.ascontiguousarray(np.broadcast_to(
-        live_seqs[:, None, :], (batch_size, beam_size, max_decode_len)))
-  else:
-    initial_index_np = np.zeros((batch_size,), np.int32)
-
-  cur, beam_cache = beam_init(batch_size, beam_size, max_decode_len, cache,
-                              cache_offset, live_seqs=live_seqs,
-                              initial_index=initial_index_np)
-  nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
-  inputs_dev = torch.as_tensor(np.ascontiguousarray(inputs_np), device=dev)
-  init_idx_dev = torch.as_tensor(initial_index_np, device=dev)
-  max_len_for_bp = max_decode_len + int(initial_index_np.max()) + 2
-  brevity = torch.as_tensor(
-      brevity_penalty(alpha, np.arange(max_len_for_bp, dtype=np.int32)),
-      device=dev).contiguous()
-  min_brevity = float(brevity_penalty(alpha, max_decode_len))  # :1268
-  min_initial = int(initial_index_np.min())
-  keep_going = torch.zeros((), dtype=torch.int32, device=dev)
-  top_alive = torch.empty((batch_size, beam_size), dtype=torch.int32,
-                          device=dev)
-  topk_bufs = None
-  vocab_size = None
-
-  def cond(state):  # :1250-1300
-    ops.beam_cond(state, min_brevity, min_log_prob, max_decode_step,
-                  min_initial, keep_going)
-    return bool(keep_going.item())
-
-  step = 0
-  while cond(cur):  # :1509
-    flat_ids = flatten_beam_dim(cur.live_seqs[:, :, step:step + 1])
-    flat_cache = cache_map(
-        functools.partial(flatten_beam_dim, offset=cache_offset), beam_cache)
-    decoding_state = DecodingState(
-        cur_index=cur.cur_index, sequences=flatten_beam_dim(cur.live_seqs),
-        cur_token=flat_ids, cache=flat_cache)
-    flat_logits, new_flat_cache = tokens_to_logits(decoding_state)
-    flat_logits = _dev(flat_logits, torch.float32).contiguous()
-    if vocab_size is None:
-      vocab_size = flat_logits.shape[-1]
-      R, k2 = batch_size * beam_size, 2 * beam_size
-      topk_bufs = (torch.empty((batch_size, k2), dtype=torch.float32,
-                               device=dev),
-                   torch.empty((batch_size, k2), dtype=torch.int32,
-                               device=dev),
-                   torch.empty((R,), dtype=torch.float32, device=dev),
-                   torch.empty((R,), dtype=torch.float32, device=dev),
-                   torch.empty((2 * R * k2,), dtype=torch.int32, device=dev))
-    new_cache = cache_map(
-        lambda x: unflatten_beam_dim(x, batch_size, beam_size, cache_offset),
-        new_flat_cache)
-    # :1340-1366 log_softmax + prefix add + top-2K over beam x vocab
-    topk_vals, topk_idx, _, _ = ops.beam_topk(flat_logits, cur.live_logprobs,
-                                              2 * beam_size, topk_bufs)
-    # :1366-1506 everything after the top-k
-    ops.beam_update(cur, nxt, topk_vals, topk_idx, inputs_dev, init_idx_dev,
-                    brevity, top_alive, vocab_size, eos_id)
-    # :1449-1457
-    beam_cache = cache_gather_beams(new_cache, top_alive, batch_size,
-                                    beam_size, beam_size, True, cache_offset)
-    cur, nxt = nxt, cur
-    step += 1
-
-  # :1516-1528 batch items with no finished sequence fall back to live ones
-  any_finished = cur.finished_flags.bool().any(dim=1)
-  finished_seqs = torch.where(any_finished[:, None, None], cur.finished_seqs,
-                              cur.live_seqs)
-  finished_scores = torch.where(any_finished[:, None], cur.finished_scores,
-                                cur.live_logprobs)
-
-  if right_aligned_input is not None:  # :1532-1564
-    seqs = finished_seqs.cpu().numpy()[:, :, 1:]
-    prompt = np.broadcast_to(
-        right_aligned_input[:, None, :],
-        (batch_size, seqs.shape[1], right_aligned_input.shape[-1]))
-    seqs = np.concatenate([prompt, seqs], axis=-1)
-    flat = _left_align_prompts(seqs.reshape(-1, seqs.shape[-1]))
-    seqs = flat.reshape(seqs.shape)[:, :, :max_decode_len - 1]
-    finished_seqs = torch.as_tensor(np.ascontiguousarray(seqs), device=dev)
-  else:
-    finished_seqs = finished_seqs[:, :, 1:]  # :1567
-  return finished_seqs, finished_scores
+  loop = BeamLoop(inputs, cache, tokens_to_logits, eos_id, num_decodes, alpha,
+                  max_decode_len, max_decode_step, min_log_prob, cache_offset,
+                  initial_index)
+  while loop.cond():  # :1509
+    loop.body()
+  return loop.finish()

@@ -271,8 +271,13 @@ class Transformer:
     a stride."""
     cfg, dev = self.config, self._dev()
     act = _TORCH_DTYPE[cfg.dtype]
+    # Rows are read in 16-byte chunks: a length that is not a multiple of 8
+    # (bf16) / 4 (f32) positions is padded up; the extra columns are never
+    # attended to (they lie beyond every cache_index).
+    el = 16 // torch.empty((), dtype=act).element_size()
+    length = (max_decode_length + el - 1) // el * el
     kv = torch.zeros((cfg.num_decoder_layers, 2, batch, cfg.num_heads,
-                      cfg.head_dim, max_decode_length), dtype=act, device=dev)
+                      cfg.head_dim, length), dtype=act, device=dev)
     idx = torch.zeros((cfg.num_decoder_layers,), dtype=torch.int32, device=dev)
     return {'decoder': {
         f'layers_{i}': {'self_attention': {
@@ -367,8 +372,8 @@ class Transformer:
       c = cache['decoder'][f'layers_{i}']['self_attention']
       ck, cv, ci = c['cached_key'], c['cached_value'], c['cache_index']
       L = ck.shape[-1]
-      if max_decode_length and L != max_decode_length:
-        raise ValueError(f'cache length {L} != max_decode_length '
+      if max_decode_length and L < max_decode_length:
+        raise ValueError(f'cache length {L} < max_decode_length '
                          f'{max_decode_length}')
       index_leaves.append(ci)
       ops.rmsnorm(x, lw['ln_self'], b.xn)
@@ -400,3 +405,54 @@ class Transformer:
         ops.add_i32(ci, 1)
     logits = b.logits.view(R, 1, cfg.vocab_size)
     return (logits, {'cache': cache}) if mutable else logits
+
+
+def init_params(cfg: T5Config, seed: int = 0, device=None,
+                with_encoder: bool = True):
+  """Synthetic random-init parameters in the reference tree layout, generated
+  on the device: every dense kernel normal(0, 1/sqrt(fan_in)) (query kernels
+  additionally / sqrt(head_dim), as the reference initialiser does,
+  t5x/examples/t5/layers.py:207-211), embedding normal(0, 1), norm scales
+  1 + 0.1 normal, relative-position table 0.5 normal."""
+  device = device or torch.device('cuda')
+  gen = torch.Generator(device=device)
+  gen.manual_seed(seed)
+  d, hd, f = cfg.emb_dim, cfg.num_heads * cfg.head_dim, cfg.mlp_dim
+
+  def w(k, n, scale=None):
+    t = torch.randn((k, n), generator=gen, device=device, dtype=torch.float32)
+    return t * (scale if scale is not None else 1.0 / np.sqrt(k))
+
+  def norm():
+    return {'scale': 1.0 + 0.1 * torch.randn((d,), generator=gen,
+                                             device=device)}
+
+  def attn():
+    return {'query': {'kernel': w(d, hd) / np.sqrt(cfg.head_dim)},
+            'key': {'kernel': w(d, hd)}, 'value': {'kernel': w(d, hd)},
+            'out': {'kernel': w(hd, d)}}
+
+  def mlp():
+    return {'wi_0': {'kernel': w(d, f)}, 'wi_1': {'kernel': w(d, f)},
+            'wo': {'kernel': w(f, d)}}
+
+  params = {'token_embedder': {'embedding': w(cfg.vocab_size, d, 1.0)}}
+  if with_encoder:
+    enc = {'relpos_bias': {'rel_embedding': w(cfg.num_heads, 32, 0.5)},
+           'encoder_norm': norm()}
+    for i in range(cfg.num_encoder_layers):
+      enc[f'layers_{i}'] = {'pre_attention_layer_norm': norm(),
+                            'attention': attn(), 'pre_mlp_layer_norm': norm(),
+                            'mlp': mlp()}
+    params['encoder'] = enc
+  dec = {'relpos_bias': {'rel_embedding': w(cfg.num_heads, 32, 0.5)},
+         'decoder_norm': norm(),
+         'logits_dense': {'kernel': w(d, cfg.vocab_size)}}
+  for i in range(cfg.num_decoder_layers):
+    dec[f'layers_{i}'] = {
+        'pre_self_attention_layer_norm': norm(), 'self_attention': attn(),
+        'pre_cross_attention_layer_norm': norm(),
+        'encoder_decoder_attention': attn(),
+        'pre_mlp_layer_norm': norm(), 'mlp': mlp()}
+  params['decoder'] = dec
+  return params

@@ -415,3 +415,41 @@ def test_end_to_end_tiny_model_greedy_matches_full_forward_argmax():
   encoded = t5.encode(params, cfg, enc)
   full = t5.decode(params, cfg, encoded, enc, dec_in, np.ones_like(dec_in))
   np.testing.assert_array_equal(out, full.argmax(-1))
+
+
+def test_bf16_pipeline_sensitivity(monkeypatch):
+  """The bf16 oracle against itself with only the matmul accumulation changed
+  (float64 instead of float32 sums): same inputs, same rounding points, yet
+  logits move by ~1e-2.  This is the noise floor any bf16 implementation is
+  compared at; float32 activations do not show it."""
+  cfg = tiny_cfg('bfloat16', emb_dim=256, num_heads=4, head_dim=64,
+                 mlp_dim=512, vocab_size=512, num_decoder_layers=3)
+  params = t5.init_params(cfg, seed=1)
+  rs = np.random.RandomState(0)
+  b, e, l = 8, 12, 6
+  enc_tokens = rs.randint(2, cfg.vocab_size, size=(b, e))
+  encoded = t5.encode(params, cfg, enc_tokens)
+  tok = rs.randint(2, cfg.vocab_size, size=(b, 1))
+
+  def run():
+    cache = t5.init_cache(cfg, b, l)
+    for _ in range(3):
+      logits, cache = t5.decode(params, cfg, encoded, enc_tokens, tok, tok,
+                                decode=True, cache=cache, max_decode_length=l)
+    return logits
+
+  base = run()
+  real = t5.dense_general
+
+  def dense64(x, kernel, dtype, out_dtype=None):
+    if isinstance(kernel, dict):
+      return real(x, kernel, dtype, out_dtype)
+    y = t5.cast(x, dtype).astype(np.float64) @ t5.cast(kernel, dtype).astype(
+        np.float64)
+    return t5.cast(y.astype(np.float32), out_dtype or dtype)
+
+  monkeypatch.setattr(t5, 'dense_general', dense64)
+  other = run()
+  err = np.abs(base - other)
+  assert 1e-4 < err.max() < 6e-2, err.max()
+  assert err.mean() < 5e-3
