@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Decode-path benchmark: T5.1.1-base, beam_search with 4 beams, batch 32,
+encoder length 512 (rows 128..512 valid), max decode length 128, bf16, on one
+MI355X.  Synthetic random-init weights and seeded synthetic tokens.
+
+A "step" is one iteration of the beam-search loop: one decoder forward for the
+128 beam rows, log_softmax + top-2K over beam x vocab, beam bookkeeping, cache
+reorder and the loop-condition check.  `value` = batch * steps / seconds
+(decoded tokens per second: every batch item emits one token per step).  The
+encoder output is synthetic and the cross-attention K/V projection, weight
+packing and upload happen before the timed region.
+
+Prints ONE JSON line.  `roofline` describes the dominant HBM-bound kernel of
+the step, timed live with HIP events on the launch stream; `cpu_baseline` is the
+NumPy oracle (a port of the reference algorithm, not the reference itself) on
+this host's cores over a bounded sample of the same workload.
+"""
+
+import argparse
+import functools
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor peak
+
+CONFIGS = {
+    # name: (size, batch, beams, enc_len, enc_min_len, max_decode_len, dtype,
+    #        weight_dtype)
+    'base-beam4': ('base', 32, 4, 512, 128, 128, 'bfloat16', None),
+    'xl-int8-beam4': ('xl', 16, 4, 512, 512, 128, 'bfloat16', 'int8'),
+    'large-greedy': ('large', 64, 1, 512, 512, 256, 'bfloat16', None),
+}
+
+
+def parse_args():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--gpus', type=int, default=1)
+  ap.add_argument('--steps', type=int, default=256)
+  ap.add_argument('--warmup', type=int, default=128)
+  ap.add_argument('--config', default='base-beam4', choices=sorted(CONFIGS))
+  ap.add_argument('--seed', type=int, default=0)
+  ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--cpu-steps', type=int, default=3,
+                  help='decode steps of the CPU oracle sample')
+  return ap.parse_args()
+
+
+class Workload:
+  """Synthetic batch + model state for repeated full decodes."""
+
+  def __init__(self, name, seed):
+    import torch
+    from t5x_amd import decoding, models, network
+    self.torch, self.decoding = torch, decoding
+    size, B, K, E, Emin, L, dtype, wdt = CONFIGS[name]
+    self.name, self.B, self.K, self.E, self.L = name, B, K, E, L
+    self.cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
+    dev = torch.device('cuda')
+    self.params = network.init_params(self.cfg, seed, dev, with_encoder=False)
+    self.module = network.Transformer(self.cfg, dev)
+    self.model = models.EncoderDecoderModel(self.module,
+                                            decode_fn=decoding.beam_search)
+    rs = np.random.Generator(np.random.PCG64(seed + 1))
+    tok = rs.integers(2, 32128, size=(B, E)).astype(np.int32)
+    lens = rs.integers(Emin, E + 1, size=(B,))
+    tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+    self.enc_lens = lens
+    self.enc_tokens = torch.as_tensor(tok, device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed + 2)
+    self.encoded = torch.randn((B, E, self.cfg.emb_dim), generator=gen,
+                               device=dev).to(network._TORCH_DTYPE[dtype])
+    self.inputs = np.zeros((B, L), np.int32)
+    self.tokens_to_logits = functools.partial(
+        self.model._compute_logits_from_slice, params=self.params,
+        encoded_inputs=network.BeamShared(self.encoded, K),
+        raw_inputs=network.BeamShared(self.enc_tokens, K),
+        max_decode_length=L)
+    self.weights = self.module.decoder_weights(self.params)
+    self.loop = None
+
+  def new_decode(self):
+    cache = self.module.init_cache(self.B, self.L)
+    self.loop = self.decoding.BeamLoop(
+        self.inputs, cache, self.tokens_to_logits, eos_id=1,
+        num_decodes=self.K, alpha=0.6)
+
+  def run_steps(self, n):
+    """Runs exactly n loop iterations, starting new decodes as needed."""
+    done = 0
+    while done < n:
+      if self.loop is None or not self.loop.cond():
+        self.new_decode()
+        if not self.loop.cond():
+          raise RuntimeError('fresh decode terminated immediately')
+      self.loop.body()
+      done += 1
+
+  # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
+  def cross_attention_bytes(self):
+    s = 2  # bf16
+    hd = self.cfg.num_heads * self.cfg.head_dim
+    R = self.B * self.K
+    return int(self.enc_lens.sum()) * hd * 2 * s + 2 * R * hd * s
+
+  def self_attention_bytes(self, t):
+    s = 2
+    hd = self.cfg.num_heads * self.cfg.head_dim
+    R = self.B * self.K
+    return R * hd * (t + 1) * 2 * s + R * hd * 2 * s + 2 * R * hd * s
+
+
+def time_kernel(torch, fn, reps):
+  """Average duration of `fn`'s single kernel launch, HIP events on the
+  current (launch) stream around `reps` back-to-back launches."""
+  fn()
+  torch.cuda.synchronize()
+  start = torch.cuda.Event(enable_timing=True)
+  end = torch.cuda.Event(enable_timing=True)
+  start.record()
+  for _ in range(reps):
+    fn()
+  end.record()
+  end.synchronize()
+  return start.elapsed_time(end) * 1e-3 / reps
+
+
+def roofline_cross_attention(w):
+  """The step's largest single stream of HBM bytes per launch: cross-attention
+  over the encoder K/V (12 launches per step, same shape every step)."""
+  from t5x_amd import ops
+  torch = w.torch
+  cross = w.module._cross[1]
+  R = w.B * w.K
+  hd = w.cfg.num_heads * w.cfg.head_dim
+  q = torch.randn((R, hd), device='cuda').to(w.encoded.dtype)
+  out = torch.empty_like(q)
+  nl = len(cross['k'])
+  state = {'i': 0}
+
+  def launch():
+    i = state['i'] = (state['i'] + 1) % nl  # walk the layers: no cache reuse
+    ops.cross_attention_step(q, cross['k'][i], cross['v'][i], cross['enc_len'],
+                             w.K, out)
+
+  sec = time_kernel(torch, launch, 20 * nl)
+  nbytes = w.cross_attention_bytes()
+  achieved = nbytes / sec / 1e9
+  return {'kernel': 'attn_step_kernel<bf16,NQ=4,cross>', 'bound': 'hbm',
+          'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS,
+          'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBPS, 4),
+          'traffic': None, 'bytes_per_launch': nbytes,
+          'avg_launch_us': round(sec * 1e6, 2)}
+
+
+def cpu_baseline(name, steps, seed):
+  """NumPy oracle on this host: `steps` beam-search iterations at the same
+  shape (decoder only, cross K/V hoisted as in the GPU path)."""
+  from oracle import decoding as odec
+  from oracle import t5 as ot5
+  size, B, K, E, Emin, L, dtype, wdt = CONFIGS[name]
+  from t5x_amd import network
+  kw = dict(network.T5_1_1[size])
+  kw['num_encoder_layers'] = 0
+  cfg = ot5.T5Config(dtype=dtype, **kw)
+  params = ot5.init_params(cfg, seed, with_encoder=False)
+  rs = np.random.Generator(np.random.PCG64(seed + 1))
+  tok = rs.integers(2, 32128, size=(B, E)).astype(np.int32)
+  lens = rs.integers(Emin, E + 1, size=(B,))
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  encoded = ot5.bf16_round(
+      rs.standard_normal((B, E, cfg.emb_dim), dtype=np.float32))
+  cross_kv = ot5.project_cross_kv(params, cfg, encoded)
+  cross_kv = [(np.repeat(k, K, 0), np.repeat(v, K, 0)) for k, v in cross_kv]
+  enc_tok_rows = np.repeat(tok, K, axis=0)
+  calls = {'n': 0, 't0': None}
+
+  def tokens_to_logits(state):
+    if calls['t0'] is None:
+      calls['t0'] = time.perf_counter()
+    calls['n'] += 1
+    t = state.cur_token
+    logits, cache = ot5.decode(params, cfg, None, enc_tok_rows, t, t,
+                               decode=True, cache=state.cache,
+                               max_decode_length=L, cross_kv=cross_kv)
+    return logits[:, 0], cache
+
+  inputs = np.zeros((B, L), np.int32)
+  odec.beam_search(inputs, ot5.init_cache(cfg, B, L), tokens_to_logits, 1,
+                   num_decodes=K, alpha=0.6, max_decode_step=steps)
+  sec = time.perf_counter() - calls['t0']
+  try:
+    from threadpoolctl import threadpool_info
+    threads = max([p.get('num_threads', 1) for p in threadpool_info()] or [1])
+  except Exception:  # pylint: disable=broad-except
+    threads = os.cpu_count() or 1
+  return {'value': round(B * calls['n'] / sec, 2), 'unit': 'tokens/s',
+          'cores': int(threads), 'kind': 'port',
+          'sample': f'{calls["n"]} beam-search steps of {name} (NumPy oracle, '
+                    f'decoder only, {sec:.1f} s)'}
+
+
+def main():
+  args = parse_args()
+  if args.gpus != 1:
+    print('bench.py: this build measures ONE GPU; --gpus must be 1 '
+          f'(got {args.gpus}). The decode path shards over batch with no '
+          'exchange; see DESIGN.md.', file=sys.stderr)
+    sys.exit(2)
+  import torch
+  if not torch.cuda.is_available():
+    print('bench.py: no GPU visible', file=sys.stderr)
+    sys.exit(3)
+  w = Workload(args.config, args.seed)
+  w.run_steps(args.warmup)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  w.run_steps(args.steps)
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+
+  size, B, K, E, Emin, L, dtype, wdt = CONFIGS[args.config]
+  out = {
+      'metric': 'decoded tokens/sec, T5.1.1-base beam=4 on 1 GPU',
+      'value': round(B * args.steps / elapsed, 1),
+      'unit': 'tokens/s',
+      'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+      'ms_per_step': round(elapsed / args.steps * 1e3, 4),
+      'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+      'dtype': 'bf16' if wdt is None else f'bf16 act / {wdt} weights',
+      'data': 'synthetic',
+      'config': {'workload': f'T5.1.1-{size} beam_search decode loop: batch '
+                             f'{B} x {K} beams, encoder {E} ({Emin}..{E} '
+                             f'valid), max decode length {L}',
+                 'name': args.config, 'beam_rows': B * K,
+                 'rows_x_steps_per_s': round(B * K * args.steps / elapsed, 1)},
+      'roofline': roofline_cross_attention(w),
+  }
+  if not args.no_cpu_baseline:
+    out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
+  print(json.dumps(out))
+
+
+if __name__ == '__main__':
+  main()
