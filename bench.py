@@ -75,11 +75,9 @@ class Workload:
     self.encoded = torch.randn((B, E, self.cfg.emb_dim), generator=gen,
                                device=dev).to(network._TORCH_DTYPE[dtype])
     self.inputs = np.zeros((B, L), np.int32)
-    self.tokens_to_logits = functools.partial(
-        self.model._compute_logits_from_slice, params=self.params,
-        encoded_inputs=network.BeamShared(self.encoded, K),
-        raw_inputs=network.BeamShared(self.enc_tokens, K),
-        max_decode_length=L)
+    self.tokens_to_logits = models.StepFunction(
+        self.model, self.params, network.BeamShared(self.encoded, K),
+        network.BeamShared(self.enc_tokens, K), L)
     self.weights = self.module.decoder_weights(self.params)
     self.loop = None
 
@@ -90,15 +88,31 @@ class Workload:
         num_decodes=self.K, alpha=0.6)
 
   def run_steps(self, n):
-    """Runs exactly n loop iterations, starting new decodes as needed."""
+    """Runs exactly n loop iterations, starting a new decode whenever the
+    current one has produced its max_decode_len tokens.  The loop condition is
+    evaluated on the device after every iteration; it is read back once per
+    decode (with these random-init weights no batch item ever finishes early,
+    which the read-back at the end of each decode verifies)."""
     done = 0
     while done < n:
-      if self.loop is None or not self.loop.cond():
+      if self.loop is None or self.loop.step >= self.L:
+        if self.loop is not None:
+          if self.loop.cond():
+            raise RuntimeError('decode did not stop at max_decode_len')
+          self.check_full_decode()
         self.new_decode()
         if not self.loop.cond():
           raise RuntimeError('fresh decode terminated immediately')
-      self.loop.body()
-      done += 1
+      take = min(n - done, self.L - self.loop.step)
+      for _ in range(take):
+        self.loop.body()
+      done += take
+
+  def check_full_decode(self):
+    cur_index = int(self.loop.cur.cur_index.item())
+    if cur_index != self.L:
+      raise RuntimeError(f'decode stopped early at step {cur_index}; the '
+                         'step count of this run would be wrong')
 
   # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
   def cross_attention_bytes(self):
@@ -137,7 +151,7 @@ def roofline_cross_attention(w):
   cross = w.module._cross[1]
   R = w.B * w.K
   hd = w.cfg.num_heads * w.cfg.head_dim
-  q = torch.randn((R, hd), device='cuda').to(w.encoded.dtype)
+  q = (0.125 * torch.randn((R, hd), device='cuda')).to(w.encoded.dtype)
   out = torch.empty_like(q)
   nl = len(cross['k'])
   state = {'i': 0}

@@ -86,9 +86,9 @@ int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
  *   out_dtype: dtype of C (T5D_F32 for the logits layer,
  *   t5x/examples/t5/network.py:286-291).
  *   T5D_EPI_GEGLU: W is a geglu-packed [K, 2F] kernel, N = 2F, C is [M, F].
- *   workspace/counters: float32 [split_k_max * M * N] scratch and int32
- *   [N/16] zero-initialised counters, needed when the call splits K over
- *   workgroups (t5d_gemm_workspace_bytes > 0); counters are left zeroed. */
+ *   workspace/counters: reserved for kernel variants that need scratch
+ *   memory; t5d_gemm_workspace_bytes currently returns 0 for every shape and
+ *   both may be NULL. */
 int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M, int K, int N);
 int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
              const void* A, const void* W, const float* scales,
@@ -114,7 +114,10 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
 /* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
  * mask :366-370).  The reference re-projects K/V from the beam-expanded
  * encoder output every step; here they are projected once per batch item:
- *   cross_key / cross_value [B, H, 64, E], shared by the item's `beams` rows;
+ *   cross_key [B, H, E, 64] (head dim contiguous) and cross_value
+ *   [B, H, 64, E] (positions contiguous), shared by the item's `beams` rows
+ *   (<= 8); these are the layouts in which a 16-byte chunk is directly an MFMA
+ *   operand of Q.K^T and P.V respectively.  E a multiple of 8 (bf16) / 4 (f32).
  *   enc_len [B]: number of leading valid (non-padding) encoder positions.
  *   q [B*beams, H*64] -> out [B*beams, H*64]. */
 int t5d_cross_attention_step(void* stream, int dtype, const void* q,
@@ -174,8 +177,8 @@ typedef struct {
 /* Everything in the beam_search loop body after the top-2K
  * (t5x/decoding.py:1366-1506): prompt forcing, sequence gather + token write,
  * EOS handling, second top-K with flip, brevity-penalised finished pool merge.
- *   in/out: `cur` is read, `next` is written (distinct buffers);
- *   next.cur_index = cur.cur_index + 1.
+ *   in/out: `cur` is read, `next` is written; they may be the same buffers
+ *   (in-place update).  next.cur_index = cur.cur_index + 1.
  *   inputs [B, Lin] prompt tokens; initial_index [B];
  *   brevity [S + max(initial_index) + 1] f32: ((5+len)/6)^alpha by length.
  *   top_alive_indices [B, K] (out): source beam of each surviving beam, the
@@ -223,6 +226,93 @@ int t5d_sample_update(void* stream, const int32_t* tokens,
                       float* log_prob, const int32_t* max_decode_len,
                       const int32_t* initial_eos_count, int32_t* all_ended,
                       int R, int S, int eos_id);
+
+/* ids[r] = live_seqs[r, *cur_index]: the token each beam row feeds to the
+ * decoder this step (t5x/decoding.py:1308-1312). live_seqs [R, S]. */
+int t5d_gather_step_ids(void* stream, const int32_t* live_seqs,
+                        const int32_t* cur_index, int32_t* ids, int R, int S);
+
+/* ---- fused entry points --------------------------------------------------
+ * One host call enqueues a whole decoder step / beam-search iteration, so the
+ * host pays one FFI crossing per step instead of one per kernel, and the call
+ * can be captured into a HIP graph once and replayed.
+ * The structs hold device pointers and are read at call time only. */
+
+typedef struct {
+  /* norm scales [d] (act dtype); kernels packed with t5d_pack_weight (or
+   * row-major float32), int8 scales or NULL */
+  const void *ln_self, *qkv, *self_out, *ln_cross, *cross_q, *cross_out,
+      *ln_mlp, *wi, *wo;
+  const float *qkv_scales, *self_out_scales, *cross_q_scales,
+      *cross_out_scales, *wi_scales, *wo_scales;
+  void *cached_key, *cached_value;        /* [R, H, 64, L] */
+  const void *cross_key;                  /* [B, H, E, 64] */
+  const void *cross_value;                /* [B, H, 64, E] */
+} t5d_layer;
+
+typedef struct {
+  int dtype, w_dtype;
+  int d, H, F, V, L, E, NL;   /* emb, heads, mlp, vocab, cache len, enc len */
+  int R, B, beams;            /* R = B * beams decoder rows */
+  const void* embedding;      /* [V, d] act dtype */
+  const void* rel_bias;       /* [H, L] act dtype, by distance */
+  const void* ln_final;
+  const void* logits_w;
+  const float* logits_scales;
+  const t5d_layer* layers;    /* HOST array of NL entries */
+  int32_t* cache_index;       /* [NL] device, consecutive */
+  const int32_t* enc_len;     /* [B] */
+  void *x, *x1, *x2, *xn;     /* [R, d] activations */
+  void *qkv;                  /* [R, 3*H*64] */
+  void *q, *ao;               /* [R, H*64] */
+  void *h;                    /* [R, F] */
+  float* logits;              /* [R, V] (out) */
+  /* optional device flag: when non-NULL and 0, every kernel of the step
+   * returns immediately (the step becomes a no-op) */
+  const int32_t* gate;
+} t5d_model_step;
+
+/* One decoder step for R rows (Decoder.__call__ with decode=True,
+ * t5x/examples/t5/network.py:229-292, as driven by
+ * _compute_logits_from_slice, t5x/models.py:484-515): ids [R] -> logits,
+ * caches updated in place, every cache_index advanced by one. */
+int t5d_decoder_step(void* stream, const t5d_model_step* model,
+                     const int32_t* ids);
+
+typedef struct {
+  t5d_beam_state state;        /* updated in place */
+  const int32_t* inputs;       /* [B, Lin] */
+  const int32_t* initial_index;/* [B] */
+  const float* brevity;        /* by length */
+  int32_t* top_alive;          /* [B, K] */
+  float* topk_vals;            /* [B, 2K] */
+  int32_t* topk_idx;           /* [B, 2K] */
+  float *row_max, *row_lse;    /* [R] */
+  void* scratch;               /* 2*R*2K*4 bytes */
+  int32_t* ids;                /* [R] */
+  int32_t* keep_going;         /* loop flag; must equal model->gate */
+  int S, Lin, eos_id;
+  float min_brevity, min_log_prob;
+  int max_decode_step, min_initial_index;
+  void* kv_base;               /* first cache tensor [B, K, H, 64, L] */
+  int64_t kv_tensor_stride_bytes;
+  int n_kv_tensors;            /* 2 * NL when all layers share one block */
+} t5d_beam_step;
+
+/* One iteration of the beam_search loop body plus the loop condition
+ * (t5x/decoding.py:1250-1506): gather ids, decoder step, log_softmax + top-2K,
+ * bookkeeping, cache reorder over the valid prefix, condition -> *keep_going.
+ * Every kernel is gated on *keep_going, so iterations enqueued after the
+ * condition turned false leave all state untouched. */
+int t5d_beam_search_step(void* stream, const t5d_model_step* model,
+                         const t5d_beam_step* beam);
+
+/* HIP graph capture on `stream` (must not be the null stream):
+ * begin, enqueue any t5d calls, end -> executable graph; launch replays it. */
+int t5d_graph_begin(void* stream);
+int t5d_graph_end(void* stream, void** graph_exec);
+int t5d_graph_launch(void* graph_exec, void* stream);
+int t5d_graph_destroy(void* graph_exec);
 
 #ifdef __cplusplus
 }

@@ -24,8 +24,48 @@ class BeamStatePtrs(Structure):
               ('finished_seqs', c_void_p), ('finished_flags', c_void_p)]
 
 
+class Layer(Structure):
+  """t5d_layer."""
+  _fields_ = [(n, c_void_p) for n in (
+      'ln_self', 'qkv', 'self_out', 'ln_cross', 'cross_q', 'cross_out',
+      'ln_mlp', 'wi', 'wo', 'qkv_scales', 'self_out_scales', 'cross_q_scales',
+      'cross_out_scales', 'wi_scales', 'wo_scales', 'cached_key',
+      'cached_value', 'cross_key', 'cross_value')]
+
+
+class ModelStep(Structure):
+  """t5d_model_step."""
+  _fields_ = ([(n, c_int) for n in (
+      'dtype', 'w_dtype', 'd', 'H', 'F', 'V', 'L', 'E', 'NL', 'R', 'B',
+      'beams')] + [(n, c_void_p) for n in (
+          'embedding', 'rel_bias', 'ln_final', 'logits_w', 'logits_scales')] +
+              [('layers', POINTER(Layer))] + [(n, c_void_p) for n in (
+                  'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
+                  'ao', 'h', 'logits', 'gate')])
+
+
+class BeamStep(Structure):
+  """t5d_beam_step."""
+  _fields_ = ([('state', BeamStatePtrs)] + [(n, c_void_p) for n in (
+      'inputs', 'initial_index', 'brevity', 'top_alive', 'topk_vals',
+      'topk_idx', 'row_max', 'row_lse', 'scratch', 'ids', 'keep_going')] +
+              [('S', c_int), ('Lin', c_int), ('eos_id', c_int),
+               ('min_brevity', c_float), ('min_log_prob', c_float),
+               ('max_decode_step', c_int), ('min_initial_index', c_int),
+               ('kv_base', c_void_p), ('kv_tensor_stride_bytes', c_int64),
+               ('n_kv_tensors', c_int)])
+
+
 _P = c_void_p
 _SIGNATURES = {
+    't5d_gather_step_ids': (c_int, [_P, _P, _P, _P, c_int, c_int]),
+    't5d_decoder_step': (c_int, [_P, POINTER(ModelStep), _P]),
+    't5d_beam_search_step': (c_int, [_P, POINTER(ModelStep),
+                                     POINTER(BeamStep)]),
+    't5d_graph_begin': (c_int, [_P]),
+    't5d_graph_end': (c_int, [_P, POINTER(c_void_p)]),
+    't5d_graph_launch': (c_int, [_P, _P]),
+    't5d_graph_destroy': (c_int, [_P]),
     't5d_version': (c_int, []),
     't5d_last_error': (c_char_p, []),
     't5d_packed_weight_bytes': (c_int64, [c_int, c_int, c_int]),

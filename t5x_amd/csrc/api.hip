@@ -6,6 +6,7 @@
 namespace t5d {
 
 static thread_local char g_error[512] = "";
+thread_local const int32_t* tls_gate = nullptr;
 
 void set_error(const char* fmt, ...) {
   va_list ap;
@@ -18,7 +19,9 @@ void set_error(const char* fmt, ...) {
 // One workgroup per row; 16-byte copies.
 __global__ void embed_kernel(const uint4* __restrict__ table,
                              const int32_t* __restrict__ ids,
-                             uint4* __restrict__ out, int vec_per_row, int V) {
+                             uint4* __restrict__ out, int vec_per_row, int V,
+                             const int32_t* gate) {
+  T5D_GATED(gate);
   const int r = blockIdx.x;
   int id = ids[r];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);
@@ -33,7 +36,8 @@ __global__ void embed_kernel(const uint4* __restrict__ table,
 template <typename T>
 __global__ void __launch_bounds__(256)
 rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
-               T* __restrict__ out, int d, float eps) {
+               T* __restrict__ out, int d, float eps, const int32_t* gate) {
+  T5D_GATED(gate);
   __shared__ float partial[4];
   const int r = blockIdx.x;
   const T* xr = x + (size_t)r * d;
@@ -54,7 +58,9 @@ rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
   }
 }
 
-__global__ void add_i32_kernel(int32_t* x, int n, int delta) {
+__global__ void add_i32_kernel(int32_t* x, int n, int delta,
+                               const int32_t* gate) {
+  T5D_GATED(gate);
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) x[i] += delta;
 }
@@ -77,7 +83,8 @@ extern "C" int t5d_embed(void* stream, int dtype, const void* table,
   T5D_REQUIRE((d * esz) % 16 == 0, T5D_EINVAL,
               "t5d_embed: row bytes %d not a multiple of 16", d * esz);
   hipLaunchKernelGGL(embed_kernel, dim3(R), dim3(128), 0, as_stream(stream),
-                     (const uint4*)table, ids, (uint4*)out, d * esz / 16, V);
+                     (const uint4*)table, ids, (uint4*)out, d * esz / 16, V,
+                     tls_gate);
   T5D_CHECK_LAUNCH("t5d_embed");
   return T5D_OK;
 }
@@ -92,11 +99,11 @@ extern "C" int t5d_rmsnorm(void* stream, int dtype, const void* x,
   if (dtype == T5D_F32)
     hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(R), dim3(256), 0,
                        as_stream(stream), (const float*)x, (const float*)scale,
-                       (float*)out, d, eps);
+                       (float*)out, d, eps, tls_gate);
   else
     hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(R), dim3(256), 0,
                        as_stream(stream), (const bf16_t*)x,
-                       (const bf16_t*)scale, (bf16_t*)out, d, eps);
+                       (const bf16_t*)scale, (bf16_t*)out, d, eps, tls_gate);
   T5D_CHECK_LAUNCH("t5d_rmsnorm");
   return T5D_OK;
 }
@@ -104,7 +111,7 @@ extern "C" int t5d_rmsnorm(void* stream, int dtype, const void* x,
 extern "C" int t5d_add_i32(void* stream, int32_t* x, int n, int delta) {
   T5D_REQUIRE(x && n > 0, T5D_EINVAL, "t5d_add_i32: x=%p n=%d", (void*)x, n);
   hipLaunchKernelGGL(add_i32_kernel, dim3((n + 63) / 64), dim3(64), 0,
-                     as_stream(stream), x, n, delta);
+                     as_stream(stream), x, n, delta, tls_gate);
   T5D_CHECK_LAUNCH("t5d_add_i32");
   return T5D_OK;
 }

@@ -33,6 +33,7 @@ struct AttnArgs {
   const int32_t* index; // self: cache_index scalar; cross: enc_len [G]
   void* out;            // [R, HD]
   int H, S, nq, q_stride;
+  const int32_t* gate;  // optional device-side enable flag
 };
 
 constexpr int kD = 64;
@@ -47,6 +48,7 @@ attn_step_kernel(AttnArgs a) {
   constexpr int BJ = 16 * EL;               // key positions per wavefront
   __shared__ float s_red[WM][NQ];
   __shared__ float s_out[WM][NQ][kD];
+  T5D_GATED(a.gate);
 
   const int h = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x & 63;
@@ -286,6 +288,111 @@ attn_step_kernel(AttnArgs a) {
   }
 }
 
+// ---- float32 cross-attention -------------------------------------------------
+// K is [B, H, E, 64] (head dim contiguous), V is [B, H, 64, E].  Lane = key
+// position for the scores (a lane reads its own 256-byte K row), lane = head
+// dim for the value product.  Float32 activations only occur in the small
+// CPU-comparable configuration; this kernel favours clarity.
+template <int NQ>
+__global__ void __launch_bounds__(1024)
+cross_attn_f32_kernel(AttnArgs a) {
+  __shared__ float s_q[NQ][kD];
+  __shared__ float s_red[kMaxWaves][NQ];
+  __shared__ float s_p[NQ][kMaxWaves * 64];
+  __shared__ float s_out[kMaxWaves][NQ][kD];
+  T5D_GATED(a.gate);
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nwaves = blockDim.x >> 6;
+  const int HD = a.H * kD;
+  int n = a.index[b];
+  n = n < 0 ? 0 : (n > a.S ? a.S : n);
+  bool uniform = false;
+  if (n == 0) { uniform = true; n = a.S; }
+  const float* kbase = reinterpret_cast<const float*>(a.k) +
+                       ((size_t)b * a.H + h) * (size_t)a.S * kD;
+  const float* vbase = reinterpret_cast<const float*>(a.v) +
+                       ((size_t)b * a.H + h) * (size_t)kD * a.S;
+  const float* qbase = reinterpret_cast<const float*>(a.q);
+  for (int e = threadIdx.x; e < NQ * kD; e += blockDim.x) {
+    const int qi = e / kD, d = e % kD;
+    s_q[qi][d] = qi < a.nq
+                     ? qbase[(size_t)(b * a.nq + qi) * a.q_stride + h * kD + d]
+                     : 0.f;
+  }
+  __syncthreads();
+  const int j = wave * 64 + lane;
+  float s[NQ];
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) s[qi] = 0.f;
+  if (j < n) {
+    const float4* row = reinterpret_cast<const float4*>(kbase + (size_t)j * kD);
+#pragma unroll
+    for (int c = 0; c < kD / 4; ++c) {
+      const float4 kv = row[c];
+#pragma unroll
+      for (int qi = 0; qi < NQ; ++qi) {
+        s[qi] = fmaf(s_q[qi][4 * c + 0], kv.x, s[qi]);
+        s[qi] = fmaf(s_q[qi][4 * c + 1], kv.y, s[qi]);
+        s[qi] = fmaf(s_q[qi][4 * c + 2], kv.z, s[qi]);
+        s[qi] = fmaf(s_q[qi][4 * c + 3], kv.w, s[qi]);
+      }
+    }
+  }
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) {
+    float x = uniform ? 0.f : s[qi];
+    x = (j < n) ? x : -INFINITY;
+    s[qi] = x;
+    const float m = wave_max(x);
+    if (lane == 0) s_red[wave][qi] = m;
+  }
+  __syncthreads();
+  float ex[NQ];
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) {
+    float m = s_red[0][qi];
+    for (int w = 1; w < nwaves; ++w) m = fmaxf(m, s_red[w][qi]);
+    ex[qi] = (s[qi] == -INFINITY) ? 0.f : expf(s[qi] - m);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) {
+    const float t = wave_sum(ex[qi]);
+    if (lane == 0) s_red[wave][qi] = t;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) {
+    float t = s_red[0][qi];
+    for (int w = 1; w < nwaves; ++w) t += s_red[w][qi];
+    s_p[qi][j] = ex[qi] / t;
+  }
+  __syncthreads();
+  // value product: lane = head dim, this wavefront's 64 positions
+  float o[NQ];
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) o[qi] = 0.f;
+  const int jb = wave * 64, je = min(n, jb + 64);
+  for (int jj = jb; jj < je; ++jj) {
+    const float v = vbase[(size_t)lane * a.S + jj];
+#pragma unroll
+    for (int qi = 0; qi < NQ; ++qi) o[qi] = fmaf(s_p[qi][jj], v, o[qi]);
+  }
+#pragma unroll
+  for (int qi = 0; qi < NQ; ++qi) s_out[wave][qi][lane] = o[qi];
+  __syncthreads();
+  for (int e = threadIdx.x; e < NQ * kD; e += blockDim.x) {
+    const int qi = e / kD, d = e % kD;
+    if (qi >= a.nq) continue;
+    float acc = s_out[0][qi][d];
+    for (int w = 1; w < nwaves; ++w) acc += s_out[w][qi][d];
+    reinterpret_cast<float*>(a.out)[(size_t)(b * a.nq + qi) * HD + h * kD + d] =
+        acc;
+  }
+}
+
 template <typename T, int NQ, bool SELF>
 static void launch_attn_nq(const AttnArgs& a, int groups, hipStream_t s) {
   constexpr int BJ = 16 * Act<T>::kElemsPer16B;
@@ -299,17 +406,22 @@ static void launch_attn_nq(const AttnArgs& a, int groups, hipStream_t s) {
     hipLaunchKernelGGL((attn_step_kernel<T, NQ, SELF, 16>), grid, block, 0, s, a);
 }
 
-template <typename T, bool SELF>
-static void launch_attn(const AttnArgs& a, int groups, hipStream_t s) {
-  if constexpr (SELF) {
-    launch_attn_nq<T, 1, true>(a, groups, s);
-  } else {
-    if (a.nq == 1) launch_attn_nq<T, 1, false>(a, groups, s);
-    else if (a.nq == 2) launch_attn_nq<T, 2, false>(a, groups, s);
-    else if (a.nq <= 4) launch_attn_nq<T, 4, false>(a, groups, s);
-    else launch_attn_nq<T, 8, false>(a, groups, s);
-  }
+static void launch_cross_f32(const AttnArgs& a, int B, hipStream_t s) {
+  const int waves = (a.S + 63) / 64;
+  dim3 grid(a.H, B), block(64 * waves);
+  if (a.nq == 1) hipLaunchKernelGGL(cross_attn_f32_kernel<1>, grid, block, 0, s, a);
+  else if (a.nq == 2) hipLaunchKernelGGL(cross_attn_f32_kernel<2>, grid, block, 0, s, a);
+  else if (a.nq <= 4) hipLaunchKernelGGL(cross_attn_f32_kernel<4>, grid, block, 0, s, a);
+  else hipLaunchKernelGGL(cross_attn_f32_kernel<8>, grid, block, 0, s, a);
 }
+
+int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
+                                const void* v, const int32_t* enc_len,
+                                void* out, int B, int beams, int H, int E);
+int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
+                               void* cv, const void* rel_bias,
+                               const int32_t* cache_index, void* out, int R,
+                               int H, int L);
 
 static int check_common(const char* name, int dtype, int H, int S) {
   T5D_REQUIRE(dtype == T5D_F32 || dtype == T5D_BF16, T5D_EINVAL, "%s: dtype %d",
@@ -345,8 +457,12 @@ extern "C" int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
   a.q = qkv; a.k = cached_key; a.v = cached_value; a.rel_bias = rel_bias;
   a.index = cache_index; a.out = out;
   a.H = H; a.S = L; a.nq = 1; a.q_stride = 3 * H * kD;
-  if (dtype == T5D_F32) launch_attn<float, true>(a, R, as_stream(stream));
-  else launch_attn<bf16_t, true>(a, R, as_stream(stream));
+  a.gate = tls_gate;
+  if (dtype == T5D_F32)
+    launch_attn_nq<float, 1, true>(a, R, as_stream(stream));
+  else
+    launch_self_attention_bf16(as_stream(stream), qkv, cached_key, cached_value,
+                               rel_bias, cache_index, out, R, H, L);
   T5D_CHECK_LAUNCH("t5d_self_attention_step");
   return T5D_OK;
 }
@@ -370,8 +486,16 @@ extern "C" int t5d_cross_attention_step(void* stream, int dtype, const void* q,
   a.v = const_cast<void*>(cross_value); a.rel_bias = nullptr;
   a.index = enc_len; a.out = out;
   a.H = H; a.S = E; a.nq = beams; a.q_stride = H * kD;
-  if (dtype == T5D_F32) launch_attn<float, false>(a, B, as_stream(stream));
-  else launch_attn<bf16_t, false>(a, B, as_stream(stream));
+  a.gate = tls_gate;
+  if (dtype == T5D_F32) {
+    T5D_REQUIRE(E <= kMaxWaves * 64, T5D_ELIMIT,
+                "t5d_cross_attention_step: float32 covers at most %d positions",
+                kMaxWaves * 64);
+    launch_cross_f32(a, B, as_stream(stream));
+  } else {
+    launch_cross_attention_bf16(as_stream(stream), q, cross_key, cross_value,
+                                enc_len, out, B, beams, H, E);
+  }
   T5D_CHECK_LAUNCH("t5d_cross_attention_step");
   return T5D_OK;
 }

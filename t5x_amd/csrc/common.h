@@ -104,4 +104,14 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Optional device-side gate.  While a fused multi-kernel entry point is
+// enqueueing work it publishes a pointer to an int32 flag here; every kernel
+// launched by this thread then receives it and returns immediately when the
+// flag is 0.  This lets a decode loop run several steps per host
+// synchronisation: once the loop condition turns false on the device, the
+// remaining enqueued steps are no-ops.  Null outside fused entry points.
+extern thread_local const int32_t* tls_gate;
+#define T5D_GATED(gate) \
+  if ((gate) != nullptr && *(gate) == 0) return
+
 }  // namespace t5d

@@ -6,15 +6,17 @@
 //     tiles stored lane-major, so one wavefront load instruction fetches one
 //     whole tile as a single contiguous 1 KB (bf16) / 512 B (int8) burst
 //     straight into the registers v_mfma_f32_16x16x32_bf16 consumes;
-//   * a workgroup owns N_TILES adjacent 16-column tiles and all M rows; its 4
-//     wavefronts split the K range (k-tile kt goes to wave kt % 4) so that
-//     every byte of the workgroup's weight slice is requested exactly once and
-//     as early as possible, then the 4 partial accumulators are summed through
-//     LDS in a fixed order (bitwise deterministic);
-//   * small-N layers additionally split K across workgroups; partial tiles go
-//     to a float32 workspace and the last workgroup to arrive (per column
-//     group) sums them in split order and applies the epilogue.
-// The activation operand (<= 128 x K) is re-read by every workgroup from L2.
+//   * a workgroup owns NT adjacent 16-column tiles and MP 16-row tiles; its 4
+//     wavefronts split the K range in pairs of k-tiles (pair p goes to wave
+//     p % 4), keep several pairs of weight tiles in flight ahead of the MFMAs,
+//     and sum their 4 partial accumulators through LDS in a fixed order
+//     (bitwise deterministic, no atomics, no cross-workgroup traffic);
+//   * small-N layers get their parallelism from splitting M across
+//     workgroups; the workgroups that share a weight slice are mapped to the
+//     same XCD (consecutive block ids go round-robin over the 8 XCDs), so the
+//     slice comes from HBM once and from that XCD's L2 afterwards.
+// The activation operand is read from L2 in full 128-byte lines (a pair of
+// k-tiles is 64 contiguous bf16 per row).
 #include "common.h"
 
 namespace t5d {
@@ -62,9 +64,9 @@ struct GemmArgs {
   const float* scales;  // [N] or null
   const void* residual; // [M, Nout] act dtype or null
   void* C;              // [M, Nout]
-  float* workspace;     // [split_k, M_pad, N] f32
-  int32_t* counters;    // [gridDim.x]
   int M, K, N;          // N = number of weight columns
+  int m_parts;          // workgroups along M
+  const int32_t* gate;  // optional device-side enable flag
   int epilogue;
   int out_f32;
 };
@@ -92,23 +94,31 @@ __device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
   reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(v);
 }
 
-template <int M_TILES, int N_TILES, typename WT>
+template <int MP, int NT, typename WT>
 __global__ void __launch_bounds__(256)
 gemm_mfma_kernel(GemmArgs g) {
-  constexpr int ACC = M_TILES * N_TILES;
-  constexpr int TN = N_TILES * 16;
+  constexpr int ACC = MP * NT;
+  constexpr int TN = NT * 16;
+  constexpr int PF = (NT >= 4) ? 2 : (NT == 2 ? 3 : 4);  // pairs in flight
   static_assert(ACC <= 16, "accumulator tile budget");
   __shared__ float red[2][ACC * 4][64];
-  __shared__ int is_last;
+  T5D_GATED(g.gate);
+
+  // XCD-aware block mapping: the m_parts workgroups of one column group get
+  // block ids 8 apart, i.e. the same XCD and adjacent dispatch slots.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int n_group = (slot / g.m_parts) * 8 + xcd;
+  const int m_part = slot % g.m_parts;
+  const int n_tiles_total = g.N >> 4;
+  const int nt0 = n_group * NT;
+  if (nt0 >= n_tiles_total) return;
+  const int m0 = m_part * MP * 16;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int KT = g.K >> 5;
-  const int n_tiles_total = g.N >> 4;
-  const int nt0 = blockIdx.x * N_TILES;
-  const int split = gridDim.y;
-  const int kt_begin = (int)(((long)KT * blockIdx.y) / split);
-  const int kt_end = (int)(((long)KT * (blockIdx.y + 1)) / split);
+  const int n_pairs = (KT + 1) >> 1;
+  const int nj = (n_pairs - wave + 3) >> 2;  // pairs owned by this wave
 
   f32x4_v acc[ACC];
 #pragma unroll
@@ -117,36 +127,56 @@ gemm_mfma_kernel(GemmArgs g) {
   const int arow = lane & 15;
   const int akoff = (lane >> 4) * 8;
   const char* wbase = reinterpret_cast<const char*>(g.W);
+  constexpr int TB = WeightTile<WT>::kTileBytes;
 
-  for (int kt = kt_begin + wave; kt < kt_end; kt += 4) {
-    Frag b[N_TILES];
+  Frag bq[PF][2][NT];
+  auto load_b = [&](int slot_, int j) {
+    const int kt = (wave + 4 * j) * 2;
 #pragma unroll
-    for (int nn = 0; nn < N_TILES; ++nn) {
-      const int nt = nt0 + nn;
-      if (nt < n_tiles_total) {
-        b[nn] = WeightTile<WT>::load(
-            wbase + ((size_t)nt * KT + kt) * WeightTile<WT>::kTileBytes, lane);
-      } else {
-        b[nn].u = make_uint4(0, 0, 0, 0);
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int nn = 0; nn < NT; ++nn) {
+        const int nt = nt0 + nn;
+        if (nt < n_tiles_total && kt + h < KT)
+          bq[slot_][h][nn] = WeightTile<WT>::load(
+              wbase + ((size_t)nt * KT + kt + h) * TB, lane);
+        else
+          bq[slot_][h][nn].u = make_uint4(0, 0, 0, 0);
+      }
+  };
+#pragma unroll
+  for (int p = 0; p < PF; ++p)
+    if (p < nj) load_b(p, p);
+
+  for (int j0 = 0; j0 < nj; j0 += PF) {
+#pragma unroll
+    for (int p = 0; p < PF; ++p) {
+      const int j = j0 + p;
+      if (j < nj) {
+        const int kt = (wave + 4 * j) * 2;
+        Frag a[2][MP];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int mt = 0; mt < MP; ++mt) {
+            const int row = m0 + mt * 16 + arow;
+            if (row < g.M && kt + h < KT)
+              a[h][mt].u = *reinterpret_cast<const uint4*>(
+                  g.A + (size_t)row * g.K + (kt + h) * 32 + akoff);
+            else
+              a[h][mt].u = make_uint4(0, 0, 0, 0);
+          }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int mt = 0; mt < MP; ++mt)
+#pragma unroll
+            for (int nn = 0; nn < NT; ++nn)
+              acc[mt * NT + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  a[h][mt].v, bq[p][h][nn].v, acc[mt * NT + nn], 0, 0, 0);
+        if (j + PF < nj) load_b(p, j + PF);
       }
     }
-    Frag a[M_TILES];
-#pragma unroll
-    for (int mt = 0; mt < M_TILES; ++mt) {
-      const int row = mt * 16 + arow;
-      if (row < g.M) {
-        a[mt].u = *reinterpret_cast<const uint4*>(g.A + (size_t)row * g.K +
-                                                  kt * 32 + akoff);
-      } else {
-        a[mt].u = make_uint4(0, 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int mt = 0; mt < M_TILES; ++mt)
-#pragma unroll
-      for (int nn = 0; nn < N_TILES; ++nn)
-        acc[mt * N_TILES + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            a[mt].v, b[nn].v, acc[mt * N_TILES + nn], 0, 0, 0);
   }
 
   // Cross-wave reduction in a fixed order: (w0 + w2) + (w1 + w3).
@@ -182,67 +212,25 @@ gemm_mfma_kernel(GemmArgs g) {
   }
   __syncthreads();
 
-  const int m_rows = M_TILES * 16;
   const bool geglu = g.epilogue == T5D_EPI_GEGLU;
-
-  auto tile_sum = [&](int m, int nl) -> float {
-    const int mt = m >> 4, i = m & 3, c = (m & 15) >> 2;
+  auto tile_sum = [&](int ml, int nl) -> float {
+    const int mt = ml >> 4, i = ml & 3, c = (ml & 15) >> 2;
     const int nn = nl >> 4, l = c * 16 + (nl & 15);
-    return red[1][(mt * N_TILES + nn) * 4 + i][l];
+    return red[1][(mt * NT + nn) * 4 + i][l];
   };
-
-  if (split == 1) {
-    for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
-      const int m = e / TN, nl = e % TN;
-      const int n = nt0 * 16 + nl;
-      if (m >= g.M || n >= g.N) continue;
-      if (geglu && (nl & 8)) continue;
-      float v = tile_sum(m, nl);
-      float vg = geglu ? tile_sum(m, nl + 8) : 0.f;
-      if (g.scales) {
-        v *= g.scales[n];
-        if (geglu) vg *= g.scales[n + 8];
-      }
-      store_result(g, m, n, v, vg);
-    }
-    return;
-  }
-
-  // Split-K: publish this workgroup's partial tile, last arrival finishes.
-  const size_t ws_stride = (size_t)m_rows * g.N;
-  float* ws = g.workspace + (size_t)blockIdx.y * ws_stride;
-  for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
-    const int m = e / TN, nl = e % TN;
-    const int n = nt0 * 16 + nl;
-    if (n < g.N) ws[(size_t)m * g.N + n] = tile_sum(m, nl);
-  }
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int prev = atomicAdd(&g.counters[blockIdx.x], 1);
-    is_last = (prev == split - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  for (int e = threadIdx.x; e < m_rows * TN; e += 256) {
-    const int m = e / TN, nl = e % TN;
-    const int n = nt0 * 16 + nl;
+  for (int e = threadIdx.x; e < MP * 16 * TN; e += 256) {
+    const int ml = e / TN, nl = e % TN;
+    const int m = m0 + ml, n = nt0 * 16 + nl;
     if (m >= g.M || n >= g.N) continue;
     if (geglu && (nl & 8)) continue;
-    float v = 0.f, vg = 0.f;
-    for (int s = 0; s < split; ++s) {
-      const float* p = g.workspace + (size_t)s * ws_stride + (size_t)m * g.N;
-      v += p[n];
-      if (geglu) vg += p[n + 8];
-    }
+    float v = tile_sum(ml, nl);
+    float vg = geglu ? tile_sum(ml, nl + 8) : 0.f;
     if (g.scales) {
       v *= g.scales[n];
       if (geglu) vg *= g.scales[n + 8];
     }
     store_result(g, m, n, v, vg);
   }
-  if (threadIdx.x == 0) g.counters[blockIdx.x] = 0;
 }
 
 // ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
@@ -251,8 +239,9 @@ template <int MB>
 __global__ void __launch_bounds__(256)
 gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
                 const float* __restrict__ residual, float* __restrict__ C,
-                int M, int K, int N, int epilogue) {
+                int M, int K, int N, int epilogue, const int32_t* gate) {
   __shared__ float red[4][2 * MB][64];
+  T5D_GATED(gate);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool geglu = epilogue == T5D_EPI_GEGLU;
@@ -330,35 +319,47 @@ __global__ void pack_weight_kernel(const WT* __restrict__ src,
 }
 
 struct GemmPlan {
-  int m_tiles, n_tiles, split_k;
+  int mp, nt, m_parts, n_groups;
 };
 
+// Pick the workgroup tile.  Model: all workgroups run in ceil(wgs / 512)
+// rounds (two resident per CU); a round costs a fixed latency plus the time
+// one workgroup needs to pull its A and B bytes.
 static GemmPlan plan_gemm(int M, int K, int N) {
-  GemmPlan p;
-  p.m_tiles = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
-  const int nt = N / 16;
-  const int kt = K / 32;
-  // Wider column groups amortise the activation re-read; keep at least ~256
-  // workgroups so every CU has work.
-  int n_tiles = 16 / p.m_tiles;       // accumulator budget: m_tiles*n_tiles<=16
-  if (n_tiles > 4) n_tiles = 4;
-  while (n_tiles > 1 && nt / n_tiles < 256) n_tiles >>= 1;
-  p.n_tiles = n_tiles;
-  const int groups = (nt + n_tiles - 1) / n_tiles;
-  int split = 1;
-  while (groups * split < 192 && kt / (split * 2) >= 4 && split < 16) split *= 2;
-  p.split_k = split;
-  return p;
+  const int mt_total = (M + 15) / 16;
+  const int n_tiles = N / 16;
+  GemmPlan best = {1, 1, 1, 1};
+  double best_cost = 1e30;
+  const int mps[4] = {1, 2, 4, 8};
+  const int nts[3] = {1, 2, 4};
+  for (int mi = 0; mi < 4; ++mi)
+    for (int ni = 0; ni < 3; ++ni) {
+      const int mp = mps[mi], nt = nts[ni];
+      if (mp * nt > 16) continue;
+      if (mp > mt_total && mp != 1 && (mp >> 1) >= mt_total) continue;
+      const int m_parts = (mt_total + mp - 1) / mp;
+      const int n_groups = (n_tiles + nt - 1) / nt;
+      const double wgs = (double)m_parts * n_groups;
+      const double rounds = (double)(long)((wgs + 511) / 512);
+      const double bytes = (double)K * 2.0 * (mp * 16 + nt * 16);
+      const double cost = rounds * (3.0 + bytes / 40e3) + wgs * bytes / 30e6;
+      if (cost < best_cost) {
+        best_cost = cost;
+        best = {mp, nt, m_parts, n_groups};
+      }
+    }
+  return best;
 }
 
 template <typename WT>
-static void launch_mfma(const GemmPlan& p, const GemmArgs& g, hipStream_t s) {
-  const int groups = (g.N / 16 + p.n_tiles - 1) / p.n_tiles;
-  dim3 grid(groups, p.split_k), block(256);
-#define T5D_GEMM_CASE(MT, NT)                                              \
-  if (p.m_tiles == MT && p.n_tiles == NT) {                                \
-    hipLaunchKernelGGL((gemm_mfma_kernel<MT, NT, WT>), grid, block, 0, s, g); \
-    return;                                                                \
+static void launch_mfma(const GemmPlan& p, GemmArgs g, hipStream_t s) {
+  g.m_parts = p.m_parts;
+  const int groups8 = (p.n_groups + 7) / 8 * 8;
+  dim3 grid(groups8 * p.m_parts), block(256);
+#define T5D_GEMM_CASE(MT, NT_)                                              \
+  if (p.mp == MT && p.nt == NT_) {                                          \
+    hipLaunchKernelGGL((gemm_mfma_kernel<MT, NT_, WT>), grid, block, 0, s, g); \
+    return;                                                                 \
   }
   T5D_GEMM_CASE(1, 1) T5D_GEMM_CASE(1, 2) T5D_GEMM_CASE(1, 4)
   T5D_GEMM_CASE(2, 1) T5D_GEMM_CASE(2, 2) T5D_GEMM_CASE(2, 4)
@@ -406,11 +407,8 @@ extern "C" int t5d_pack_weight(void* stream, int w_dtype, const void* src,
 
 extern "C" int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M,
                                             int K, int N) {
-  (void)w_dtype;
-  if (dtype != T5D_BF16 || M <= 0 || M > 128 || K % 32 || N % 16) return 0;
-  GemmPlan p = plan_gemm(M, K, N);
-  if (p.split_k == 1) return 0;
-  return (int64_t)p.split_k * p.m_tiles * 16 * N * 4;
+  (void)dtype; (void)w_dtype; (void)M; (void)K; (void)N;
+  return 0;  // no kernel variant needs scratch memory
 }
 
 extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
@@ -435,12 +433,14 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
       dim3 grid((ncols + 63) / 64, 1);
       hipLaunchKernelGGL(gemm_f32_kernel<8>, grid, dim3(256), 0, s,
                          (const float*)A, (const float*)W,
-                         (const float*)residual, (float*)C, M, K, N, epilogue);
+                         (const float*)residual, (float*)C, M, K, N, epilogue,
+                         tls_gate);
     } else {
       dim3 grid((ncols + 63) / 64, (M + 15) / 16);
       hipLaunchKernelGGL(gemm_f32_kernel<16>, grid, dim3(256), 0, s,
                          (const float*)A, (const float*)W,
-                         (const float*)residual, (float*)C, M, K, N, epilogue);
+                         (const float*)residual, (float*)C, M, K, N, epilogue,
+                         tls_gate);
     }
     T5D_CHECK_LAUNCH("t5d_gemm(f32)");
     return T5D_OK;
@@ -459,18 +459,17 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
               "t5d_gemm: K=%d N=%d must tile 32x16", K, N);
   T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
               "t5d_gemm: A/W must be 16-byte aligned");
+  (void)workspace; (void)counters;
   GemmPlan p = plan_gemm(M, K, N);
-  T5D_REQUIRE(p.split_k == 1 || (workspace && counters), T5D_EINVAL,
-              "t5d_gemm: split-K plan needs workspace and counters");
   GemmArgs g;
   g.A = (const bf16_t*)A;
   g.W = W;
   g.scales = w_dtype == T5D_I8 ? scales : nullptr;
   g.residual = residual;
   g.C = C;
-  g.workspace = (float*)workspace;
-  g.counters = counters;
   g.M = M; g.K = K; g.N = N;
+  g.m_parts = 1;
+  g.gate = tls_gate;
   g.epilogue = epilogue;
   g.out_f32 = out_dtype == T5D_F32;
   if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);

@@ -21,11 +21,13 @@ struct GatherArgs {
   const int32_t* valid_len;
   int valid_off;
   int beams, inner, row_bytes, elem_bytes, L;
+  const int32_t* gate;  // optional device-side enable flag
 };
 
 template <int BEAMS>
 __global__ void __launch_bounds__(256)
 cache_gather_kernel(GatherArgs a) {
+  T5D_GATED(a.gate);
   const int b = blockIdx.y;
   int src[BEAMS];
   bool identity = true;
@@ -100,6 +102,7 @@ extern "C" int t5d_cache_gather_beams(void* stream, void* cache,
   a.valid_off = valid_len_offset;
   a.beams = beams; a.inner = inner; a.row_bytes = L * elem_bytes;
   a.elem_bytes = elem_bytes; a.L = L;
+  a.gate = tls_gate;
   const size_t work = (size_t)inner * (a.row_bytes / 16);
   int gx = (int)((work + 255) / 256);
   gx = gx < 1 ? 1 : (gx > 256 ? 256 : gx);

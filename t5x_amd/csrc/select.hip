@@ -122,10 +122,11 @@ beam_row_topk_kernel(const float* __restrict__ logits,
                      const float* __restrict__ live_logprobs,
                      float* __restrict__ row_max, float* __restrict__ row_lse,
                      float* __restrict__ cand_vals, int32_t* __restrict__ cand_idx,
-                     int V, int beams, int k) {
+                     int V, int beams, int k, const int32_t* gate) {
   __shared__ Cand scratch[4];
   __shared__ float fscratch[4];
   __shared__ double dscratch[4];
+  T5D_GATED(gate);
   const int r = blockIdx.x;
   const float* x = logits + (size_t)r * V;
   float m = -INFINITY;
@@ -185,9 +186,10 @@ __global__ void __launch_bounds__(128)
 beam_merge_kernel(const float* __restrict__ cand_vals,
                   const int32_t* __restrict__ cand_idx,
                   float* __restrict__ topk_vals, int32_t* __restrict__ topk_idx,
-                  int beams, int k) {
+                  int beams, int k, const int32_t* gate) {
   __shared__ float sv[128];
   __shared__ int si[128];
+  T5D_GATED(gate);
   const int b = blockIdx.x, tid = threadIdx.x;
   const int n = beams * k;
   float v = -INFINITY;
@@ -221,6 +223,7 @@ struct BeamUpdateArgs {
   const float* brevity;
   int32_t* top_alive_indices;
   int B, K, S, Lin, V, eos_id;
+  const int32_t* gate;
 };
 
 // Stable descending order of n values (ties keep index order).
@@ -234,6 +237,10 @@ __device__ __forceinline__ void stable_order_desc(const float* v, int n,
   }
 }
 
+// One workgroup per batch item.  Thread 0 does the (tiny, order-sensitive)
+// scalar bookkeeping into LDS; then every thread owns sequence COLUMNS: for a
+// column it reads the item's K live and K finished entries into registers
+// before writing any, so `cur` and `next` may be the same buffers.
 __global__ void __launch_bounds__(64)
 beam_update_kernel(BeamUpdateArgs a) {
   __shared__ int s_src_live[kMaxBeams];       // source live beam of new live e
@@ -241,6 +248,10 @@ beam_update_kernel(BeamUpdateArgs a) {
   __shared__ int s_fin_from[kMaxBeams];       // <K: old finished; else K+cand
   __shared__ int s_cand_beam[2 * kMaxBeams];
   __shared__ int s_cand_tok[2 * kMaxBeams];
+  __shared__ float s_live_lp[kMaxBeams];
+  __shared__ float s_fin_score[kMaxBeams];
+  __shared__ int s_fin_flag[kMaxBeams];
+  T5D_GATED(a.gate);
   const int b = blockIdx.x;
   const int K = a.K, K2 = 2 * a.K, S = a.S;
   const int cur = *a.cur.cur_index;
@@ -269,8 +280,7 @@ beam_update_kernel(BeamUpdateArgs a) {
     stable_order_desc(new_lp, K2, order);
     for (int e = 0; e < K; ++e) {
       const int c = order[K - 1 - e];
-      a.next.live_logprobs[(size_t)b * K + e] = new_lp[c];
-      a.top_alive_indices[(size_t)b * K + e] = beam[c];
+      s_live_lp[e] = new_lp[c];
       s_src_live[e] = beam[c];
       s_tok_live[e] = id[c];
     }
@@ -284,41 +294,81 @@ beam_update_kernel(BeamUpdateArgs a) {
     for (int e = 0; e < K; ++e) {
       const int src = order[K - 1 - e];
       s_fin_from[e] = src;
-      a.next.finished_scores[(size_t)b * K + e] = pool[src];
-      a.next.finished_flags[(size_t)b * K + e] =
-          src < K ? a.cur.finished_flags[(size_t)b * K + src]
-                  : (uint8_t)fin[src - K];
+      s_fin_score[e] = pool[src];
+      s_fin_flag[e] = src < K ? a.cur.finished_flags[(size_t)b * K + src]
+                              : (int)fin[src - K];
     }
-    if (b == 0) *a.next.cur_index = cur + 1;
+    for (int e = 0; e < K; ++e) {
+      a.next.live_logprobs[(size_t)b * K + e] = s_live_lp[e];
+      a.top_alive_indices[(size_t)b * K + e] = s_src_live[e];
+      a.next.finished_scores[(size_t)b * K + e] = s_fin_score[e];
+      a.next.finished_flags[(size_t)b * K + e] = (uint8_t)s_fin_flag[e];
+    }
   }
   __syncthreads();
 
-  const int32_t* live = a.cur.live_seqs + (size_t)b * K * S;
-  for (int e = 0; e < K; ++e) {
-    int32_t* dst = a.next.live_seqs + ((size_t)b * K + e) * S;
-    const int32_t* src = live + (size_t)s_src_live[e] * S;
-    for (int j = threadIdx.x; j < S; j += 64)
-      dst[j] = (j == cur + 1) ? s_tok_live[e] : src[j];
-    int32_t* fdst = a.next.finished_seqs + ((size_t)b * K + e) * S;
-    const int from = s_fin_from[e];
-    if (from < K) {
-      const int32_t* fsrc = a.cur.finished_seqs + ((size_t)b * K + from) * S;
-      for (int j = threadIdx.x; j < S; j += 64) fdst[j] = fsrc[j];
-    } else {
-      const int c = from - K;
-      const int32_t* fsrc = live + (size_t)s_cand_beam[c] * S;
-      const int tok = s_cand_tok[c];
-      for (int j = threadIdx.x; j < S; j += 64)
-        fdst[j] = (j == cur + 1) ? tok : fsrc[j];
+  const size_t base = (size_t)b * K * S;
+  for (int j = threadIdx.x; j < S; j += 64) {
+    int live[kMaxBeams], fin[kMaxBeams];
+#pragma unroll
+    for (int e = 0; e < kMaxBeams; ++e) {
+      if (e < K) {
+        live[e] = a.cur.live_seqs[base + (size_t)e * S + j];
+        fin[e] = a.cur.finished_seqs[base + (size_t)e * S + j];
+      }
+    }
+    const bool tokcol = j == cur + 1;
+#pragma unroll
+    for (int e = 0; e < kMaxBeams; ++e) {
+      if (e < K) {
+        int lv = live[0], fv;
+#pragma unroll
+        for (int q = 1; q < kMaxBeams; ++q)
+          lv = (s_src_live[e] == q) ? live[q] : lv;
+        const int from = s_fin_from[e];
+        if (from < K) {
+          fv = fin[0];
+#pragma unroll
+          for (int q = 1; q < kMaxBeams; ++q) fv = (from == q) ? fin[q] : fv;
+        } else {
+          const int cb = s_cand_beam[from - K];
+          fv = live[0];
+#pragma unroll
+          for (int q = 1; q < kMaxBeams; ++q) fv = (cb == q) ? live[q] : fv;
+          if (tokcol) fv = s_cand_tok[from - K];
+        }
+        a.next.live_seqs[base + (size_t)e * S + j] =
+            tokcol ? s_tok_live[e] : lv;
+        a.next.finished_seqs[base + (size_t)e * S + j] = fv;
+      }
     }
   }
+  // cur_index is read by every workgroup at entry; a separate 1-thread kernel
+  // advances it after this one.
+}
+
+__global__ void advance_index_kernel(const int32_t* cur, int32_t* next,
+                                     const int32_t* gate) {
+  T5D_GATED(gate);
+  *next = *cur + 1;
+}
+
+// ids[r] = live_seqs[r, cur_index] (t5x/decoding.py:1308-1312).
+__global__ void gather_ids_kernel(const int32_t* __restrict__ live_seqs,
+                                  const int32_t* __restrict__ cur_index,
+                                  int32_t* __restrict__ ids, int R, int S,
+                                  const int32_t* gate) {
+  T5D_GATED(gate);
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < R) ids[r] = live_seqs[(size_t)r * S + *cur_index];
 }
 
 __global__ void __launch_bounds__(256)
 beam_cond_kernel(t5d_beam_state st, int B, int K, int S, float min_brevity,
                  float min_log_prob, int max_decode_step, int min_initial_index,
-                 int32_t* keep_going) {
+                 int32_t* keep_going, const int32_t* gate) {
   __shared__ int iscratch[4];
+  T5D_GATED(gate);
   const int cur = *st.cur_index;
   const float raw_min = min_log_prob / min_brevity;
   int not_terminated = 0, passes_min = 0;
@@ -627,18 +677,18 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
   if (k <= 4)
     hipLaunchKernelGGL(beam_row_topk_kernel<4>, dim3(R), dim3(256), 0, s,
                        logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k);
+                       cand_idx, V, beams, k, tls_gate);
   else if (k <= 8)
     hipLaunchKernelGGL(beam_row_topk_kernel<8>, dim3(R), dim3(256), 0, s,
                        logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k);
+                       cand_idx, V, beams, k, tls_gate);
   else
     hipLaunchKernelGGL(beam_row_topk_kernel<16>, dim3(R), dim3(256), 0, s,
                        logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k);
+                       cand_idx, V, beams, k, tls_gate);
   T5D_CHECK_LAUNCH("t5d_beam_topk(rows)");
   hipLaunchKernelGGL(beam_merge_kernel, dim3(B), dim3(128), 0, s, cand_vals,
-                     cand_idx, topk_vals, topk_idx, beams, k);
+                     cand_idx, topk_vals, topk_idx, beams, k, tls_gate);
   T5D_CHECK_LAUNCH("t5d_beam_topk(merge)");
   return T5D_OK;
 }
@@ -669,18 +719,20 @@ extern "C" int t5d_beam_update(void* stream, const t5d_beam_state* cur,
               "t5d_beam_update: B=%d K=%d S=%d Lin=%d V=%d", B, K, S, Lin, V);
   T5D_REQUIRE(K <= kMaxBeams, T5D_ELIMIT, "t5d_beam_update: K=%d > %d", K,
               kMaxBeams);
-  T5D_REQUIRE(cur->live_seqs != next->live_seqs &&
-                  cur->finished_seqs != next->finished_seqs,
-              T5D_EINVAL, "t5d_beam_update: cur and next must be distinct");
   BeamUpdateArgs a;
   a.cur = *cur; a.next = *next;
   a.topk_vals = topk_vals; a.topk_idx = topk_idx; a.inputs = inputs;
   a.initial_index = initial_index; a.brevity = brevity;
   a.top_alive_indices = top_alive_indices;
   a.B = B; a.K = K; a.S = S; a.Lin = Lin; a.V = V; a.eos_id = eos_id;
+  a.gate = tls_gate;
   hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_beam_update");
+  hipLaunchKernelGGL(advance_index_kernel, dim3(1), dim3(1), 0,
+                     as_stream(stream), cur->cur_index, next->cur_index,
+                     tls_gate);
+  T5D_CHECK_LAUNCH("t5d_beam_update(index)");
   return T5D_OK;
 }
 
@@ -695,7 +747,7 @@ extern "C" int t5d_beam_cond(void* stream, const t5d_beam_state* state, int B,
   hipLaunchKernelGGL(beam_cond_kernel, dim3(1), dim3(256), 0,
                      as_stream(stream), *state, B, K, S, min_brevity,
                      min_log_prob, max_decode_step, min_initial_index,
-                     keep_going);
+                     keep_going, tls_gate);
   T5D_CHECK_LAUNCH("t5d_beam_cond");
   return T5D_OK;
 }
@@ -760,5 +812,17 @@ extern "C" int t5d_gather_beams(void* stream, const void* src, void* dst,
                      as_stream(stream), (const char*)src, (char*)dst,
                      beam_indices, old_beams, new_beams, (size_t)inner_bytes);
   T5D_CHECK_LAUNCH("t5d_gather_beams");
+  return T5D_OK;
+}
+
+extern "C" int t5d_gather_step_ids(void* stream, const int32_t* live_seqs,
+                                   const int32_t* cur_index, int32_t* ids,
+                                   int R, int S) {
+  T5D_REQUIRE(live_seqs && cur_index && ids && R > 0 && S > 0, T5D_EINVAL,
+              "t5d_gather_step_ids: null pointer or R=%d S=%d", R, S);
+  hipLaunchKernelGGL(gather_ids_kernel, dim3((R + 63) / 64), dim3(64), 0,
+                     as_stream(stream), live_seqs, cur_index, ids, R, S,
+                     tls_gate);
+  T5D_CHECK_LAUNCH("t5d_gather_step_ids");
   return T5D_OK;
 }

@@ -1,0 +1,162 @@
+// Fused host-side entry points: one call enqueues every kernel of a decoder
+// step (and of a whole beam-search iteration) on the caller's stream, and a
+// thin wrapper over HIP graph capture lets the caller record that call once
+// and replay it every step.  Nothing here synchronises with the device.
+#include <vector>
+
+#include "common.h"
+
+using namespace t5d;
+
+namespace {
+
+struct GateScope {
+  explicit GateScope(const int32_t* g) { tls_gate = g; }
+  ~GateScope() { tls_gate = nullptr; }
+};
+
+#define T5D_TRY(call)        \
+  do {                       \
+    int rc_ = (call);        \
+    if (rc_ != T5D_OK) return rc_; \
+  } while (0)
+
+int check_model(const t5d_model_step* m) {
+  T5D_REQUIRE(m && m->layers, T5D_EINVAL, "t5d step: null model description");
+  T5D_REQUIRE(m->dtype == T5D_F32 || m->dtype == T5D_BF16, T5D_EINVAL,
+              "t5d step: dtype %d", m->dtype);
+  T5D_REQUIRE(m->d > 0 && m->H > 0 && m->F > 0 && m->V > 0 && m->L > 0 &&
+                  m->E > 0 && m->NL > 0 && m->R > 0 && m->B > 0 &&
+                  m->beams > 0 && m->R == m->B * m->beams,
+              T5D_EINVAL,
+              "t5d step: d=%d H=%d F=%d V=%d L=%d E=%d NL=%d R=%d B=%d beams=%d",
+              m->d, m->H, m->F, m->V, m->L, m->E, m->NL, m->R, m->B, m->beams);
+  T5D_REQUIRE(m->embedding && m->rel_bias && m->ln_final && m->logits_w &&
+                  m->cache_index && m->enc_len && m->x && m->x1 && m->x2 &&
+                  m->xn && m->qkv && m->q && m->ao && m->h && m->logits,
+              T5D_EINVAL, "t5d step: null buffer");
+  return T5D_OK;
+}
+
+}  // namespace
+
+extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
+                                const int32_t* ids) {
+  T5D_TRY(check_model(m));
+  T5D_REQUIRE(ids, T5D_EINVAL, "t5d_decoder_step: null ids");
+  GateScope gate(m->gate);
+  const int dt = m->dtype, wd = m->w_dtype;
+  const int R = m->R, d = m->d, HD = m->H * 64, F = m->F;
+  T5D_TRY(t5d_embed(stream, dt, m->embedding, ids, m->x, R, d, m->V));
+  const void* x = m->x;
+  for (int l = 0; l < m->NL; ++l) {
+    const t5d_layer& w = m->layers[l];
+    T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
+                     m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
+    T5D_TRY(t5d_self_attention_step(stream, dt, m->qkv, w.cached_key,
+                                    w.cached_value, m->rel_bias,
+                                    m->cache_index + l, m->ao, R, m->H, m->L));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.self_out, w.self_out_scales,
+                     x, m->x1, R, HD, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
+    T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q, w.cross_q_scales,
+                     nullptr, m->q, R, d, HD, T5D_EPI_NONE, nullptr, nullptr));
+    T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
+                                     w.cross_value, m->enc_len, m->ao, m->B,
+                                     m->beams, m->H, m->E));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
+                     w.cross_out_scales, m->x1, m->x2, R, HD, d,
+                     T5D_EPI_RESIDUAL, nullptr, nullptr));
+    T5D_TRY(t5d_rmsnorm(stream, dt, m->x2, w.ln_mlp, m->xn, R, d, 1e-6f));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.wi, w.wi_scales, nullptr,
+                     m->h, R, d, 2 * F, T5D_EPI_GEGLU, nullptr, nullptr));
+    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->h, w.wo, w.wo_scales, m->x2, m->x,
+                     R, F, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
+    x = m->x;
+  }
+  T5D_TRY(t5d_rmsnorm(stream, dt, x, m->ln_final, m->xn, R, d, 1e-6f));
+  T5D_TRY(t5d_gemm(stream, dt, wd, T5D_F32, m->xn, m->logits_w,
+                   m->logits_scales, nullptr, m->logits, R, d, m->V,
+                   T5D_EPI_NONE, nullptr, nullptr));
+  T5D_TRY(t5d_add_i32(stream, m->cache_index, m->NL, 1));
+  return T5D_OK;
+}
+
+extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
+                                    const t5d_beam_step* b) {
+  T5D_TRY(check_model(m));
+  T5D_REQUIRE(b && b->ids && b->topk_vals && b->topk_idx && b->row_max &&
+                  b->row_lse && b->scratch && b->top_alive && b->keep_going &&
+                  b->inputs && b->initial_index && b->brevity && b->kv_base,
+              T5D_EINVAL, "t5d_beam_search_step: null buffer");
+  T5D_REQUIRE(m->gate == b->keep_going, T5D_EINVAL,
+              "t5d_beam_search_step: the model gate must be the loop flag");
+  const int R = m->R, K = m->beams, B = m->B;
+  {
+    GateScope gate(b->keep_going);
+    T5D_TRY(t5d_gather_step_ids(stream, b->state.live_seqs, b->state.cur_index,
+                                b->ids, R, b->S));
+  }
+  T5D_TRY(t5d_decoder_step(stream, m, b->ids));
+  GateScope gate(b->keep_going);
+  T5D_TRY(t5d_beam_topk(stream, m->logits, b->state.live_logprobs,
+                        b->topk_vals, b->topk_idx, b->row_max, b->row_lse,
+                        b->scratch, B, K, m->V, 2 * K));
+  T5D_TRY(t5d_beam_update(stream, &b->state, &b->state, b->topk_vals,
+                          b->topk_idx, b->inputs, b->initial_index, b->brevity,
+                          b->top_alive, B, K, b->S, b->Lin, m->V, b->eos_id));
+  // After the update cur_index == number of valid cache columns.
+  if (K > 1)
+    T5D_TRY(t5d_cache_gather_beams(
+        stream, b->kv_base, b->kv_tensor_stride_bytes, b->n_kv_tensors,
+        m->dtype == T5D_F32 ? 4 : 2, B, K, m->H * 64, m->L, b->top_alive,
+        b->state.cur_index, 0));
+  T5D_TRY(t5d_beam_cond(stream, &b->state, B, K, b->S, b->min_brevity,
+                        b->min_log_prob, b->max_decode_step,
+                        b->min_initial_index, b->keep_going));
+  return T5D_OK;
+}
+
+// ---- HIP graph capture --------------------------------------------------------
+
+extern "C" int t5d_graph_begin(void* stream) {
+  hipError_t e = hipStreamBeginCapture(as_stream(stream),
+                                       hipStreamCaptureModeThreadLocal);
+  T5D_REQUIRE(e == hipSuccess, T5D_EHIP, "t5d_graph_begin: %s",
+              hipGetErrorString(e));
+  return T5D_OK;
+}
+
+extern "C" int t5d_graph_end(void* stream, void** graph_exec) {
+  T5D_REQUIRE(graph_exec, T5D_EINVAL, "t5d_graph_end: null output");
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
+  T5D_REQUIRE(e == hipSuccess && graph, T5D_EHIP, "t5d_graph_end: %s",
+              hipGetErrorString(e));
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  T5D_REQUIRE(e == hipSuccess && exec, T5D_EHIP,
+              "t5d_graph_end: instantiate: %s", hipGetErrorString(e));
+  *graph_exec = exec;
+  return T5D_OK;
+}
+
+extern "C" int t5d_graph_launch(void* graph_exec, void* stream) {
+  T5D_REQUIRE(graph_exec, T5D_EINVAL, "t5d_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph_exec),
+                                as_stream(stream));
+  T5D_REQUIRE(e == hipSuccess, T5D_EHIP, "t5d_graph_launch: %s",
+              hipGetErrorString(e));
+  return T5D_OK;
+}
+
+extern "C" int t5d_graph_destroy(void* graph_exec) {
+  if (!graph_exec) return T5D_OK;
+  hipError_t e =
+      hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph_exec));
+  T5D_REQUIRE(e == hipSuccess, T5D_EHIP, "t5d_graph_destroy: %s",
+              hipGetErrorString(e));
+  return T5D_OK;
+}

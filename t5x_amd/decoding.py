@@ -514,10 +514,19 @@ class BeamLoop:
     else:
       initial_index_np = np.zeros((batch_size,), np.int32)
 
+    # A step function that can run whole iterations on the device exposes
+    # `fused_beam_step(loop)`; it then owns the beam-expanded caches (the
+    # incoming cache must be the untouched zero cache) and the state is
+    # updated in place.
+    factory = getattr(tokens_to_logits, 'fused_beam_step', None)
+    use_fused = (factory is not None and initial_index is None and
+                 getattr(cache, 'fresh', False))
+    self.fused = None
     self.cur, self.beam_cache = beam_init(
-        batch_size, beam_size, max_decode_len, cache, cache_offset,
-        live_seqs=live_seqs, initial_index=initial_index_np)
-    self.nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
+        batch_size, beam_size, max_decode_len, {} if use_fused else cache,
+        cache_offset, live_seqs=live_seqs, initial_index=initial_index_np)
+    self.nxt = (self.cur if use_fused else
+                ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev))
     self.inputs_dev = torch.as_tensor(np.ascontiguousarray(inputs_np),
                                       device=dev)
     self.init_idx_dev = torch.as_tensor(initial_index_np, device=dev)
@@ -533,15 +542,41 @@ class BeamLoop:
     self.topk_bufs = None
     self.vocab_size = None
     self.step = 0
+    if use_fused:
+      self.fused = factory(self)
+      if self.fused is None:  # configuration not covered: generic path
+        self.cur, self.beam_cache = beam_init(
+            batch_size, beam_size, max_decode_len, cache, cache_offset)
+        self.nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
+      else:
+        self.beam_cache = self.fused.cache_tree()
 
   def cond(self) -> bool:
     """:1250-1300 (reads one flag back from the device)."""
+    if self.fused is not None:
+      return self.fused.keep_going()
     ops.beam_cond(self.cur, self.min_brevity, self.min_log_prob,
                   self.max_decode_step, self.min_initial, self.keep_going)
     return bool(self.keep_going.item())
 
+  def run(self, check_every: int = 8):
+    """Runs the loop to termination.  With a fused step the condition is read
+    back only every `check_every` iterations: iterations enqueued after it
+    turned false are no-ops on the device, so the final state is the same."""
+    if self.fused is None:
+      while self.cond():
+        self.body()
+      return
+    while self.fused.keep_going():
+      self.fused.launch(check_every)
+      self.step += check_every
+
   def body(self):
     """:1302-1506."""
+    if self.fused is not None:
+      self.fused.launch(1)
+      self.step += 1
+      return
     cur, nxt = self.cur, self.nxt
     B, K, dev = self.batch_size, self.beam_size, cur.live_seqs.device
     step, off = self.step, self.cache_offset
@@ -579,6 +614,8 @@ class BeamLoop:
 
   def finish(self):
     """:1513-1569."""
+    if self.fused is not None:
+      self.fused.finish()
     cur, dev = self.cur, self.cur.live_seqs.device
     # batch items with no finished sequence fall back to the live ones
     any_finished = cur.finished_flags.bool().any(dim=1)
@@ -612,6 +649,5 @@ def beam_search(
   loop = BeamLoop(inputs, cache, tokens_to_logits, eos_id, num_decodes, alpha,
                   max_decode_len, max_decode_step, min_log_prob, cache_offset,
                   initial_index)
-  while loop.cond():  # :1509
-    loop.body()
+  loop.run()  # :1509
   return loop.finish()

@@ -29,8 +29,26 @@ class Vocabulary:
   eos_id: int = 1
 
 
-def _is_array(x):
-  return isinstance(x, (np.ndarray, torch.Tensor))
+class StepFunction:
+  """`tokens_ids_to_logits` of t5x/models.py:703-715: the bound
+  `_compute_logits_from_slice`, as an object so the decode loop can also ask
+  for a fused on-device step (`fused_beam_step`)."""
+
+  def __init__(self, model, params, encoded_inputs, raw_inputs,
+               max_decode_length):
+    self.model, self.params = model, params
+    self.encoded_inputs, self.raw_inputs = encoded_inputs, raw_inputs
+    self.max_decode_length = max_decode_length
+    module = model.module
+    if hasattr(module, 'make_fused_beam_step'):
+      self.fused_beam_step = lambda loop: module.make_fused_beam_step(
+          loop, params, encoded_inputs, raw_inputs)
+
+  def __call__(self, decoding_state):
+    return self.model._compute_logits_from_slice(
+        decoding_state, params=self.params,
+        encoded_inputs=self.encoded_inputs, raw_inputs=self.raw_inputs,
+        max_decode_length=self.max_decode_length)
 
 
 class EncoderDecoderModel:
@@ -138,11 +156,9 @@ class EncoderDecoderModel:
       expand = lambda x: network.BeamShared(x, num_decodes)
     else:
       expand = lambda x: decoding.flat_batch_beam_expand(x, num_decodes)
-    tokens_ids_to_logits = functools.partial(
-        self._compute_logits_from_slice, params=params,
-        encoded_inputs=expand(encoded_inputs),
-        raw_inputs=expand(encoder_input_tokens),
-        max_decode_length=decoder_input_tokens.shape[1])
+    tokens_ids_to_logits = StepFunction(
+        self, params, expand(encoded_inputs), expand(encoder_input_tokens),
+        decoder_input_tokens.shape[1])
 
     if decoder_params is None:
       decoder_params = {}

@@ -89,6 +89,13 @@ def relative_position_bucket(relative_position, bidirectional=True,
   return ret + np.where(is_small, n, val_if_large)
 
 
+class FreshCache(dict):
+  """The zero cache as returned by cache initialisation.  The marker lets a
+  decode loop that owns its (beam-expanded) caches skip expanding this one;
+  any tree derived from it through cache_map is a plain dict again."""
+  fresh = True
+
+
 class BeamShared:
   """An array that is logically `flat_batch_beam_expand(x, beams)` but stored
   once per batch item.  `EncoderDecoderModel.predict_batch_with_aux` hands the
@@ -229,6 +236,7 @@ class Transformer:
     self._enc_weights = {}
     self._bufs = {}
     self._cross = None
+    self._step_cache = None
 
   # -- plumbing ---------------------------------------------------------------
   def _dev(self):
@@ -279,11 +287,12 @@ class Transformer:
     kv = torch.zeros((cfg.num_decoder_layers, 2, batch, cfg.num_heads,
                       cfg.head_dim, length), dtype=act, device=dev)
     idx = torch.zeros((cfg.num_decoder_layers,), dtype=torch.int32, device=dev)
-    return {'decoder': {
+    tree = FreshCache({'decoder': {
         f'layers_{i}': {'self_attention': {
             'cached_key': kv[i, 0], 'cached_value': kv[i, 1],
             'cache_index': idx[i]}}
-        for i in range(cfg.num_decoder_layers)}}
+        for i in range(cfg.num_decoder_layers)}})
+    return tree
 
   def _call(self, variables, encoder_input_tokens, decoder_input_tokens,
             decoder_target_tokens, enable_dropout=False, decode=False,
@@ -314,9 +323,13 @@ class Transformer:
         y = torch.matmul(x, kern)  # float32 accumulate, one rounding
         if scale is not None:
           y = (torch.matmul(x.float(), kern.float()) * scale).to(x.dtype)
-        y = y.view(B, E, H, D).permute(0, 2, 3, 1)  # [B, H, D, E]
-        buf = torch.zeros((B, H, D, Ep), dtype=x.dtype, device=x.device)
-        buf[..., :E] = y
+        y = y.view(B, E, H, D)
+        if dst is ks:  # keys: [B, H, E, D], head dim contiguous
+          buf = torch.zeros((B, H, Ep, D), dtype=x.dtype, device=x.device)
+          buf[:, :, :E] = y.permute(0, 2, 1, 3)
+        else:  # values: [B, H, D, E], positions contiguous
+          buf = torch.zeros((B, H, D, Ep), dtype=x.dtype, device=x.device)
+          buf[..., :E] = y.permute(0, 2, 3, 1)
         dst.append(buf)
     tok = enc_tokens.reshape(B, E)
     valid = tok > 0
@@ -332,6 +345,46 @@ class Transformer:
     return out
 
   # -- the decode step -------------------------------------------------------------
+  def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
+                  L, gate=None):
+    """Fills a t5d_model_step for one call of t5d_decoder_step."""
+    from t5x_amd import _lib
+    cfg = self.config
+    P = _lib.ptr
+    layers = (_lib.Layer * cfg.num_decoder_layers)()
+    for i, lw in enumerate(w.layers):
+      ck, cv = layer_caches[i]
+      l = layers[i]
+      l.ln_self, l.ln_cross, l.ln_mlp = (P(lw['ln_self']), P(lw['ln_cross']),
+                                         P(lw['ln_mlp']))
+      for name in ('qkv', 'self_out', 'cross_q', 'cross_out', 'wi', 'wo'):
+        setattr(l, name, P(lw[name].data))
+        setattr(l, name + '_scales', P(lw[name].scales))
+      l.cached_key, l.cached_value = P(ck), P(cv)
+      l.cross_key, l.cross_value = P(cross['k'][i]), P(cross['v'][i])
+    m = _lib.ModelStep()
+    m.dtype = _lib.dtype_code(w.act_dtype)
+    m.w_dtype = w.layers[0]['qkv'].w_dtype
+    m.d, m.H, m.F, m.V = (cfg.emb_dim, cfg.num_heads, cfg.mlp_dim,
+                          cfg.vocab_size)
+    m.L, m.E, m.NL = L, cross['E'], cfg.num_decoder_layers
+    m.R, m.B, m.beams = R, cross['B'], beams
+    m.embedding, m.rel_bias = P(w.embedding), P(w.rel_bias(L))
+    m.ln_final, m.logits_w = P(w.ln_final), P(w.logits.data)
+    m.logits_scales = P(w.logits.scales)
+    m.layers = layers
+    m.cache_index, m.enc_len = P(cache_index), P(cross['enc_len'])
+    for name in ('x', 'x1', 'x2', 'xn', 'qkv', 'q', 'ao', 'h', 'logits'):
+      setattr(m, name, P(getattr(bufs, name)))
+    m.gate = P(gate)
+    m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate)
+    return m
+
+  def _step_buffers(self, R, w):
+    if R not in self._bufs:
+      self._bufs[R] = _StepBuffers(self.config, R, self._dev(), w.act_dtype)
+    return self._bufs[R]
+
   def _decode(self, variables, encoded, encoder_input_tokens,
               decoder_input_tokens, decoder_target_tokens,
               enable_dropout=False, decode=False, max_decode_length=None,
@@ -339,6 +392,7 @@ class Transformer:
     del decoder_target_tokens, enable_dropout
     if not decode:
       raise NotImplementedError('only decode=True (single-step) is implemented')
+    from t5x_amd import _lib
     cfg, dev = self.config, self._dev()
     w = self.decoder_weights(variables['params'])
     cache = variables['cache']
@@ -359,52 +413,184 @@ class Transformer:
                        '%s instead got %s.' % ((R, 1), tuple(ids.shape)))
     if R != cross['B'] * beams:
       raise ValueError(f'{R} decoder rows vs {cross["B"]} x {beams} encoder rows')
-    key = (R,)
-    if key not in self._bufs:
-      self._bufs[key] = _StepBuffers(cfg, R, dev, w.act_dtype)
-    b = self._bufs[key]
+    b = self._step_buffers(R, w)
     b.ids.copy_(ids.reshape(R).to(torch.int32))
 
-    ops.embed(w.embedding, b.ids, b.x)
-    x = b.x
-    index_leaves = []
-    for i, lw in enumerate(w.layers):
+    layer_caches, index_leaves = [], []
+    for i in range(cfg.num_decoder_layers):
       c = cache['decoder'][f'layers_{i}']['self_attention']
-      ck, cv, ci = c['cached_key'], c['cached_value'], c['cache_index']
-      L = ck.shape[-1]
-      if max_decode_length and L < max_decode_length:
-        raise ValueError(f'cache length {L} < max_decode_length '
-                         f'{max_decode_length}')
-      index_leaves.append(ci)
-      ops.rmsnorm(x, lw['ln_self'], b.xn)
-      ops.gemm(b.xn, lw['qkv'], b.qkv)
-      ops.self_attention_step(b.qkv, ck, cv, w.rel_bias(L), ci, b.ao)
-      ops.gemm(b.ao, lw['self_out'], b.x1, residual=x)
-      ops.rmsnorm(b.x1, lw['ln_cross'], b.xn)
-      ops.gemm(b.xn, lw['cross_q'], b.q)
-      ops.cross_attention_step(b.q, cross['k'][i], cross['v'][i],
-                               cross['enc_len'], beams, b.ao)
-      ops.gemm(b.ao, lw['cross_out'], b.x2, residual=b.x1)
-      ops.rmsnorm(b.x2, lw['ln_mlp'], b.xn)
-      ops.gemm(b.xn, lw['wi'], b.h)
-      ops.gemm(b.h, lw['wo'], b.x, residual=b.x2)
-      x = b.x
-    ops.rmsnorm(x, w.ln_final, b.xn)
-    ops.gemm(b.xn, w.logits, b.logits, out_dtype=torch.float32)
-    # cache_index += 1 for every layer (layers.py:275): one launch when the
-    # leaves are consecutive elements of one vector.
+      ck, cv = c['cached_key'], c['cached_value']
+      for t in (ck, cv):
+        if (not t.is_contiguous() or t.dtype != w.act_dtype or
+            tuple(t.shape[:3]) != (R, cfg.num_heads, cfg.head_dim)):
+          raise ValueError(f'cache leaf of layer {i}: shape {tuple(t.shape)} '
+                           f'dtype {t.dtype} contiguous={t.is_contiguous()}')
+      layer_caches.append((ck, cv))
+      index_leaves.append(c['cache_index'])
+    L = layer_caches[0][0].shape[-1]
+    if max_decode_length and L < max_decode_length:
+      raise ValueError(f'cache length {L} < max_decode_length '
+                       f'{max_decode_length}')
+    # cache_index leaves are consecutive elements of one int32 vector when the
+    # tree came from init_cache; otherwise gather them into one.
     first = index_leaves[0]
-    contiguous = all(
-        ci.data_ptr() == first.data_ptr() + 4 * j
-        for j, ci in enumerate(index_leaves))
-    if contiguous:
-      base = first.as_strided((len(index_leaves),), (1,))
-      ops.add_i32(base, 1)
+    consecutive = all(ci.dtype == torch.int32 and ci.is_cuda and
+                      ci.data_ptr() == first.data_ptr() + 4 * j
+                      for j, ci in enumerate(index_leaves))
+    if consecutive:
+      index_vec = first.as_strided((len(index_leaves),), (1,))
     else:
-      for ci in index_leaves:
-        ops.add_i32(ci, 1)
+      index_vec = torch.stack([ci.reshape(()).to(dev, torch.int32)
+                               for ci in index_leaves])
+    key = (id(w), R, beams, L, layer_caches[0][0].data_ptr(),
+           layer_caches[-1][1].data_ptr(), index_vec.data_ptr(),
+           cross['k'][0].data_ptr())
+    if self._step_cache is None or self._step_cache[0] != key:
+      self._step_cache = (key, self._model_step(w, cross, b, layer_caches,
+                                                index_vec, R, beams, L))
+    m = self._step_cache[1]
+    _lib.call('t5d_decoder_step', _lib.stream_handle(), m, b.ids.data_ptr())
+    if not consecutive:
+      for j, name in enumerate(cache['decoder']):
+        cache['decoder'][name]['self_attention']['cache_index'] = index_vec[j]
     logits = b.logits.view(R, 1, cfg.vocab_size)
     return (logits, {'cache': cache}) if mutable else logits
+
+  # -- fused beam search: one graph replay per loop iteration ------------------------
+  def make_fused_beam_step(self, loop, params, encoded, enc_tokens):
+    """Returns a FusedBeamStep driving `loop` (a decoding.BeamLoop), or None
+    when this configuration has to use the generic per-call path."""
+    if not isinstance(encoded, BeamShared) or loop.cache_offset != 0:
+      return None
+    if loop.beam_size > 8:
+      return None
+    return FusedBeamStep(self, loop, params, encoded, enc_tokens)
+
+
+class FusedBeamStep:
+  """Whole beam-search iterations as replays of one captured HIP graph.
+
+  Owns the beam-expanded self-attention caches as one block
+  [layers, 2, B*K, H, 64, L] (so the reorder is a single launch over the valid
+  prefix) and runs on its own stream.  The loop flag lives on the device and
+  gates every kernel, so iterations enqueued after the loop condition turned
+  false change nothing."""
+
+  def __init__(self, module, loop, params, encoded, enc_tokens):
+    from t5x_amd import _lib
+    self._lib = _lib
+    cfg, dev = module.config, module._dev()
+    self.module, self.loop = module, loop
+    w = module.decoder_weights(params)
+    enc_tok = enc_tokens.x
+    enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
+        enc_tok, torch.Tensor) else enc_tok.to(dev)
+    cross = module._cross_kv(w, encoded.x, enc_tok, encoded.beams)
+    B, K = loop.batch_size, loop.beam_size
+    if cross['B'] != B or encoded.beams != K:
+      raise ValueError('encoder batch / beams do not match the decode loop')
+    R, S = B * K, loop.max_decode_len
+    act = w.act_dtype
+    el = 16 // torch.empty((), dtype=act).element_size()
+    L = (S - 1 + el - 1) // el * el
+    nl = cfg.num_decoder_layers
+    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
+                          dtype=act, device=dev)
+    self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
+    self.bufs = _StepBuffers(cfg, R, dev, act)
+    k2 = 2 * K
+    f32, i32 = torch.float32, torch.int32
+    self.topk_vals = torch.empty((B, k2), dtype=f32, device=dev)
+    self.topk_idx = torch.empty((B, k2), dtype=i32, device=dev)
+    self.row_max = torch.empty((R,), dtype=f32, device=dev)
+    self.row_lse = torch.empty((R,), dtype=f32, device=dev)
+    self.scratch = torch.empty((2 * R * k2,), dtype=i32, device=dev)
+    layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
+    self.model = module._model_step(w, cross, self.bufs, layer_caches,
+                                    self.cache_index, R, K, L,
+                                    gate=loop.keep_going)
+    st = loop.cur
+    bs = _lib.BeamStep()
+    bs.state = st._ptrs
+    P = _lib.ptr
+    bs.inputs, bs.initial_index = P(loop.inputs_dev), P(loop.init_idx_dev)
+    bs.brevity, bs.top_alive = P(loop.brevity), P(loop.top_alive)
+    bs.topk_vals, bs.topk_idx = P(self.topk_vals), P(self.topk_idx)
+    bs.row_max, bs.row_lse = P(self.row_max), P(self.row_lse)
+    bs.scratch, bs.ids = P(self.scratch), P(self.bufs.ids)
+    bs.keep_going = P(loop.keep_going)
+    bs.S, bs.Lin, bs.eos_id = S, loop.inputs_dev.shape[1], int(loop.eos_id)
+    bs.min_brevity, bs.min_log_prob = loop.min_brevity, loop.min_log_prob
+    bs.max_decode_step = int(loop.max_decode_step)
+    bs.min_initial_index = loop.min_initial
+    bs.kv_base = P(self.kv)
+    bs.kv_tensor_stride_bytes = self.kv[0, 0].numel() * self.kv.element_size()
+    bs.n_kv_tensors = 2 * nl
+    self.beam = bs
+    self.stream = torch.cuda.Stream(device=dev)
+    self.graph = None
+    self._capture()
+
+  def _enqueue(self):
+    self._lib.call('t5d_beam_search_step', self.stream.cuda_stream,
+                   self.model, self.beam)
+
+  def _capture(self):
+    lib, loop = self._lib, self.loop
+    self.stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(self.stream):
+      # First launches load the code objects; do them with the gate closed so
+      # nothing is computed, then open the gate with the real loop condition.
+      loop.keep_going.zero_()
+      self._enqueue()
+      self.stream.synchronize()
+      lib.call('t5d_graph_begin', self.stream.cuda_stream)
+      try:
+        self._enqueue()
+      finally:
+        handle = ctypes_void_p()
+        lib.call('t5d_graph_end', self.stream.cuda_stream, handle_ref(handle))
+      self.graph = handle
+      from t5x_amd import ops
+      ops.beam_cond(loop.cur, loop.min_brevity, loop.min_log_prob,
+                    loop.max_decode_step, loop.min_initial, loop.keep_going)
+    self.stream.synchronize()
+
+  def launch(self, n=1):
+    for _ in range(n):
+      self._lib.call('t5d_graph_launch', self.graph, self.stream.cuda_stream)
+
+  def keep_going(self) -> bool:
+    self.stream.synchronize()
+    return bool(self.loop.keep_going.item())
+
+  def finish(self):
+    torch.cuda.current_stream().wait_stream(self.stream)
+
+  def cache_tree(self):
+    """The caches in the reference's tree layout (views of the block)."""
+    nl = self.kv.shape[0]
+    return {'decoder': {
+        f'layers_{i}': {'self_attention': {
+            'cached_key': self.kv[i, 0], 'cached_value': self.kv[i, 1],
+            'cache_index': self.cache_index[i]}} for i in range(nl)}}
+
+  def __del__(self):
+    try:
+      if self.graph is not None:
+        self._lib.call('t5d_graph_destroy', self.graph)
+    except Exception:  # pylint: disable=broad-except
+      pass
+
+
+def ctypes_void_p():
+  import ctypes
+  return ctypes.c_void_p()
+
+
+def handle_ref(h):
+  import ctypes
+  return ctypes.byref(h)
 
 
 def init_params(cfg: T5Config, seed: int = 0, device=None,

@@ -237,11 +237,13 @@ def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
   _chk(cross_key, 'cross_key', q.dtype, 4)
   _chk(cross_value, 'cross_value', q.dtype, 4)
   _chk(enc_len, 'enc_len', torch.int32, 1)
-  B, H, D, E = cross_key.shape
+  B, H, E, D = cross_key.shape
   if D != 64:
     raise ValueError('head_dim must be 64')
-  if cross_value.shape != cross_key.shape:
-    raise ValueError('cross_key / cross_value shapes differ')
+  if tuple(cross_value.shape) != (B, H, D, E):
+    raise ValueError(f'cross_key {tuple(cross_key.shape)} is [B, H, E, 64]; '
+                     f'cross_value must be [B, H, 64, E], got '
+                     f'{tuple(cross_value.shape)}')
   if tuple(q.shape) != (B * beams, H * D):
     raise ValueError(f'q shape {tuple(q.shape)} != {(B * beams, H * D)}')
   if enc_len.shape[0] != B:

@@ -233,8 +233,8 @@ def test_cross_attention_step(ops, dt, B, beams, H, E):
       params, q[:, None, :], None, mask, None, num_heads=H, head_dim=D,
       dtype=od, projected_kv=(np.repeat(k, beams, axis=0),
                               np.repeat(v, beams, axis=0)))
-  kd = dev(np.ascontiguousarray(k.transpose(0, 2, 3, 1)), dt)
-  vd = dev(np.ascontiguousarray(v.transpose(0, 2, 3, 1)), dt)
+  kd = dev(np.ascontiguousarray(k.transpose(0, 2, 1, 3)), dt)  # [B,H,E,D]
+  vd = dev(np.ascontiguousarray(v.transpose(0, 2, 3, 1)), dt)  # [B,H,D,E]
   out = ops.cross_attention_step(dev(q, dt), kd, vd, dev(lens), beams)
   np.testing.assert_allclose(host(out), want[:, 0], atol=TOL[dt],
                              rtol=TOL[dt])
