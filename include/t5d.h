@@ -111,6 +111,19 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
                             const void* rel_bias, const int32_t* cache_index,
                             void* out, int R, int H, int L);
 
+/* As t5d_self_attention_step for the B*beams rows of a beam search, but first
+ * applying a beam gather that the caller deferred
+ * (cache_gather_beams, t5x/decoding.py:1449-1457): row (b, e) attends over the
+ * cache of row (b, pending_src[b, e]) and, if the item's beams were permuted,
+ * that cache is written into slot (b, e).  After the call the caches equal
+ * gather-then-step.  bfloat16 only; beams * ceil(L/128) <= 16. */
+int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
+                                   void* cached_key, void* cached_value,
+                                   const void* rel_bias,
+                                   const int32_t* cache_index, void* out,
+                                   int B, int beams, int H, int L,
+                                   const int32_t* pending_src);
+
 /* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
  * mask :366-370).  The reference re-projects K/V from the beam-expanded
  * encoder output every step; here they are projected once per batch item:
@@ -270,6 +283,9 @@ typedef struct {
   /* optional device flag: when non-NULL and 0, every kernel of the step
    * returns immediately (the step becomes a no-op) */
   const int32_t* gate;
+  /* optional [B, beams] source-beam indices of a deferred cache gather, applied
+   * inside the self-attention kernels (t5d_self_attention_step_gather) */
+  const int32_t* pending_src;
 } t5d_model_step;
 
 /* One decoder step for R rows (Decoder.__call__ with decode=True,
@@ -301,7 +317,9 @@ typedef struct {
 
 /* One iteration of the beam_search loop body plus the loop condition
  * (t5x/decoding.py:1250-1506): gather ids, decoder step, log_softmax + top-2K,
- * bookkeeping, cache reorder over the valid prefix, condition -> *keep_going.
+ * bookkeeping, cache reorder over the valid prefix (done here, or deferred to
+ * the next step's self-attention when model->pending_src == beam->top_alive;
+ * top_alive must then start as the identity), condition -> *keep_going.
  * Every kernel is gated on *keep_going, so iterations enqueued after the
  * condition turned false leave all state untouched. */
 int t5d_beam_search_step(void* stream, const t5d_model_step* model,

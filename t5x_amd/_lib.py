@@ -41,7 +41,7 @@ class ModelStep(Structure):
           'embedding', 'rel_bias', 'ln_final', 'logits_w', 'logits_scales')] +
               [('layers', POINTER(Layer))] + [(n, c_void_p) for n in (
                   'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
-                  'ao', 'h', 'logits', 'gate')])
+                  'ao', 'h', 'logits', 'gate', 'pending_src')])
 
 
 class BeamStep(Structure):
@@ -77,6 +77,9 @@ _SIGNATURES = {
                          c_int, c_int, c_int, _P, _P]),
     't5d_self_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P,
                                         c_int, c_int, c_int]),
+    't5d_self_attention_step_gather': (c_int, [_P, c_int, _P, _P, _P, _P, _P,
+                                               _P, c_int, c_int, c_int, c_int,
+                                               _P]),
     't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
                                          c_int, c_int, c_int]),
     't5d_add_i32': (c_int, [_P, _P, c_int, c_int]),

@@ -54,9 +54,16 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
     T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
                      m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
-    T5D_TRY(t5d_self_attention_step(stream, dt, m->qkv, w.cached_key,
-                                    w.cached_value, m->rel_bias,
-                                    m->cache_index + l, m->ao, R, m->H, m->L));
+    if (m->pending_src)
+      T5D_TRY(t5d_self_attention_step_gather(
+          stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
+          m->cache_index + l, m->ao, m->B, m->beams, m->H, m->L,
+          m->pending_src));
+    else
+      T5D_TRY(t5d_self_attention_step(stream, dt, m->qkv, w.cached_key,
+                                      w.cached_value, m->rel_bias,
+                                      m->cache_index + l, m->ao, R, m->H,
+                                      m->L));
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.self_out, w.self_out_scales,
                      x, m->x1, R, HD, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
     T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
@@ -92,6 +99,9 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
               T5D_EINVAL, "t5d_beam_search_step: null buffer");
   T5D_REQUIRE(m->gate == b->keep_going, T5D_EINVAL,
               "t5d_beam_search_step: the model gate must be the loop flag");
+  T5D_REQUIRE(m->pending_src == nullptr || m->pending_src == b->top_alive,
+              T5D_EINVAL,
+              "t5d_beam_search_step: pending_src must be the top_alive buffer");
   const int R = m->R, K = m->beams, B = m->B;
   {
     GateScope gate(b->keep_going);
@@ -106,8 +116,10 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
   T5D_TRY(t5d_beam_update(stream, &b->state, &b->state, b->topk_vals,
                           b->topk_idx, b->inputs, b->initial_index, b->brevity,
                           b->top_alive, B, K, b->S, b->Lin, m->V, b->eos_id));
-  // After the update cur_index == number of valid cache columns.
-  if (K > 1)
+  // After the update cur_index == number of valid cache columns.  When the
+  // model applies pending gathers inside its self-attention (pending_src ==
+  // top_alive) the reorder happens there, on the next step.
+  if (K > 1 && m->pending_src == nullptr)
     T5D_TRY(t5d_cache_gather_beams(
         stream, b->kv_base, b->kv_tensor_stride_bytes, b->n_kv_tensors,
         m->dtype == T5D_F32 ? 4 : 2, B, K, m->H * 64, m->L, b->top_alive,
@@ -136,7 +148,7 @@ extern "C" int t5d_graph_end(void* stream, void** graph_exec) {
               hipGetErrorString(e));
   hipGraphExec_t exec = nullptr;
   e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-  hipGraphDestroy(graph);
+  (void)hipGraphDestroy(graph);
   T5D_REQUIRE(e == hipSuccess && exec, T5D_EHIP,
               "t5d_graph_end: instantiate: %s", hipGetErrorString(e));
   *graph_exec = exec;

@@ -346,7 +346,7 @@ class Transformer:
 
   # -- the decode step -------------------------------------------------------------
   def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
-                  L, gate=None):
+                  L, gate=None, pending_src=None):
     """Fills a t5d_model_step for one call of t5d_decoder_step."""
     from t5x_amd import _lib
     cfg = self.config
@@ -377,7 +377,9 @@ class Transformer:
     for name in ('x', 'x1', 'x2', 'xn', 'qkv', 'q', 'ao', 'h', 'logits'):
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
-    m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate)
+    m.pending_src = P(pending_src)
+    m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
+                    pending_src)
     return m
 
   def _step_buffers(self, R, w):
@@ -506,9 +508,17 @@ class FusedBeamStep:
     self.row_lse = torch.empty((R,), dtype=f32, device=dev)
     self.scratch = torch.empty((2 * R * k2,), dtype=i32, device=dev)
     layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
-    self.model = module._model_step(w, cross, self.bufs, layer_caches,
-                                    self.cache_index, R, K, L,
-                                    gate=loop.keep_going)
+    # With bfloat16 caches the reorder of a step is deferred into the next
+    # step's self-attention kernels, which read each row's cache from its
+    # source beam anyway; the permutation in flight lives in loop.top_alive.
+    self.deferred_gather = (K > 1 and act == torch.bfloat16 and
+                            K * ((L + 127) // 128) <= 16)
+    loop.top_alive.copy_(torch.arange(K, dtype=torch.int32,
+                                      device=dev).expand(B, K))
+    self.model = module._model_step(
+        w, cross, self.bufs, layer_caches, self.cache_index, R, K, L,
+        gate=loop.keep_going,
+        pending_src=loop.top_alive if self.deferred_gather else None)
     st = loop.cur
     bs = _lib.BeamStep()
     bs.state = st._ptrs
@@ -570,6 +580,18 @@ class FusedBeamStep:
   def cache_tree(self):
     """The caches in the reference's tree layout (views of the block)."""
     nl = self.kv.shape[0]
+    if self.deferred_gather:
+      # Apply the reorder still in flight, then mark it done.
+      from t5x_amd import ops
+      B, K = self.loop.top_alive.shape
+      with torch.cuda.stream(self.stream):
+        ops.cache_gather_beams(
+            self.kv[0, 0].view(B, K, *self.kv.shape[3:]), self.loop.top_alive,
+            n_tensors=2 * nl,
+            tensor_stride_bytes=self.kv[0, 0].numel() * self.kv.element_size())
+        self.loop.top_alive.copy_(torch.arange(
+            K, dtype=torch.int32, device=self.kv.device).expand(B, K))
+      self.stream.synchronize()
     return {'decoder': {
         f'layers_{i}': {'self_attention': {
             'cached_key': self.kv[i, 0], 'cached_value': self.kv[i, 1],

@@ -205,7 +205,9 @@ def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
 
 
 def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
-                        out=None):
+                        out=None, pending_src=None):
+  """One cached self-attention step; with pending_src [B, beams] the rows'
+  caches are first gathered from their source beams inside the kernel."""
   _chk(qkv, 'qkv', ndim=2)
   _chk(cached_key, 'cached_key', qkv.dtype, 4)
   _chk(cached_value, 'cached_value', qkv.dtype, 4)
@@ -225,6 +227,17 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
   if out is None:
     out = torch.empty((R, H * D), dtype=qkv.dtype, device=qkv.device)
   _chk(out, 'out', qkv.dtype, 2)
+  if pending_src is not None:
+    _chk(pending_src, 'pending_src', torch.int32, 2)
+    B, beams = pending_src.shape
+    if B * beams != R:
+      raise ValueError(f'pending_src {(B, beams)} does not cover {R} rows')
+    _lib.call('t5d_self_attention_step_gather', _s(),
+              _lib.dtype_code(qkv.dtype), qkv.data_ptr(),
+              cached_key.data_ptr(), cached_value.data_ptr(),
+              rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), B,
+              beams, H, L, pending_src.data_ptr())
+    return out
   _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
             qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),
             rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), R, H,

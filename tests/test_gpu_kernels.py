@@ -208,6 +208,45 @@ def test_self_attention_step(ops, dt, R, H, L, t):
   np.testing.assert_allclose(host(out), want, atol=TOL[dt], rtol=TOL[dt])
 
 
+@pytest.mark.parametrize('B,beams,H,L,t', [(3, 4, 2, 128, 0), (3, 4, 2, 128, 1),
+                                           (3, 4, 3, 128, 77),
+                                           (2, 4, 2, 128, 127),
+                                           (2, 2, 2, 32, 9), (2, 8, 2, 256, 200),
+                                           (2, 3, 2, 384, 300),
+                                           (32, 4, 12, 128, 64)])
+def test_self_attention_step_with_pending_gather(ops, B, beams, H, L, t):
+  """The deferred reorder inside the kernel == cache_gather_beams followed by
+  the plain step, bit for bit (outputs and both caches).  The first batch item
+  keeps its beams in place, the second duplicates one beam (the common case
+  after a beam-search step), the rest are random."""
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(B * 131 + beams * 17 + L + t)
+  R, D, dt = B * beams, 64, torch.bfloat16
+  ck = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  cv = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  qkv = torch.randn((R, 3 * H * D), generator=gen, device='cuda').to(dt)
+  rel_bias = torch.randn((H, L), generator=gen, device='cuda').to(dt)
+  src = torch.randint(0, beams, (B, beams), generator=gen, device='cuda',
+                      dtype=torch.int32)
+  src[0] = torch.arange(beams, dtype=torch.int32)
+  src[1] = 0
+  idx = torch.tensor(t, dtype=torch.int32, device='cuda')
+
+  ck_a, cv_a = ck.clone(), cv.clone()
+  valid = torch.tensor(t, dtype=torch.int32, device='cuda')
+  for c in (ck_a, cv_a):
+    ops.cache_gather_beams(c.view(B, beams, H, D, L), src, valid_len=valid)
+  want = ops.self_attention_step(qkv, ck_a, cv_a, rel_bias, idx)
+
+  ck_b, cv_b = ck.clone(), cv.clone()
+  got = ops.self_attention_step(qkv, ck_b, cv_b, rel_bias, idx,
+                                pending_src=src)
+  assert torch.equal(got, want)
+  # columns 0..t are defined by the algorithm; the rest is never read
+  assert torch.equal(ck_b[..., :t + 1], ck_a[..., :t + 1])
+  assert torch.equal(cv_b[..., :t + 1], cv_a[..., :t + 1])
+
+
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('B,beams,H,E', [(2, 1, 3, 64), (3, 4, 2, 512),
                                          (2, 2, 2, 128), (1, 8, 2, 264),

@@ -297,3 +297,99 @@ def test_decoder_step_at_base_size_matches_oracle():
   print(f'base-size step: max |dlogit| = {err.max():.3g}, mean '
         f'{err.mean():.3g}, p99.9 {np.quantile(err, 0.999):.3g}')
   check_logits(host(got)[:, 0], want[:, 0], 'bfloat16', 'base')
+
+
+def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
+  """A step function over synthetic encoder output, as predict_batch builds
+  it.  eos_bias > 0 scales up the logits column of EOS so decodes finish early."""
+  from t5x_amd import decoding, models, network
+  _, gcfg = tiny(dtype)
+  dev = torch.device('cuda')
+  params = network.init_params(gcfg, seed, dev, with_encoder=False)
+  if eos_bias:
+    params['decoder']['logits_dense']['kernel'][:, 1] *= eos_bias
+  module = network.Transformer(gcfg, dev)
+  model = models.EncoderDecoderModel(module, decode_fn=decoding.beam_search)
+  rs = np.random.RandomState(seed)
+  tok = torch.as_tensor(ragged_tokens(rs, B, E, gcfg.vocab_size, 3), device=dev)
+  gen = torch.Generator(device=dev)
+  gen.manual_seed(seed)
+  encoded = torch.randn((B, E, gcfg.emb_dim), generator=gen,
+                        device=dev).to(network._TORCH_DTYPE[dtype])
+  fn = models.StepFunction(model, params, network.BeamShared(encoded, K),
+                           network.BeamShared(tok, K), L)
+  return module, fn
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+@pytest.mark.parametrize('B,K,L', [(3, 4, 12), (2, 2, 140), (5, 1, 9)])
+def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L):
+  """The captured whole-iteration graph (in-place state, gated kernels,
+  reorder deferred into the next step's attention for bf16) and the
+  kernel-per-call loop run the same kernels on the same values: sequences and
+  scores must be bit-identical, and so must the caches after every few steps."""
+  from t5x_amd import decoding
+  module, fn = _decode_setup(dtype, B, K, 24, L, seed=7)
+  inputs = np.zeros((B, L), np.int32)
+
+  fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                            num_decodes=K)
+  assert fused.fused is not None
+  plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
+                            eos_id=1, num_decodes=K)
+  assert plain.fused is None
+  step = -1
+  while True:
+    keep = plain.cond()
+    assert fused.cond() == keep, step
+    if not keep:
+      break
+    step += 1
+    fused.body()
+    plain.body()
+    if step % 5 == 2 or step >= L - 3:
+      for name in ('live_logprobs', 'finished_scores', 'live_seqs',
+                   'finished_seqs', 'finished_flags', 'cur_index'):
+        a = getattr(fused.cur, name)
+        fused.fused.stream.synchronize()
+        assert torch.equal(a, getattr(plain.cur, name)), (step, name)
+      fc = fused.fused.cache_tree()['decoder']
+      pc = plain.beam_cache['decoder']
+      n = step + 1
+      assert len(fc) == 3
+      for layer in fc:
+        for which in ('cached_key', 'cached_value'):
+          a = fc[layer]['self_attention'][which]
+          b = pc[layer]['self_attention'][which]
+          b = b.reshape(a.shape[0], *b.shape[-3:])
+          assert torch.equal(a[..., :n], b[..., :n]), (step, layer, which)
+  assert step >= L - 3, step
+  got, gs = fused.finish()
+  want, ws = plain.finish()
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
+
+
+@pytest.mark.parametrize('check_every', [1, 3, 8])
+def test_fused_loop_early_stop_is_independent_of_check_interval(check_every):
+  """With EOS made likely the loop ends long before max_decode_len; iterations
+  enqueued after the device-side condition turned false must change nothing,
+  and replaying the graph many times must keep giving the eager loop's result."""
+  from t5x_amd import decoding
+  B, K, L = 4, 4, 48
+  module, fn = _decode_setup('bfloat16', B, K, 16, L, seed=11, eos_bias=6.0)
+  inputs = np.zeros((B, L), np.int32)
+  plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
+                            eos_id=1, num_decodes=K)
+  plain.run()
+  want, ws = plain.finish()
+  steps = int(plain.cur.cur_index.item())
+  assert 0 < steps < L - 8, steps   # the case does stop early
+
+  fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                            num_decodes=K)
+  fused.run(check_every=check_every)
+  got, gs = fused.finish()
+  assert int(fused.cur.cur_index.item()) == steps
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
