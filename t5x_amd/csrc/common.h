@@ -41,16 +41,19 @@ __device__ __forceinline__ float bf16lo_to_f32(uint32_t packed) {
 __device__ __forceinline__ float bf16hi_to_f32(uint32_t packed) {
   return __uint_as_float(packed & 0xFFFF0000u);
 }
-// Round to nearest even (inputs are finite on this path).
+// Round to nearest even with the hardware conversion (v_cvt_pk_bf16_f32).
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_v;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_v;
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float round_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return __uint_as_float(u & 0xFFFF0000u);
+  return __uint_as_float(((uint32_t)f32_to_bf16(f)) << 16);
+}
+// Two values rounded and packed (lo in bits 0..15) by one instruction.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_v v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_v));
 }
 
 // Activation-dtype traits: how a value is rounded / loaded / stored.

@@ -180,6 +180,174 @@ beam_row_topk_kernel(const float* __restrict__ logits,
   }
 }
 
+// Fast path of the same computation for 16-byte aligned rows of at most 32768
+// elements with V % 4 == 0: 1024 threads per row, the row lives in registers
+// (8 float4 per thread, all loads issued at once), so logits are read from
+// memory exactly once.  Every thread keeps the best two of its 32 elements;
+// each wavefront then extracts its k best by k rounds of a 64-lane arg-best
+// (a lane that runs out of candidates rescans its registers for the next two
+// below the last one it gave away: rare, and skipped by a wave-uniform
+// branch), and wavefront 0 merges the 16 sorted lists the same way.
+constexpr int kFastTopkVec = 8;
+
+__device__ __forceinline__ void top2_insert(float f, int fi, float& v0, int& i0,
+                                            float& v1, int& i1) {
+  if (better(f, fi, v1, i1)) {
+    if (better(f, fi, v0, i0)) {
+      v1 = v0; i1 = i0; v0 = f; i0 = fi;
+    } else {
+      v1 = f; i1 = fi;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(1024)
+beam_row_topk_fast_kernel(const float* __restrict__ logits,
+                          const float* __restrict__ live_logprobs,
+                          float* __restrict__ row_max,
+                          float* __restrict__ row_lse,
+                          float* __restrict__ cand_vals,
+                          int32_t* __restrict__ cand_idx, int V, int beams,
+                          int k, const int32_t* gate) {
+  __shared__ float s_f[16];
+  __shared__ double s_d[16];
+  __shared__ float s_cv[16][16];
+  __shared__ int s_ci[16][16];
+  T5D_GATED(gate);
+  constexpr int kNone = 0x7FFFFFFF;
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const float4* x4 = reinterpret_cast<const float4*>(logits + (size_t)r * V);
+  const int nvec = V >> 2;
+  float4 x[kFastTopkVec];
+#pragma unroll
+  for (int u = 0; u < kFastTopkVec; ++u) {
+    const int vi = u * 1024 + tid;
+    x[u] = vi < nvec ? x4[vi]
+                     : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  }
+  const float lp = live_logprobs[r];
+
+  float m = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < kFastTopkVec; ++u)
+    m = fmaxf(fmaxf(m, fmaxf(x[u].x, x[u].y)), fmaxf(x[u].z, x[u].w));
+  m = wave_max(m);
+  if (lane == 0) s_f[wave] = m;
+  __syncthreads();
+  m = s_f[lane & 15];
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+
+  double sum = 0.0;
+#pragma unroll
+  for (int u = 0; u < kFastTopkVec; ++u) {
+    // exp(-inf) == 0 for the padding
+    sum += (double)expf(x[u].x - m);
+    sum += (double)expf(x[u].y - m);
+    sum += (double)expf(x[u].z - m);
+    sum += (double)expf(x[u].w - m);
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  if (lane == 0) s_d[wave] = sum;
+  __syncthreads();
+  sum = s_d[lane & 15];
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  const float lse = (float)log(sum);
+  if (tid == 0) {
+    row_max[r] = m;
+    row_lse[r] = lse;
+  }
+
+  // f(j) = ((x[j] - max) - lse) + live_logprob, in place.
+  const int base = (r % beams) * V;
+  float v0 = -INFINITY, v1 = -INFINITY;
+  int i0 = kNone, i1 = kNone;
+#pragma unroll
+  for (int u = 0; u < kFastTopkVec; ++u) {
+    const int vi = u * 1024 + tid;
+    const int j = base + 4 * vi;
+    const bool in = vi < nvec;
+    x[u].x = ((x[u].x - m) - lse) + lp;
+    x[u].y = ((x[u].y - m) - lse) + lp;
+    x[u].z = ((x[u].z - m) - lse) + lp;
+    x[u].w = ((x[u].w - m) - lse) + lp;
+    if (in) {
+      top2_insert(x[u].x, j, v0, i0, v1, i1);
+      top2_insert(x[u].y, j + 1, v0, i0, v1, i1);
+      top2_insert(x[u].z, j + 2, v0, i0, v1, i1);
+      top2_insert(x[u].w, j + 3, v0, i0, v1, i1);
+    }
+  }
+
+  // k rounds per wavefront.  `have` counts the valid entries of (v0, v1);
+  // (lv, li) is the last candidate this lane gave away.
+  int have = 2;
+  float lv = INFINITY;
+  int li = -1;
+  for (int out = 0; out < k; ++out) {
+    if (__builtin_amdgcn_ballot_w64(have == 0) != 0) {
+      if (have == 0) {  // rescan: best two strictly after (lv, li)
+        v0 = v1 = -INFINITY;
+        i0 = i1 = kNone;
+#pragma unroll
+        for (int u = 0; u < kFastTopkVec; ++u) {
+          const int vi = u * 1024 + tid;
+          const int j = base + 4 * vi;
+          if (vi < nvec) {
+            if (better(lv, li, x[u].x, j))
+              top2_insert(x[u].x, j, v0, i0, v1, i1);
+            if (better(lv, li, x[u].y, j + 1))
+              top2_insert(x[u].y, j + 1, v0, i0, v1, i1);
+            if (better(lv, li, x[u].z, j + 2))
+              top2_insert(x[u].z, j + 2, v0, i0, v1, i1);
+            if (better(lv, li, x[u].w, j + 3))
+              top2_insert(x[u].w, j + 3, v0, i0, v1, i1);
+          }
+        }
+        have = 2;  // entries may be (-inf, none): they lose every comparison
+      }
+    }
+    Cand head = {v0, i0};
+    Cand best = wave_best(head);
+    if (head.i == best.i && best.i != kNone) {  // indices are unique
+      lv = v0; li = i0;
+      v0 = v1; i0 = i1;
+      v1 = -INFINITY; i1 = kNone;
+      --have;
+    }
+    if (lane == 0) {
+      s_cv[wave][out] = best.v;
+      s_ci[wave][out] = best.i;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // Merge the 16 best-first lists: lane w < 16 walks list w.
+  int pos = 0;
+  for (int out = 0; out < k; ++out) {
+    Cand head = {-INFINITY, kNone};
+    if (lane < 16 && pos < k) {
+      head.v = s_cv[lane][pos];
+      head.i = s_ci[lane][pos];
+    }
+    Cand best = head;
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) {
+      float v = __shfl_xor(best.v, o, 64);
+      int i = __shfl_xor(best.i, o, 64);
+      if (better(v, i, best.v, best.i)) { best.v = v; best.i = i; }
+    }
+    if (lane < 16 && head.i == best.i && best.i != kNone) ++pos;
+    if (lane == 0) {
+      cand_vals[(size_t)r * k + out] = best.v;
+      cand_idx[(size_t)r * k + out] = best.i;
+    }
+  }
+}
+
 // Merge the beams' per-row candidates of one batch item: one candidate per
 // thread (beams*k <= 128), rank by counting better candidates.
 __global__ void __launch_bounds__(128)
@@ -674,7 +842,11 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
   float* cand_vals = (float*)scratch;
   int32_t* cand_idx = (int32_t*)((char*)scratch + (size_t)R * k * 4);
   hipStream_t s = as_stream(stream);
-  if (k <= 4)
+  if (V % 4 == 0 && V <= kFastTopkVec * 4096 && ((uintptr_t)logits % 16) == 0)
+    hipLaunchKernelGGL(beam_row_topk_fast_kernel, dim3(R), dim3(1024), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k, tls_gate);
+  else if (k <= 4)
     hipLaunchKernelGGL(beam_row_topk_kernel<4>, dim3(R), dim3(256), 0, s,
                        logits, live_logprobs, row_max, row_lse, cand_vals,
                        cand_idx, V, beams, k, tls_gate);

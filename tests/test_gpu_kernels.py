@@ -320,6 +320,45 @@ def test_beam_topk(ops, B, beams, V):
   np.testing.assert_array_equal(host(vals), wv)
 
 
+@pytest.mark.parametrize('V', [32128, 4096 * 8, 4100, 512, 250])
+@pytest.mark.parametrize('pattern', ['one_thread', 'one_wave', 'all_equal',
+                                     'descending'])
+def test_beam_topk_adversarial_placements(ops, V, pattern):
+  """Placements that stress how the row kernel splits the vocabulary over
+  lanes: all winners in the registers of one thread (consecutive elements and
+  elements 4096 apart), all in one wavefront, a constant row (pure index
+  ties), and a sorted row.  Selection must equal the oracle's top_k exactly."""
+  B, beams = 2, 4
+  k = 2 * beams
+  rs = np.random.RandomState(V)
+  logits = rs.randn(B * beams, V).astype(np.float32)
+  if pattern == 'one_thread':
+    hot = [4 * 77 + c for c in range(4)] + [4 * 77 + 4096 * u for u in range(1, 8)]
+    hot = [j for j in hot if j < V]
+    logits[:, hot] += 20 + rs.rand(B * beams, len(hot)).astype(np.float32)
+  elif pattern == 'one_wave':
+    hot = np.arange(4 * 64 * 3, min(V, 4 * 64 * 4))[:40]
+    logits[:, hot] += 20
+  elif pattern == 'all_equal':
+    logits[:] = 0.5
+  else:
+    logits[:] = -np.arange(V, dtype=np.float32)[None, :] / 64
+  live = np.sort(-np.abs(rs.randn(B, beams)).astype(np.float32), axis=1)
+  if pattern == 'all_equal':
+    live[:] = -1.0
+  vals, idx, row_max, row_lse = ops.beam_topk(dev(logits), dev(live), k)
+  cand = ((logits - host(row_max)[:, None]) - host(row_lse)[:, None]).astype(
+      np.float32)
+  flat = (cand.reshape(B, beams, V) + live[:, :, None]).astype(
+      np.float32).reshape(B, beams * V)
+  wv, wi = odec.top_k(flat, k)
+  np.testing.assert_array_equal(host(idx), wi)
+  np.testing.assert_array_equal(host(vals), wv)
+  lp = odec.log_softmax(logits)
+  want_lse = -(lp - (logits - logits.max(-1, keepdims=True)))[:, 0]
+  np.testing.assert_allclose(host(row_lse), want_lse, atol=1e-5, rtol=1e-6)
+
+
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('B,beams,H,L,valid', [(2, 2, 2, 32, None),
                                                (3, 4, 3, 128, 57),
