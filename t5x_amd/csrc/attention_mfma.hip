@@ -66,19 +66,21 @@ __device__ long long t5d_probe_buf[64 * 16];
 #endif
 
 // ---- cross-attention -----------------------------------------------------------
-// NQP: query rows padded to a multiple of 4 (4, 8).  WM: max wavefronts.
+// scores^T = K·Q^T with the K tile (16 positions x 32 dims) as the A operand
+// and Q^T as the B operand whose 16 columns are the NQP (4 or 8) query rows
+// repeated REP = 16 / NQP times.  The repeats cost nothing on the matrix
+// cores and leave every score in REP lanes; copy s of a column keeps the
+// tiles jt = s (mod REP), so the softmax runs on all 64 lanes with 32 / REP
+// scores each instead of 32 scores in 16 lanes.  out^T = V·P^T likewise (V
+// tile as A, P^T with repeated query columns as B).
 template <int NQP, int WM>
 __global__ void __launch_bounds__(64 * WM)
 cross_attn_mfma_kernel(AttnMfmaArgs a) {
-  __shared__ float s_red[WM][NQP];
-  // s_p (probabilities, bf16) and s_out (partial outputs, f32) are used one
-  // after the other and share storage.
-  __shared__ __attribute__((aligned(16))) float s_raw[WM * NQP * kHeadDim];
-  bf16_t (*s_p)[NQP][kBlockJ] =
-      reinterpret_cast<bf16_t (*)[NQP][kBlockJ]>(s_raw);
-  float (*s_out)[NQP][kHeadDim] =
-      reinterpret_cast<float (*)[NQP][kHeadDim]>(s_raw);
-  static_assert(sizeof(bf16_t) * kBlockJ <= sizeof(float) * kHeadDim, "alias");
+  constexpr int REP = 16 / NQP;   // copies of each query column
+  constexpr int TPL = 8 / REP;    // score tiles a lane keeps
+  __shared__ float s_red[2][WM][16];
+  __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][NQP][kBlockJ];
+  __shared__ __attribute__((aligned(16))) float s_out[WM][NQP][kHeadDim];
   T5D_GATED(a.gate);
 
   const int h = blockIdx.x, b = blockIdx.y;
@@ -86,226 +88,236 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nwaves = blockDim.x >> 6;
   const int n16 = lane & 15, g = lane >> 4;
+  const int q = n16 % NQP, rep = n16 / NQP;
   const int HD = a.H * kHeadDim;
 
-  T5D_STAMP(0);
   int n = a.index[b];
   n = n < 0 ? 0 : (n > a.S ? a.S : n);
   bool uniform = false;  // no valid key: the masked softmax is uniform
   if (n == 0) { uniform = true; n = a.S; }
-  T5D_STAMP(1);
 
-  const int jw = wave * kBlockJ;          // first position of this wavefront
-  const bool wave_live = jw < n;
+  const int jw = wave * kBlockJ;  // first position of this wavefront
   const bf16_t* kbase = a.k + ((size_t)b * a.H + h) * (size_t)a.S * kHeadDim;
   const bf16_t* vbase = a.v + ((size_t)b * a.H + h) * (size_t)kHeadDim * a.S;
+  const int nw = n - jw;  // valid positions of this wavefront (may be <= 0)
 
-  // A operand of Q·K^T: lane (m = n16, g) holds Q[m][32c + 8g .. +8].
-  Frag16 qa[2];
-  {
-    const bool qrow = n16 < a.nq;
-    const bf16_t* qp = a.q + (size_t)(b * a.nq + (qrow ? n16 : 0)) * a.q_stride +
-                       h * kHeadDim + 8 * g;
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      if (qrow) qa[c].u = *reinterpret_cast<const uint4*>(qp + 32 * c);
-      else qa[c].u = make_uint4(0, 0, 0, 0);
-    }
-  }
-
-  // Every K and V chunk this lane needs is requested up front, before any of
-  // it is consumed, so one memory round trip covers the whole stream.
-  //   K: B operand of Q·K^T, lane (n = j%16, g) holds K[j][32c + 8g .. +8];
-  //   V: B operand of P·V,   lane (n = d%16, g) holds V[16dt + n16][32jb + 8g .. +8].
+  // Every K and V chunk is requested up front (whole 16 / 32 position tiles,
+  // skipped by wave-uniform branches beyond the valid length; inside a tile
+  // the tail past the valid length is read and masked, it must be finite).
+  //   K: A operand, lane (row = position n16, g) holds K[j][32c + 8g .. +8];
+  //   V: A operand, lane (row = d n16, g) holds V[16dt + n16][32jb + 8g .. +8].
+  // S is a multiple of 8 but not of the tile sizes: addresses are clamped to
+  // the last row / last 8 positions (those positions are masked anyway).
   Frag16 kb[8][2];
   Frag16 vb[4][4];
 #pragma unroll
   for (int jt = 0; jt < 8; ++jt) {
-    const int j = jw + 16 * jt + n16;
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      if (j < n)  // rows beyond the valid prefix are never requested
-        kb[jt][c].u = *reinterpret_cast<const uint4*>(
-            kbase + (size_t)j * kHeadDim + 32 * c + 8 * g);
-      else
-        kb[jt][c].u = make_uint4(0, 0, 0, 0);
-    }
-  }
-#pragma unroll
-  for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
-      const int j0 = jw + 32 * jb + 8 * g;
-      if (j0 < n)
-        vb[jb][dt].u = *reinterpret_cast<const uint4*>(
-            vbase + (size_t)(16 * dt + n16) * a.S + j0);
-      else
-        vb[jb][dt].u = make_uint4(0, 0, 0, 0);
-    }
-
-  // scores: tile jt covers positions jw + 16 jt .. +16; lane holds column
-  // n16 of the tile and rows q = 4g + i.
-  f32x4_v sc[8];
-#pragma unroll
-  for (int jt = 0; jt < 8; ++jt) sc[jt] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
-  if (wave_live) {
-#pragma unroll
-    for (int jt = 0; jt < 8; ++jt)
+    if (16 * jt < nw) {
 #pragma unroll
       for (int c = 0; c < 2; ++c)
-        sc[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[c].v, kb[jt][c].v,
-                                                         sc[jt], 0, 0, 0);
+        kb[jt][c].u = *reinterpret_cast<const uint4*>(
+            kbase + (size_t)min(jw + 16 * jt + n16, a.S - 1) * kHeadDim +
+            32 * c + 8 * g);
+    } else {
+      kb[jt][0].u = kb[jt][1].u = make_uint4(0, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int jb = 0; jb < 4; ++jb) {
+    if (32 * jb < nw) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+        vb[jb][dt].u = *reinterpret_cast<const uint4*>(
+            vbase + (size_t)(16 * dt + n16) * a.S +
+            min(jw + 32 * jb + 8 * g, a.S - 8));
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);
+    }
+  }
+  // B operand of K·Q^T: lane (col n16 -> query q, g) holds Q[q][32c + 8g .. +8].
+  Frag16 qb[2];
+  {
+    const bool qrow = q < a.nq;
+    const bf16_t* qp = a.q + (size_t)(b * a.nq + (qrow ? q : 0)) * a.q_stride +
+                       h * kHeadDim + 8 * g;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      qb[c].u = *reinterpret_cast<const uint4*>(qp + 32 * c);
+      if (!qrow) qb[c].u = make_uint4(0, 0, 0, 0);
+    }
   }
 
-  T5D_STAMP(2);
-  // Softmax over all positions of the workgroup, per query row q = 4g + i.
-  const bool rows_live = 4 * g < a.nq;
-  float mx[4];
+  // Tile jt: lane (n16, g) gets scores of positions 16 jt + 4g + i, query q.
+  // It keeps the tiles with jt % REP == rep.
+  float sc[TPL][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float m = -INFINITY;
+  for (int t = 0; t < TPL; ++t)
 #pragma unroll
-    for (int jt = 0; jt < 8; ++jt) {
-      const int j = jw + 16 * jt + n16;
-      float x = round_bf16(sc[jt][i]);
-      if (uniform) x = 0.f;
-      x = (j < n && rows_live) ? x : -INFINITY;
-      sc[jt][i] = x;
+    for (int r = 0; r < REP; ++r) {
+      const int jt = t * REP + r;
+      f32x4_v acc = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+      if (16 * jt < nw) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[jt][c].v, qb[c].v,
+                                                        acc, 0, 0, 0);
+      }
+      if (REP == 1 || r == rep) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sc[t][i] = acc[i];
+      }
+    }
+
+  // Softmax over all positions of the workgroup for query q.  The 16 lanes
+  // that share q differ in lane bits {2,3 (if REP == 4) | 3 (REP == 2)} and
+  // in g (bits 4, 5).
+  float m = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < TPL; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = 16 * (t * REP + rep) + 4 * g + i;  // within the wavefront
+      float x = uniform ? 0.f : round_bf16(sc[t][i]);
+      x = j < nw ? x : -INFINITY;
+      sc[t][i] = x;
       m = fmaxf(m, x);
     }
 #pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    mx[i] = m;
-  }
+  for (int o = NQP; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
   if (nwaves > 1) {
-    if (n16 == 0 && 4 * g < NQP) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) s_red[wave][4 * g + i] = mx[i];
-    }
+    if (lane < 16) s_red[0][wave][lane] = m;  // lanes 0..15: q = lane % NQP
     __syncthreads();
-    if (4 * g < NQP) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float m = s_red[0][4 * g + i];
-        for (int w = 1; w < nwaves; ++w) m = fmaxf(m, s_red[w][4 * g + i]);
-        mx[i] = m;
-      }
-    }
-    __syncthreads();
+    m = s_red[0][0][n16];
+    for (int w = 1; w < nwaves; ++w) m = fmaxf(m, s_red[0][w][n16]);
   }
-  T5D_STAMP(3);
-  float sum[4];
+  float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float s = 0.f;
-#pragma unroll
-    for (int jt = 0; jt < 8; ++jt) {
-      const float x = sc[jt][i];
-      const float ex = (x == -INFINITY) ? 0.f : __expf(x - mx[i]);
-      sc[jt][i] = ex;
-      s += ex;
-    }
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
-    sum[i] = s;
-  }
-  if (nwaves > 1) {
-    if (n16 == 0 && 4 * g < NQP) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) s_red[wave][4 * g + i] = sum[i];
-    }
-    __syncthreads();
-    if (4 * g < NQP) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float s = s_red[0][4 * g + i];
-        for (int w = 1; w < nwaves; ++w) s += s_red[w][4 * g + i];
-        sum[i] = s;
-      }
-    }
-  }
-  T5D_STAMP(4);
-  // Normalise, round to bf16, hand to the P·V A-operand layout through LDS.
-  if (4 * g < NQP) {
+  for (int t = 0; t < TPL; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float inv = rows_live ? 1.0f / sum[i] : 0.f;
+      const float ex = __expf(sc[t][i] - m);  // exp(-inf) == 0
+      sc[t][i] = ex;
+      sum += ex;
+    }
 #pragma unroll
-      for (int jt = 0; jt < 8; ++jt)
-        s_p[wave][4 * g + i][16 * jt + n16] = f32_to_bf16(sc[jt][i] * inv);
+  for (int o = NQP; o < 64; o <<= 1) sum += __shfl_xor(sum, o, 64);
+  if (nwaves > 1) {
+    if (lane < 16) s_red[1][wave][lane] = sum;
+    __syncthreads();
+    sum = s_red[1][0][n16];
+    for (int w = 1; w < nwaves; ++w) sum += s_red[1][w][n16];
+  }
+  // Normalise, round to bf16 (where the reference rounds), hand over to the
+  // B-operand layout of V·P^T through LDS: 4 consecutive positions per tile.
+  {
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int t = 0; t < TPL; ++t) {
+      uint2 pk;
+      pk.x = pack_bf16x2(sc[t][0] * inv, sc[t][1] * inv);
+      pk.y = pack_bf16x2(sc[t][2] * inv, sc[t][3] * inv);
+      *reinterpret_cast<uint2*>(&s_p[wave][q][16 * (t * REP + rep) + 4 * g]) = pk;
     }
   }
   __syncthreads();
 
-  T5D_STAMP(5);
-  // out[q][d] = sum_j P[q][j] V[d][j]; A lane (m = n16, g) holds
-  // P[m][32 jb + 8g .. +8].
+  // out^T[d][q] = sum_j V[d][j] P[q][j]; B lane (col n16 -> q, g) holds
+  // P[q][32 jb + 8g .. +8].
   f32x4_v oc[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
-  if (wave_live) {
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      Frag16 pa;
-      if (n16 < NQP)
-        pa.u = *reinterpret_cast<const uint4*>(&s_p[wave][n16][32 * jb + 8 * g]);
-      else
-        pa.u = make_uint4(0, 0, 0, 0);
+  for (int jb = 0; jb < 4; ++jb) {
+    if (32 * jb < nw) {
+      Frag16 pb;
+      pb.u = *reinterpret_cast<const uint4*>(&s_p[wave][q][32 * jb + 8 * g]);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
-        oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vb[jb][dt].v,
+        oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb[jb][dt].v, pb.v,
                                                          oc[dt], 0, 0, 0);
     }
   }
-  T5D_STAMP(6);
-  // oc[dt][i] in lane (n16, g) is out[q = 4g + i][d = 16 dt + n16].
+  // oc[dt][i] in lane (n16, g) is out[q][d = 16 dt + 4g + i] (all REP copies).
   if (nwaves == 1) {
-    if (rows_live) {
+    if (rep == 0 && q < a.nq) {
+      bf16_t* o = a.out + (size_t)(b * a.nq + q) * HD + h * kHeadDim + 4 * g;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int q = 4 * g + i;
-        if (q < a.nq) {
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
-            a.out[(size_t)(b * a.nq + q) * HD + h * kHeadDim + 16 * dt + n16] =
-                f32_to_bf16(oc[dt][i]);
-        }
+      for (int dt = 0; dt < 4; ++dt) {
+        uint2 pk;
+        pk.x = pack_bf16x2(oc[dt][0], oc[dt][1]);
+        pk.y = pack_bf16x2(oc[dt][2], oc[dt][3]);
+        *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
       }
     }
     return;
   }
-  __syncthreads();  // every wavefront is done reading s_p
-  if (4 * g < NQP) {
+  if (rep == 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-        s_out[wave][4 * g + i][16 * dt + n16] = oc[dt][i];
+    for (int dt = 0; dt < 4; ++dt)
+      *reinterpret_cast<float4*>(&s_out[wave][q][16 * dt + 4 * g]) =
+          make_float4(oc[dt][0], oc[dt][1], oc[dt][2], oc[dt][3]);
   }
   __syncthreads();
   for (int e = threadIdx.x; e < a.nq * kHeadDim; e += blockDim.x) {
-    const int q = e / kHeadDim, d = e % kHeadDim;
-    float acc = s_out[0][q][d];
-    for (int w = 1; w < nwaves; ++w) acc += s_out[w][q][d];
-    a.out[(size_t)(b * a.nq + q) * HD + h * kHeadDim + d] = f32_to_bf16(acc);
+    const int qq = e / kHeadDim, d = e % kHeadDim;
+    float acc = s_out[0][qq][d];
+    for (int w = 1; w < nwaves; ++w) acc += s_out[w][qq][d];
+    a.out[(size_t)(b * a.nq + qq) * HD + h * kHeadDim + d] = f32_to_bf16(acc);
   }
-  T5D_STAMP(7);
 }
 
 // ---- self-attention ------------------------------------------------------------
-// Optionally applies a pending beam gather on the fly: when `pending` is set,
-// a workgroup handles the `beams` rows of one batch item (wavefront = beam x
-// 128-position block), every wavefront reads the cache of its SOURCE beam
-// pending[b, e], and — if the item's beams were actually permuted — writes what
-// it read into its own slot after a workgroup barrier (all reads are in
-// registers by then, so the in-place permutation is safe).  This replaces a
-// separate read+write pass over every cache by the writes alone.
+// Sum across the 4 row groups of a wavefront (lane bits 4 and 5) of 8 values,
+// leaving each lane with 2 of the 8 totals (reduce-scatter): one
+// v_permlane32_swap / v_permlane16_swap plus one add per pair of registers.
+// Lane (bit5, bit4) ends with totals 4*bit5 + 2*bit4 + {0, 1}.
+__device__ __forceinline__ void reduce_scatter_8(const float (&s)[8],
+                                                 float (&out)[2]) {
+  float r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    auto w = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[e]),
+                                              __float_as_uint(s[e + 4]), false,
+                                              false);
+    r[e] = __uint_as_float(w[0]) + __uint_as_float(w[1]);
+  }
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    auto w = __builtin_amdgcn_permlane16_swap(__float_as_uint(r[e]),
+                                              __float_as_uint(r[e + 2]), false,
+                                              false);
+    out[e] = __uint_as_float(w[0]) + __uint_as_float(w[1]);
+  }
+}
+
+// One wavefront per (row, 128-position block).  Optionally applies a pending
+// beam gather on the fly: when `pending` is set, a workgroup handles the
+// `beams` rows of one batch item, every wavefront reads the cache of its
+// SOURCE beam pending[b, e], and — if the item's beams were actually permuted —
+// writes what it read into its own slot after a workgroup barrier (all reads
+// are in registers by then, so the in-place permutation is safe).  This
+// replaces a separate read+write pass over every cache by the writes alone.
+//
+//   scores: vector ALU.  Lane (dg = lane / 16, jc = lane % 16) multiplies head
+//     dims 16 dg .. +16 of the query with positions 8 jc .. +8 of the key
+//     cache (one 16-byte load per dim), the 4 dg partials are reduce-scattered
+//     so each lane softmaxes 2 positions.
+//   out^T = V·P^T on the matrix cores: V chunks are the A operand (rows = head
+//     dim, k = position), P^T the B operand with the single query repeated in
+//     all 16 columns, so every lane ends with 4 consecutive outputs per tile.
+//   The column being written (position t) never goes through the cache: its
+//   score comes from the new key, its output share from the new value.
+constexpr int kMaxSelfLen = 2048;
+
 template <int WM>
 __global__ void __launch_bounds__(64 * WM)
 self_attn_mfma_kernel(AttnMfmaArgs a) {
-  __shared__ float s_red[WM];
-  __shared__ float s_out[WM][kHeadDim];
+  __shared__ float s_red[2][WM];
+  __shared__ float s_pt[WM];
+  __shared__ __attribute__((aligned(16))) float s_out[WM][kHeadDim];
   __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][kBlockJ];
+  __shared__ float s_bias[kMaxSelfLen];
   T5D_GATED(a.gate);
 
   const int h = blockIdx.x;
@@ -336,7 +348,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   const int t = *a.index;
   const int n = t + 1;
   const int jw = blk * kBlockJ;
-  const bool wave_live = jw < n;
+  const int nw = n - jw;  // positions of this wavefront in use (may be <= 0)
   const bool wave_has_t = t >= jw && t < jw + kBlockJ;
   const size_t slot = (size_t)kHeadDim * S;
   const bf16_t* ksrc = a.k + ((size_t)rs * a.H + h) * slot;
@@ -345,194 +357,200 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   bf16_t* vdst = a.v + ((size_t)r * a.H + h) * slot;
   const bf16_t* qrow = a.q + (size_t)r * a.q_stride + h * kHeadDim;
 
-  // Query and (for the wavefront holding column t) new key, for this lane's
-  // 16 head-dim rows d = dg + 4i; new value for its 4 MFMA rows 16 dt + n16.
-  float qv[16], knew[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    qv[i] = bf16_to_f32(qrow[dg + 4 * i]);
-    knew[i] = wave_has_t ? bf16_to_f32(qrow[HD + dg + 4 * i]) : 0.f;
-  }
-  bf16_t vnew[4];
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-    vnew[dt] = wave_has_t ? qrow[2 * HD + 16 * dt + n16] : (bf16_t)0;
+  // Relative-position bias of this head, by distance, for the softmax below.
+  for (int i = threadIdx.x; i < n; i += blockDim.x)
+    s_bias[i] = bf16_to_f32(a.rel_bias[(size_t)h * S + i]);
 
-  // Scores on the vector ALU: lane (dg, jc) owns positions j0 .. j0 + 7.
+  // All K and V chunks are requested before anything is consumed.  K: lanes
+  // whose 8 positions lie beyond the current length skip their loads (one
+  // predicated region; what they compute is masked).  V: whole 32-position
+  // groups are skipped by wave-uniform branches, together with their matrix
+  // products.  Offsets are clamped to the row end when S is not a multiple of
+  // the tile (those positions are masked).
   const int j0 = jw + 8 * jc;
   const bool live = j0 < n;
-  const bool ins = wave_has_t && (t >= j0) && (t < j0 + 8);
-  const int e_t = t - j0;
-  const int jv = jw + 8 * g;  // + 32 jb: first position of a value chunk
-  // All K and V chunks are requested before anything is consumed.
+  const uint32_t koff = (uint32_t)(16 * dg * S + min(j0, S - 8)) * 2u;
   uint4 kc[16];
-  Frag16 vb[4][4];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    if (live)
-      kc[i] = *reinterpret_cast<const uint4*>(ksrc + (size_t)(dg + 4 * i) * S + j0);
-    else
-      kc[i] = make_uint4(0, 0, 0, 0);
-  }
-#pragma unroll
-  for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
-      if (jv + 32 * jb < n)
-        vb[jb][dt].u = *reinterpret_cast<const uint4*>(
-            vsrc + (size_t)(16 * dt + n16) * S + jv + 32 * jb);
-      else
-        vb[jb][dt].u = make_uint4(0, 0, 0, 0);
-    }
-  float s[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) s[e] = 0.f;
   if (live) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float kf[8];
-      unpack16(kc[i], kf);
+    for (int i = 0; i < 16; ++i)
+      kc[i] = *reinterpret_cast<const uint4*>(
+          reinterpret_cast<const char*>(ksrc + (size_t)i * S) + koff);
+  }
+  uint32_t voff[4];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s[e] = fmaf(qv[i], kf[e], s[e]);
+  for (int jb = 0; jb < 4; ++jb)
+    voff[jb] = (uint32_t)(n16 * S + min(jw + 32 * jb + 8 * g, S - 8)) * 2u;
+  Frag16 vb[4][4];
+#pragma unroll
+  for (int jb = 0; jb < 4; ++jb) {
+    if (32 * jb < nw) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+        vb[jb][dt].u = *reinterpret_cast<const uint4*>(
+            reinterpret_cast<const char*>(vsrc + (size_t)(16 * dt) * S) +
+            voff[jb]);
     }
   }
-  // Score of the position being written, from the new key (the cache column
-  // itself still holds its old content in the registers above).
-  float snew = 0.f;
+  // Query: this lane's 16 head dims.  New key / value / query element of
+  // head dim `lane` for the column being written.
+  float qv[16];
+  {
+    const uint4* qp = reinterpret_cast<const uint4*>(qrow + 16 * dg);
+    float f[8];
+    unpack16(qp[0], f);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) snew = fmaf(qv[i], knew[i], snew);
+    for (int e = 0; e < 8; ++e) qv[e] = f[e];
+    unpack16(qp[1], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[8 + e] = f[e];
+  }
+  const bf16_t knew_d = qrow[HD + lane];
+  const bf16_t vnew_d = qrow[2 * HD + lane];
+  // Score of position t from the new key.
+  float snew = wave_sum(bf16_to_f32(qrow[lane]) * bf16_to_f32(knew_d));
+
+  float s8[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s8[e] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float kf[8];
+    unpack16(kc[i], kf);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s8[e] = fmaf(qv[i], kf[e], s8[e]);
+  }
 
   if (permuted) {
-    // Every wavefront of the workgroup has its source data in registers (the
-    // scores above consumed K; V is forced below) before any slot is written.
+    // Every wavefront of the workgroup has its source data in registers
+    // before any slot is written.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (r != rs) {
+      if (live) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (live)
-          *reinterpret_cast<uint4*>(kdst + (size_t)(dg + 4 * i) * S + j0) = kc[i];
+        for (int i = 0; i < 16; ++i)
+          *reinterpret_cast<uint4*>(
+              reinterpret_cast<char*>(kdst + (size_t)i * S) + koff) = kc[i];
+      }
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
+      for (int jb = 0; jb < 4; ++jb) {
+        if (32 * jb < nw) {
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-          if (jv + 32 * jb < n)
-            *reinterpret_cast<uint4*>(vdst + (size_t)(16 * dt + n16) * S + jv +
-                                      32 * jb) = vb[jb][dt].u;
+          for (int dt = 0; dt < 4; ++dt)
+            *reinterpret_cast<uint4*>(
+                reinterpret_cast<char*>(vdst + (size_t)(16 * dt) * S) +
+                voff[jb]) = vb[jb][dt].u;
+        }
+      }
       // the column written below must land after the chunks that cover it
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+  } else {
+    __syncthreads();  // s_bias
   }
-  // The column being written: K by the 4 score lanes whose chunk holds t,
-  // V by the 16 MFMA lanes whose chunk holds t.
-  if (ins) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      kdst[(size_t)(dg + 4 * i) * S + t] = qrow[HD + dg + 4 * i];
-  }
-  const int tl = t - jw;  // position of column t inside this wavefront
-  const int jb_t = tl >> 5, g_t = (tl & 31) >> 3, ev = tl & 7;
-  if (wave_has_t && g == g_t) {
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-      vdst[(size_t)(16 * dt + n16) * S + t] = vnew[dt];
+  // The column being written: lane d stores element d of the new key / value.
+  if (wave_has_t) {
+    kdst[(size_t)lane * S + t] = knew_d;
+    vdst[(size_t)lane * S + t] = vnew_d;
   }
 
-  // Reduce the 4 row groups, add the relative-position bias, mask, softmax.
-  snew += __shfl_xor(snew, 16, 64);
-  snew += __shfl_xor(snew, 32, 64);
+  // 2 positions per lane: bias, mask, softmax.
+  float sc[2];
+  reduce_scatter_8(s8, sc);
+  const int jp = j0 + 4 * (dg >> 1) + 2 * (dg & 1);  // first of the 2 positions
   float m = -INFINITY;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    float x = s[e];
-    x += __shfl_xor(x, 16, 64);
-    x += __shfl_xor(x, 32, 64);
-    x = (ins && e == e_t) ? snew : x;
-    const int j = j0 + e;
+  for (int e = 0; e < 2; ++e) {
+    const int j = jp + e;
+    float x = (j == t) ? snew : sc[e];
     x = round_bf16(x);
-    if (j < n) x = round_bf16(x + bf16_to_f32(a.rel_bias[(size_t)h * S + (t - j)]));
-    x = (j < n) ? x : -INFINITY;
-    s[e] = x;
+    if (j < n) x = round_bf16(x + s_bias[t - j]);
+    else x = -INFINITY;
+    sc[e] = x;
     m = fmaxf(m, x);
   }
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  m = wave_max(m);
   if (nblk > 1) {
-    if (lane == 0) s_red[wave] = m;
+    if (lane == 0) s_red[0][wave] = m;
     __syncthreads();
-    m = s_red[wave0];
-    for (int w = 1; w < nblk; ++w) m = fmaxf(m, s_red[wave0 + w]);
-    __syncthreads();
+    m = s_red[0][wave0];
+    for (int w = 1; w < nblk; ++w) m = fmaxf(m, s_red[0][wave0 + w]);
   }
   float sum = 0.f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float ex = (s[e] == -INFINITY) ? 0.f : __expf(s[e] - m);
-    s[e] = ex;
-    sum += ex;
+  for (int e = 0; e < 2; ++e) {
+    sc[e] = __expf(sc[e] - m);  // exp(-inf) == 0
+    sum += sc[e];
   }
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  sum = wave_sum(sum);
   if (nblk > 1) {
-    if (lane == 0) s_red[wave] = sum;
+    if (lane == 0) s_red[1][wave] = sum;
     __syncthreads();
-    sum = s_red[wave0];
-    for (int w = 1; w < nblk; ++w) sum += s_red[wave0 + w];
+    sum = s_red[1][wave0];
+    for (int w = 1; w < nblk; ++w) sum += s_red[1][wave0 + w];
   }
-  if (dg == 0) {
-    Frag16 pk;
+  {
+    // Normalised probabilities, rounded to bf16 where the reference rounds.
+    // Position t is kept out of the matrix product (the V registers hold the
+    // column's old content): its probability goes to s_pt instead.
     const float inv = 1.0f / sum;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) pk.h[e] = f32_to_bf16(s[e] * inv);
-    *reinterpret_cast<uint4*>(&s_p[wave][8 * jc]) = pk.u;
+    float p0 = round_bf16(sc[0] * inv), p1 = round_bf16(sc[1] * inv);
+    if (jp == t) { s_pt[wave] = p0; p0 = 0.f; }
+    if (jp + 1 == t) { s_pt[wave] = p1; p1 = 0.f; }
+    *reinterpret_cast<uint32_t*>(&s_p[wave][jp - jw]) = pack_bf16x2(p0, p1);
   }
   __syncthreads();
 
-  // P·V on the matrix cores; only A row 0 (lanes with n16 == 0) is non-zero.
-  // Column t is taken out of the matrix product (the V registers still hold
-  // the column's old content) and added from the new value below.
-  const float p_t = wave_has_t ? bf16_to_f32(s_p[wave][tl]) : 0.f;
+  // out^T tile dt: lane (n16, g) gets out[16 dt + 4g + i], i < 4, in every
+  // column n16.  B lane (col, g) holds P[32 jb + 8g .. +8].
   f32x4_v oc[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
-  if (wave_live) {
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      Frag16 pa;
-      if (n16 == 0)
-        pa.u = *reinterpret_cast<const uint4*>(&s_p[wave][32 * jb + 8 * g]);
-      else
-        pa.u = make_uint4(0, 0, 0, 0);
-      if (wave_has_t && jb == jb_t && g == g_t) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e == ev) pa.h[e] = 0;
-      }
+  for (int jb = 0; jb < 4; ++jb) {
+    if (32 * jb < nw) {
+      Frag16 pb;
+      pb.u = *reinterpret_cast<const uint4*>(&s_p[wave][32 * jb + 8 * g]);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
-        oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vb[jb][dt].v,
+        oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb[jb][dt].v, pb.v,
                                                          oc[dt], 0, 0, 0);
     }
   }
-  // Row 0 of the result: lanes 0..15, element 0 -> out[d = 16 dt + lane].
+  if (wave_has_t) {
+    const float p_t = s_pt[wave];
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-    oc[dt][0] = fmaf(p_t, bf16_to_f32(vnew[dt]), oc[dt][0]);
+    for (int dt = 0; dt < 4; ++dt) {
+      const uint2 vn = *reinterpret_cast<const uint2*>(qrow + 2 * HD + 16 * dt +
+                                                       4 * g);
+      oc[dt][0] = fmaf(p_t, bf16lo_to_f32(vn.x), oc[dt][0]);
+      oc[dt][1] = fmaf(p_t, bf16hi_to_f32(vn.x), oc[dt][1]);
+      oc[dt][2] = fmaf(p_t, bf16lo_to_f32(vn.y), oc[dt][2]);
+      oc[dt][3] = fmaf(p_t, bf16hi_to_f32(vn.y), oc[dt][3]);
+    }
+  }
   if (nblk == 1) {
-    if (g == 0) {
+    if (n16 == 0) {
+      bf16_t* o = a.out + (size_t)r * HD + h * kHeadDim + 4 * g;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-        a.out[(size_t)r * HD + h * kHeadDim + 16 * dt + n16] =
-            f32_to_bf16(oc[dt][0]);
+      for (int dt = 0; dt < 4; ++dt) {
+        uint2 pk;
+        pk.x = pack_bf16x2(oc[dt][0], oc[dt][1]);
+        pk.y = pack_bf16x2(oc[dt][2], oc[dt][3]);
+        *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
+      }
     }
     return;
   }
-  if (g == 0) {
+  if (n16 == 0) {
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) s_out[wave][16 * dt + n16] = oc[dt][0];
+    for (int dt = 0; dt < 4; ++dt)
+      *reinterpret_cast<float4*>(&s_out[wave][16 * dt + 4 * g]) =
+          make_float4(oc[dt][0], oc[dt][1], oc[dt][2], oc[dt][3]);
   }
   __syncthreads();
-  if (blk == 0 && lane < kHeadDim) {
+  if (blk == 0) {
     float acc = s_out[wave0][lane];
     for (int w = 1; w < nblk; ++w) acc += s_out[wave0 + w][lane];
     a.out[(size_t)r * HD + h * kHeadDim + lane] = f32_to_bf16(acc);
