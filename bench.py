@@ -44,6 +44,8 @@ def parse_args():
   ap.add_argument('--config', default='base-beam4', choices=sorted(CONFIGS))
   ap.add_argument('--seed', type=int, default=0)
   ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--lanes', type=int, default=None,
+                  help='batch slices stepped concurrently (default: library)')
   ap.add_argument('--cpu-steps', type=int, default=3,
                   help='decode steps of the CPU oracle sample')
   return ap.parse_args()
@@ -52,7 +54,7 @@ def parse_args():
 class Workload:
   """Synthetic batch + model state for repeated full decodes."""
 
-  def __init__(self, name, seed):
+  def __init__(self, name, seed, lanes=None):
     import torch
     from t5x_amd import decoding, models, network
     self.torch, self.decoding = torch, decoding
@@ -62,6 +64,8 @@ class Workload:
     dev = torch.device('cuda')
     self.params = network.init_params(self.cfg, seed, dev, with_encoder=False)
     self.module = network.Transformer(self.cfg, dev)
+    if lanes:
+      self.module.decode_lanes = lanes
     self.model = models.EncoderDecoderModel(self.module,
                                             decode_fn=decoding.beam_search)
     rs = np.random.Generator(np.random.PCG64(seed + 1))
@@ -229,7 +233,7 @@ def main():
   if not torch.cuda.is_available():
     print('bench.py: no GPU visible', file=sys.stderr)
     sys.exit(3)
-  w = Workload(args.config, args.seed)
+  w = Workload(args.config, args.seed, args.lanes)
   w.run_steps(args.warmup)
   torch.cuda.synchronize()
   t0 = time.perf_counter()

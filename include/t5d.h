@@ -313,6 +313,10 @@ typedef struct {
   void* kv_base;               /* first cache tensor [B, K, H, 64, L] */
   int64_t kv_tensor_stride_bytes;
   int n_kv_tensors;            /* 2 * NL when all layers share one block */
+  /* non-zero: *keep_going is only read (as the gate); the caller runs
+   * t5d_beam_cond itself, e.g. once over all slices of a batch that it steps
+   * on separate streams */
+  int skip_cond;
 } t5d_beam_step;
 
 /* One iteration of the beam_search loop body plus the loop condition

@@ -53,7 +53,7 @@ class BeamStep(Structure):
                ('min_brevity', c_float), ('min_log_prob', c_float),
                ('max_decode_step', c_int), ('min_initial_index', c_int),
                ('kv_base', c_void_p), ('kv_tensor_stride_bytes', c_int64),
-               ('n_kv_tensors', c_int)])
+               ('n_kv_tensors', c_int), ('skip_cond', c_int)])
 
 
 _P = c_void_p

@@ -37,7 +37,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                T* __restrict__ out, int d, float eps, const int32_t* gate) {
-  T5D_GATED(gate);
+  T5D_GATE_READ(gate);
   __shared__ float partial[4];
   const int r = blockIdx.x;
   const T* xr = x + (size_t)r * d;
@@ -46,6 +46,7 @@ rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
     float v = Act<T>::load(xr + i);
     ss += v * v;
   }
+  T5D_GATE_TEST();
   ss = wave_sum(ss);
   if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
   __syncthreads();

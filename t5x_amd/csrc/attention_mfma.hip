@@ -81,7 +81,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   __shared__ float s_red[2][WM][16];
   __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][NQP][kBlockJ];
   __shared__ __attribute__((aligned(16))) float s_out[WM][NQP][kHeadDim];
-  T5D_GATED(a.gate);
+  T5D_GATE_READ(a.gate);
 
   const int h = blockIdx.x, b = blockIdx.y;
   const int lane = threadIdx.x & 63;
@@ -91,7 +91,10 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   const int q = n16 % NQP, rep = n16 / NQP;
   const int HD = a.H * kHeadDim;
 
+  T5D_STAMP(0);
   int n = a.index[b];
+  T5D_GATE_TEST();  // after both scalar loads are in flight
+  T5D_STAMP(1);
   n = n < 0 ? 0 : (n > a.S ? a.S : n);
   bool uniform = false;  // no valid key: the masked softmax is uniform
   if (n == 0) { uniform = true; n = a.S; }
@@ -169,6 +172,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       }
     }
 
+  T5D_STAMP(2);
   // Softmax over all positions of the workgroup for query q.  The 16 lanes
   // that share q differ in lane bits {2,3 (if REP == 4) | 3 (REP == 2)} and
   // in g (bits 4, 5).
@@ -191,6 +195,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     m = s_red[0][0][n16];
     for (int w = 1; w < nwaves; ++w) m = fmaxf(m, s_red[0][w][n16]);
   }
+  T5D_STAMP(3);
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < TPL; ++t)
@@ -208,6 +213,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     sum = s_red[1][0][n16];
     for (int w = 1; w < nwaves; ++w) sum += s_red[1][w][n16];
   }
+  T5D_STAMP(4);
   // Normalise, round to bf16 (where the reference rounds), hand over to the
   // B-operand layout of V·P^T through LDS: 4 consecutive positions per tile.
   {
@@ -221,6 +227,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     }
   }
   __syncthreads();
+  T5D_STAMP(5);
 
   // out^T[d][q] = sum_j V[d][j] P[q][j]; B lane (col n16 -> q, g) holds
   // P[q][32 jb + 8g .. +8].
@@ -238,6 +245,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
                                                          oc[dt], 0, 0, 0);
     }
   }
+  T5D_STAMP(6);
   // oc[dt][i] in lane (n16, g) is out[q][d = 16 dt + 4g + i] (all REP copies).
   if (nwaves == 1) {
     if (rep == 0 && q < a.nq) {
@@ -265,6 +273,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int w = 1; w < nwaves; ++w) acc += s_out[w][qq][d];
     a.out[(size_t)(b * a.nq + qq) * HD + h * kHeadDim + d] = f32_to_bf16(acc);
   }
+  T5D_STAMP(7);
 }
 
 // ---- self-attention ------------------------------------------------------------
@@ -318,7 +327,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   __shared__ __attribute__((aligned(16))) float s_out[WM][kHeadDim];
   __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][kBlockJ];
   __shared__ float s_bias[kMaxSelfLen];
-  T5D_GATED(a.gate);
+  T5D_GATE_READ(a.gate);
 
   const int h = blockIdx.x;
   const int lane = threadIdx.x & 63;
@@ -345,7 +354,10 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     r = rs = blockIdx.y;
   }
 
+  T5D_STAMP(8);
   const int t = *a.index;
+  T5D_GATE_TEST();  // after the scalar loads above are in flight
+  T5D_STAMP(9);
   const int n = t + 1;
   const int jw = blk * kBlockJ;
   const int nw = n - jw;  // positions of this wavefront in use (may be <= 0)
@@ -421,6 +433,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int e = 0; e < 8; ++e) s8[e] = fmaf(qv[i], kf[e], s8[e]);
   }
 
+  T5D_STAMP(10);
   if (permuted) {
     // Every wavefront of the workgroup has its source data in registers
     // before any slot is written.
@@ -455,6 +468,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     vdst[(size_t)lane * S + t] = vnew_d;
   }
 
+  T5D_STAMP(11);
   // 2 positions per lane: bias, mask, softmax.
   float sc[2];
   reduce_scatter_8(s8, sc);
@@ -477,6 +491,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     m = s_red[0][wave0];
     for (int w = 1; w < nblk; ++w) m = fmaxf(m, s_red[0][wave0 + w]);
   }
+  T5D_STAMP(12);
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
@@ -501,6 +516,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     *reinterpret_cast<uint32_t*>(&s_p[wave][jp - jw]) = pack_bf16x2(p0, p1);
   }
   __syncthreads();
+  T5D_STAMP(13);
 
   // out^T tile dt: lane (n16, g) gets out[16 dt + 4g + i], i < 4, in every
   // column n16.  B lane (col, g) holds P[32 jb + 8g .. +8].
@@ -530,6 +546,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       oc[dt][3] = fmaf(p_t, bf16hi_to_f32(vn.y), oc[dt][3]);
     }
   }
+  T5D_STAMP(14);
   if (nblk == 1) {
     if (n16 == 0) {
       bf16_t* o = a.out + (size_t)r * HD + h * kHeadDim + 4 * g;
@@ -541,6 +558,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
         *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
       }
     }
+    T5D_STAMP(15);
     return;
   }
   if (n16 == 0) {

@@ -116,5 +116,11 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 extern thread_local const int32_t* tls_gate;
 #define T5D_GATED(gate) \
   if ((gate) != nullptr && *(gate) == 0) return
+// Two-part form: read the flag first, test it after the kernel has issued its
+// first (side-effect free) loads, so the flag's memory latency overlaps theirs.
+#define T5D_GATE_READ(gate) \
+  const int t5d_gate_open_ = (gate) != nullptr ? *(gate) : 1
+#define T5D_GATE_TEST() \
+  if (t5d_gate_open_ == 0) return
 
 }  // namespace t5d

@@ -71,9 +71,10 @@ struct GemmArgs {
   int out_f32;
 };
 
-// Apply scale + epilogue to one finished column (pair) of row m.
+// Apply scale + epilogue to one finished column (pair) of row m; `res` is the
+// residual element (fetched early by the caller).
 __device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
-                                             float v, float v_gate) {
+                                             float v, float v_gate, float res) {
   if (g.epilogue == T5D_EPI_GEGLU) {
     const int f = (n >> 4) * 8 + (n & 7);
     const int F = g.N >> 1;
@@ -87,10 +88,7 @@ __device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
     reinterpret_cast<float*>(g.C)[o] = v;
     return;
   }
-  if (g.epilogue == T5D_EPI_RESIDUAL) {
-    float r = bf16_to_f32(reinterpret_cast<const bf16_t*>(g.residual)[o]);
-    v = round_bf16(v) + r;
-  }
+  if (g.epilogue == T5D_EPI_RESIDUAL) v = round_bf16(v) + res;
   reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(v);
 }
 
@@ -101,8 +99,11 @@ gemm_mfma_kernel(GemmArgs g) {
   constexpr int TN = NT * 16;
   constexpr int PF = (NT >= 4) ? 2 : (NT == 2 ? 3 : 4);  // pairs in flight
   static_assert(ACC <= 16, "accumulator tile budget");
-  __shared__ float red[2][ACC * 4][64];
-  T5D_GATED(g.gate);
+  // Small tiles: every wavefront parks its partial sums and one barrier
+  // suffices; large tiles: two buffers and a tree (LDS budget).
+  constexpr bool FLAT = ACC <= 4;
+  __shared__ float red[FLAT ? 4 : 2][ACC * 4][64];
+  T5D_GATE_READ(g.gate);
 
   // XCD-aware block mapping: the m_parts workgroups of one column group get
   // block ids 8 apart, i.e. the same XCD and adjacent dispatch slots.
@@ -147,6 +148,20 @@ gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
   for (int p = 0; p < PF; ++p)
     if (p < nj) load_b(p, p);
+  // The residual elements this thread will need in the epilogue.
+  float res[FLAT ? ACC : 1];
+  if (FLAT && g.epilogue == T5D_EPI_RESIDUAL) {
+#pragma unroll
+    for (int p = 0; p < (FLAT ? ACC : 0); ++p) {
+      const int e = threadIdx.x + 256 * p;
+      const int m = m0 + e / TN, n = nt0 * 16 + e % TN;
+      res[p] = (m < g.M && n < g.N)
+                   ? bf16_to_f32(reinterpret_cast<const bf16_t*>(
+                         g.residual)[(size_t)m * g.N + n])
+                   : 0.f;
+    }
+  }
+  T5D_GATE_TEST();
 
   for (int j0 = 0; j0 < nj; j0 += PF) {
 #pragma unroll
@@ -182,54 +197,82 @@ gemm_mfma_kernel(GemmArgs g) {
   // Cross-wave reduction in a fixed order: (w0 + w2) + (w1 + w3).
   // Accumulator element i of tile (mt, nn) in lane l is
   // C[16*mt + 4*(l/16) + i][16*nn + l%16].
-  if (wave >= 2) {
+  if constexpr (FLAT) {
 #pragma unroll
     for (int t = 0; t < ACC; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave - 2][t * 4 + i][lane] = acc[t][i];
+      for (int i = 0; i < 4; ++i) red[wave][t * 4 + i][lane] = acc[t][i];
+    __syncthreads();
+  } else {
+    if (wave >= 2) {
+#pragma unroll
+      for (int t = 0; t < ACC; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave - 2][t * 4 + i][lane] = acc[t][i];
+    }
+    __syncthreads();
+    if (wave < 2) {
+#pragma unroll
+      for (int t = 0; t < ACC; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] += red[wave][t * 4 + i][lane];
+    }
+    __syncthreads();
+    if (wave == 1) {
+#pragma unroll
+      for (int t = 0; t < ACC; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[0][t * 4 + i][lane] = acc[t][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < ACC; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          red[1][t * 4 + i][lane] = acc[t][i] + red[0][t * 4 + i][lane];
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  if (wave < 2) {
-#pragma unroll
-    for (int t = 0; t < ACC; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[t][i] += red[wave][t * 4 + i][lane];
-  }
-  __syncthreads();
-  if (wave == 1) {
-#pragma unroll
-    for (int t = 0; t < ACC; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[0][t * 4 + i][lane] = acc[t][i];
-  }
-  __syncthreads();
-  if (wave == 0) {
-#pragma unroll
-    for (int t = 0; t < ACC; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        red[1][t * 4 + i][lane] = acc[t][i] + red[0][t * 4 + i][lane];
-  }
-  __syncthreads();
 
   const bool geglu = g.epilogue == T5D_EPI_GEGLU;
   auto tile_sum = [&](int ml, int nl) -> float {
     const int mt = ml >> 4, i = ml & 3, c = (ml & 15) >> 2;
     const int nn = nl >> 4, l = c * 16 + (nl & 15);
-    return red[1][(mt * NT + nn) * 4 + i][l];
+    const int idx = (mt * NT + nn) * 4 + i;
+    if constexpr (FLAT)
+      return (red[0][idx][l] + red[2][idx][l]) +
+             (red[1][idx][l] + red[3][idx][l]);
+    else
+      return red[1][idx][l];
   };
-  for (int e = threadIdx.x; e < MP * 16 * TN; e += 256) {
+  auto finish = [&](int e, float r) {
     const int ml = e / TN, nl = e % TN;
     const int m = m0 + ml, n = nt0 * 16 + nl;
-    if (m >= g.M || n >= g.N) continue;
-    if (geglu && (nl & 8)) continue;
+    if (m >= g.M || n >= g.N) return;
+    if (geglu && (nl & 8)) return;
     float v = tile_sum(ml, nl);
     float vg = geglu ? tile_sum(ml, nl + 8) : 0.f;
     if (g.scales) {
       v *= g.scales[n];
       if (geglu) vg *= g.scales[n + 8];
     }
-    store_result(g, m, n, v, vg);
+    store_result(g, m, n, v, vg, r);
+  };
+  if constexpr (FLAT) {
+#pragma unroll
+    for (int p = 0; p < ACC; ++p) finish(threadIdx.x + 256 * p, res[p]);
+  } else {
+    for (int e = threadIdx.x; e < MP * 16 * TN; e += 256) {
+      float r = 0.f;
+      if (g.epilogue == T5D_EPI_RESIDUAL) {
+        const int m = m0 + e / TN, n = nt0 * 16 + e % TN;
+        if (m < g.M && n < g.N)
+          r = bf16_to_f32(reinterpret_cast<const bf16_t*>(
+              g.residual)[(size_t)m * g.N + n]);
+      }
+      finish(e, r);
+    }
   }
 }
 

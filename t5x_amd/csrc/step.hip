@@ -124,9 +124,10 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
         stream, b->kv_base, b->kv_tensor_stride_bytes, b->n_kv_tensors,
         m->dtype == T5D_F32 ? 4 : 2, B, K, m->H * 64, m->L, b->top_alive,
         b->state.cur_index, 0));
-  T5D_TRY(t5d_beam_cond(stream, &b->state, B, K, b->S, b->min_brevity,
-                        b->min_log_prob, b->max_decode_step,
-                        b->min_initial_index, b->keep_going));
+  if (!b->skip_cond)
+    T5D_TRY(t5d_beam_cond(stream, &b->state, B, K, b->S, b->min_brevity,
+                          b->min_log_prob, b->max_decode_step,
+                          b->min_initial_index, b->keep_going));
   return T5D_OK;
 }
 

@@ -221,6 +221,11 @@ class Transformer:
   """
 
   scan_layers = False
+  # Batch slices a fused beam search steps on separate streams.  On MI355X
+  # kernels of different streams do overlap, but the dispatch rate (about one
+  # kernel per 1.5 us) is shared by all streams, and a decode step is bound by
+  # its kernel count, so more lanes only add dispatches: 1 is fastest.
+  decode_lanes = 1
 
   def __init__(self, config: T5Config, device=None):
     if config.head_dim != 64:
@@ -469,20 +474,95 @@ class Transformer:
     return FusedBeamStep(self, loop, params, encoded, enc_tokens)
 
 
+class _BeamLane:
+  """One independent slice [b0, b1) of the batch: its own caches, activations,
+  loop flag, position counter, stream and captured graph."""
+
+  def __init__(self, owner, index, b0, b1, w, cross):
+    from t5x_amd import _lib
+    module, loop = owner.module, owner.loop
+    cfg, dev = module.config, owner.device
+    B, K = b1 - b0, loop.beam_size
+    self.b0, self.b1 = b0, b1
+    R, S, L = B * K, loop.max_decode_len, owner.L
+    act = w.act_dtype
+    nl = cfg.num_decoder_layers
+    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
+                          dtype=act, device=dev)
+    self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
+    self.bufs = _StepBuffers(cfg, R, dev, act)
+    self.keep_going = loop.keep_going      # one flag for the whole batch
+    self.cur_index = owner.lane_cur_index[index]
+    k2 = 2 * K
+    f32, i32 = torch.float32, torch.int32
+    self.topk_vals = torch.empty((B, k2), dtype=f32, device=dev)
+    self.topk_idx = torch.empty((B, k2), dtype=i32, device=dev)
+    self.row_max = torch.empty((R,), dtype=f32, device=dev)
+    self.row_lse = torch.empty((R,), dtype=f32, device=dev)
+    self.scratch = torch.empty((2 * R * k2,), dtype=i32, device=dev)
+    self.top_alive = loop.top_alive[b0:b1]
+    lane_cross = dict(k=[t[b0:b1] for t in cross['k']],
+                      v=[t[b0:b1] for t in cross['v']],
+                      enc_len=cross['enc_len'][b0:b1], B=B, beams=K,
+                      E=cross['E'])
+    layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
+    self.model = module._model_step(
+        w, lane_cross, self.bufs, layer_caches, self.cache_index, R, K, L,
+        gate=self.keep_going,
+        pending_src=self.top_alive if owner.deferred_gather else None)
+    st = loop.cur
+    P = _lib.ptr
+    ptrs = _lib.BeamStatePtrs()
+    ptrs.cur_index = P(self.cur_index)
+    ptrs.live_logprobs = P(st.live_logprobs[b0:b1])
+    ptrs.finished_scores = P(st.finished_scores[b0:b1])
+    ptrs.live_seqs = P(st.live_seqs[b0:b1])
+    ptrs.finished_seqs = P(st.finished_seqs[b0:b1])
+    ptrs.finished_flags = P(st.finished_flags[b0:b1])
+    self.state_ptrs = ptrs
+    bs = _lib.BeamStep()
+    bs.state = ptrs
+    bs.inputs = P(loop.inputs_dev[b0:b1])
+    bs.initial_index = P(loop.init_idx_dev[b0:b1])
+    bs.brevity, bs.top_alive = P(loop.brevity), P(self.top_alive)
+    bs.topk_vals, bs.topk_idx = P(self.topk_vals), P(self.topk_idx)
+    bs.row_max, bs.row_lse = P(self.row_max), P(self.row_lse)
+    bs.scratch, bs.ids = P(self.scratch), P(self.bufs.ids)
+    bs.keep_going = P(self.keep_going)
+    bs.S, bs.Lin, bs.eos_id = S, loop.inputs_dev.shape[1], int(loop.eos_id)
+    bs.min_brevity, bs.min_log_prob = loop.min_brevity, loop.min_log_prob
+    bs.max_decode_step = int(loop.max_decode_step)
+    bs.min_initial_index = loop.min_initial
+    bs.kv_base = P(self.kv)
+    bs.kv_tensor_stride_bytes = self.kv[0, 0].numel() * self.kv.element_size()
+    bs.n_kv_tensors = 2 * nl
+    bs.skip_cond = 1 if owner.n_lanes > 1 else 0
+    self.beam = bs
+    self.stream = torch.cuda.Stream(device=dev)
+    self.event = torch.cuda.Event()
+    self.graph = None
+
+
 class FusedBeamStep:
-  """Whole beam-search iterations as replays of one captured HIP graph.
+  """Whole beam-search iterations as replays of captured HIP graphs.
 
-  Owns the beam-expanded self-attention caches as one block
-  [layers, 2, B*K, H, 64, L] (so the reorder is a single launch over the valid
-  prefix) and runs on its own stream.  The loop flag lives on the device and
-  gates every kernel, so iterations enqueued after the loop condition turned
-  false change nothing."""
+  The batch is cut into lanes (batch items never interact in beam search).
+  Each lane owns its beam-expanded self-attention caches as one block
+  [layers, 2, rows, H, 64, L], its activations and its position counter, and
+  replays its own graph on its own stream, so the lanes' kernels overlap on
+  the device: while one lane sits in a latency-bound phase another one
+  streams.  The loop condition stays the reference's single whole-batch
+  condition: after every iteration the lanes' streams join, one kernel
+  evaluates it over the whole (contiguous) beam state into the one device
+  flag that gates every kernel of every lane, and the lanes fork again, all
+  without the host.  Iterations enqueued after the flag turned 0 change
+  nothing, so the host may look at it only every few iterations."""
 
-  def __init__(self, module, loop, params, encoded, enc_tokens):
+  def __init__(self, module, loop, params, encoded, enc_tokens, lanes=None):
     from t5x_amd import _lib
     self._lib = _lib
     cfg, dev = module.config, module._dev()
-    self.module, self.loop = module, loop
+    self.module, self.loop, self.device = module, loop, dev
     w = module.decoder_weights(params)
     enc_tok = enc_tokens.x
     enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
@@ -491,23 +571,10 @@ class FusedBeamStep:
     B, K = loop.batch_size, loop.beam_size
     if cross['B'] != B or encoded.beams != K:
       raise ValueError('encoder batch / beams do not match the decode loop')
-    R, S = B * K, loop.max_decode_len
+    S = loop.max_decode_len
     act = w.act_dtype
     el = 16 // torch.empty((), dtype=act).element_size()
-    L = (S - 1 + el - 1) // el * el
-    nl = cfg.num_decoder_layers
-    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
-                          dtype=act, device=dev)
-    self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
-    self.bufs = _StepBuffers(cfg, R, dev, act)
-    k2 = 2 * K
-    f32, i32 = torch.float32, torch.int32
-    self.topk_vals = torch.empty((B, k2), dtype=f32, device=dev)
-    self.topk_idx = torch.empty((B, k2), dtype=i32, device=dev)
-    self.row_max = torch.empty((R,), dtype=f32, device=dev)
-    self.row_lse = torch.empty((R,), dtype=f32, device=dev)
-    self.scratch = torch.empty((2 * R * k2,), dtype=i32, device=dev)
-    layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
+    self.L = L = (S - 1 + el - 1) // el * el
     # With bfloat16 caches the reorder of a step is deferred into the next
     # step's self-attention kernels, which read each row's cache from its
     # source beam anyway; the permutation in flight lives in loop.top_alive.
@@ -515,92 +582,121 @@ class FusedBeamStep:
                             K * ((L + 127) // 128) <= 16)
     loop.top_alive.copy_(torch.arange(K, dtype=torch.int32,
                                       device=dev).expand(B, K))
-    self.model = module._model_step(
-        w, cross, self.bufs, layer_caches, self.cache_index, R, K, L,
-        gate=loop.keep_going,
-        pending_src=loop.top_alive if self.deferred_gather else None)
-    st = loop.cur
-    bs = _lib.BeamStep()
-    bs.state = st._ptrs
-    P = _lib.ptr
-    bs.inputs, bs.initial_index = P(loop.inputs_dev), P(loop.init_idx_dev)
-    bs.brevity, bs.top_alive = P(loop.brevity), P(loop.top_alive)
-    bs.topk_vals, bs.topk_idx = P(self.topk_vals), P(self.topk_idx)
-    bs.row_max, bs.row_lse = P(self.row_max), P(self.row_lse)
-    bs.scratch, bs.ids = P(self.scratch), P(self.bufs.ids)
-    bs.keep_going = P(loop.keep_going)
-    bs.S, bs.Lin, bs.eos_id = S, loop.inputs_dev.shape[1], int(loop.eos_id)
-    bs.min_brevity, bs.min_log_prob = loop.min_brevity, loop.min_log_prob
-    bs.max_decode_step = int(loop.max_decode_step)
-    bs.min_initial_index = loop.min_initial
-    bs.kv_base = P(self.kv)
-    bs.kv_tensor_stride_bytes = self.kv[0, 0].numel() * self.kv.element_size()
-    bs.n_kv_tensors = 2 * nl
-    self.beam = bs
-    self.stream = torch.cuda.Stream(device=dev)
-    self.graph = None
+    if lanes is None:
+      lanes = module.decode_lanes
+    n = max(1, min(int(lanes), B))
+    self.n_lanes = n
+    bounds = [B * i // n for i in range(n + 1)]
+    self.lane_cur_index = loop.cur.cur_index.to(torch.int32).reshape(1).repeat(n)
+    self.cond_event = torch.cuda.Event()
+    self.lanes = [_BeamLane(self, i, bounds[i], bounds[i + 1], w, cross)
+                  for i in range(n)]
     self._capture()
 
-  def _enqueue(self):
-    self._lib.call('t5d_beam_search_step', self.stream.cuda_stream,
-                   self.model, self.beam)
+  def _enqueue(self, lane):
+    self._lib.call('t5d_beam_search_step', lane.stream.cuda_stream,
+                   lane.model, lane.beam)
+
+  def _cond(self, stream):
+    """The whole-batch loop condition -> loop.keep_going, on `stream`."""
+    loop = self.loop
+    st = self._lib.BeamStatePtrs()
+    P = self._lib.ptr
+    st.cur_index = P(self.lane_cur_index)  # lane 0's counter; all are equal
+    st.live_logprobs = P(loop.cur.live_logprobs)
+    st.finished_scores = P(loop.cur.finished_scores)
+    st.live_seqs = P(loop.cur.live_seqs)
+    st.finished_seqs = P(loop.cur.finished_seqs)
+    st.finished_flags = P(loop.cur.finished_flags)
+    self._lib.call('t5d_beam_cond', stream.cuda_stream, handle_ref(st),
+                   loop.batch_size, loop.beam_size, loop.max_decode_len,
+                   float(loop.min_brevity), float(loop.min_log_prob),
+                   int(loop.max_decode_step), int(loop.min_initial),
+                   loop.keep_going.data_ptr())
 
   def _capture(self):
     lib, loop = self._lib, self.loop
-    self.stream.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(self.stream):
-      # First launches load the code objects; do them with the gate closed so
-      # nothing is computed, then open the gate with the real loop condition.
-      loop.keep_going.zero_()
-      self._enqueue()
-      self.stream.synchronize()
-      lib.call('t5d_graph_begin', self.stream.cuda_stream)
-      try:
-        self._enqueue()
-      finally:
-        handle = ctypes_void_p()
-        lib.call('t5d_graph_end', self.stream.cuda_stream, handle_ref(handle))
-      self.graph = handle
-      from t5x_amd import ops
-      ops.beam_cond(loop.cur, loop.min_brevity, loop.min_log_prob,
-                    loop.max_decode_step, loop.min_initial, loop.keep_going)
-    self.stream.synchronize()
+    cur = torch.cuda.current_stream()
+    for lane in self.lanes:
+      lane.stream.wait_stream(cur)
+      with torch.cuda.stream(lane.stream):
+        # First launches load the code objects; do them with the gate closed
+        # so nothing is computed, then open the gate with the real condition.
+        loop.keep_going.zero_()
+        self._enqueue(lane)
+        lane.stream.synchronize()
+        lib.call('t5d_graph_begin', lane.stream.cuda_stream)
+        try:
+          self._enqueue(lane)
+        finally:
+          handle = ctypes_void_p()
+          lib.call('t5d_graph_end', lane.stream.cuda_stream,
+                   handle_ref(handle))
+        lane.graph = handle
+      lane.stream.synchronize()
+    self._cond(self.lanes[0].stream)
+    self.lanes[0].stream.synchronize()
 
   def launch(self, n=1):
+    lanes, lib = self.lanes, self._lib
+    first = lanes[0].stream
     for _ in range(n):
-      self._lib.call('t5d_graph_launch', self.graph, self.stream.cuda_stream)
+      for lane in lanes:
+        lib.call('t5d_graph_launch', lane.graph, lane.stream.cuda_stream)
+      if len(lanes) > 1:
+        # join -> one condition for the whole batch -> fork
+        for lane in lanes[1:]:
+          lane.event.record(lane.stream)
+          first.wait_event(lane.event)
+        self._cond(first)
+        self.cond_event.record(first)
+        for lane in lanes[1:]:
+          lane.stream.wait_event(self.cond_event)
+
+  def synchronize(self):
+    for lane in self.lanes:
+      lane.stream.synchronize()
+    # the lanes advance in lock step
+    self.loop.cur.cur_index.copy_(self.lane_cur_index[0])
 
   def keep_going(self) -> bool:
-    self.stream.synchronize()
+    self.synchronize()
     return bool(self.loop.keep_going.item())
 
   def finish(self):
-    torch.cuda.current_stream().wait_stream(self.stream)
+    self.synchronize()
 
   def cache_tree(self):
-    """The caches in the reference's tree layout (views of the block)."""
-    nl = self.kv.shape[0]
-    if self.deferred_gather:
-      # Apply the reorder still in flight, then mark it done.
-      from t5x_amd import ops
-      B, K = self.loop.top_alive.shape
-      with torch.cuda.stream(self.stream):
+    """The caches in the reference's tree layout (copies; pending reorders
+    are applied first)."""
+    self.synchronize()
+    from t5x_amd import ops
+    K = self.loop.beam_size
+    for lane in self.lanes:
+      if self.deferred_gather:
+        # Apply the reorder still in flight, then mark it done.
+        nl = lane.kv.shape[0]
+        B = lane.b1 - lane.b0
         ops.cache_gather_beams(
-            self.kv[0, 0].view(B, K, *self.kv.shape[3:]), self.loop.top_alive,
+            lane.kv[0, 0].view(B, K, *lane.kv.shape[3:]), lane.top_alive,
             n_tensors=2 * nl,
-            tensor_stride_bytes=self.kv[0, 0].numel() * self.kv.element_size())
-        self.loop.top_alive.copy_(torch.arange(
-            K, dtype=torch.int32, device=self.kv.device).expand(B, K))
-      self.stream.synchronize()
+            tensor_stride_bytes=lane.kv[0, 0].numel() * lane.kv.element_size())
+        lane.top_alive.copy_(torch.arange(
+            K, dtype=torch.int32, device=self.device).expand(B, K))
+    torch.cuda.synchronize()
+    nl = self.lanes[0].kv.shape[0]
+    kv = torch.cat([lane.kv for lane in self.lanes], dim=2)
+    idx = self.lanes[0].cache_index
     return {'decoder': {
         f'layers_{i}': {'self_attention': {
-            'cached_key': self.kv[i, 0], 'cached_value': self.kv[i, 1],
-            'cache_index': self.cache_index[i]}} for i in range(nl)}}
+            'cached_key': kv[i, 0], 'cached_value': kv[i, 1],
+            'cache_index': idx[i]}} for i in range(nl)}}
 
   def __del__(self):
     try:
-      if self.graph is not None:
-        self._lib.call('t5d_graph_destroy', self.graph)
+      for lane in self.lanes:
+        if lane.graph is not None:
+          self._lib.call('t5d_graph_destroy', lane.graph)
     except Exception:  # pylint: disable=broad-except
       pass
 

@@ -322,14 +322,17 @@ def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
 
 
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
-@pytest.mark.parametrize('B,K,L', [(3, 4, 12), (2, 2, 140), (5, 1, 9)])
-def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L):
+@pytest.mark.parametrize('B,K,L,lanes', [(3, 4, 12, 1), (3, 4, 12, 2),
+                                         (2, 2, 140, 2), (5, 1, 9, 3),
+                                         (5, 3, 20, 8)])
+def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L, lanes):
   """The captured whole-iteration graph (in-place state, gated kernels,
   reorder deferred into the next step's attention for bf16) and the
   kernel-per-call loop run the same kernels on the same values: sequences and
   scores must be bit-identical, and so must the caches after every few steps."""
   from t5x_amd import decoding
   module, fn = _decode_setup(dtype, B, K, 24, L, seed=7)
+  module.decode_lanes = lanes  # batch slices stepped on separate streams
   inputs = np.zeros((B, L), np.int32)
 
   fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
@@ -351,7 +354,7 @@ def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L):
       for name in ('live_logprobs', 'finished_scores', 'live_seqs',
                    'finished_seqs', 'finished_flags', 'cur_index'):
         a = getattr(fused.cur, name)
-        fused.fused.stream.synchronize()
+        fused.fused.synchronize()
         assert torch.equal(a, getattr(plain.cur, name)), (step, name)
       fc = fused.fused.cache_tree()['decoder']
       pc = plain.beam_cache['decoder']
@@ -370,14 +373,16 @@ def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L):
   assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
 
 
-@pytest.mark.parametrize('check_every', [1, 3, 8])
-def test_fused_loop_early_stop_is_independent_of_check_interval(check_every):
+@pytest.mark.parametrize('check_every,lanes', [(1, 1), (3, 2), (8, 2), (8, 4)])
+def test_fused_loop_early_stop_is_independent_of_check_interval(check_every,
+                                                                lanes):
   """With EOS made likely the loop ends long before max_decode_len; iterations
   enqueued after the device-side condition turned false must change nothing,
   and replaying the graph many times must keep giving the eager loop's result."""
   from t5x_amd import decoding
   B, K, L = 4, 4, 48
   module, fn = _decode_setup('bfloat16', B, K, 16, L, seed=11, eos_bias=6.0)
+  module.decode_lanes = lanes
   inputs = np.zeros((B, L), np.int32)
   plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
                             eos_id=1, num_decodes=K)
