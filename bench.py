@@ -46,6 +46,9 @@ def parse_args():
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--lanes', type=int, default=None,
                   help='batch slices stepped concurrently (default: library)')
+  ap.add_argument('--roofline-only', action='store_true',
+                  help='only the dominant-kernel replay plus a plain copy of '
+                       'known size (for counter runs under rocprofv3 --pmc)')
   ap.add_argument('--cpu-steps', type=int, default=3,
                   help='decode steps of the CPU oracle sample')
   return ap.parse_args()
@@ -132,24 +135,62 @@ class Workload:
     return R * hd * (t + 1) * 2 * s + R * hd * 2 * s + 2 * R * hd * s
 
 
-def time_kernel(torch, fn, reps):
-  """Average duration of `fn`'s single kernel launch, HIP events on the
-  current (launch) stream around `reps` back-to-back launches."""
-  fn()
-  torch.cuda.synchronize()
-  start = torch.cuda.Event(enable_timing=True)
-  end = torch.cuda.Event(enable_timing=True)
-  start.record()
-  for _ in range(reps):
+def time_kernel(torch, fn, launches, replays=5):
+  """Average duration of one kernel launch of `fn`: `launches` launches are
+  captured into a HIP graph on a side stream (so the host launch rate does not
+  enter), the graph is replayed `replays` times, and HIP events recorded on
+  that same stream bracket the replays."""
+  import ctypes
+  from t5x_amd import _lib
+  st = torch.cuda.Stream()
+  st.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(st):
     fn()
-  end.record()
-  end.synchronize()
-  return start.elapsed_time(end) * 1e-3 / reps
+    st.synchronize()
+    _lib.call('t5d_graph_begin', st.cuda_stream)
+    try:
+      for _ in range(launches):
+        fn()
+    finally:
+      graph = ctypes.c_void_p()
+      _lib.call('t5d_graph_end', st.cuda_stream, ctypes.byref(graph))
+    _lib.call('t5d_graph_launch', graph, st.cuda_stream)
+    st.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record(st)
+    for _ in range(replays):
+      _lib.call('t5d_graph_launch', graph, st.cuda_stream)
+    end.record(st)
+    end.synchronize()
+  _lib.call('t5d_graph_destroy', graph)
+  return start.elapsed_time(end) * 1e-3 / (launches * replays)
 
 
-def roofline_cross_attention(w):
+PROFILE_NOTE = os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                            'profiles',
+                            'cross_attn_mfma_kernel_base-beam4_pmc.txt')
+
+
+def measured_traffic(name):
+  """HBM bytes per launch of the dominant kernel from the committed counter
+  summary (FETCH_SIZE + WRITE_SIZE, calibrated against a plain copy), or None
+  when no summary exists for this workload."""
+  if name != 'base-beam4' or not os.path.exists(PROFILE_NOTE):
+    return None
+  with open(PROFILE_NOTE) as f:
+    for line in f:
+      if line.startswith('traffic_bytes_per_launch:'):
+        return int(float(line.split(':', 1)[1]))
+  return None
+
+
+def roofline_cross_attention(w, reps_per_layer=4):
   """The step's largest single stream of HBM bytes per launch: cross-attention
-  over the encoder K/V (12 launches per step, same shape every step)."""
+  over the encoder K/V (one launch per layer per step, same shape every step).
+  Replayed here back to back, walking the layers so no launch finds its K/V in
+  a cache (12 x 31 MB > the 256 MB memory-side cache only partly; L2 holds
+  none of it), and timed with HIP events on the launch stream."""
   from t5x_amd import ops
   torch = w.torch
   cross = w.module._cross[1]
@@ -165,14 +206,26 @@ def roofline_cross_attention(w):
     ops.cross_attention_step(q, cross['k'][i], cross['v'][i], cross['enc_len'],
                              w.K, out)
 
-  sec = time_kernel(torch, launch, 20 * nl)
+  sec = time_kernel(torch, launch, reps_per_layer * nl)
   nbytes = w.cross_attention_bytes()
   achieved = nbytes / sec / 1e9
-  return {'kernel': 'attn_step_kernel<bf16,NQ=4,cross>', 'bound': 'hbm',
+  return {'kernel': 'cross_attn_mfma_kernel<4,4>', 'bound': 'hbm',
           'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS,
           'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBPS, 4),
-          'traffic': None, 'bytes_per_launch': nbytes,
+          'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes,
           'avg_launch_us': round(sec * 1e6, 2)}
+
+
+def copy_calibration(torch, nbytes=256 << 20, reps=5):
+  """A plain device copy of known size, so FETCH_SIZE / WRITE_SIZE readings can
+  be scaled: it reads nbytes and writes nbytes."""
+  src = torch.empty(nbytes, dtype=torch.uint8, device='cuda')
+  src.zero_()
+  dst = torch.empty_like(src)
+  for _ in range(reps):
+    dst.copy_(src)
+  torch.cuda.synchronize()
+  return nbytes
 
 
 def cpu_baseline(name, steps, seed):
@@ -234,6 +287,12 @@ def main():
     print('bench.py: no GPU visible', file=sys.stderr)
     sys.exit(3)
   w = Workload(args.config, args.seed, args.lanes)
+  if args.roofline_only:
+    w.new_decode()  # builds the cross-attention K/V
+    r = roofline_cross_attention(w, reps_per_layer=1)
+    r['copy_bytes'] = copy_calibration(torch)
+    print(json.dumps(r))
+    return
   w.run_steps(args.warmup)
   torch.cuda.synchronize()
   t0 = time.perf_counter()
