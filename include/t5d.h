@@ -138,6 +138,22 @@ int t5d_cross_attention_step(void* stream, int dtype, const void* q,
                              const int32_t* enc_len, void* out, int B,
                              int beams, int H, int E);
 
+/* t5d_rmsnorm + the query projection (t5d_gemm) + t5d_cross_attention_step
+ * in one kernel (pre_cross_attention_layer_norm, the `query` DenseGeneral and
+ * the attention of t5x/examples/t5/network.py:149-159): every workgroup
+ * normalises its batch item's rows of x and multiplies them with its head's
+ * 64 columns of the packed query kernel while its K stream is in flight.
+ *   x [B*beams, d] residual stream; ln_scale [d]; query_kernel: packed
+ *   (t5d_pack_weight) [d, H*64] bfloat16 kernel.  bfloat16 only; E <= 512;
+ *   d a multiple of 64, <= 1024. */
+int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
+                                    const void* x, const void* ln_scale,
+                                    float eps, const void* query_kernel,
+                                    const void* cross_key,
+                                    const void* cross_value,
+                                    const int32_t* enc_len, void* out, int B,
+                                    int beams, int H, int E, int d);
+
 /* Add `delta` to n int32 values (cache_index += 1, layers.py:275). */
 int t5d_add_i32(void* stream, int32_t* x, int n, int delta);
 

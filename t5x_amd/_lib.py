@@ -82,6 +82,10 @@ _SIGNATURES = {
                                                _P]),
     't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
                                          c_int, c_int, c_int]),
+    't5d_cross_attention_step_norm_q': (c_int, [_P, c_int, c_int, _P, _P,
+                                                c_float, _P, _P, _P, _P, _P,
+                                                c_int, c_int, c_int, c_int,
+                                                c_int]),
     't5d_add_i32': (c_int, [_P, _P, c_int, c_int]),
     't5d_cache_gather_beams': (c_int, [_P, _P, c_int64, c_int, c_int, c_int,
                                        c_int, c_int, c_int, _P, _P, c_int]),

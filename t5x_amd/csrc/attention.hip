@@ -417,7 +417,9 @@ static void launch_cross_f32(const AttnArgs& a, int B, hipStream_t s) {
 
 int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 const void* v, const int32_t* enc_len,
-                                void* out, int B, int beams, int H, int E);
+                                void* out, int B, int beams, int H, int E,
+                                const void* x, const void* ln, const void* wq,
+                                int d, float eps);
 int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                void* cv, const void* rel_bias,
                                const int32_t* cache_index, void* out, int R,
@@ -522,8 +524,42 @@ extern "C" int t5d_cross_attention_step(void* stream, int dtype, const void* q,
     launch_cross_f32(a, B, as_stream(stream));
   } else {
     launch_cross_attention_bf16(as_stream(stream), q, cross_key, cross_value,
-                                enc_len, out, B, beams, H, E);
+                                enc_len, out, B, beams, H, E, nullptr, nullptr,
+                                nullptr, 0, 0.f);
   }
   T5D_CHECK_LAUNCH("t5d_cross_attention_step");
+  return T5D_OK;
+}
+
+extern "C" int t5d_cross_attention_step_norm_q(
+    void* stream, int dtype, int w_dtype, const void* x, const void* ln_scale,
+    float eps, const void* query_kernel, const void* cross_key,
+    const void* cross_value, const int32_t* enc_len, void* out, int B,
+    int beams, int H, int E, int d) {
+  int rc = check_common("t5d_cross_attention_step_norm_q", dtype, H, E);
+  if (rc) return rc;
+  T5D_REQUIRE(dtype == T5D_BF16 && w_dtype == T5D_BF16, T5D_EINVAL,
+              "t5d_cross_attention_step_norm_q: bfloat16 activations and "
+              "weights only");
+  T5D_REQUIRE(x && ln_scale && query_kernel && cross_key && cross_value &&
+                  enc_len && out && B > 0,
+              T5D_EINVAL,
+              "t5d_cross_attention_step_norm_q: null pointer or B=%d", B);
+  T5D_REQUIRE(beams >= 1 && beams <= 8, T5D_ELIMIT,
+              "t5d_cross_attention_step_norm_q: beams=%d (supported: 1..8)",
+              beams);
+  T5D_REQUIRE(E <= 512 && d >= 64 && d % 64 == 0 && d <= 1024, T5D_ELIMIT,
+              "t5d_cross_attention_step_norm_q: E=%d (<= 512), d=%d (multiple "
+              "of 64, <= 1024)", E, d);
+  T5D_REQUIRE(((uintptr_t)cross_key % 16) == 0 &&
+                  ((uintptr_t)cross_value % 16) == 0 &&
+                  ((uintptr_t)x % 16) == 0 && ((uintptr_t)ln_scale % 16) == 0 &&
+                  ((uintptr_t)query_kernel % 16) == 0,
+              T5D_EINVAL,
+              "t5d_cross_attention_step_norm_q: operands not 16-byte aligned");
+  launch_cross_attention_bf16(as_stream(stream), nullptr, cross_key, cross_value,
+                              enc_len, out, B, beams, H, E, x, ln_scale,
+                              query_kernel, d, eps);
+  T5D_CHECK_LAUNCH("t5d_cross_attention_step_norm_q");
   return T5D_OK;
 }

@@ -48,6 +48,12 @@ struct AttnMfmaArgs {
   // self-attention only
   const int32_t* pending;  // [B, beams] source beam per row, or null
   int beams, nblk;         // rows per workgroup, wavefronts per row
+  // cross-attention with the query projection fused in (q == nullptr)
+  const bf16_t* x;         // [R, d] residual stream
+  const bf16_t* ln;        // [d] pre-attention layer-norm scale
+  const void* wq;          // packed [d, H*64] query kernel (bf16 tiles)
+  int d;
+  float eps;
 };
 
 constexpr int kHeadDim = 64;
@@ -60,9 +66,16 @@ __device__ long long t5d_probe_buf[64 * 16];
   if (lane == 0 && wave == 0 && (blockIdx.x + blockIdx.y * gridDim.x) % 37 == 0 && \
       (blockIdx.x + blockIdx.y * gridDim.x) / 37 < 64)                      \
     t5d_probe_buf[((blockIdx.x + blockIdx.y * gridDim.x) / 37) * 16 + (i)] = \
-        __builtin_readcyclecounter()
+        wall_clock64()
 #else
 #define T5D_STAMP(i)
+#endif
+#ifdef T5D_PROBE_FQ  // slots 8..15 go to the fused projection instead
+#define T5D_STAMP_SELF(i)
+#define T5D_STAMP_FQ(i) T5D_STAMP(i)
+#else
+#define T5D_STAMP_SELF(i) T5D_STAMP(i)
+#define T5D_STAMP_FQ(i)
 #endif
 
 // ---- cross-attention -----------------------------------------------------------
@@ -73,12 +86,25 @@ __device__ long long t5d_probe_buf[64 * 16];
 // tiles jt = s (mod REP), so the softmax runs on all 64 lanes with 32 / REP
 // scores each instead of 32 scores in 16 lanes.  out^T = V·P^T likewise (V
 // tile as A, P^T with repeated query columns as B).
-template <int NQP, int WM>
-__global__ void __launch_bounds__(64 * WM)
+//
+// NJ > 0 fuses the pre-attention layer norm and the query projection in: the
+// workgroup (4 wavefronts) normalises the item's NQP rows of the residual
+// stream and multiplies them with the head's 64 columns of the query kernel
+// while its K stream is in flight — same k-tile split over wavefronts, same
+// accumulation and summation order as gemm_mfma_kernel, so q has the same
+// bits as the stand-alone dense layer given the same row statistics.  NJ is
+// the number of k-tile pairs per wavefront (d / 256, rounded up).
+template <int NQP, int WM, int NJ>
+__global__ void __launch_bounds__(64 * WM, NJ > 0 ? 2 : 1)  // fused: 2 WGs per CU
 cross_attn_mfma_kernel(AttnMfmaArgs a) {
   constexpr int REP = 16 / NQP;   // copies of each query column
   constexpr int TPL = 8 / REP;    // score tiles a lane keeps
+  constexpr bool FQ = NJ > 0;
+  static_assert(!FQ || WM == 4, "the fused projection splits K over 4 waves");
   __shared__ float s_red[2][WM][16];
+  __shared__ float s_ss[FQ ? 4 : 1][16];
+  __shared__ __attribute__((aligned(16))) float s_qp[FQ ? 4 : 1][NQP][kHeadDim];
+  __shared__ __attribute__((aligned(16))) bf16_t s_qb[FQ ? NQP : 1][kHeadDim];
   __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][NQP][kBlockJ];
   __shared__ __attribute__((aligned(16))) float s_out[WM][NQP][kHeadDim];
   T5D_GATE_READ(a.gate);
@@ -113,6 +139,28 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   // the last row / last 8 positions (those positions are masked anyway).
   Frag16 kb[8][2];
   Frag16 vb[4][4];
+  // Fused projection: this wavefront's k-tile pairs p = wave + 4 j.
+  Frag16 xa[FQ ? NJ : 1][2];      // A: rows of x (row n16), k = 8g .. +8
+  uint4 lnv[FQ ? NJ : 1][2];      // layer-norm scale for the same k
+  Frag16 wt[FQ ? NJ : 1][2][4];   // B: query-kernel tiles of this head
+  const int KT = FQ ? a.d >> 5 : 0;
+  if constexpr (FQ) {
+    const int xr = b * a.nq + (n16 < a.nq ? n16 : 0);
+    const bf16_t* xrow = a.x + (size_t)xr * a.d + 8 * g;
+    const char* wbase = reinterpret_cast<const char*>(a.wq);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
+        xa[j][hh].u = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+        lnv[j][hh] = *reinterpret_cast<const uint4*>(a.ln + 32 * kt + 8 * g);
+#pragma unroll
+        for (int nn = 0; nn < 4; ++nn)
+          wt[j][hh][nn].u = reinterpret_cast<const uint4*>(
+              wbase + ((size_t)(4 * h + nn) * KT + kt) * 1024)[lane];
+      }
+  }
 #pragma unroll
   for (int jt = 0; jt < 8; ++jt) {
     if (16 * jt < nw) {
@@ -125,22 +173,25 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       kb[jt][0].u = kb[jt][1].u = make_uint4(0, 0, 0, 0);
     }
   }
+  auto load_v = [&]() {
 #pragma unroll
-  for (int jb = 0; jb < 4; ++jb) {
-    if (32 * jb < nw) {
+    for (int jb = 0; jb < 4; ++jb) {
+      if (32 * jb < nw) {
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-        vb[jb][dt].u = *reinterpret_cast<const uint4*>(
-            vbase + (size_t)(16 * dt + n16) * a.S +
-            min(jw + 32 * jb + 8 * g, a.S - 8));
-    } else {
+        for (int dt = 0; dt < 4; ++dt)
+          vb[jb][dt].u = *reinterpret_cast<const uint4*>(
+              vbase + (size_t)(16 * dt + n16) * a.S +
+              min(jw + 32 * jb + 8 * g, a.S - 8));
+      } else {
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);
+        for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);
+      }
     }
-  }
+  };
   // B operand of K·Q^T: lane (col n16 -> query q, g) holds Q[q][32c + 8g .. +8].
   Frag16 qb[2];
-  {
+  if constexpr (!FQ) {
+    load_v();
     const bool qrow = q < a.nq;
     const bf16_t* qp = a.q + (size_t)(b * a.nq + (qrow ? q : 0)) * a.q_stride +
                        h * kHeadDim + 8 * g;
@@ -149,6 +200,83 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       qb[c].u = *reinterpret_cast<const uint4*>(qp + 32 * c);
       if (!qrow) qb[c].u = make_uint4(0, 0, 0, 0);
     }
+  } else {
+    T5D_STAMP_FQ(8);
+    // Row statistics: sum of squares of row n16 over this wavefront's k range.
+    const int n_pairs = KT >> 1;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (wave + 4 * j < n_pairs) {
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          float f[8];
+          unpack16(xa[j][hh].u, f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+        }
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    T5D_STAMP_FQ(9);
+    if (g == 0) s_ss[wave][n16] = n16 < a.nq ? ss : 0.f;
+    __syncthreads();
+    T5D_STAMP_FQ(10);
+    const float tot = (s_ss[0][n16] + s_ss[2][n16]) + (s_ss[1][n16] + s_ss[3][n16]);
+    const float inv = 1.0f / sqrtf(tot / (float)a.d + a.eps);
+    f32x4_v qacc[4];
+#pragma unroll
+    for (int nn = 0; nn < 4; ++nn) qacc[nn] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (wave + 4 * j < n_pairs) {
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          float xf[8], sf[8];
+          unpack16(xa[j][hh].u, xf);
+          unpack16(lnv[j][hh], sf);
+          uint32_t o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float y0 = round_bf16(xf[2 * e] * inv);
+            const float y1 = round_bf16(xf[2 * e + 1] * inv);
+            o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
+          }
+          Frag16 an;
+          an.u = n16 < a.nq ? make_uint4(o[0], o[1], o[2], o[3])
+                            : make_uint4(0, 0, 0, 0);
+#pragma unroll
+          for (int nn = 0; nn < 4; ++nn)
+            qacc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                an.v, wt[j][hh][nn].v, qacc[nn], 0, 0, 0);
+        }
+      }
+    }
+    T5D_STAMP_FQ(11);
+    // qacc[nn][i] in lane (n16, g) is the partial q[row 4g + i][16 nn + n16].
+    if (4 * g < NQP) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int nn = 0; nn < 4; ++nn)
+          s_qp[wave][4 * g + i][16 * nn + n16] = qacc[nn][i];
+    }
+    load_v();  // the V stream follows K while the projection is reduced
+    T5D_STAMP_FQ(12);
+    __syncthreads();
+    T5D_STAMP_FQ(13);
+    for (int e = threadIdx.x; e < NQP * kHeadDim; e += 64 * WM) {
+      const int row = e / kHeadDim, col = e % kHeadDim;
+      const float v = (s_qp[0][row][col] + s_qp[2][row][col]) +
+                      (s_qp[1][row][col] + s_qp[3][row][col]);
+      s_qb[row][col] = f32_to_bf16(v);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      qb[c].u = *reinterpret_cast<const uint4*>(&s_qb[q][32 * c + 8 * g]);
+    T5D_STAMP_FQ(14);
   }
 
   // Tile jt: lane (n16, g) gets scores of positions 16 jt + 4g + i, query q.
@@ -354,10 +482,10 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     r = rs = blockIdx.y;
   }
 
-  T5D_STAMP(8);
+  T5D_STAMP_SELF(8);
   const int t = *a.index;
   T5D_GATE_TEST();  // after the scalar loads above are in flight
-  T5D_STAMP(9);
+  T5D_STAMP_SELF(9);
   const int n = t + 1;
   const int jw = blk * kBlockJ;
   const int nw = n - jw;  // positions of this wavefront in use (may be <= 0)
@@ -433,7 +561,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int e = 0; e < 8; ++e) s8[e] = fmaf(qv[i], kf[e], s8[e]);
   }
 
-  T5D_STAMP(10);
+  T5D_STAMP_SELF(10);
   if (permuted) {
     // Every wavefront of the workgroup has its source data in registers
     // before any slot is written.
@@ -468,7 +596,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     vdst[(size_t)lane * S + t] = vnew_d;
   }
 
-  T5D_STAMP(11);
+  T5D_STAMP_SELF(11);
   // 2 positions per lane: bias, mask, softmax.
   float sc[2];
   reduce_scatter_8(s8, sc);
@@ -491,7 +619,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     m = s_red[0][wave0];
     for (int w = 1; w < nblk; ++w) m = fmaxf(m, s_red[0][wave0 + w]);
   }
-  T5D_STAMP(12);
+  T5D_STAMP_SELF(12);
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
@@ -516,7 +644,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     *reinterpret_cast<uint32_t*>(&s_p[wave][jp - jw]) = pack_bf16x2(p0, p1);
   }
   __syncthreads();
-  T5D_STAMP(13);
+  T5D_STAMP_SELF(13);
 
   // out^T tile dt: lane (n16, g) gets out[16 dt + 4g + i], i < 4, in every
   // column n16.  B lane (col, g) holds P[32 jb + 8g .. +8].
@@ -546,7 +674,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       oc[dt][3] = fmaf(p_t, bf16hi_to_f32(vn.y), oc[dt][3]);
     }
   }
-  T5D_STAMP(14);
+  T5D_STAMP_SELF(14);
   if (nblk == 1) {
     if (n16 == 0) {
       bf16_t* o = a.out + (size_t)r * HD + h * kHeadDim + 4 * g;
@@ -558,7 +686,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
         *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
       }
     }
-    T5D_STAMP(15);
+    T5D_STAMP_SELF(15);
     return;
   }
   if (n16 == 0) {
@@ -580,18 +708,33 @@ template <int NQP>
 static void launch_cross(const AttnMfmaArgs& a, int B, hipStream_t s) {
   const int waves = (a.S + kBlockJ - 1) / kBlockJ;
   dim3 grid(a.H, B), block(64 * waves);
+  if (a.q == nullptr) {  // fused query projection: always 4 wavefronts
+    block = dim3(256);
+    const int nj = (a.d / 64 + 3) / 4;
+    if (nj <= 3)
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 3>), grid, block, 0, s,
+                         a);
+    else
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 4>), grid, block, 0, s,
+                         a);
+    return;
+  }
   if (waves <= 4)
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 0>), grid, block, 0, s, a);
   else if (waves <= 8)
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 8>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 8, 0>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 16>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 16, 0>), grid, block, 0, s, a);
 }
 
 int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 const void* v, const int32_t* enc_len,
-                                void* out, int B, int beams, int H, int E) {
+                                void* out, int B, int beams, int H, int E,
+                                const void* x, const void* ln, const void* wq,
+                                int d, float eps) {
   AttnMfmaArgs a;
+  a.x = (const bf16_t*)x; a.ln = (const bf16_t*)ln; a.wq = wq;
+  a.d = d; a.eps = eps;
   a.q = (const bf16_t*)q; a.k = (bf16_t*)k; a.v = (bf16_t*)v;
   a.rel_bias = nullptr; a.index = enc_len; a.out = (bf16_t*)out;
   a.H = H; a.S = E; a.nq = beams; a.q_stride = H * kHeadDim;
@@ -612,6 +755,7 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
   a.out = (bf16_t*)out;
   a.H = H; a.S = L; a.nq = 1; a.q_stride = 3 * H * kHeadDim;
   a.gate = tls_gate;
+  a.x = nullptr; a.ln = nullptr; a.wq = nullptr; a.d = 0; a.eps = 0.f;
   a.nblk = (L + kBlockJ - 1) / kBlockJ;
   a.pending = pending;
   a.beams = pending ? beams : 1;

@@ -49,6 +49,10 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
   const int R = m->R, d = m->d, HD = m->H * 64, F = m->F;
   T5D_TRY(t5d_embed(stream, dt, m->embedding, ids, m->x, R, d, m->V));
   const void* x = m->x;
+  // Layer norm + query projection ride inside the cross-attention kernel when
+  // its limits allow (bfloat16 weights, E <= 512, d <= 1024).
+  const bool fuse_cross_q = dt == T5D_BF16 && wd == T5D_BF16 && m->E <= 512 &&
+                            d % 64 == 0 && d <= 1024;
   for (int l = 0; l < m->NL; ++l) {
     const t5d_layer& w = m->layers[l];
     T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
@@ -66,12 +70,19 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
                                       m->L));
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.self_out, w.self_out_scales,
                      x, m->x1, R, HD, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
-    T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
-    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q, w.cross_q_scales,
-                     nullptr, m->q, R, d, HD, T5D_EPI_NONE, nullptr, nullptr));
-    T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
-                                     w.cross_value, m->enc_len, m->ao, m->B,
-                                     m->beams, m->H, m->E));
+    if (fuse_cross_q) {
+      T5D_TRY(t5d_cross_attention_step_norm_q(
+          stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
+          w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d));
+    } else {
+      T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
+      T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q, w.cross_q_scales,
+                       nullptr, m->q, R, d, HD, T5D_EPI_NONE, nullptr,
+                       nullptr));
+      T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
+                                       w.cross_value, m->enc_len, m->ao, m->B,
+                                       m->beams, m->H, m->E));
+    }
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
                      w.cross_out_scales, m->x1, m->x2, R, HD, d,
                      T5D_EPI_RESIDUAL, nullptr, nullptr));

@@ -270,6 +270,33 @@ def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
   return out
 
 
+def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
+                                cross_value, enc_len, beams, out=None,
+                                eps=1e-6):
+  """rmsnorm(x, ln_scale) @ wq followed by cross_attention_step, one kernel."""
+  _chk(x, 'x', torch.bfloat16, 2)
+  _chk(ln_scale, 'ln_scale', torch.bfloat16, 1)
+  _chk(cross_key, 'cross_key', x.dtype, 4)
+  _chk(cross_value, 'cross_value', x.dtype, 4)
+  _chk(enc_len, 'enc_len', torch.int32, 1)
+  B, H, E, D = cross_key.shape
+  R, d = x.shape
+  if D != 64 or tuple(cross_value.shape) != (B, H, D, E):
+    raise ValueError('cross_key must be [B, H, E, 64], cross_value [B, H, 64, E]')
+  if R != B * beams or ln_scale.shape[0] != d or enc_len.shape[0] != B:
+    raise ValueError('x / ln_scale / enc_len do not match the batch')
+  if wq.K != d or wq.N != H * D or wq.geglu:
+    raise ValueError(f'query kernel must be [{d}, {H * D}]')
+  if out is None:
+    out = torch.empty((R, H * D), dtype=x.dtype, device=x.device)
+  _chk(out, 'out', x.dtype, 2)
+  _lib.call('t5d_cross_attention_step_norm_q', _s(), _lib.dtype_code(x.dtype),
+            wq.w_dtype, x.data_ptr(), ln_scale.data_ptr(), float(eps),
+            wq.data.data_ptr(), cross_key.data_ptr(), cross_value.data_ptr(),
+            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E, d)
+  return out
+
+
 def add_i32(x, delta):
   _chk(x, 'x', torch.int32)
   _lib.call('t5d_add_i32', _s(), x.data_ptr(), x.numel(), int(delta))

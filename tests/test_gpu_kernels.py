@@ -320,6 +320,38 @@ def test_beam_topk(ops, B, beams, V):
   np.testing.assert_array_equal(host(vals), wv)
 
 
+@pytest.mark.parametrize('B,beams,H,E,d', [(3, 4, 2, 512, 768),
+                                           (2, 8, 3, 264, 256),
+                                           (32, 4, 12, 512, 768),
+                                           (2, 1, 2, 64, 1024),
+                                           (2, 3, 2, 128, 64),
+                                           (2, 4, 2, 384, 832)])
+def test_cross_attention_with_fused_norm_and_query_projection(ops, B, beams, H,
+                                                              E, d):
+  """One kernel against rmsnorm -> dense -> cross_attention_step.  The
+  projection uses the dense kernel's split and summation order, so the only
+  source of difference is the order of the sum of squares (one ulp of 1/rms,
+  which now and then flips a bf16 rounding of a normalised element)."""
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(B * 7 + beams + E + d)
+  bf = torch.bfloat16
+  R, HD = B * beams, H * 64
+  rnd = lambda *shape: torch.randn(shape, generator=gen, device='cuda')
+  x = (2 * rnd(R, d)).to(bf)
+  scale = (1 + 0.1 * rnd(d)).to(bf)
+  wq = ops.pack_weight(rnd(d, HD) / (8 * d ** 0.5), bf)
+  ck, cv = rnd(B, H, E, 64).to(bf), rnd(B, H, 64, E).to(bf)
+  lens = torch.randint(1, E + 1, (B,), generator=gen, device='cuda',
+                       dtype=torch.int32)
+  lens[0] = E
+  q = ops.gemm(ops.rmsnorm(x, scale), wq)
+  want = ops.cross_attention_step(q, ck, cv, lens, beams)
+  got = ops.cross_attention_step_norm_q(x, scale, wq, ck, cv, lens, beams)
+  diff = (got.float() - want.float()).abs()
+  assert float((diff > 0).float().mean()) < 0.02, float((diff > 0).float().mean())
+  assert float(diff.max()) <= 2e-2, float(diff.max())
+
+
 @pytest.mark.parametrize('V', [32128, 4096 * 8, 4100, 512, 250])
 @pytest.mark.parametrize('pattern', ['one_thread', 'one_wave', 'all_equal',
                                      'descending'])
