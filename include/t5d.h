@@ -95,6 +95,17 @@ int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
              const void* residual, void* C, int M, int K, int N, int epilogue,
              void* workspace, int32_t* counters);
 
+/* t5d_rmsnorm followed by t5d_gemm in one kernel (a pre-attention / pre-MLP
+ * LayerNorm feeding its dense layer, t5x/examples/t5/network.py:134-139,
+ * 166-171): the rows of A are normalised on their way into the matrix product,
+ * with the same two roundings to bfloat16 as t5d_rmsnorm and the same
+ * summation order of the product as t5d_gemm.  bfloat16 activations and
+ * packed bfloat16 weights; K a multiple of 64, <= 1024; epilogue NONE or
+ * GEGLU. */
+int t5d_norm_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
+                  const void* A, const void* norm_scale, float eps,
+                  const void* W, void* C, int M, int K, int N, int epilogue);
+
 /* One step of cached decoder self-attention
  * (MultiHeadDotProductAttention decode branch,
  * t5x/examples/t5/layers.py:223-346, and dot_product_attention :52-129).

@@ -75,6 +75,8 @@ _SIGNATURES = {
     't5d_gemm_workspace_bytes': (c_int64, [c_int] * 5),
     't5d_gemm': (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
                          c_int, c_int, c_int, _P, _P]),
+    't5d_norm_gemm': (c_int, [_P, c_int, c_int, c_int, _P, _P, c_float, _P, _P,
+                              c_int, c_int, c_int, c_int]),
     't5d_self_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P,
                                         c_int, c_int, c_int]),
     't5d_self_attention_step_gather': (c_int, [_P, c_int, _P, _P, _P, _P, _P,

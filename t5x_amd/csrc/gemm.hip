@@ -69,6 +69,8 @@ struct GemmArgs {
   const int32_t* gate;  // optional device-side enable flag
   int epilogue;
   int out_f32;
+  const bf16_t* norm_scale;  // norm_gemm_kernel: [K] layer-norm scale
+  float eps;
 };
 
 // Apply scale + epilogue to one finished column (pair) of row m; `res` is the
@@ -273,6 +275,131 @@ gemm_mfma_kernel(GemmArgs g) {
       }
       finish(e, r);
     }
+  }
+}
+
+// ---- layer norm + dense in one kernel -------------------------------------------
+// y = bf16(bf16(x / rms(x)) * scale) feeds the matrix cores directly.  A
+// workgroup owns 16 rows and NT column tiles; its 4 wavefronts split K in
+// k-tile pairs exactly like gemm_mfma_kernel (same accumulation and summation
+// order) and hold ALL their operand fragments in registers (K <= 256 * NJ), so
+// the row statistics come from the fragments already loaded for the product:
+// one exchange through LDS, no second pass over x, and only 16 rows per
+// workgroup to normalise.
+template <int NT, int NJ>
+__global__ void __launch_bounds__(256)
+norm_gemm_kernel(GemmArgs g) {
+  constexpr int TN = NT * 16;
+  __shared__ float red[4][NT * 4][64];
+  __shared__ float s_ss[4][16];
+  T5D_GATE_READ(g.gate);
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int n_group = (slot / g.m_parts) * 8 + xcd;
+  const int m_part = slot % g.m_parts;
+  const int n_tiles_total = g.N >> 4;
+  const int nt0 = n_group * NT;
+  if (nt0 >= n_tiles_total) return;
+  const int m0 = m_part * 16;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n16 = lane & 15, gq = lane >> 4;
+  const int KT = g.K >> 5, n_pairs = KT >> 1;
+  const int row = m0 + n16;
+  const bool row_ok = row < g.M;
+
+  Frag xa[NJ][2], wt[NJ][2][NT];
+  uint4 lnv[NJ][2];
+  {
+    const bf16_t* xrow = g.A + (size_t)(row_ok ? row : g.M - 1) * g.K + 8 * gq;
+    const char* wbase = reinterpret_cast<const char*>(g.W);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
+        xa[j][hh].u = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+        lnv[j][hh] =
+            *reinterpret_cast<const uint4*>(g.norm_scale + 32 * kt + 8 * gq);
+#pragma unroll
+        for (int nn = 0; nn < NT; ++nn)
+          wt[j][hh][nn].u = reinterpret_cast<const uint4*>(
+              wbase + ((size_t)min(nt0 + nn, n_tiles_total - 1) * KT + kt) *
+                          1024)[lane];
+      }
+  }
+  T5D_GATE_TEST();
+
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (wave + 4 * j < n_pairs) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        float f[8];
+        unpack16(xa[j][hh].u, f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+      }
+    }
+  }
+  ss += __shfl_xor(ss, 16, 64);
+  ss += __shfl_xor(ss, 32, 64);
+  if (gq == 0) s_ss[wave][n16] = ss;
+  __syncthreads();
+  const float tot = (s_ss[0][n16] + s_ss[2][n16]) + (s_ss[1][n16] + s_ss[3][n16]);
+  const float inv = 1.0f / sqrtf(tot / (float)g.K + g.eps);
+
+  f32x4_v acc[NT];
+#pragma unroll
+  for (int nn = 0; nn < NT; ++nn) acc[nn] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (wave + 4 * j < n_pairs) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        float xf[8], sf[8];
+        unpack16(xa[j][hh].u, xf);
+        unpack16(lnv[j][hh], sf);
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(xf[2 * e] * inv);
+          const float y1 = round_bf16(xf[2 * e + 1] * inv);
+          o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
+        }
+        Frag an;
+        an.u = row_ok ? make_uint4(o[0], o[1], o[2], o[3])
+                      : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int nn = 0; nn < NT; ++nn)
+          acc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              an.v, wt[j][hh][nn].v, acc[nn], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t * 4 + i][lane] = acc[t][i];
+  __syncthreads();
+
+  const bool geglu = g.epilogue == T5D_EPI_GEGLU;
+  auto tile_sum = [&](int ml, int nl) -> float {
+    const int i = ml & 3, c = (ml & 15) >> 2;
+    const int nn = nl >> 4, l = c * 16 + (nl & 15);
+    const int idx = nn * 4 + i;
+    return (red[0][idx][l] + red[2][idx][l]) + (red[1][idx][l] + red[3][idx][l]);
+  };
+#pragma unroll
+  for (int p = 0; p < NT; ++p) {
+    const int e = threadIdx.x + 256 * p;
+    const int ml = e / TN, nl = e % TN;
+    const int m = m0 + ml, n = nt0 * 16 + nl;
+    if (m >= g.M || n >= g.N) continue;
+    if (geglu && (nl & 8)) continue;
+    const float v = tile_sum(ml, nl);
+    const float vg = geglu ? tile_sum(ml, nl + 8) : 0.f;
+    store_result(g, m, n, v, vg, 0.f);
   }
 }
 
@@ -515,8 +642,61 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
   g.gate = tls_gate;
   g.epilogue = epilogue;
   g.out_f32 = out_dtype == T5D_F32;
+  g.norm_scale = nullptr;
+  g.eps = 0.f;
   if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);
   else launch_mfma<int8_t>(p, g, s);
   T5D_CHECK_LAUNCH("t5d_gemm");
+  return T5D_OK;
+}
+
+extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
+                             int out_dtype, const void* A,
+                             const void* norm_scale, float eps, const void* W,
+                             void* C, int M, int K, int N, int epilogue) {
+  T5D_REQUIRE(A && norm_scale && W && C, T5D_EINVAL,
+              "t5d_norm_gemm: null pointer");
+  T5D_REQUIRE(dtype == T5D_BF16 && w_dtype == T5D_BF16, T5D_EINVAL,
+              "t5d_norm_gemm: bfloat16 activations and weights only");
+  T5D_REQUIRE(out_dtype == T5D_BF16 ||
+                  (out_dtype == T5D_F32 && epilogue == T5D_EPI_NONE),
+              T5D_EINVAL, "t5d_norm_gemm: out_dtype %d with epilogue %d",
+              out_dtype, epilogue);
+  T5D_REQUIRE(epilogue == T5D_EPI_NONE || epilogue == T5D_EPI_GEGLU, T5D_EINVAL,
+              "t5d_norm_gemm: epilogue %d (none or geglu)", epilogue);
+  T5D_REQUIRE(M > 0 && M <= 128, T5D_ELIMIT, "t5d_norm_gemm: M=%d (1..128)", M);
+  T5D_REQUIRE(K >= 64 && K % 64 == 0 && K <= 1024 && N > 0 && N % 16 == 0,
+              T5D_ELIMIT,
+              "t5d_norm_gemm: K=%d (multiple of 64, <= 1024), N=%d (multiple "
+              "of 16)", K, N);
+  T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 &&
+                  ((uintptr_t)norm_scale % 16) == 0,
+              T5D_EINVAL, "t5d_norm_gemm: operands must be 16-byte aligned");
+  GemmArgs g;
+  g.A = (const bf16_t*)A; g.W = W; g.scales = nullptr; g.residual = nullptr;
+  g.C = C; g.M = M; g.K = K; g.N = N;
+  g.m_parts = (M + 15) / 16;
+  g.gate = tls_gate;
+  g.epilogue = epilogue;
+  g.out_f32 = out_dtype == T5D_F32;
+  g.norm_scale = (const bf16_t*)norm_scale;
+  g.eps = eps;
+  const int n_tiles = N / 16;
+  // 64-column tiles unless that leaves too few workgroups to fill the chip
+  const int nt = (n_tiles / 4) * g.m_parts >= 256 ? 4 : (n_tiles >= 64 ? 2 : 1);
+  const int n_groups = (n_tiles + nt - 1) / nt;
+  dim3 grid((n_groups + 7) / 8 * 8 * g.m_parts), block(256);
+  hipStream_t s = as_stream(stream);
+  const int nj = (K / 64 + 3) / 4;
+#define T5D_NG_CASE(NT_)                                                     \
+  if (nt == NT_) {                                                           \
+    if (nj <= 3)                                                             \
+      hipLaunchKernelGGL((norm_gemm_kernel<NT_, 3>), grid, block, 0, s, g);  \
+    else                                                                     \
+      hipLaunchKernelGGL((norm_gemm_kernel<NT_, 4>), grid, block, 0, s, g);  \
+  }
+  T5D_NG_CASE(1) T5D_NG_CASE(2) T5D_NG_CASE(4)
+#undef T5D_NG_CASE
+  T5D_CHECK_LAUNCH("t5d_norm_gemm");
   return T5D_OK;
 }

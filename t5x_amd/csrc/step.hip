@@ -53,11 +53,19 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
   // its limits allow (bfloat16 weights, E <= 512, d <= 1024).
   const bool fuse_cross_q = dt == T5D_BF16 && wd == T5D_BF16 && m->E <= 512 &&
                             d % 64 == 0 && d <= 1024;
+  // Likewise the pre-attention / pre-MLP norms ride inside their dense layers.
+  const bool fuse_norm = dt == T5D_BF16 && wd == T5D_BF16 && d % 64 == 0 &&
+                         d <= 1024;
   for (int l = 0; l < m->NL; ++l) {
     const t5d_layer& w = m->layers[l];
-    T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
-    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
-                     m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
+    if (fuse_norm) {
+      T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, x, w.ln_self, 1e-6f, w.qkv,
+                            m->qkv, R, d, 3 * HD, T5D_EPI_NONE));
+    } else {
+      T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
+      T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
+                       m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
+    }
     if (m->pending_src)
       T5D_TRY(t5d_self_attention_step_gather(
           stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
@@ -86,9 +94,14 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
                      w.cross_out_scales, m->x1, m->x2, R, HD, d,
                      T5D_EPI_RESIDUAL, nullptr, nullptr));
-    T5D_TRY(t5d_rmsnorm(stream, dt, m->x2, w.ln_mlp, m->xn, R, d, 1e-6f));
-    T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.wi, w.wi_scales, nullptr,
-                     m->h, R, d, 2 * F, T5D_EPI_GEGLU, nullptr, nullptr));
+    if (fuse_norm) {
+      T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, m->x2, w.ln_mlp, 1e-6f, w.wi,
+                            m->h, R, d, 2 * F, T5D_EPI_GEGLU));
+    } else {
+      T5D_TRY(t5d_rmsnorm(stream, dt, m->x2, w.ln_mlp, m->xn, R, d, 1e-6f));
+      T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.wi, w.wi_scales, nullptr,
+                       m->h, R, d, 2 * F, T5D_EPI_GEGLU, nullptr, nullptr));
+    }
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->h, w.wo, w.wo_scales, m->x2, m->x,
                      R, F, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
     x = m->x;

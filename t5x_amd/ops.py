@@ -169,8 +169,9 @@ def _default_scratch(device):
 
 
 def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
-         scratch=None):
-  """C = epilogue(a @ W).  a [M, K]; geglu weights give [M, F]."""
+         scratch=None, norm_scale=None, eps=1e-6):
+  """C = epilogue(a @ W).  a [M, K]; geglu weights give [M, F].  With
+  norm_scale [K] the rows of a are RMS-normalised first, in the same kernel."""
   _chk(a, 'a', ndim=2)
   M, K = a.shape
   if K != w.K:
@@ -189,6 +190,14 @@ def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
     if tuple(residual.shape) != (M, n_out):
       raise ValueError('residual shape mismatch')
   dt = _lib.dtype_code(a.dtype)
+  if norm_scale is not None:
+    _chk(norm_scale, 'norm_scale', a.dtype, 1)
+    if norm_scale.numel() != K or residual is not None:
+      raise ValueError('norm_scale must be [K]; no residual with a fused norm')
+    _lib.call('t5d_norm_gemm', _s(), dt, w.w_dtype,
+              _lib.dtype_code(out_dtype), a.data_ptr(), norm_scale.data_ptr(),
+              float(eps), w.data.data_ptr(), out.data_ptr(), M, K, w.N, epi)
+    return out
   ws_bytes = _lib.load().t5d_gemm_workspace_bytes(dt, w.w_dtype, M, K, w.N)
   ws = cnt = None
   if ws_bytes:

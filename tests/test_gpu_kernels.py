@@ -93,6 +93,59 @@ def test_gemm_bf16(ops, M, K, N, epi):
   np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
 
 
+@pytest.mark.parametrize('M,K,N', [(1, 768, 768), (5, 256, 512), (32, 768, 2304),
+                                   (128, 768, 768), (128, 768, 4096),
+                                   (100, 1024, 1024), (128, 64, 48),
+                                   (128, 832, 2304)])
+@pytest.mark.parametrize('mode', ['none', 'geglu', 'f32out'])
+def test_norm_gemm_equals_rmsnorm_then_gemm(ops, M, K, N, mode):
+  """The layer norm fused into the dense kernel against the two-kernel
+  sequence: the normalised operand is rounded to bf16 exactly as the
+  stand-alone kernel rounds it and the product is summed in the same order, so
+  the results agree bit for bit unless the differently ordered sum of squares
+  moves 1/rms by an ulp AND that flips a bf16 rounding; and against the
+  oracle's layer_norm + dense to the dense-layer tolerance."""
+  rs = np.random.RandomState(M + K + N)
+  x = dev(rs.randn(M, K).astype(np.float32) * 3, torch.bfloat16)
+  scale = dev(1 + 0.1 * rs.randn(K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  kw = {}
+  if mode == 'geglu':
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, gate_kernel=dev(w1))
+  else:
+    pw = ops.pack_weight(dev(w0), torch.bfloat16)
+    if mode == 'f32out':
+      kw['out_dtype'] = torch.float32
+  two = ops.gemm(ops.rmsnorm(x, scale), pw, **kw)
+  one = ops.gemm(x, pw, norm_scale=scale, **kw)
+  diff = (one.float() - two.float()).abs()
+  assert float((diff > 0).float().mean()) < 0.02, float((diff > 0).float().mean())
+  assert float(diff.max()) <= 2e-2
+  xn = ot5.layer_norm(host(x), host(scale), 'bfloat16')
+  if mode == 'geglu':
+    want = ot5.mlp_block(
+        {'wi_0': {'kernel': w0}, 'wi_1': {'kernel': w1},
+         'wo': {'kernel': np.eye(N, dtype=np.float32)}}, xn,
+        ('gelu', 'linear'), 'bfloat16')
+  elif mode == 'f32out':
+    want = xn @ ot5.bf16_round(w0)
+  else:
+    want = ot5.dense_general(xn, w0, 'bfloat16')
+  np.testing.assert_allclose(host(one), want, atol=2e-2, rtol=2**-7)
+
+
+def test_norm_gemm_rejects_what_it_does_not_cover(ops):
+  x = dev(np.zeros((4, 64), np.float32))
+  pw = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.float32)
+  with pytest.raises(ValueError, match='bfloat16'):
+    ops.gemm(x, pw, norm_scale=dev(np.ones(64, np.float32)))
+  xb = dev(np.zeros((4, 2048), np.float32), torch.bfloat16)
+  pwb = ops.pack_weight(dev(np.zeros((2048, 32), np.float32)), torch.bfloat16)
+  with pytest.raises(Exception, match='1024'):
+    ops.gemm(xb, pwb, norm_scale=dev(np.ones(2048, np.float32), torch.bfloat16))
+
+
 @pytest.mark.parametrize('M', [8, 128])
 def test_gemm_logits_f32_out(ops, M):
   K, N = 768, 32128
