@@ -17,13 +17,16 @@ void set_error(const char* fmt, ...) {
 
 // ---- embedding gather --------------------------------------------------------
 // One workgroup per row; 16-byte copies.
+// ids == nullptr: the id of row r is seqs[r * S + *cur_index].
 __global__ void embed_kernel(const uint4* __restrict__ table,
                              const int32_t* __restrict__ ids,
                              uint4* __restrict__ out, int vec_per_row, int V,
-                             const int32_t* gate) {
+                             const int32_t* gate,
+                             const int32_t* __restrict__ seqs,
+                             const int32_t* __restrict__ cur_index, int S) {
   T5D_GATED(gate);
   const int r = blockIdx.x;
-  int id = ids[r];
+  int id = ids != nullptr ? ids[r] : seqs[(size_t)r * S + *cur_index];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);
   const uint4* src = table + (size_t)id * vec_per_row;
   uint4* dst = out + (size_t)r * vec_per_row;
@@ -85,8 +88,23 @@ extern "C" int t5d_embed(void* stream, int dtype, const void* table,
               "t5d_embed: row bytes %d not a multiple of 16", d * esz);
   hipLaunchKernelGGL(embed_kernel, dim3(R), dim3(128), 0, as_stream(stream),
                      (const uint4*)table, ids, (uint4*)out, d * esz / 16, V,
-                     tls_gate);
+                     tls_gate, nullptr, nullptr, 0);
   T5D_CHECK_LAUNCH("t5d_embed");
+  return T5D_OK;
+}
+
+int t5d::launch_embed_from_seqs(hipStream_t s, int dtype, const void* table,
+                                const int32_t* seqs, const int32_t* cur_index,
+                                int S, void* out, int R, int d, int V) {
+  T5D_REQUIRE(table && seqs && cur_index && out && R > 0 && S > 0, T5D_EINVAL,
+              "embed(from sequences): null pointer or R=%d S=%d", R, S);
+  const int esz = dtype == T5D_F32 ? 4 : 2;
+  T5D_REQUIRE((d * esz) % 16 == 0, T5D_EINVAL,
+              "embed: row bytes %d not a multiple of 16", d * esz);
+  hipLaunchKernelGGL(embed_kernel, dim3(R), dim3(128), 0, s,
+                     (const uint4*)table, (const int32_t*)nullptr, (uint4*)out,
+                     d * esz / 16, V, tls_gate, seqs, cur_index, S);
+  T5D_CHECK_LAUNCH("embed(from sequences)");
   return T5D_OK;
 }
 

@@ -123,4 +123,29 @@ extern thread_local const int32_t* tls_gate;
 #define T5D_GATE_TEST() \
   if (t5d_gate_open_ == 0) return
 
+// ---- internal launches used by the fused step (not part of the C ABI) -------
+// Embedding rows of the current tokens, read straight from the sequences:
+// ids[r] = seqs[r, *cur_index] (t5d_gather_step_ids + t5d_embed in one kernel).
+int launch_embed_from_seqs(hipStream_t s, int dtype, const void* table,
+                           const int32_t* seqs, const int32_t* cur_index,
+                           int S, void* out, int R, int d, int V);
+// log_softmax + prefix add + per-row top-2K, then one kernel that merges the
+// rows' candidates and does all the beam bookkeeping of the iteration
+// (t5d_beam_topk + t5d_beam_update without the index advance).
+int launch_beam_select(hipStream_t s, const float* logits,
+                       const t5d_beam_state* st, float* topk_vals,
+                       int32_t* topk_idx, float* row_max, float* row_lse,
+                       void* scratch, const int32_t* inputs,
+                       const int32_t* initial_index, const float* brevity,
+                       int32_t* top_alive, int B, int K, int S, int Lin, int V,
+                       int eos_id);
+// End of a beam-search iteration in one single-workgroup kernel: advance
+// *state.cur_index, add 1 to `counters[0..n_counters)` (the layers' cache
+// indices), and, if do_cond, evaluate the loop condition into *keep_going.
+int launch_beam_tail(hipStream_t s, const t5d_beam_state* state, int B, int K,
+                     int S, float min_brevity, float min_log_prob,
+                     int max_decode_step, int min_initial_index,
+                     int32_t* keep_going, int do_cond, int32_t* counters,
+                     int n_counters);
+
 }  // namespace t5d

@@ -392,6 +392,12 @@ struct BeamUpdateArgs {
   int32_t* top_alive_indices;
   int B, K, S, Lin, V, eos_id;
   const int32_t* gate;
+  // optional merge of per-row candidates [B, K, 2K] first (then topk_vals /
+  // topk_idx above are not read; the merged top 2K goes to *_out)
+  const float* cand_vals;
+  const int32_t* cand_idx;
+  float* topk_vals_out;
+  int32_t* topk_idx_out;
 };
 
 // Stable descending order of n values (ties keep index order).
@@ -405,10 +411,14 @@ __device__ __forceinline__ void stable_order_desc(const float* v, int n,
   }
 }
 
-// One workgroup per batch item.  Thread 0 does the (tiny, order-sensitive)
-// scalar bookkeeping into LDS; then every thread owns sequence COLUMNS: for a
-// column it reads the item's K live and K finished entries into registers
-// before writing any, so `cur` and `next` may be the same buffers.
+// One workgroup (one wavefront) per batch item.  Optionally first merges the
+// beams' per-row candidates (cand_* != null) into the item's top 2K.  The
+// order-sensitive bookkeeping is done in parallel, one candidate / pool entry
+// per lane, ranks by counting under the total order (value descending, index
+// ascending), which is what the reference's stable sorts produce.  Then every
+// thread owns sequence COLUMNS: for a column it reads the item's K live and K
+// finished entries into registers before writing any, so `cur` and `next`
+// may be the same buffers.
 __global__ void __launch_bounds__(64)
 beam_update_kernel(BeamUpdateArgs a) {
   __shared__ int s_src_live[kMaxBeams];       // source live beam of new live e
@@ -419,59 +429,105 @@ beam_update_kernel(BeamUpdateArgs a) {
   __shared__ float s_live_lp[kMaxBeams];
   __shared__ float s_fin_score[kMaxBeams];
   __shared__ int s_fin_flag[kMaxBeams];
+  __shared__ float s_mv[128];                 // candidates being merged
+  __shared__ int s_mi[128];
+  __shared__ float s_top_v[2 * kMaxBeams];    // the item's top 2K
+  __shared__ int s_top_i[2 * kMaxBeams];
+  __shared__ float s_new_lp[2 * kMaxBeams], s_lp[2 * kMaxBeams];
+  __shared__ int s_fin[2 * kMaxBeams];
+  __shared__ float s_pool[3 * kMaxBeams];
   T5D_GATED(a.gate);
-  const int b = blockIdx.x;
+  const int b = blockIdx.x, lane = threadIdx.x;
   const int K = a.K, K2 = 2 * a.K, S = a.S;
   const int cur = *a.cur.cur_index;
 
-  if (threadIdx.x == 0) {
-    float lp[2 * kMaxBeams], new_lp[2 * kMaxBeams];
-    float pool[3 * kMaxBeams];
-    int id[2 * kMaxBeams], beam[2 * kMaxBeams];
-    bool fin[2 * kMaxBeams];
-    int order[3 * kMaxBeams];
-    const int col = min(cur + 1, a.Lin - 1);
-    const int nxt = a.inputs[(size_t)b * a.Lin + col];
-    const bool oop = nxt == 0;
-    for (int c = 0; c < K2; ++c) {
-      const float raw = a.topk_vals[(size_t)b * K2 + c];
-      const int fi = a.topk_idx[(size_t)b * K2 + c];
-      beam[c] = fi / a.V;
-      id[c] = oop ? fi % a.V : nxt;
-      lp[c] = oop ? raw : (c == 0 ? 0.f : kNegInf);
-      fin[c] = id[c] == a.eos_id;
-      new_lp[c] = lp[c] + (fin[c] ? kNegInf : 0.f);
-      s_cand_beam[c] = beam[c];
-      s_cand_tok[c] = id[c];
+  if (a.cand_vals != nullptr) {
+    // top 2K of the K rows' 2K candidates each
+    const int n = K * K2;
+    for (int c = lane; c < n; c += 64) {
+      s_mv[c] = a.cand_vals[(size_t)b * n + c];
+      s_mi[c] = a.cand_idx[(size_t)b * n + c];
     }
-    // live beams: top K of the 2K, ascending (lax.top_k then flip)
-    stable_order_desc(new_lp, K2, order);
-    for (int e = 0; e < K; ++e) {
-      const int c = order[K - 1 - e];
-      s_live_lp[e] = new_lp[c];
-      s_src_live[e] = beam[c];
-      s_tok_live[e] = id[c];
+    __syncthreads();
+    for (int c = lane; c < n; c += 64) {
+      const float v = s_mv[c];
+      const int i = s_mi[c];
+      int rank = 0;
+      for (int o = 0; o < n; ++o)
+        if (better(s_mv[o], s_mi[o], v, i)) ++rank;
+      if (rank < K2) {
+        s_top_v[rank] = v;
+        s_top_i[rank] = i;
+        a.topk_vals_out[(size_t)b * K2 + rank] = v;
+        a.topk_idx_out[(size_t)b * K2 + rank] = i;
+      }
     }
-    // finished pool: K old + 2K new, brevity-penalised
-    const int len = a.initial_index[b] + cur + 1;
-    const float bp = a.brevity[len];
-    for (int e = 0; e < K; ++e) pool[e] = a.cur.finished_scores[(size_t)b * K + e];
-    for (int c = 0; c < K2; ++c)
-      pool[K + c] = lp[c] / bp + (fin[c] ? 0.f : kNegInf);
-    stable_order_desc(pool, 3 * K, order);
-    for (int e = 0; e < K; ++e) {
-      const int src = order[K - 1 - e];
-      s_fin_from[e] = src;
-      s_fin_score[e] = pool[src];
-      s_fin_flag[e] = src < K ? a.cur.finished_flags[(size_t)b * K + src]
-                              : (int)fin[src - K];
+  } else if (lane < K2) {
+    s_top_v[lane] = a.topk_vals[(size_t)b * K2 + lane];
+    s_top_i[lane] = a.topk_idx[(size_t)b * K2 + lane];
+  }
+  __syncthreads();
+
+  const int col = min(cur + 1, a.Lin - 1);
+  const int nxt = a.inputs[(size_t)b * a.Lin + col];
+  const bool oop = nxt == 0;
+  if (lane < K2) {
+    const int c = lane;
+    const float raw = s_top_v[c];
+    const int fi = s_top_i[c];
+    const int beam = fi / a.V;
+    const int id = oop ? fi % a.V : nxt;
+    const float lp = oop ? raw : (c == 0 ? 0.f : kNegInf);
+    const bool fin = id == a.eos_id;
+    s_cand_beam[c] = beam;
+    s_cand_tok[c] = id;
+    s_lp[c] = lp;
+    s_fin[c] = fin;
+    s_new_lp[c] = lp + (fin ? kNegInf : 0.f);
+  }
+  const int len = a.initial_index[b] + cur + 1;
+  const float bp = a.brevity[len];
+  __syncthreads();
+  // finished pool: K old + 2K new, brevity-penalised
+  if (lane < 3 * K) {
+    s_pool[lane] = lane < K
+        ? a.cur.finished_scores[(size_t)b * K + lane]
+        : s_lp[lane - K] / bp + (s_fin[lane - K] ? 0.f : kNegInf);
+  }
+  __syncthreads();
+  // live beams: top K of the 2K, ascending (lax.top_k then flip)
+  if (lane < K2) {
+    const float v = s_new_lp[lane];
+    int rank = 0;
+    for (int o = 0; o < K2; ++o)
+      if (better(s_new_lp[o], o, v, lane)) ++rank;
+    if (rank < K) {
+      const int e = K - 1 - rank;
+      s_live_lp[e] = v;
+      s_src_live[e] = s_cand_beam[lane];
+      s_tok_live[e] = s_cand_tok[lane];
     }
-    for (int e = 0; e < K; ++e) {
-      a.next.live_logprobs[(size_t)b * K + e] = s_live_lp[e];
-      a.top_alive_indices[(size_t)b * K + e] = s_src_live[e];
-      a.next.finished_scores[(size_t)b * K + e] = s_fin_score[e];
-      a.next.finished_flags[(size_t)b * K + e] = (uint8_t)s_fin_flag[e];
+  }
+  if (lane < 3 * K) {
+    const float v = s_pool[lane];
+    int rank = 0;
+    for (int o = 0; o < 3 * K; ++o)
+      if (better(s_pool[o], o, v, lane)) ++rank;
+    if (rank < K) {
+      const int e = K - 1 - rank;
+      s_fin_from[e] = lane;
+      s_fin_score[e] = v;
+      s_fin_flag[e] = lane < K ? a.cur.finished_flags[(size_t)b * K + lane]
+                               : s_fin[lane - K];
     }
+  }
+  __syncthreads();
+  if (lane < K) {
+    const int e = lane;
+    a.next.live_logprobs[(size_t)b * K + e] = s_live_lp[e];
+    a.top_alive_indices[(size_t)b * K + e] = s_src_live[e];
+    a.next.finished_scores[(size_t)b * K + e] = s_fin_score[e];
+    a.next.finished_flags[(size_t)b * K + e] = (uint8_t)s_fin_flag[e];
   }
   __syncthreads();
 
@@ -534,10 +590,19 @@ __global__ void gather_ids_kernel(const int32_t* __restrict__ live_seqs,
 __global__ void __launch_bounds__(256)
 beam_cond_kernel(t5d_beam_state st, int B, int K, int S, float min_brevity,
                  float min_log_prob, int max_decode_step, int min_initial_index,
-                 int32_t* keep_going, const int32_t* gate) {
+                 int32_t* keep_going, const int32_t* gate, int advance,
+                 int do_cond, int32_t* counters, int n_counters) {
   __shared__ int iscratch[4];
   T5D_GATED(gate);
-  const int cur = *st.cur_index;
+  // advance: this launch also ends the iteration (cur_index and the layers'
+  // cache indices move on before the condition looks at them).
+  const int cur = *st.cur_index + (advance ? 1 : 0);
+  if (advance) {
+    __syncthreads();  // every thread has read the old value
+    if (threadIdx.x == 0) *st.cur_index = cur;
+    if ((int)threadIdx.x < n_counters) counters[threadIdx.x] += 1;
+  }
+  if (!do_cond) return;
   const float raw_min = min_log_prob / min_brevity;
   int not_terminated = 0, passes_min = 0;
   for (int b = threadIdx.x; b < B; b += 256) {
@@ -824,6 +889,30 @@ extern "C" int t5d_top_k(void* stream, const float* x, float* vals,
   return T5D_OK;
 }
 
+static int launch_row_topk(hipStream_t s, const float* logits,
+                           const float* live_logprobs, float* row_max,
+                           float* row_lse, float* cand_vals, int32_t* cand_idx,
+                           int R, int V, int beams, int k) {
+  if (V % 4 == 0 && V <= kFastTopkVec * 4096 && ((uintptr_t)logits % 16) == 0)
+    hipLaunchKernelGGL(beam_row_topk_fast_kernel, dim3(R), dim3(1024), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k, tls_gate);
+  else if (k <= 4)
+    hipLaunchKernelGGL(beam_row_topk_kernel<4>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k, tls_gate);
+  else if (k <= 8)
+    hipLaunchKernelGGL(beam_row_topk_kernel<8>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k, tls_gate);
+  else
+    hipLaunchKernelGGL(beam_row_topk_kernel<16>, dim3(R), dim3(256), 0, s,
+                       logits, live_logprobs, row_max, row_lse, cand_vals,
+                       cand_idx, V, beams, k, tls_gate);
+  T5D_CHECK_LAUNCH("beam top-k (rows)");
+  return T5D_OK;
+}
+
 extern "C" int t5d_beam_topk(void* stream, const float* logits,
                              const float* live_logprobs, float* topk_vals,
                              int32_t* topk_idx, float* row_max, float* row_lse,
@@ -842,23 +931,9 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
   float* cand_vals = (float*)scratch;
   int32_t* cand_idx = (int32_t*)((char*)scratch + (size_t)R * k * 4);
   hipStream_t s = as_stream(stream);
-  if (V % 4 == 0 && V <= kFastTopkVec * 4096 && ((uintptr_t)logits % 16) == 0)
-    hipLaunchKernelGGL(beam_row_topk_fast_kernel, dim3(R), dim3(1024), 0, s,
-                       logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k, tls_gate);
-  else if (k <= 4)
-    hipLaunchKernelGGL(beam_row_topk_kernel<4>, dim3(R), dim3(256), 0, s,
-                       logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k, tls_gate);
-  else if (k <= 8)
-    hipLaunchKernelGGL(beam_row_topk_kernel<8>, dim3(R), dim3(256), 0, s,
-                       logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k, tls_gate);
-  else
-    hipLaunchKernelGGL(beam_row_topk_kernel<16>, dim3(R), dim3(256), 0, s,
-                       logits, live_logprobs, row_max, row_lse, cand_vals,
-                       cand_idx, V, beams, k, tls_gate);
-  T5D_CHECK_LAUNCH("t5d_beam_topk(rows)");
+  int rc = launch_row_topk(s, logits, live_logprobs, row_max, row_lse, cand_vals,
+                           cand_idx, R, V, beams, k);
+  if (rc) return rc;
   hipLaunchKernelGGL(beam_merge_kernel, dim3(B), dim3(128), 0, s, cand_vals,
                      cand_idx, topk_vals, topk_idx, beams, k, tls_gate);
   T5D_CHECK_LAUNCH("t5d_beam_topk(merge)");
@@ -898,6 +973,8 @@ extern "C" int t5d_beam_update(void* stream, const t5d_beam_state* cur,
   a.top_alive_indices = top_alive_indices;
   a.B = B; a.K = K; a.S = S; a.Lin = Lin; a.V = V; a.eos_id = eos_id;
   a.gate = tls_gate;
+  a.cand_vals = nullptr; a.cand_idx = nullptr;
+  a.topk_vals_out = nullptr; a.topk_idx_out = nullptr;
   hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_beam_update");
@@ -919,8 +996,59 @@ extern "C" int t5d_beam_cond(void* stream, const t5d_beam_state* state, int B,
   hipLaunchKernelGGL(beam_cond_kernel, dim3(1), dim3(256), 0,
                      as_stream(stream), *state, B, K, S, min_brevity,
                      min_log_prob, max_decode_step, min_initial_index,
-                     keep_going, tls_gate);
+                     keep_going, tls_gate, 0, 1, nullptr, 0);
   T5D_CHECK_LAUNCH("t5d_beam_cond");
+  return T5D_OK;
+}
+
+int t5d::launch_beam_select(hipStream_t s, const float* logits,
+                            const t5d_beam_state* st, float* topk_vals,
+                            int32_t* topk_idx, float* row_max, float* row_lse,
+                            void* scratch, const int32_t* inputs,
+                            const int32_t* initial_index, const float* brevity,
+                            int32_t* top_alive, int B, int K, int S, int Lin,
+                            int V, int eos_id) {
+  int rc = check_state("beam select", st);
+  if (rc) return rc;
+  T5D_REQUIRE(K <= kMaxBeams, T5D_ELIMIT, "beam select: K=%d > %d", K,
+              kMaxBeams);
+  const int k = 2 * K, R = B * K;
+  float* cand_vals = (float*)scratch;
+  int32_t* cand_idx = (int32_t*)((char*)scratch + (size_t)R * k * 4);
+  rc = launch_row_topk(s, logits, st->live_logprobs, row_max, row_lse,
+                       cand_vals, cand_idx, R, V, K, k);
+  if (rc) return rc;
+  BeamUpdateArgs a;
+  a.cur = *st; a.next = *st;
+  a.topk_vals = nullptr; a.topk_idx = nullptr; a.inputs = inputs;
+  a.initial_index = initial_index; a.brevity = brevity;
+  a.top_alive_indices = top_alive;
+  a.B = B; a.K = K; a.S = S; a.Lin = Lin; a.V = V; a.eos_id = eos_id;
+  a.gate = tls_gate;
+  a.cand_vals = cand_vals; a.cand_idx = cand_idx;
+  a.topk_vals_out = topk_vals; a.topk_idx_out = topk_idx;
+  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0, s, a);
+  T5D_CHECK_LAUNCH("beam select");
+  return T5D_OK;
+}
+
+int t5d::launch_beam_tail(hipStream_t s, const t5d_beam_state* state, int B,
+                          int K, int S, float min_brevity, float min_log_prob,
+                          int max_decode_step, int min_initial_index,
+                          int32_t* keep_going, int do_cond, int32_t* counters,
+                          int n_counters) {
+  int rc = check_state("beam tail", state);
+  if (rc) return rc;
+  T5D_REQUIRE((keep_going || !do_cond) && B > 0 && K > 0 && S > 1 &&
+                  n_counters >= 0 && n_counters <= 256 &&
+                  (counters || n_counters == 0),
+              T5D_EINVAL, "beam tail: B=%d K=%d S=%d counters=%d", B, K, S,
+              n_counters);
+  hipLaunchKernelGGL(beam_cond_kernel, dim3(1), dim3(256), 0, s, *state, B, K,
+                     S, min_brevity, min_log_prob, max_decode_step,
+                     min_initial_index, keep_going, tls_gate, 1, do_cond,
+                     counters, n_counters);
+  T5D_CHECK_LAUNCH("beam tail");
   return T5D_OK;
 }
 

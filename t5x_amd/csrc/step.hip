@@ -40,14 +40,22 @@ int check_model(const t5d_model_step* m) {
 
 }  // namespace
 
-extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
-                                const int32_t* ids) {
-  T5D_TRY(check_model(m));
-  T5D_REQUIRE(ids, T5D_EINVAL, "t5d_decoder_step: null ids");
+namespace {
+// One decoder step.  ids == nullptr: the current tokens are read from
+// seqs[r, *cur_index] inside the embedding kernel.  bump_index: add 1 to the
+// layers' cache indices at the end (the beam-search step does that in its
+// tail kernel instead).
+int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
+                      const int32_t* seqs, const int32_t* cur_index, int S,
+                      bool bump_index) {
   GateScope gate(m->gate);
   const int dt = m->dtype, wd = m->w_dtype;
   const int R = m->R, d = m->d, HD = m->H * 64, F = m->F;
-  T5D_TRY(t5d_embed(stream, dt, m->embedding, ids, m->x, R, d, m->V));
+  if (ids)
+    T5D_TRY(t5d_embed(stream, dt, m->embedding, ids, m->x, R, d, m->V));
+  else
+    T5D_TRY(launch_embed_from_seqs(as_stream(stream), dt, m->embedding, seqs,
+                                   cur_index, S, m->x, R, d, m->V));
   const void* x = m->x;
   // Layer norm + query projection ride inside the cross-attention kernel when
   // its limits allow (bfloat16 weights, E <= 512, d <= 1024).
@@ -110,8 +118,16 @@ extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
   T5D_TRY(t5d_gemm(stream, dt, wd, T5D_F32, m->xn, m->logits_w,
                    m->logits_scales, nullptr, m->logits, R, d, m->V,
                    T5D_EPI_NONE, nullptr, nullptr));
-  T5D_TRY(t5d_add_i32(stream, m->cache_index, m->NL, 1));
+  if (bump_index) T5D_TRY(t5d_add_i32(stream, m->cache_index, m->NL, 1));
   return T5D_OK;
+}
+}  // namespace
+
+extern "C" int t5d_decoder_step(void* stream, const t5d_model_step* m,
+                                const int32_t* ids) {
+  T5D_TRY(check_model(m));
+  T5D_REQUIRE(ids, T5D_EINVAL, "t5d_decoder_step: null ids");
+  return decoder_step_impl(stream, m, ids, nullptr, nullptr, 0, true);
 }
 
 extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
@@ -126,32 +142,30 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
   T5D_REQUIRE(m->pending_src == nullptr || m->pending_src == b->top_alive,
               T5D_EINVAL,
               "t5d_beam_search_step: pending_src must be the top_alive buffer");
-  const int R = m->R, K = m->beams, B = m->B;
-  {
-    GateScope gate(b->keep_going);
-    T5D_TRY(t5d_gather_step_ids(stream, b->state.live_seqs, b->state.cur_index,
-                                b->ids, R, b->S));
-  }
-  T5D_TRY(t5d_decoder_step(stream, m, b->ids));
+  const int K = m->beams, B = m->B;
+  T5D_TRY(decoder_step_impl(stream, m, nullptr, b->state.live_seqs,
+                            b->state.cur_index, b->S, false));
   GateScope gate(b->keep_going);
-  T5D_TRY(t5d_beam_topk(stream, m->logits, b->state.live_logprobs,
-                        b->topk_vals, b->topk_idx, b->row_max, b->row_lse,
-                        b->scratch, B, K, m->V, 2 * K));
-  T5D_TRY(t5d_beam_update(stream, &b->state, &b->state, b->topk_vals,
-                          b->topk_idx, b->inputs, b->initial_index, b->brevity,
-                          b->top_alive, B, K, b->S, b->Lin, m->V, b->eos_id));
-  // After the update cur_index == number of valid cache columns.  When the
-  // model applies pending gathers inside its self-attention (pending_src ==
-  // top_alive) the reorder happens there, on the next step.
+  hipStream_t hs = as_stream(stream);
+  T5D_TRY(launch_beam_select(hs, m->logits, &b->state, b->topk_vals,
+                             b->topk_idx, b->row_max, b->row_lse, b->scratch,
+                             b->inputs, b->initial_index, b->brevity,
+                             b->top_alive, B, K, b->S, b->Lin, m->V,
+                             b->eos_id));
+  // When the model applies pending gathers inside its self-attention
+  // (pending_src == top_alive) the reorder happens there, on the next step.
+  // Otherwise reorder now: cur_index + 1 columns are valid.
   if (K > 1 && m->pending_src == nullptr)
     T5D_TRY(t5d_cache_gather_beams(
         stream, b->kv_base, b->kv_tensor_stride_bytes, b->n_kv_tensors,
         m->dtype == T5D_F32 ? 4 : 2, B, K, m->H * 64, m->L, b->top_alive,
-        b->state.cur_index, 0));
-  if (!b->skip_cond)
-    T5D_TRY(t5d_beam_cond(stream, &b->state, B, K, b->S, b->min_brevity,
-                          b->min_log_prob, b->max_decode_step,
-                          b->min_initial_index, b->keep_going));
+        b->state.cur_index, 1));
+  // The tail advances cur_index and the cache indices and evaluates the loop
+  // condition.
+  T5D_TRY(launch_beam_tail(hs, &b->state, B, K, b->S, b->min_brevity,
+                           b->min_log_prob, b->max_decode_step,
+                           b->min_initial_index, b->keep_going, !b->skip_cond,
+                           m->cache_index, m->NL));
   return T5D_OK;
 }
 
