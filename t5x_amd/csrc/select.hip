@@ -190,6 +190,19 @@ beam_row_topk_kernel(const float* __restrict__ logits,
 // branch), and wavefront 0 merges the 16 sorted lists the same way.
 constexpr int kFastTopkVec = 8;
 
+// exp(x) for x <= 0 to about 1 ulp with the hardware exp2: the rounding error
+// of x * log2(e) is recovered with an fma and folded back in as a first-order
+// correction.  Anything below -1e30 (padding, -inf logits) gives exactly 0.
+__device__ __forceinline__ float exp_nonpositive(float x) {
+  const float kL2eHi = 1.44269502162933349609375f;    // float(log2(e))
+  const float kL2eLo = 1.92596299112661746e-8f;       // log2(e) - kL2eHi
+  const float hi = x * kL2eHi;
+  const float lo = fmaf(x, kL2eHi, -hi) + x * kL2eLo;
+  const float e = __builtin_amdgcn_exp2f(hi);
+  const float r = fmaf(e, lo * 0.693147180559945309f, e);
+  return x < -1.0e30f ? 0.f : r;
+}
+
 __device__ __forceinline__ void top2_insert(float f, int fi, float& v0, int& i0,
                                             float& v1, int& i1) {
   if (better(f, fi, v1, i1)) {
@@ -243,10 +256,10 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
 #pragma unroll
   for (int u = 0; u < kFastTopkVec; ++u) {
     // exp(-inf) == 0 for the padding
-    sum += (double)expf(x[u].x - m);
-    sum += (double)expf(x[u].y - m);
-    sum += (double)expf(x[u].z - m);
-    sum += (double)expf(x[u].w - m);
+    sum += (double)exp_nonpositive(x[u].x - m);
+    sum += (double)exp_nonpositive(x[u].y - m);
+    sum += (double)exp_nonpositive(x[u].z - m);
+    sum += (double)exp_nonpositive(x[u].w - m);
   }
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
