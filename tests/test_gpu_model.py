@@ -23,6 +23,7 @@ logit tolerance.
 """
 
 import functools
+import types
 
 import numpy as np
 import pytest
@@ -398,3 +399,26 @@ def test_fused_loop_early_stop_is_independent_of_check_interval(check_every,
   assert int(fused.cur.cur_index.item()) == steps
   assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
   assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
+
+
+def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
+  """The reference's host loop (get_infer_fn) around predict_batch_with_aux:
+  5 examples at batch 2 (one pad), float32 so tokens are exact."""
+  from t5x_amd import infer
+  ocfg, om, gm = _models('float32', 'beam_search', alpha=0.6)
+  params = ot5.init_params(ocfg, seed=9)
+  rs = np.random.RandomState(4)
+  enc = ragged_tokens(rs, 5, 12, ocfg.vocab_size, 3)
+  ds = [(np.int64(i), {'encoder_input_tokens': enc[i],
+                       'decoder_input_tokens': np.zeros((8,), np.int32)})
+        for i in range(5)]
+  fn = infer.get_infer_fn(gm.predict_batch_with_aux, 2)
+  got, aux = fn(ds, types.SimpleNamespace(params=params, flax_mutables=None))
+  assert [i for i, _ in got] == list(range(5))
+  assert len(aux['scores']) == 5
+  for i, tokens in got:
+    batch = {'encoder_input_tokens': enc[i:i + 1],
+             'decoder_input_tokens': np.zeros((1, 8), np.int32)}
+    want, waux = om.predict_batch_with_aux(params, batch)
+    np.testing.assert_array_equal(np.asarray(tokens), want[0])
+    np.testing.assert_allclose(aux['scores'][i], waux['scores'][0], atol=1e-4)

@@ -1,0 +1,124 @@
+"""Host loop around predict_batch (t5x/utils.py:1543-1817) against the
+reference's own expectation (t5x/utils_test.py:1024-1110: 8 examples, batch 2,
+with and without flax_mutables -> indices 0..7 and element-wise results in
+dataset order) and the properties the reference code fixes: padding with index
+-1 is dropped, shard interleaving is undone, aux dicts are kept un-flattened,
+the step signature decides whether rng / flax_mutables are passed."""
+
+import types
+
+import numpy as np
+import pytest
+
+from t5x_amd import infer
+
+
+def _dataset(n):
+  col = np.transpose(np.tile(np.arange(n), (2, 1)))  # [n, 2]
+  return [(np.int64(i), {'a': col[i], 'b': col[i]}) for i in range(n)]
+
+
+@pytest.mark.parametrize('use_flax_mutables', [True, False])
+def test_get_infer_fn_predict_reference_vector(use_flax_mutables):
+  batch_size, weight_const = 2, 7
+  mutable_const = 5 if use_flax_mutables else 0
+
+  def predict_batch(params, batch, flax_mutables):
+    result = (flax_mutables['mutable_w'] * batch['b']
+              if use_flax_mutables else 0)
+    return result + params['weight'] * batch['a']
+
+  train_state = types.SimpleNamespace(
+      params={'weight': np.full((1,), weight_const)},
+      flax_mutables=({'mutable_w': np.full((1,), mutable_const)}
+                     if use_flax_mutables else None))
+  layout = types.SimpleNamespace(batch_size=2, shard_id=0, num_shards=1,
+                                 is_first_host_in_replica_set=True)
+  partitioner = types.SimpleNamespace(get_data_layout=lambda bs: layout)
+  infer_fn = infer.get_infer_fn(predict_batch, batch_size, None,
+                                partitioner=partitioner)
+  all_indices, all_inferences = zip(*infer_fn(_dataset(8), train_state))
+  np.testing.assert_equal(all_indices, np.arange(8))
+  np.testing.assert_equal(
+      all_inferences,
+      np.transpose(np.tile(np.arange(8) * (weight_const + mutable_const),
+                           (2, 1))))
+
+
+def test_padding_is_added_and_removed():
+  seen = []
+
+  def step(params, batch):
+    seen.append(batch['a'].shape[0])
+    return batch['a'][:, 0] * 10
+
+  out = infer.get_infer_fn(step, 4)(_dataset(6), {'w': 1})
+  assert seen == [4, 4]               # 6 examples padded to 8
+  assert out == [(i, i * 10) for i in range(6)]
+
+
+def test_more_than_one_data_shard_is_refused():
+  layout = types.SimpleNamespace(shard_id=0, num_shards=2)
+  part = types.SimpleNamespace(get_data_layout=lambda bs: layout)
+  with pytest.raises(NotImplementedError, match='one GPU'):
+    infer.get_infer_fn(lambda p, b: b, 4, None, part)
+
+
+def test_rng_is_split_per_batch_and_passed_by_signature():
+  class Key:
+    def __init__(self, path=()):
+      self.path = path
+    def split(self):
+      return Key(self.path + (0,)), Key(self.path + (1,))
+
+  got = []
+
+  def step(params, batch, rng):
+    got.append(rng.path)
+    return batch['a'][:, 0]
+
+  infer.get_infer_fn(step, 2)(_dataset(6), None, rng=Key())
+  # step_rng, rng = split(rng): first child goes to the step, second carries on
+  assert got == [(0,), (1, 0), (1, 1, 0)]
+
+
+def test_rng_none_is_passed_as_none():
+  got = []
+
+  def step(params, batch, rng):
+    got.append(rng)
+    return batch['a'][:, 0]
+
+  infer.get_infer_fn(step, 2)(_dataset(4), None)
+  assert got == [None, None]
+
+
+@pytest.mark.parametrize('keep_numpy', [False, True])
+def test_aux_values_stay_a_dict_of_sequences(keep_numpy):
+  def step(params, batch):
+    a = batch['a'][:, 0]
+    return np.stack([a, a + 1], axis=1), {'scores': a * 0.5}
+
+  out, aux = infer.get_infer_fn(step, 3, keep_aux_as_numpy=keep_numpy)(
+      _dataset(5), None)
+  assert out == [(i, [i, i + 1]) for i in range(5)]
+  assert list(aux) == ['scores'] and len(aux['scores']) == 5
+  np.testing.assert_allclose(np.asarray(aux['scores']), np.arange(5) * 0.5)
+  if keep_numpy:
+    assert isinstance(aux["scores"][0], (np.ndarray, np.generic))
+  else:
+    assert isinstance(aux['scores'][0], float)
+
+
+def test_structured_inferences_keep_their_structure_per_example():
+  def step(params, batch):
+    a = batch['a'][:, 0]
+    return {'x': a, 'y': (a * 2, a * 3)}
+
+  out = infer.get_infer_fn(step, 2)(_dataset(4), None)
+  assert out[3] == (3, {'x': 3, 'y': (6, 9)})
+
+
+def test_unsized_dataset_raises_like_the_reference():
+  with pytest.raises(TypeError, match='dataset length is unknown.'):
+    infer.get_infer_fn(lambda p, b: b, 2)(iter(_dataset(4)), None)
