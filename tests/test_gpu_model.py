@@ -422,3 +422,32 @@ def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
     want, waux = om.predict_batch_with_aux(params, batch)
     np.testing.assert_array_equal(np.asarray(tokens), want[0])
     np.testing.assert_allclose(aux['scores'][i], waux['scores'][0], atol=1e-4)
+
+
+@pytest.mark.parametrize('decode_fn_name,kw', [
+    ('beam_search', dict(alpha=0.6)),
+    ('temperature_sample', dict(temperature=0.0))])
+def test_predict_batch_with_decoder_prompts_float32_exact(decode_fn_name, kw):
+  """prompt_with_targets=True: the decoder inputs (minus EOS) are forced as a
+  prefix (t5x/models.py:623-634, decoding.py:1374-1397 / :596-606); ragged
+  prompt lengths, float32 so the continuation must match token for token."""
+  ocfg, om, gm = _models('float32', decode_fn_name, **kw)
+  params = ot5.init_params(ocfg, seed=21)
+  rs = np.random.RandomState(6)
+  dec = np.zeros((4, 12), np.int32)
+  for i, n in enumerate((0, 3, 5, 1)):       # shifted-right targets: 0 first
+    dec[i, 1:1 + n] = rs.randint(2, ocfg.vocab_size, size=n)
+  batch = {'encoder_input_tokens': ragged_tokens(rs, 4, 14, ocfg.vocab_size, 3),
+           'decoder_input_tokens': dec}
+  extra = dict(num_decodes=3, return_all_decodes=True) if (
+      decode_fn_name == 'beam_search') else {}
+  want, waux = om.predict_batch_with_aux(params, batch,
+                                         prompt_with_targets=True, **extra)
+  got, gaux = gm.predict_batch_with_aux(params, batch,
+                                        prompt_with_targets=True, **extra)
+  np.testing.assert_array_equal(host(got), want)
+  np.testing.assert_allclose(host(gaux['scores']), waux['scores'], atol=1e-4)
+  # the forced prefix is reproduced in every returned decode
+  flat = host(got).reshape(4, -1, 12)
+  for i, n in enumerate((0, 3, 5, 1)):
+    assert (flat[i, :, :n] == dec[i, 1:1 + n]).all()
