@@ -48,6 +48,13 @@ enum {
   T5D_EPI_GEGLU = 2      /* C[:, f] = act(act(gelu(act(a0))) * act(a1)) */
 };
 
+/* Output layouts of t5d_gemm_rows. */
+enum {
+  T5D_OUT_ROWS = 0,        /* row-major [M, N] */
+  T5D_OUT_HEADS_KEY = 1,   /* [B, H, Ep, 64]: cross-attention keys */
+  T5D_OUT_HEADS_VALUE = 2  /* [B, H, 64, Ep]: cross-attention values */
+};
+
 int t5d_version(void);
 const char* t5d_last_error(void);
 
@@ -105,6 +112,20 @@ int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
 int t5d_norm_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
                   const void* A, const void* norm_scale, float eps,
                   const void* W, void* C, int M, int K, int N, int epilogue);
+
+/* Bias-free dense layer over any number of rows (the encoder's DenseGeneral /
+ * MlpBlock layers, t5x/examples/t5/layers.py:364-414,434-487, residual adds of
+ * network.py:73,87, and the once-per-batch key / value projections of the
+ * decoder's cross-attention, network.py:149-159).  bfloat16 activations;
+ * W packed by t5d_pack_weight (bfloat16 or int8 + scales); epilogues as
+ * t5d_gemm.  out_layout T5D_OUT_HEADS_*: row m = b * E + e, column
+ * n = h * 64 + d is written to [B, H, Ep, 64] / [B, H, 64, Ep] (what
+ * t5d_cross_attention_step reads); rows e >= E of those buffers are left
+ * untouched. */
+int t5d_gemm_rows(void* stream, int w_dtype, const void* A, const void* W,
+                  const float* scales, const void* residual, void* C,
+                  int64_t M, int K, int N, int epilogue, int out_layout, int E,
+                  int Ep);
 
 /* One step of cached decoder self-attention
  * (MultiHeadDotProductAttention decode branch,
@@ -164,6 +185,21 @@ int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
                                     const void* cross_value,
                                     const int32_t* enc_len, void* out, int B,
                                     int beams, int H, int E, int d);
+
+/* Encoder self-attention over whole sequences, bfloat16
+ * (MultiHeadDotProductAttention without cache, t5x/examples/t5/layers.py:
+ * 137-221,305-346, dot_product_attention :52-129, with the encoder's
+ * bidirectional relative-position bias and padding mask,
+ * t5x/examples/t5/network.py:47-96,325-328).
+ *   q, k [B*E, *_stride]: head h in columns h*64 .. h*64+63 (row-major
+ *   projections); v_t [B, H, 64, Ep] (t5d_gemm_rows, T5D_OUT_HEADS_VALUE);
+ *   rel_bias [H, 2E-1] bfloat16 indexed by (key - query + E - 1);
+ *   enc_len [B]: keys and queries at positions >= enc_len[b] are padding
+ *   (masked with -1e10 as in the reference); out [B*E, H*64]. */
+int t5d_encoder_attention(void* stream, const void* q, const void* k,
+                          const void* v_t, const void* rel_bias,
+                          const int32_t* enc_len, void* out, int B, int H,
+                          int E, int Ep, int q_stride, int k_stride);
 
 /* Add `delta` to n int32 values (cache_index += 1, layers.py:275). */
 int t5d_add_i32(void* stream, int32_t* x, int n, int delta);

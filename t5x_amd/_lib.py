@@ -12,6 +12,7 @@ from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int32,
 
 F32, BF16, I8 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_GEGLU = 0, 1, 2
+OUT_ROWS, OUT_HEADS_KEY, OUT_HEADS_VALUE = 0, 1, 2
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, 'csrc', 'libt5d.so')
@@ -75,6 +76,10 @@ _SIGNATURES = {
     't5d_gemm_workspace_bytes': (c_int64, [c_int] * 5),
     't5d_gemm': (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
                          c_int, c_int, c_int, _P, _P]),
+    't5d_encoder_attention': (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int,
+                                      c_int, c_int, c_int, c_int, c_int]),
+    't5d_gemm_rows': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int,
+                              c_int, c_int, c_int, c_int, c_int]),
     't5d_norm_gemm': (c_int, [_P, c_int, c_int, c_int, _P, _P, c_float, _P, _P,
                               c_int, c_int, c_int, c_int]),
     't5d_self_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P,

@@ -1,0 +1,190 @@
+// Encoder self-attention over whole sequences (bfloat16), once per batch:
+// out = softmax(Q K^T + relative-position bias + padding mask) V per
+// (batch item, head), t5x/examples/t5/layers.py:52-129 with the encoder's
+// bidirectional bias (layers.py:560-677) and mask (network.py:325-328).
+//
+// A workgroup takes 64 queries of one (item, head), a wavefront 16 of them.
+// Two passes over the keys, 16 at a time, both on the matrix cores:
+//   pass 1: S^T = K Q^T (keys as MFMA rows, so a lane ends up with 4
+//           consecutive keys of ONE query), scores rounded where the reference
+//           rounds them, running max / sum per lane, combined at the end;
+//   pass 2: S^T again, P = bf16(exp(s - max) / sum) written 4 keys at a time
+//           into a small LDS tile, read back as the B operand of
+//           out^T = V^T P^T, 32 keys per step.  V is given transposed
+//           ([B, H, 64, Ep], what t5d_gemm_rows' value layout writes), so its
+//           fragments are contiguous 16-byte loads.
+// Masked keys get the reference's -1e10 (so a padded query attends uniformly,
+// as it does there); keys beyond E do not exist and get -inf.
+#include <math.h>
+
+#include "common.h"
+
+namespace t5d {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_e;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_e;
+
+union FragE {
+  uint4 u;
+  bf16x8_e v;
+};
+
+struct EncAttnArgs {
+  const bf16_t* q;    // [B*E, q_stride]: head h at columns h*64 .. +64
+  const bf16_t* k;    // same layout as q
+  const bf16_t* vt;   // [B, H, 64, Ep]
+  const bf16_t* bias; // [H, 2E-1]: by (key - query + E - 1)
+  const int32_t* len; // [B] valid prefix length
+  bf16_t* out;        // [B*E, H*64]
+  int H, E, Ep, q_stride, k_stride;
+};
+
+__global__ void __launch_bounds__(256)
+enc_attn_kernel(EncAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t s_p[4][16][32];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, gq = lane >> 4;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int q0 = blockIdx.x * 64 + wave * 16;
+  if (q0 >= a.E) return;
+  const int E = a.E;
+  int n = a.len[b];
+  n = n < 0 ? 0 : (n > E ? E : n);
+  const float kMasked = -9.9857e9f;  // bf16(-1e10), layers.py:309-311
+  const size_t row0 = (size_t)b * E;
+
+  // B operand of S^T: lane (col = query l16, g) holds Q[q][32c + 8g .. +8]
+  const int qi = min(q0 + l16, E - 1);
+  FragE qb[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+    qb[c].u = *reinterpret_cast<const uint4*>(
+        a.q + (row0 + qi) * a.q_stride + h * 64 + 32 * c + 8 * gq);
+  const bool q_valid = (q0 + l16) < n;
+  const bf16_t* bias_row = a.bias + (size_t)h * (2 * E - 1) + (E - 1) - qi;
+
+  // scores of key tile kt for this lane: keys 16 kt + 4 g + i of query l16
+  auto score_tile = [&](int kt, float (&s)[4]) {
+    const int key_row = min(16 * kt + l16, E - 1);
+    f32x4_e acc = (f32x4_e){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      FragE ka;
+      ka.u = *reinterpret_cast<const uint4*>(
+          a.k + (row0 + key_row) * a.k_stride + h * 64 + 32 * c + 8 * gq);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qb[c].v, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = 16 * kt + 4 * gq + i;
+      float x = round_bf16(acc[i]);
+      if (key < E) {
+        const bool ok = q_valid && key < n;
+        x = ok ? round_bf16(x + bf16_to_f32(bias_row[key])) : kMasked;
+      } else {
+        x = -INFINITY;
+      }
+      s[i] = x;
+    }
+  };
+
+  const int n_tiles = (E + 15) >> 4;
+  float m = -INFINITY, l = 0.f;
+  for (int kt = 0; kt < n_tiles; ++kt) {
+    float s[4];
+    score_tile(kt, s);
+    const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    const float nm = fmaxf(m, tm);
+    float add = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) add += __expf(s[i] - nm);
+    l = l * __expf(m - nm) + add;  // exp(-inf - finite) == 0 on the first tile
+    m = nm;
+  }
+  // combine the 4 lanes (g) that share a query
+#pragma unroll
+  for (int o = 16; o <= 32; o <<= 1) {
+    const float om = __shfl_xor(m, o, 64), ol = __shfl_xor(l, o, 64);
+    const float nm = fmaxf(m, om);
+    l = l * __expf(m - nm) + ol * __expf(om - nm);
+    m = nm;
+  }
+  const float inv = 1.0f / l;
+
+  f32x4_e oc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_e){0.f, 0.f, 0.f, 0.f};
+  const bf16_t* vbase = a.vt + ((size_t)b * a.H + h) * 64 * (size_t)a.Ep;
+  for (int kb = 0; kb < n_tiles; kb += 2) {  // 32 keys per step
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float s[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (kb + t < n_tiles) score_tile(kb + t, s);
+      uint2 pk;
+      pk.x = pack_bf16x2(__expf(s[0] - m) * inv, __expf(s[1] - m) * inv);
+      pk.y = pack_bf16x2(__expf(s[2] - m) * inv, __expf(s[3] - m) * inv);
+      *reinterpret_cast<uint2*>(&s_p[wave][l16][16 * t + 4 * gq]) = pk;
+    }
+    // LDS traffic stays inside the wavefront: its own writes are visible to it
+    // once they have completed.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    FragE pb;  // B: lane (col = query l16, g) holds P[q][8g .. +8] of the 32
+    pb.u = *reinterpret_cast<const uint4*>(&s_p[wave][l16][8 * gq]);
+    const int key0 = min(16 * kb + 8 * gq, a.Ep - 8);
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      FragE va;  // A: lane (row = d l16, g) holds V^T[16 dt + l16][key0 .. +8]
+      va.u = *reinterpret_cast<const uint4*>(
+          vbase + (size_t)(16 * dt + l16) * a.Ep + key0);
+      oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, oc[dt], 0, 0,
+                                                       0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // oc[dt][i]: out[q = l16][d = 16 dt + 4 g + i]
+  if (q0 + l16 < E) {
+    bf16_t* o = a.out + (row0 + q0 + l16) * (size_t)(a.H * 64) + h * 64 + 4 * gq;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      uint2 pk;
+      pk.x = pack_bf16x2(oc[dt][0], oc[dt][1]);
+      pk.y = pack_bf16x2(oc[dt][2], oc[dt][3]);
+      *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
+    }
+  }
+}
+
+}  // namespace t5d
+
+using namespace t5d;
+
+extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
+                                     const void* v_t, const void* rel_bias,
+                                     const int32_t* enc_len, void* out, int B,
+                                     int H, int E, int Ep, int q_stride,
+                                     int k_stride) {
+  T5D_REQUIRE(q && k && v_t && rel_bias && enc_len && out, T5D_EINVAL,
+              "t5d_encoder_attention: null pointer");
+  T5D_REQUIRE(B > 0 && H > 0 && E > 0 && Ep >= E && Ep % 8 == 0 && Ep >= 8,
+              T5D_EINVAL, "t5d_encoder_attention: B=%d H=%d E=%d Ep=%d", B, H,
+              E, Ep);
+  T5D_REQUIRE(q_stride >= H * 64 && k_stride >= H * 64 && q_stride % 8 == 0 &&
+                  k_stride % 8 == 0,
+              T5D_EINVAL, "t5d_encoder_attention: row strides %d / %d", q_stride,
+              k_stride);
+  T5D_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 &&
+                  ((uintptr_t)v_t % 16) == 0 && ((uintptr_t)out % 8) == 0,
+              T5D_EINVAL, "t5d_encoder_attention: operand alignment");
+  T5D_REQUIRE(H <= 65535 && B <= 65535, T5D_ELIMIT,
+              "t5d_encoder_attention: H=%d B=%d beyond the launch grid", H, B);
+  EncAttnArgs a;
+  a.q = (const bf16_t*)q; a.k = (const bf16_t*)k; a.vt = (const bf16_t*)v_t;
+  a.bias = (const bf16_t*)rel_bias; a.len = enc_len; a.out = (bf16_t*)out;
+  a.H = H; a.E = E; a.Ep = Ep; a.q_stride = q_stride; a.k_stride = k_stride;
+  dim3 grid((E + 63) / 64, H, B), block(256);
+  hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
+  T5D_CHECK_LAUNCH("t5d_encoder_attention");
+  return T5D_OK;
+}

@@ -1,10 +1,13 @@
 """T5.1.1 encoder forward (t5x/examples/t5/network.py:47-96,182-219,315-343),
 run once per batch before the decode loop.
 
-This is not part of the per-step hot path: it is compute-bound full-sequence
-work and uses library GEMMs and softmax through torch, with the reference's
-rounding points (every op result in the activation dtype, float32
-accumulation).  The decode step never calls into this module.
+bfloat16: hand-written HIP kernels — the many-row dense kernel
+(t5d_gemm_rows: fused residual / gated-GELU epilogues, value projection written
+transposed), whole-sequence self-attention on the matrix cores
+(t5d_encoder_attention), the embedding gather and the RMS norm of the decode
+path.  float32 (the exactness-test dtype): library GEMMs and softmax through
+torch with the reference's rounding points.  The decode step never calls into
+this module.
 """
 
 import numpy as np
@@ -60,17 +63,94 @@ def _rms(x, scale, eps=1e-6):
   return y * scale
 
 
+class EncoderKernelWeights:
+  """Encoder parameters packed for the HIP kernels (bfloat16 activations)."""
+
+  def __init__(self, cfg, params, device):
+    from t5x_amd import ops
+    act = torch.bfloat16
+    wdt = network._TORCH_DTYPE[cfg.weight_dtype or cfg.dtype]
+    enc = params['encoder']
+    f = lambda x: network._f32(x, device)
+    self.embedding = f(params['token_embedder']['embedding']).to(act).contiguous()
+    self.rel_embedding = f(enc['relpos_bias']['rel_embedding']).to(act)
+    self.layers = []
+    for i in range(cfg.num_encoder_layers):
+      p = enc[f'layers_{i}']
+      a, m = p['attention'], p['mlp']
+      qk = torch.cat([f(a['query']['kernel']), f(a['key']['kernel'])],
+                     dim=1).contiguous()
+      self.layers.append(dict(
+          ln_attn=f(p['pre_attention_layer_norm']['scale']).to(act),
+          qk=ops.pack_weight(qk, act, wdt),
+          v=ops.pack_weight(f(a['value']['kernel']), act, wdt),
+          o=ops.pack_weight(f(a['out']['kernel']), act, wdt),
+          ln_mlp=f(p['pre_mlp_layer_norm']['scale']).to(act),
+          wi=ops.pack_weight(f(m['wi_0']['kernel']), act, wdt,
+                             gate_kernel=f(m['wi_1']['kernel'])),
+          wo=ops.pack_weight(f(m['wo']['kernel']), act, wdt)))
+    self.ln_final = f(enc['encoder_norm']['scale']).to(act)
+    self._bias = {}
+
+  def rel_bias(self, E):
+    """[H, 2E-1] bias by (key - query + E - 1), bidirectional buckets."""
+    if E not in self._bias:
+      bucket = network.relative_position_bucket(np.arange(-(E - 1), E),
+                                                bidirectional=True)
+      idx = torch.as_tensor(bucket.astype(np.int64),
+                            device=self.rel_embedding.device)
+      self._bias[E] = self.rel_embedding[:, idx].contiguous()
+    return self._bias[E]
+
+
+def _encode_hip(module, params, tokens):
+  """bfloat16 encoder on the HIP kernels; tokens [B, E] int64 on the device."""
+  from t5x_amd import _lib, ops
+  cfg, dev = module.config, module._dev()
+  key = ('hip', id(params))
+  if key not in module._enc_weights:
+    module._enc_weights[key] = (params, EncoderKernelWeights(cfg, params, dev))
+  w = module._enc_weights[key][1]
+  B, E = tokens.shape
+  H = cfg.num_heads
+  HD = H * 64
+  valid = tokens > 0
+  lens = valid.sum(dim=1).to(torch.int32)
+  prefix = torch.arange(E, device=dev)[None, :] < lens[:, None]
+  if not bool((prefix == valid).all()):
+    raise ValueError('encoder padding must be a suffix of zeros')
+  lens = lens.contiguous()
+  Ep = (E + 7) // 8 * 8
+  bias = w.rel_bias(E)
+  ids = tokens.reshape(-1).to(torch.int32).contiguous()
+  x = ops.embed(w.embedding, ids)
+  M = B * E
+  v_t = torch.zeros((B, H, 64, Ep), dtype=x.dtype, device=dev)
+  for l in w.layers:
+    xn = ops.rmsnorm(x, l['ln_attn'])
+    qk = ops.gemm_rows(xn, l['qk'])                       # [M, q | k]
+    ops.gemm_rows(xn, l['v'], out=v_t, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep)
+    attn = ops.encoder_attention(qk[:, :HD], qk[:, HD:], v_t, bias, lens)
+    x = ops.gemm_rows(attn, l['o'], residual=x)
+    y = ops.rmsnorm(x, l['ln_mlp'])
+    h = ops.gemm_rows(y, l['wi'])
+    x = ops.gemm_rows(h, l['wo'], residual=x)
+  return ops.rmsnorm(x, w.ln_final).view(B, E, cfg.emb_dim)
+
+
 def encode(module, params, encoder_input_tokens):
   cfg, dev = module.config, module._dev()
-  key = id(params)
-  if key not in module._enc_weights:
-    module._enc_weights[key] = (params, EncoderWeights(cfg, params, dev))
-  w = module._enc_weights[key][1]
   tokens = encoder_input_tokens
   if not isinstance(tokens, torch.Tensor):
     tokens = torch.as_tensor(np.asarray(tokens), device=dev)
   tokens = tokens.to(dev).long()
   B, E = tokens.shape
+  if cfg.dtype == 'bfloat16' and E % 4 == 0:
+    return _encode_hip(module, params, tokens)
+  key = id(params)
+  if key not in module._enc_weights:
+    module._enc_weights[key] = (params, EncoderWeights(cfg, params, dev))
+  w = module._enc_weights[key][1]
   H, D = cfg.num_heads, cfg.head_dim
   act = w.embedding.dtype
   bucket = network.relative_position_bucket(

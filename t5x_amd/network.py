@@ -155,11 +155,17 @@ class DecoderWeights:
           wi=ops.pack_weight(g(n, mlp, 'wi_0', 'kernel'), act, wdt,
                              gate_kernel=g(n, mlp, 'wi_1', 'kernel')),
           wo=ops.pack_weight(g(n, mlp, 'wo', 'kernel'), act, wdt),
-          # once-per-batch cross K/V projection (library GEMM)
+          # once-per-batch cross K/V projection: packed for t5d_gemm_rows
+          # (bfloat16 activations), library layout for the float32 path
           cross_k=self._dense_for_library(g(n, ca, 'key', 'kernel'), act, wdt),
           cross_v=self._dense_for_library(g(n, ca, 'value', 'kernel'), act,
                                           wdt),
       )
+      if act == torch.bfloat16:
+        layer['cross_k_packed'] = ops.pack_weight(g(n, ca, 'key', 'kernel'),
+                                                  act, wdt)
+        layer['cross_v_packed'] = ops.pack_weight(g(n, ca, 'value', 'kernel'),
+                                                  act, wdt)
       self.layers.append(layer)
     self.ln_final = g('decoder_norm', 'scale').to(act)
     # Logits layer: float32 in the reference; bf16 configs stream it as bf16
@@ -321,9 +327,19 @@ class Transformer:
     H, D = cfg.num_heads, cfg.head_dim
     el = 16 // encoded.element_size()
     Ep = (E + el - 1) // el * el  # rows padded to 16-byte multiples
-    x = encoded.reshape(B * E, d)
+    x = encoded.reshape(B * E, d).contiguous()
     ks, vs = [], []
+    hip = x.dtype == torch.bfloat16 and E % 4 == 0
     for l in w.layers:
+      if hip:
+        # [B, H, Ep, 64] keys and [B, H, 64, Ep] values straight from the
+        # dense kernel's epilogue; the padding rows e >= E stay zero
+        from t5x_amd import _lib
+        ks.append(ops.gemm_rows(x, l['cross_k_packed'],
+                                layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep))
+        vs.append(ops.gemm_rows(x, l['cross_v_packed'],
+                                layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep))
+        continue
       for (kern, scale), dst in ((l['cross_k'], ks), (l['cross_v'], vs)):
         y = torch.matmul(x, kern)  # float32 accumulate, one rounding
         if scale is not None:

@@ -306,6 +306,63 @@ def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
   return out
 
 
+def gemm_rows(a, w: PackedWeight, out=None, residual=None,
+              layout=_lib.OUT_ROWS, E=0, Ep=0):
+  """Dense layer over any number of rows (bfloat16).  layout OUT_HEADS_KEY /
+  OUT_HEADS_VALUE writes [B, H, Ep, 64] / [B, H, 64, Ep] (rows m = b*E + e)."""
+  _chk(a, 'a', torch.bfloat16, 2)
+  M, K = a.shape
+  if K != w.K or w.w_dtype == F32:
+    raise ValueError(f'a is [{M}, {K}]; kernel K={w.K}, packed weights only')
+  epi = EPI_GEGLU if w.geglu else (EPI_RESIDUAL if residual is not None
+                                   else EPI_NONE)
+  if layout == _lib.OUT_ROWS:
+    if out is None:
+      out = torch.empty((M, w.out_features), dtype=a.dtype, device=a.device)
+    if tuple(out.shape) != (M, w.out_features):
+      raise ValueError(f'out shape {tuple(out.shape)}')
+  else:
+    B, H = M // max(E, 1), w.N // 64
+    want = (B, H, Ep, 64) if layout == _lib.OUT_HEADS_KEY else (B, H, 64, Ep)
+    if out is None:
+      out = torch.zeros(want, dtype=a.dtype, device=a.device)
+    if tuple(out.shape) != want:
+      raise ValueError(f'out shape {tuple(out.shape)} != {want}')
+  _chk(out, 'out', a.dtype)
+  if residual is not None:
+    _chk(residual, 'residual', a.dtype, 2)
+    if tuple(residual.shape) != (M, w.N):
+      raise ValueError('residual shape mismatch')
+  _lib.call('t5d_gemm_rows', _s(), w.w_dtype, a.data_ptr(), w.data.data_ptr(),
+            _lib.ptr(w.scales), _lib.ptr(residual), out.data_ptr(), M, K, w.N,
+            epi, int(layout), int(E), int(Ep))
+  return out
+
+
+def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
+  """q, k: [B*E, >= H*64] row-major views (row stride = stride(0)); v_t
+  [B, H, 64, Ep]; rel_bias [H, 2E-1]; enc_len [B] -> out [B*E, H*64]."""
+  _chk(v_t, 'v_t', torch.bfloat16, 4)
+  _chk(rel_bias, 'rel_bias', torch.bfloat16, 2)
+  _chk(enc_len, 'enc_len', torch.int32, 1)
+  B, H, D, Ep = v_t.shape
+  E = (rel_bias.shape[1] + 1) // 2
+  for name, t in (('q', q), ('k', k)):
+    if (not t.is_cuda or t.dtype != torch.bfloat16 or t.dim() != 2 or
+        t.stride(1) != 1 or t.shape[0] != B * E or t.shape[1] != H * 64):
+      raise ValueError(f'{name} must be a [B*E, H*64] bfloat16 view with unit '
+                       f'column stride, got {tuple(t.shape)}')
+  if D != 64 or rel_bias.shape[0] != H or enc_len.shape[0] != B:
+    raise ValueError('v_t [B, H, 64, Ep], rel_bias [H, 2E-1], enc_len [B]')
+  if out is None:
+    out = torch.empty((B * E, H * 64), dtype=torch.bfloat16, device=v_t.device)
+  _chk(out, 'out', torch.bfloat16, 2)
+  _lib.call('t5d_encoder_attention', _s(), q.data_ptr(), k.data_ptr(),
+            v_t.data_ptr(), rel_bias.data_ptr(), enc_len.data_ptr(),
+            out.data_ptr(), B, H, E, Ep, q.stride(0), k.stride(0))
+  return out
+
+
 def add_i32(x, delta):
   _chk(x, 'x', torch.int32)
   _lib.call('t5d_add_i32', _s(), x.data_ptr(), x.numel(), int(delta))

@@ -1,0 +1,182 @@
+"""Encoder-side kernels (once per batch): large-row dense layers and
+whole-sequence self-attention, against the oracle; then the whole encoder and
+the cross-attention K/V projection."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import t5 as ot5
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def ops():
+  from t5x_amd import ops as _ops
+  return _ops
+
+
+def dev(x, dtype=None):
+  t = torch.as_tensor(np.asarray(x), device='cuda')
+  return t.to(dtype) if dtype is not None else t
+
+
+def host(t):
+  return (t.detach().float() if t.is_floating_point() else t.detach()).cpu().numpy()
+
+
+@pytest.mark.parametrize('M,K,N', [(128, 64, 128), (1000, 768, 768),
+                                   (257, 256, 2304), (4096, 768, 4096),
+                                   (50, 2048, 80), (16384, 768, 768)])
+@pytest.mark.parametrize('mode', ['none', 'residual', 'geglu', 'int8',
+                                  'int8_geglu'])
+def test_gemm_rows(ops, M, K, N, mode):
+  rs = np.random.RandomState(M + K + N)
+  if M * N > 4e7 and mode != 'none':
+    pytest.skip('largest shape once')
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  wd = torch.int8 if mode.startswith('int8') else torch.bfloat16
+  q0 = ot5.quantize_int8(w0) if wd == torch.int8 else w0
+  if mode.endswith('geglu'):
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    q1 = ot5.quantize_int8(w1) if wd == torch.int8 else w1
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, wd, gate_kernel=dev(w1))
+    out = ops.gemm_rows(a, pw)
+    want = ot5.mlp_block({'wi_0': {'kernel': q0}, 'wi_1': {'kernel': q1},
+                          'wo': {'kernel': np.eye(N, dtype=np.float32)}},
+                         host(a), ('gelu', 'linear'), 'bfloat16')
+  else:
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, wd)
+    res = None
+    want = ot5.dense_general(host(a), q0, 'bfloat16')
+    if mode == 'residual':
+      res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+      want = ot5.bf16_round(want + host(res))
+    out = ops.gemm_rows(a, pw, residual=res)
+  assert out.shape == want.shape
+  np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
+  if M <= 128 and not mode.startswith('int8'):
+    # same weights, same rounding points as the decode-step kernel
+    small = ops.gemm(a, pw, residual=None if mode != 'residual' else res)
+    np.testing.assert_allclose(host(out), host(small), atol=2e-2, rtol=2**-7)
+
+
+@pytest.mark.parametrize('B,E,Ep,H,d', [(2, 16, 16, 1, 64), (3, 40, 40, 2, 128),
+                                        (2, 100, 104, 3, 256),
+                                        (4, 512, 512, 12, 768)])
+def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
+  """Key layout [B, H, Ep, 64] and value layout [B, H, 64, Ep] hold exactly the
+  row-major result, re-arranged; padding rows stay untouched (zero)."""
+  rs = np.random.RandomState(B + E + H)
+  x = dev(rs.randn(B * E, d).astype(np.float32), torch.bfloat16)
+  w = dev((rs.randn(d, H * 64) / np.sqrt(d)).astype(np.float32))
+  from t5x_amd import _lib
+  pw = ops.pack_weight(w, torch.bfloat16)
+  rows = ops.gemm_rows(x, pw).view(B, E, H, 64)
+  keys = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep)
+  vals = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep)
+  assert torch.equal(keys[:, :, :E], rows.permute(0, 2, 1, 3))
+  assert torch.equal(vals[..., :E], rows.permute(0, 2, 3, 1))
+  assert not keys[:, :, E:].any() and not vals[..., E:].any()
+
+
+def _enc_attn_oracle(q, k, v, rel_emb, lens):
+  B, E, H, D = q.shape
+  tokens = (np.arange(E)[None, :] < lens[:, None])
+  mask = ot5.make_attention_mask(tokens, tokens)
+  bias = ot5.relpos_bias(rel_emb, E, E, True, 'bfloat16')
+  total = ot5.combine_biases(
+      np.where(mask > 0, 0.0, -1e10).astype(np.float32), bias) if hasattr(
+          ot5, 'combine_biases') else None
+  if total is None:
+    total = ot5.bf16_round(np.where(mask > 0, 0.0, -1e10).astype(np.float32) +
+                           bias)
+  return ot5.dot_product_attention(q, k, v, total, 'bfloat16')
+
+
+@pytest.mark.parametrize('B,E,H', [(2, 16, 1), (3, 40, 2), (2, 100, 3),
+                                   (2, 512, 4), (1, 700, 2)])
+def test_encoder_attention(ops, B, E, H):
+  from t5x_amd import network
+  rs = np.random.RandomState(B * 1000 + E + H)
+  bf = lambda x: ot5.bf16_round(x.astype(np.float32))
+  q = bf(rs.randn(B, E, H, 64) * 0.125)
+  k = bf(rs.randn(B, E, H, 64))
+  v = bf(rs.randn(B, E, H, 64))
+  rel_emb = rs.randn(H, 32).astype(np.float32)
+  lens = rs.randint(1, E + 1, size=(B,)).astype(np.int32)
+  lens[0] = E
+  want = _enc_attn_oracle(q, k, v, rel_emb, lens)
+
+  Ep = (E + 7) // 8 * 8
+  bucket = network.relative_position_bucket(
+      np.arange(-(E - 1), E), bidirectional=True)        # key - query
+  rel_bias = dev(ot5.bf16_round(rel_emb)[:, bucket], torch.bfloat16).contiguous()
+  v_t = torch.zeros((B, H, 64, Ep), dtype=torch.bfloat16, device='cuda')
+  v_t[..., :E] = dev(v, torch.bfloat16).permute(0, 2, 3, 1)
+  qk = torch.stack([dev(q, torch.bfloat16).reshape(B * E, H * 64),
+                    dev(k, torch.bfloat16).reshape(B * E, H * 64)], dim=1)
+  qk = qk.reshape(B * E, 2 * H * 64)                      # strided q | k views
+  out = ops.encoder_attention(qk[:, :H * 64], qk[:, H * 64:], v_t, rel_bias,
+                              dev(lens))
+  got = host(out).reshape(B, E, H, 64)
+  # rows of valid queries: to the attention tolerance; padded queries attend
+  # uniformly in both (their values are never used downstream)
+  np.testing.assert_allclose(got, want, atol=2e-2, rtol=2**-6)
+
+
+def _tiny_cfgs(**kw):
+  base = dict(vocab_size=512, dtype='bfloat16', emb_dim=256, num_heads=4,
+              num_encoder_layers=3, num_decoder_layers=2, head_dim=64,
+              mlp_dim=512)
+  base.update(kw)
+  from t5x_amd import network
+  wd = base.pop('weight_dtype', None)
+  return ot5.T5Config(**base), network.T5Config(weight_dtype=wd, **base)
+
+
+@pytest.mark.parametrize('B,E', [(2, 16), (3, 40), (2, 132)])
+def test_encoder_forward_matches_oracle(B, E):
+  """Whole bf16 encoder on the HIP kernels.  Per-op agreement is to a bf16 ulp;
+  over 3 layers the same chaotic amplification as in the decoder applies, so
+  the bound is on the bulk of the outputs (normalised, |x| ~ 1)."""
+  from t5x_amd import network
+  ocfg, gcfg = _tiny_cfgs()
+  params = ot5.init_params(ocfg, seed=E)
+  rs = np.random.RandomState(E)
+  tok = rs.randint(2, ocfg.vocab_size, size=(B, E)).astype(np.int32)
+  lens = rs.randint(3, E + 1, size=(B,))
+  lens[0] = E
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  want = ot5.encode(params, ocfg, tok)
+  module = network.Transformer(gcfg, torch.device('cuda'))
+  got = host(module.apply({'params': params}, tok, enable_dropout=False,
+                          method=module.encode))
+  valid = np.arange(E)[None, :] < lens[:, None]
+  err = np.abs(got - want)[valid]
+  assert (err >= 4e-2).mean() < 0.01, (err >= 4e-2).mean()
+  assert err.mean() < 1e-2, err.mean()
+  assert err.max() < 0.25, err.max()
+
+
+def test_cross_kv_projection_layouts_match_oracle():
+  from t5x_amd import network
+  ocfg, gcfg = _tiny_cfgs()
+  params = ot5.init_params(ocfg, seed=5)
+  rs = np.random.RandomState(1)
+  B, E, K = 3, 24, 2
+  encoded = ot5.bf16_round(rs.randn(B, E, ocfg.emb_dim).astype(np.float32))
+  tok = np.ones((B, E), np.int32)
+  tok[1, 10:] = 0
+  want = ot5.project_cross_kv(params, ocfg, encoded)
+  module = network.Transformer(gcfg, torch.device('cuda'))
+  w = module.decoder_weights(params)
+  cross = module._cross_kv(w, dev(encoded, torch.bfloat16), dev(tok), K)
+  assert cross['enc_len'].tolist() == [24, 10, 24]
+  for (wk, wv), gk, gv in zip(want, cross['k'], cross['v']):
+    np.testing.assert_allclose(host(gk)[:, :, :E].transpose(0, 2, 1, 3), wk,
+                               atol=2e-2, rtol=2**-7)
+    np.testing.assert_allclose(host(gv)[..., :E].transpose(0, 3, 1, 2), wv,
+                               atol=2e-2, rtol=2**-7)
