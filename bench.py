@@ -123,10 +123,14 @@ class Workload:
 
   # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
   def cross_attention_bytes(self):
+    """Valid K and V rows once per batch item, the residual-stream rows and
+    layer-norm scale in, the query kernel once, the attention output out."""
     s = 2  # bf16
     hd = self.cfg.num_heads * self.cfg.head_dim
+    d = self.cfg.emb_dim
     R = self.B * self.K
-    return int(self.enc_lens.sum()) * hd * 2 * s + 2 * R * hd * s
+    return (int(self.enc_lens.sum()) * hd * 2 * s + R * d * s + d * s +
+            d * hd * s + R * hd * s)
 
   def self_attention_bytes(self, t):
     s = 2
@@ -186,30 +190,32 @@ def measured_traffic(name):
 
 
 def roofline_cross_attention(w, reps_per_layer=4):
-  """The step's largest single stream of HBM bytes per launch: cross-attention
-  over the encoder K/V (one launch per layer per step, same shape every step).
-  Replayed here back to back, walking the layers so no launch finds its K/V in
-  a cache (12 x 31 MB > the 256 MB memory-side cache only partly; L2 holds
-  none of it), and timed with HIP events on the launch stream."""
+  """The step's largest single stream of HBM bytes per launch: the
+  cross-attention kernel (pre-attention layer norm and query projection fused
+  in) over the encoder K/V, one launch per layer per step, same shape every
+  step.  Replayed here back to back, walking the layers so no launch finds its
+  K/V in a cache, and timed with HIP events on the launch stream."""
   from t5x_amd import ops
   torch = w.torch
   cross = w.module._cross[1]
   R = w.B * w.K
   hd = w.cfg.num_heads * w.cfg.head_dim
-  q = (0.125 * torch.randn((R, hd), device='cuda')).to(w.encoded.dtype)
-  out = torch.empty_like(q)
+  x = torch.randn((R, w.cfg.emb_dim), device='cuda').to(w.encoded.dtype)
+  out = torch.empty((R, hd), dtype=x.dtype, device='cuda')
+  layers = w.weights.layers
   nl = len(cross['k'])
   state = {'i': 0}
 
   def launch():
     i = state['i'] = (state['i'] + 1) % nl  # walk the layers: no cache reuse
-    ops.cross_attention_step(q, cross['k'][i], cross['v'][i], cross['enc_len'],
-                             w.K, out)
+    ops.cross_attention_step_norm_q(x, layers[i]['ln_cross'],
+                                    layers[i]['cross_q'], cross['k'][i],
+                                    cross['v'][i], cross['enc_len'], w.K, out)
 
   sec = time_kernel(torch, launch, reps_per_layer * nl)
   nbytes = w.cross_attention_bytes()
   achieved = nbytes / sec / 1e9
-  return {'kernel': 'cross_attn_mfma_kernel<4,4>', 'bound': 'hbm',
+  return {'kernel': 'cross_attn_mfma_kernel<4,4,3>', 'bound': 'hbm',
           'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS,
           'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBPS, 4),
           'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes,
