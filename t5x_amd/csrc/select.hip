@@ -183,12 +183,28 @@ beam_row_topk_kernel(const float* __restrict__ logits,
 // Fast path of the same computation for 16-byte aligned rows of at most 32768
 // elements with V % 4 == 0: 1024 threads per row, the row lives in registers
 // (8 float4 per thread, all loads issued at once), so logits are read from
-// memory exactly once.  Every thread keeps the best two of its 32 elements;
-// each wavefront then extracts its k best by k rounds of a 64-lane arg-best
-// (a lane that runs out of candidates rescans its registers for the next two
-// below the last one it gave away: rare, and skipped by a wave-uniform
-// branch), and wavefront 0 merges the 16 sorted lists the same way.
+// memory exactly once.  Selection is by threshold: f is monotone in x, so with
+// t = the k-th largest of the 16 wavefront maxima at least k elements have
+// f >= f(t) and nothing below f(t) can be among the k best.  The few elements
+// that pass (about 16 (H_16 - H_(16-k)) of an exchangeable row: 11 for k = 8)
+// are appended to a list in LDS and ranked there by counting.  A row with more
+// than kTopkCap elements at or above the threshold (long runs of equal values)
+// takes the slow path instead: every thread keeps the best two of its 32
+// elements, each wavefront extracts its k best by k rounds of a 64-lane
+// arg-best (a lane that runs out of candidates rescans its registers for the
+// next two below the last one it gave away), and wavefront 0 merges the 16
+// sorted lists the same way.
+constexpr int kTopkCap = 512;
 constexpr int kFastTopkVec = 8;
+
+// Phase timestamps for kernel tuning; compiled out unless T5D_PROBE is set.
+#ifdef T5D_PROBE
+__device__ long long t5d_select_probe_buf[128 * 8];
+#define T5D_SEL_STAMP(i) \
+  if (tid == 0) t5d_select_probe_buf[blockIdx.x * 8 + (i)] = wall_clock64()
+#else
+#define T5D_SEL_STAMP(i)
+#endif
 
 // exp(x) for x <= 0 to about 1 ulp with the hardware exp2: the rounding error
 // of x * log2(e) is recovered with an fma and folded back in as a first-order
@@ -205,13 +221,13 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
 
 __device__ __forceinline__ void top2_insert(float f, int fi, float& v0, int& i0,
                                             float& v1, int& i1) {
-  if (better(f, fi, v1, i1)) {
-    if (better(f, fi, v0, i0)) {
-      v1 = v0; i1 = i0; v0 = f; i0 = fi;
-    } else {
-      v1 = f; i1 = fi;
-    }
-  }
+  // selects only: a branchy form makes the compiler index the pair in memory
+  const bool b0 = better(f, fi, v0, i0);
+  const bool b1 = better(f, fi, v1, i1);
+  v1 = b0 ? v0 : (b1 ? f : v1);
+  i1 = b0 ? i0 : (b1 ? fi : i1);
+  v0 = b0 ? f : v0;
+  i0 = b0 ? fi : i0;
 }
 
 __global__ void __launch_bounds__(1024)
@@ -226,10 +242,14 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   __shared__ double s_d[16];
   __shared__ float s_cv[16][16];
   __shared__ int s_ci[16][16];
+  __shared__ float s_lv[kTopkCap];
+  __shared__ int s_li[kTopkCap];
+  __shared__ int s_count;
   T5D_GATED(gate);
   constexpr int kNone = 0x7FFFFFFF;
   const int r = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
+  T5D_SEL_STAMP(0);
   const float4* x4 = reinterpret_cast<const float4*>(logits + (size_t)r * V);
   const int nvec = V >> 2;
   float4 x[kFastTopkVec];
@@ -245,12 +265,25 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
 #pragma unroll
   for (int u = 0; u < kFastTopkVec; ++u)
     m = fmaxf(fmaxf(m, fmaxf(x[u].x, x[u].y)), fmaxf(x[u].z, x[u].w));
+  T5D_SEL_STAMP(1);
   m = wave_max(m);
   if (lane == 0) s_f[wave] = m;
+  if (tid == 0) s_count = 0;
   __syncthreads();
-  m = s_f[lane & 15];
+  const float wmax = s_f[lane & 15];
+  m = wmax;
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  // k-th largest wavefront maximum (k <= 16; ties ordered by wavefront)
+  int wrank = 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const float o = s_f[j];
+    wrank += (o > wmax || (o == wmax && j < (lane & 15))) ? 1 : 0;
+  }
+  const unsigned long long whit = __builtin_amdgcn_ballot_w64(wrank == k - 1);
+  const float tx = __shfl(wmax, (int)__builtin_ctzll(whit | (1ull << 63)), 64);
+  T5D_SEL_STAMP(2);
 
   double sum = 0.0;
 #pragma unroll
@@ -268,26 +301,70 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   sum = s_d[lane & 15];
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  T5D_SEL_STAMP(3);
   const float lse = (float)log(sum);
   if (tid == 0) {
     row_max[r] = m;
     row_lse[r] = lse;
   }
+  T5D_SEL_STAMP(4);
 
-  // f(j) = ((x[j] - max) - lse) + live_logprob, in place.
+  // f(j) = ((x[j] - max) - lse) + live_logprob, in place; elements at or
+  // above the threshold go to the list.
   const int base = (r % beams) * V;
+  const float tf = ((tx - m) - lse) + lp;
+#pragma unroll
+  for (int u = 0; u < kFastTopkVec; ++u) {
+    const int vi = u * 1024 + tid;
+    const int j = base + 4 * vi;
+    x[u].x = ((x[u].x - m) - lse) + lp;
+    x[u].y = ((x[u].y - m) - lse) + lp;
+    x[u].z = ((x[u].z - m) - lse) + lp;
+    x[u].w = ((x[u].w - m) - lse) + lp;
+    const float top = fmaxf(fmaxf(x[u].x, x[u].y), fmaxf(x[u].z, x[u].w));
+    if (vi < nvec && top >= tf) {
+      const float e[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (e[c] >= tf) {
+          const int p = atomicAdd(&s_count, 1);
+          if (p < kTopkCap) { s_lv[p] = e[c]; s_li[p] = j + c; }
+        }
+      }
+    }
+  }
+  T5D_SEL_STAMP(5);
+  __syncthreads();
+  const int ncand = s_count;
+  if (ncand <= kTopkCap) {
+    // rank by counting; indices are unique, so ranks are too
+    if (tid < ncand) {
+      const float v = s_lv[tid];
+      const int i = s_li[tid];
+      int rank = 0;
+      for (int c = 0; c < ncand; ++c)
+        rank += better(s_lv[c], s_li[c], v, i) ? 1 : 0;
+      if (rank < k) {
+        cand_vals[(size_t)r * k + rank] = v;
+        cand_idx[(size_t)r * k + rank] = i;
+      }
+    } else if (tid < k) {  // fewer than k elements in the row
+      cand_vals[(size_t)r * k + tid] = -INFINITY;
+      cand_idx[(size_t)r * k + tid] = kNone;
+    }
+    T5D_SEL_STAMP(6);
+    T5D_SEL_STAMP(7);
+    return;
+  }
+
+  // Slow path.
   float v0 = -INFINITY, v1 = -INFINITY;
   int i0 = kNone, i1 = kNone;
 #pragma unroll
   for (int u = 0; u < kFastTopkVec; ++u) {
     const int vi = u * 1024 + tid;
     const int j = base + 4 * vi;
-    const bool in = vi < nvec;
-    x[u].x = ((x[u].x - m) - lse) + lp;
-    x[u].y = ((x[u].y - m) - lse) + lp;
-    x[u].z = ((x[u].z - m) - lse) + lp;
-    x[u].w = ((x[u].w - m) - lse) + lp;
-    if (in) {
+    if (vi < nvec) {
       top2_insert(x[u].x, j, v0, i0, v1, i1);
       top2_insert(x[u].y, j + 1, v0, i0, v1, i1);
       top2_insert(x[u].z, j + 2, v0, i0, v1, i1);
@@ -338,6 +415,7 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   }
   __syncthreads();
   if (wave != 0) return;
+  T5D_SEL_STAMP(6);
   // Merge the 16 best-first lists: lane w < 16 walks list w.
   int pos = 0;
   for (int out = 0; out < k; ++out) {
@@ -359,7 +437,15 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
       cand_idx[(size_t)r * k + out] = best.i;
     }
   }
+  T5D_SEL_STAMP(7);
 }
+
+#ifdef T5D_PROBE
+extern "C" int t5d_select_probe_read(long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t5d_select_probe_buf),
+                                  sizeof(long long) * 128 * 8);
+}
+#endif
 
 // Merge the beams' per-row candidates of one batch item: one candidate per
 // thread (beams*k <= 128), rank by counting better candidates.
@@ -424,15 +510,19 @@ __device__ __forceinline__ void stable_order_desc(const float* v, int n,
   }
 }
 
-// One workgroup (one wavefront) per batch item.  Optionally first merges the
+// One workgroup per batch item.  Optionally first merges the
 // beams' per-row candidates (cand_* != null) into the item's top 2K.  The
 // order-sensitive bookkeeping is done in parallel, one candidate / pool entry
 // per lane, ranks by counting under the total order (value descending, index
 // ascending), which is what the reference's stable sorts produce.  Then every
 // thread owns sequence COLUMNS: for a column it reads the item's K live and K
 // finished entries into registers before writing any, so `cur` and `next`
-// may be the same buffers.
-__global__ void __launch_bounds__(64)
+// may be the same buffers.  Everything that does not depend on another load
+// (candidates, the finished pool, the first column of every thread) is
+// requested before the first wait, so the chain of cold misses is two deep
+// (cur_index, then the forced token and the brevity penalty).
+constexpr int kUpdateThreads = 256;
+__global__ void __launch_bounds__(kUpdateThreads)
 beam_update_kernel(BeamUpdateArgs a) {
   __shared__ int s_src_live[kMaxBeams];       // source live beam of new live e
   __shared__ int s_tok_live[kMaxBeams];
@@ -452,17 +542,34 @@ beam_update_kernel(BeamUpdateArgs a) {
   T5D_GATED(a.gate);
   const int b = blockIdx.x, lane = threadIdx.x;
   const int K = a.K, K2 = 2 * a.K, S = a.S;
+  const size_t base = (size_t)b * K * S;
+  int live[kMaxBeams], fin[kMaxBeams];
+#pragma unroll
+  for (int e = 0; e < kMaxBeams; ++e) {
+    if (e < K && lane < S) {
+      live[e] = a.cur.live_seqs[base + (size_t)e * S + lane];
+      fin[e] = a.cur.finished_seqs[base + (size_t)e * S + lane];
+    }
+  }
+  float old_score = 0.f;
+  int old_flag = 0;
+  if (lane < K) {
+    old_score = a.cur.finished_scores[(size_t)b * K + lane];
+    old_flag = a.cur.finished_flags[(size_t)b * K + lane];
+  }
+  const int first = a.initial_index[b];
   const int cur = *a.cur.cur_index;
 
   if (a.cand_vals != nullptr) {
     // top 2K of the K rows' 2K candidates each
     const int n = K * K2;
-    for (int c = lane; c < n; c += 64) {
-      s_mv[c] = a.cand_vals[(size_t)b * n + c];
-      s_mi[c] = a.cand_idx[(size_t)b * n + c];
+    if (lane < n) {
+      s_mv[lane] = a.cand_vals[(size_t)b * n + lane];
+      s_mi[lane] = a.cand_idx[(size_t)b * n + lane];
     }
     __syncthreads();
-    for (int c = lane; c < n; c += 64) {
+    if (lane < n) {
+      const int c = lane;
       const float v = s_mv[c];
       const int i = s_mi[c];
       int rank = 0;
@@ -498,13 +605,13 @@ beam_update_kernel(BeamUpdateArgs a) {
     s_fin[c] = fin;
     s_new_lp[c] = lp + (fin ? kNegInf : 0.f);
   }
-  const int len = a.initial_index[b] + cur + 1;
+  const int len = first + cur + 1;
   const float bp = a.brevity[len];
   __syncthreads();
   // finished pool: K old + 2K new, brevity-penalised
   if (lane < 3 * K) {
     s_pool[lane] = lane < K
-        ? a.cur.finished_scores[(size_t)b * K + lane]
+        ? old_score
         : s_lp[lane - K] / bp + (s_fin[lane - K] ? 0.f : kNegInf);
   }
   __syncthreads();
@@ -530,8 +637,7 @@ beam_update_kernel(BeamUpdateArgs a) {
       const int e = K - 1 - rank;
       s_fin_from[e] = lane;
       s_fin_score[e] = v;
-      s_fin_flag[e] = lane < K ? a.cur.finished_flags[(size_t)b * K + lane]
-                               : s_fin[lane - K];
+      s_fin_flag[e] = lane < K ? old_flag : s_fin[lane - K];
     }
   }
   __syncthreads();
@@ -544,14 +650,14 @@ beam_update_kernel(BeamUpdateArgs a) {
   }
   __syncthreads();
 
-  const size_t base = (size_t)b * K * S;
-  for (int j = threadIdx.x; j < S; j += 64) {
-    int live[kMaxBeams], fin[kMaxBeams];
+  for (int j = lane; j < S; j += kUpdateThreads) {
+    if (j != lane) {
 #pragma unroll
-    for (int e = 0; e < kMaxBeams; ++e) {
-      if (e < K) {
-        live[e] = a.cur.live_seqs[base + (size_t)e * S + j];
-        fin[e] = a.cur.finished_seqs[base + (size_t)e * S + j];
+      for (int e = 0; e < kMaxBeams; ++e) {
+        if (e < K) {
+          live[e] = a.cur.live_seqs[base + (size_t)e * S + j];
+          fin[e] = a.cur.finished_seqs[base + (size_t)e * S + j];
+        }
       }
     }
     const bool tokcol = j == cur + 1;
@@ -988,7 +1094,7 @@ extern "C" int t5d_beam_update(void* stream, const t5d_beam_state* cur,
   a.gate = tls_gate;
   a.cand_vals = nullptr; a.cand_idx = nullptr;
   a.topk_vals_out = nullptr; a.topk_idx_out = nullptr;
-  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0,
+  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(kUpdateThreads), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_beam_update");
   hipLaunchKernelGGL(advance_index_kernel, dim3(1), dim3(1), 0,
@@ -1040,7 +1146,7 @@ int t5d::launch_beam_select(hipStream_t s, const float* logits,
   a.gate = tls_gate;
   a.cand_vals = cand_vals; a.cand_idx = cand_idx;
   a.topk_vals_out = topk_vals; a.topk_idx_out = topk_idx;
-  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(64), 0, s, a);
+  hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(kUpdateThreads), 0, s, a);
   T5D_CHECK_LAUNCH("beam select");
   return T5D_OK;
 }
