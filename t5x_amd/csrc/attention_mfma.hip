@@ -217,8 +217,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
         }
       }
     }
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
+    ss = rows_sum(ss);
     T5D_STAMP_FQ(9);
     if (g == 0) s_ss[wave][n16] = n16 < a.nq ? ss : 0.f;
     __syncthreads();
@@ -315,8 +314,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       sc[t][i] = x;
       m = fmaxf(m, x);
     }
-#pragma unroll
-  for (int o = NQP; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if (NQP <= 4) m = fmaxf(m, lane_xor4(m));
+  if (NQP <= 8) m = fmaxf(m, lane_xor8(m));
+  m = rows_max(m);
   if (nwaves > 1) {
     if (lane < 16) s_red[0][wave][lane] = m;  // lanes 0..15: q = lane % NQP
     __syncthreads();
@@ -333,8 +333,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       sc[t][i] = ex;
       sum += ex;
     }
-#pragma unroll
-  for (int o = NQP; o < 64; o <<= 1) sum += __shfl_xor(sum, o, 64);
+  if (NQP <= 4) sum += lane_xor4(sum);
+  if (NQP <= 8) sum += lane_xor8(sum);
+  sum = rows_sum(sum);
   if (nwaves > 1) {
     if (lane < 16) s_red[1][wave][lane] = sum;
     __syncthreads();
@@ -584,17 +585,20 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
                 voff[jb]) = vb[jb][dt].u;
         }
       }
-      // the column written below must land after the chunks that cover it
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
   } else {
     __syncthreads();  // s_bias
   }
   // The column being written: lane d stores element d of the new key / value.
-  if (wave_has_t) {
-    kdst[(size_t)lane * S + t] = knew_d;
-    vdst[(size_t)lane * S + t] = vnew_d;
-  }
+  // It must land after this wavefront's chunk stores above that cover it, so
+  // it is issued last, when waiting for those stores costs nothing.
+  auto store_column = [&]() {
+    if (wave_has_t) {
+      if (r != rs) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      kdst[(size_t)lane * S + t] = knew_d;
+      vdst[(size_t)lane * S + t] = vnew_d;
+    }
+  };
 
   T5D_STAMP_SELF(11);
   // 2 positions per lane: bias, mask, softmax.
@@ -686,6 +690,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
         *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
       }
     }
+    store_column();
     T5D_STAMP_SELF(15);
     return;
   }
@@ -701,6 +706,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int w = 1; w < nblk; ++w) acc += s_out[wave0 + w][lane];
     a.out[(size_t)r * HD + h * kHeadDim + lane] = f32_to_bf16(acc);
   }
+  store_column();
 }
 
 // ---- dispatch -------------------------------------------------------------------

@@ -88,16 +88,89 @@ __device__ __forceinline__ void unpack16(const uint4& v, float (&f)[4]) {
 }
 
 // ---- wavefront (64 lanes) reductions ---------------------------------------
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+// All-reduce butterflies on the data-parallel-primitive path (no LDS round
+// trips): lane^1 and lane^2 by quad permutes, then the mirror of each 8 and
+// of each 16 lanes (the partner holds the other half's partial by then), then
+// v_permlane16_swap / v_permlane32_swap of the value with itself, which hand
+// every lane both 16-lane (32-lane) partials.  Every lane ends with the same
+// bits: both partners of a step combine the same two operands.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(
+      0, (int)__float_as_uint(v), CTRL, 0xF, 0xF, true));
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i within 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15 - i within 16
+
+constexpr int kDppReverse4 = 0x1B;    // quad_perm [3,2,1,0]
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(
+      0, (int)(uint32_t)b, CTRL, 0xF, 0xF, true);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(
+      0, (int)(uint32_t)(b >> 32), CTRL, 0xF, 0xF, true);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
 }
+// The exact lane ^ 4 and lane ^ 8 partners, two moves each.
+__device__ __forceinline__ float lane_xor4(float v) {
+  return dpp_move<kDppReverse4>(dpp_move<kDppHalfMirror>(v));
+}
+__device__ __forceinline__ float lane_xor8(float v) {
+  return dpp_move<kDppMirror>(dpp_move<kDppHalfMirror>(v));
+}
+
+// Over the 16 lanes of a row (lanes 16 r .. 16 r + 15).
+__device__ __forceinline__ float lanes16_max(float v) {
+  v = fmaxf(v, dpp_move<kDppXor1>(v));
+  v = fmaxf(v, dpp_move<kDppXor2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  return fmaxf(v, dpp_move<kDppMirror>(v));
+}
+template <typename T>
+__device__ __forceinline__ T lanes16_sum(T v) {
+  v += dpp_move<kDppXor1>(v);
+  v += dpp_move<kDppXor2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  return v + dpp_move<kDppMirror>(v);
+}
+// Over the 4 lanes lane % 16 + {0, 16, 32, 48}.
+__device__ __forceinline__ float rows_max(float v) {
+  auto w = __builtin_amdgcn_permlane16_swap(__float_as_uint(v),
+                                            __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(w[0]), __uint_as_float(w[1]));
+  w = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v),
+                                       false, false);
+  return fmaxf(__uint_as_float(w[0]), __uint_as_float(w[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  auto w = __builtin_amdgcn_permlane16_swap(__float_as_uint(v),
+                                            __float_as_uint(v), false, false);
+  v = __uint_as_float(w[0]) + __uint_as_float(w[1]);
+  w = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v),
+                                       false, false);
+  return __uint_as_float(w[0]) + __uint_as_float(w[1]);
+}
+__device__ __forceinline__ double rows_sum(double v) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  uint32_t lo = (uint32_t)b, hi = (uint32_t)(b >> 32);
+  auto wl = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
+  auto wh = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+  v = __builtin_bit_cast(double, ((uint64_t)wh[0] << 32) | wl[0]) +
+      __builtin_bit_cast(double, ((uint64_t)wh[1] << 32) | wl[1]);
+  const uint64_t c = __builtin_bit_cast(uint64_t, v);
+  lo = (uint32_t)c; hi = (uint32_t)(c >> 32);
+  wl = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+  wh = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+  return __builtin_bit_cast(double, ((uint64_t)wh[0] << 32) | wl[0]) +
+         __builtin_bit_cast(double, ((uint64_t)wh[1] << 32) | wl[1]);
+}
+
+__device__ __forceinline__ float wave_max(float v) { return rows_max(lanes16_max(v)); }
+__device__ __forceinline__ float wave_sum(float v) { return rows_sum(lanes16_sum(v)); }
+__device__ __forceinline__ double wave_sum(double v) { return rows_sum(lanes16_sum(v)); }
 
 // T5 tanh-approximate GELU in float32.
 __device__ __forceinline__ float gelu_tanh(float x) {

@@ -342,8 +342,7 @@ norm_gemm_kernel(GemmArgs g) {
       }
     }
   }
-  ss += __shfl_xor(ss, 16, 64);
-  ss += __shfl_xor(ss, 32, 64);
+  ss = rows_sum(ss);
   if (gq == 0) s_ss[wave][n16] = ss;
   __syncthreads();
   const float tot = (s_ss[0][n16] + s_ss[2][n16]) + (s_ss[1][n16] + s_ss[3][n16]);

@@ -271,9 +271,7 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   if (tid == 0) s_count = 0;
   __syncthreads();
   const float wmax = s_f[lane & 15];
-  m = wmax;
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  m = lanes16_max(wmax);
   // k-th largest wavefront maximum (k <= 16; ties ordered by wavefront)
   int wrank = 0;
 #pragma unroll
@@ -294,13 +292,10 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
     sum += (double)exp_nonpositive(x[u].z - m);
     sum += (double)exp_nonpositive(x[u].w - m);
   }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  sum = wave_sum(sum);
   if (lane == 0) s_d[wave] = sum;
   __syncthreads();
-  sum = s_d[lane & 15];
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  sum = lanes16_sum(s_d[lane & 15]);
   T5D_SEL_STAMP(3);
   const float lse = (float)log(sum);
   if (tid == 0) {

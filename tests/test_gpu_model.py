@@ -254,39 +254,41 @@ def test_predict_batch_mock_module_and_rng_rules():
       "`decoder_params['decode_rng']` (3). Please specify one or the other.")
 
 
-def test_decoder_step_at_base_size_matches_oracle():
-  """One decode step at the full T5.1.1-base / beam-4 shape (R=128, E=512 with
-  ragged lengths, L=128) in the middle of a decode (t=77): caches are
-  pre-filled with the same random prefix on both sides."""
+def _step_at_width(name, emb, heads, mlp, B, K, E, Emin, L, t,
+                   weight_dtype=None):
+  """One decode step of a 2-layer decoder at a real model width, in the middle
+  of a decode (position t): caches are pre-filled with the same random prefix
+  on both sides."""
   from t5x_amd import network
-  kw = dict(vocab_size=32128, dtype='bfloat16', emb_dim=768, num_heads=12,
+  kw = dict(vocab_size=32128, dtype='bfloat16', emb_dim=emb, num_heads=heads,
             num_encoder_layers=0, num_decoder_layers=2, head_dim=64,
-            mlp_dim=2048)
-  ocfg, cfg = ot5.T5Config(**kw), network.T5Config(**kw)
+            mlp_dim=mlp)
+  ocfg = ot5.T5Config(**kw)
+  cfg = network.T5Config(weight_dtype=weight_dtype, **kw)
   params = ot5.init_params(ocfg, seed=11, with_encoder=False)
+  oparams = quantized_tree(params) if weight_dtype == 'int8' else params
   rs = np.random.RandomState(3)
-  B, K, E, L, t = 32, 4, 512, 128, 77
   R = B * K
-  enc_tok = ragged_tokens(rs, B, E, 32128, 128)
-  encoded = ot5.bf16_round(rs.randn(B, E, 768).astype(np.float32))
+  enc_tok = ragged_tokens(rs, B, E, 32128, Emin)
+  encoded = ot5.bf16_round(rs.randn(B, E, emb).astype(np.float32))
   ocache = ot5.init_cache(ocfg, R, L)
   for lyr in ocache['decoder'].values():
     sa = lyr['self_attention']
     for n in ('cached_key', 'cached_value'):
       sa[n][..., :t] = ot5.bf16_round(
-          rs.randn(R, 12, 64, t).astype(np.float32))
+          rs.randn(R, heads, 64, t).astype(np.float32))
     sa['cache_index'] = np.array(t, np.int32)
   module = network.Transformer(cfg)
   gcache = module.init_cache(R, L)
-  for name, lyr in gcache['decoder'].items():
-    sa, osa = lyr['self_attention'], ocache['decoder'][name]['self_attention']
+  for lname, lyr in gcache['decoder'].items():
+    sa, osa = lyr['self_attention'], ocache['decoder'][lname]['self_attention']
     for n in ('cached_key', 'cached_value'):
-      sa[n].copy_(torch.as_tensor(osa[n]).to(torch.bfloat16))
+      sa[n][..., :L].copy_(torch.as_tensor(osa[n]).to(torch.bfloat16))
     sa['cache_index'].fill_(t)
   tok = rs.randint(2, 32128, size=(R, 1)).astype(np.int32)
-  cross_kv = ot5.project_cross_kv(params, ocfg, encoded)
+  cross_kv = ot5.project_cross_kv(oparams, ocfg, encoded)
   cross_kv = [(np.repeat(k, K, 0), np.repeat(v, K, 0)) for k, v in cross_kv]
-  want, _ = ot5.decode(params, ocfg, None, np.repeat(enc_tok, K, axis=0), tok,
+  want, _ = ot5.decode(oparams, ocfg, None, np.repeat(enc_tok, K, axis=0), tok,
                        tok, decode=True, cache=ocache, max_decode_length=L,
                        cross_kv=cross_kv)
   got = module.apply(
@@ -295,9 +297,29 @@ def test_decoder_step_at_base_size_matches_oracle():
       network.BeamShared(enc_tok, K), torch.as_tensor(tok, device='cuda'),
       None, decode=True, max_decode_length=L, method=module.decode)
   err = np.abs(host(got)[:, 0] - want[:, 0])
-  print(f'base-size step: max |dlogit| = {err.max():.3g}, mean '
+  print(f'{name}-size step: max |dlogit| = {err.max():.3g}, mean '
         f'{err.mean():.3g}, p99.9 {np.quantile(err, 0.999):.3g}')
-  check_logits(host(got)[:, 0], want[:, 0], 'bfloat16', 'base')
+  check_logits(host(got)[:, 0], want[:, 0], 'bfloat16', name)
+
+
+def test_decoder_step_at_base_size_matches_oracle():
+  """The full T5.1.1-base / beam-4 shape: R=128, E=512 with ragged lengths,
+  L=128, t=77."""
+  _step_at_width('base', 768, 12, 2048, B=32, K=4, E=512, Emin=128, L=128,
+                 t=77)
+
+
+@pytest.mark.parametrize('name,emb,heads,mlp,B,K,E,Emin,L,t,wdt', [
+    # T5.1.1-large rows of the sampling workload (no beams, 256 positions)
+    ('large', 1024, 16, 2816, 64, 1, 128, 40, 256, 141, None),
+    # T5.1.1-XL, int8 weight-only, 4 beams
+    ('xl-int8', 2048, 32, 5120, 4, 4, 128, 30, 128, 50, 'int8'),
+    # T5.1.1-XXL width, greedy rows, encoder 1024
+    ('xxl', 4096, 64, 10240, 8, 1, 1024, 700, 256, 200, None),
+])
+def test_decoder_step_at_other_widths_matches_oracle(name, emb, heads, mlp, B,
+                                                     K, E, Emin, L, t, wdt):
+  _step_at_width(name, emb, heads, mlp, B, K, E, Emin, L, t, wdt)
 
 
 def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
