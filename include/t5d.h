@@ -392,6 +392,37 @@ typedef struct {
 int t5d_beam_search_step(void* stream, const t5d_model_step* model,
                          const t5d_beam_step* beam);
 
+typedef struct {
+  int32_t* sequences;              /* [R, S], S = L + 2; updated in place */
+  int32_t* cur_index;              /* [R] */
+  int32_t* cur_token;              /* [R]: the ids the decoder step consumes */
+  uint8_t* ended;                  /* [R] */
+  float* log_prob;                 /* [R] */
+  const int32_t* max_decode_len;   /* [R] */
+  const int32_t* initial_eos_count;/* [R] */
+  const float* temperature;        /* [R] */
+  /* Gumbel noise for the coming steps, [noise_ring, R, V] f32: executed step n
+   * reads slot n % noise_ring.  May be NULL when every temperature <= 1e-4. */
+  const float* gumbel;
+  int noise_ring;
+  int32_t* step_count;             /* device counter of executed steps */
+  int32_t* tokens;                 /* [R] scratch */
+  float* token_logprobs;           /* [R] scratch */
+  int32_t* all_ended;              /* out: every row ended */
+  int32_t* keep_going;             /* loop flag = !all_ended; == model->gate */
+  int S, eos_id, topk, rescale;
+  float topp;
+} t5d_sample_step;
+
+/* One iteration of the temperature_sample loop body plus its condition
+ * (t5x/decoding.py:509-700): decoder step on cur_token, token choice
+ * (t5d_sample_tokens), bookkeeping (t5d_sample_update); the layers' cache
+ * indices and *step_count advance, *keep_going = !all_ended.  Every kernel is
+ * gated by *keep_going, so iterations enqueued after the last row ended change
+ * nothing.  Covers the loop without state / logit callbacks. */
+int t5d_temperature_sample_step(void* stream, const t5d_model_step* model,
+                                const t5d_sample_step* sample);
+
 /* HIP graph capture on `stream` (must not be the null stream):
  * begin, enqueue any t5d calls, end -> executable graph; launch replays it. */
 int t5d_graph_begin(void* stream);

@@ -57,12 +57,26 @@ class BeamStep(Structure):
                ('n_kv_tensors', c_int), ('skip_cond', c_int)])
 
 
+class SampleStep(Structure):
+  """t5d_sample_step."""
+  _fields_ = ([(n, c_void_p) for n in (
+      'sequences', 'cur_index', 'cur_token', 'ended', 'log_prob',
+      'max_decode_len', 'initial_eos_count', 'temperature', 'gumbel')] +
+              [('noise_ring', c_int)] + [(n, c_void_p) for n in (
+                  'step_count', 'tokens', 'token_logprobs', 'all_ended',
+                  'keep_going')] +
+              [('S', c_int), ('eos_id', c_int), ('topk', c_int),
+               ('rescale', c_int), ('topp', c_float)])
+
+
 _P = c_void_p
 _SIGNATURES = {
     't5d_gather_step_ids': (c_int, [_P, _P, _P, _P, c_int, c_int]),
     't5d_decoder_step': (c_int, [_P, POINTER(ModelStep), _P]),
     't5d_beam_search_step': (c_int, [_P, POINTER(ModelStep),
                                      POINTER(BeamStep)]),
+    't5d_temperature_sample_step': (c_int, [_P, POINTER(ModelStep),
+                                            POINTER(SampleStep)]),
     't5d_graph_begin': (c_int, [_P]),
     't5d_graph_end': (c_int, [_P, POINTER(c_void_p)]),
     't5d_graph_launch': (c_int, [_P, _P]),

@@ -221,4 +221,11 @@ int launch_beam_tail(hipStream_t s, const t5d_beam_state* state, int B, int K,
                      int32_t* keep_going, int do_cond, int32_t* counters,
                      int n_counters);
 
+// The two kernels of a temperature_sample iteration after the decoder step:
+// token choice, then the bookkeeping, which also advances `counters` (the
+// layers' cache indices) and the step count and sets the loop flag.
+int launch_sample_step(hipStream_t s, const float* logits,
+                       const t5d_sample_step* st, int R, int V,
+                       int32_t* counters, int n_counters);
+
 }  // namespace t5d

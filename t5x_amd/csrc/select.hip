@@ -757,12 +757,15 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
 
 struct SampleArgs {
   const float* logits;
-  const float* gumbel;
+  const float* gumbel;       // [noise_ring, R, V]; slot *noise_step % noise_ring
   const float* temperature;
   int32_t* tokens;
   float* logprobs;
   int V, topk, rescale;
   float topp;
+  const int32_t* noise_step; // null: slot 0
+  int noise_ring, R;
+  const int32_t* gate;
 };
 
 // One workgroup per row.
@@ -773,10 +776,13 @@ sample_tokens_kernel(SampleArgs a) {
   __shared__ double dscratch[4];
   __shared__ int iscratch[4];
   __shared__ unsigned hist[256];
+  T5D_GATED(a.gate);
   const int r = blockIdx.x;
   const int V = a.V;
   const float* x = a.logits + (size_t)r * V;
   const float T = a.temperature[r];
+  const int slot = a.noise_step ? *a.noise_step % a.noise_ring : 0;
+  const float* noise = a.gumbel + ((size_t)slot * a.R + r) * V;
   const float kMinT = 1e-4f;
 
   if (!(T > kMinT)) {  // greedy (t5x/decoding.py:575-592)
@@ -890,7 +896,7 @@ sample_tokens_kernel(SampleArgs a) {
       const float pr = expf(y - smax) / ssum;
       y = (pr >= pcut) ? y : kNegInf;
     }
-    const float z = y + a.gumbel[(size_t)r * V + j];
+    const float z = y + noise[j];
     if (better(z, j, best.v, best.i)) { best.v = z; best.i = j; }
     m = fmaxf(m, a.rescale ? y : x[j]);
   }
@@ -933,11 +939,20 @@ struct SampleUpdateArgs {
   const int32_t* initial_eos_count;
   int32_t* all_ended;
   int R, S, eos_id;
+  // fused loop only: the loop flag (= !all_ended, also the gate of this
+  // launch), the count of executed steps, and counters that advance with it
+  // (the layers' cache indices)
+  int32_t* keep_going;
+  int32_t* step_count;
+  int32_t* counters;
+  int n_counters;
+  const int32_t* gate;
 };
 
 __global__ void __launch_bounds__(256)
 sample_update_kernel(SampleUpdateArgs a) {
   __shared__ int iscratch[4];
+  T5D_GATED(a.gate);
   int not_ended = 0;
   for (int r = threadIdx.x; r < a.R; r += 256) {
     int32_t* seq = a.sequences + (size_t)r * a.S;
@@ -960,7 +975,13 @@ sample_update_kernel(SampleUpdateArgs a) {
     if (!ended) ++not_ended;
   }
   not_ended = block_sum_i32(not_ended, iscratch);
-  if (threadIdx.x == 0) *a.all_ended = not_ended == 0 ? 1 : 0;
+  if (threadIdx.x == 0) {
+    *a.all_ended = not_ended == 0 ? 1 : 0;
+    if (a.step_count) *a.step_count += 1;
+    // the gate was read by every thread before the reduction's barriers
+    if (a.keep_going) *a.keep_going = not_ended == 0 ? 0 : 1;
+  }
+  if ((int)threadIdx.x < a.n_counters) a.counters[threadIdx.x] += 1;
 }
 
 // ---- generic beam-axis gather (out of place) -----------------------------------
@@ -1181,9 +1202,35 @@ extern "C" int t5d_sample_tokens(void* stream, const float* logits,
   a.logits = logits; a.gumbel = gumbel; a.temperature = temperature;
   a.tokens = tokens; a.logprobs = logprobs;
   a.V = V; a.topk = topk; a.rescale = rescale; a.topp = topp;
+  a.noise_step = nullptr; a.noise_ring = 1; a.R = R; a.gate = tls_gate;
   hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_sample_tokens");
+  return T5D_OK;
+}
+
+int t5d::launch_sample_step(hipStream_t s, const float* logits,
+                            const t5d_sample_step* st, int R, int V,
+                            int32_t* counters, int n_counters) {
+  SampleArgs a;
+  a.logits = logits; a.gumbel = st->gumbel; a.temperature = st->temperature;
+  a.tokens = st->tokens; a.logprobs = st->token_logprobs;
+  a.V = V; a.topk = st->topk; a.rescale = st->rescale; a.topp = st->topp;
+  a.noise_step = st->step_count; a.noise_ring = st->noise_ring; a.R = R;
+  a.gate = tls_gate;
+  hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0, s, a);
+  T5D_CHECK_LAUNCH("sample step (tokens)");
+  SampleUpdateArgs u;
+  u.tokens = st->tokens; u.token_logprobs = st->token_logprobs;
+  u.sequences = st->sequences; u.cur_index = st->cur_index;
+  u.cur_token = st->cur_token; u.ended = st->ended; u.log_prob = st->log_prob;
+  u.max_decode_len = st->max_decode_len;
+  u.initial_eos_count = st->initial_eos_count; u.all_ended = st->all_ended;
+  u.R = R; u.S = st->S; u.eos_id = st->eos_id;
+  u.keep_going = st->keep_going; u.step_count = st->step_count;
+  u.counters = counters; u.n_counters = n_counters; u.gate = tls_gate;
+  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(256), 0, s, u);
+  T5D_CHECK_LAUNCH("sample step (update)");
   return T5D_OK;
 }
 
@@ -1205,6 +1252,8 @@ extern "C" int t5d_sample_update(void* stream, const int32_t* tokens,
   a.log_prob = log_prob; a.max_decode_len = max_decode_len;
   a.initial_eos_count = initial_eos_count; a.all_ended = all_ended;
   a.R = R; a.S = S; a.eos_id = eos_id;
+  a.keep_going = nullptr; a.step_count = nullptr; a.counters = nullptr;
+  a.n_counters = 0; a.gate = tls_gate;
   hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(256), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_sample_update");

@@ -169,6 +169,34 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
   return T5D_OK;
 }
 
+extern "C" int t5d_temperature_sample_step(void* stream,
+                                           const t5d_model_step* m,
+                                           const t5d_sample_step* s) {
+  T5D_TRY(check_model(m));
+  T5D_REQUIRE(s && s->sequences && s->cur_index && s->cur_token && s->ended &&
+                  s->log_prob && s->max_decode_len && s->initial_eos_count &&
+                  s->temperature && s->step_count && s->tokens &&
+                  s->token_logprobs && s->all_ended && s->keep_going,
+              T5D_EINVAL, "t5d_temperature_sample_step: null buffer");
+  T5D_REQUIRE(m->gate == s->keep_going, T5D_EINVAL,
+              "t5d_temperature_sample_step: the model gate must be the loop "
+              "flag");
+  T5D_REQUIRE(m->pending_src == nullptr, T5D_EINVAL,
+              "t5d_temperature_sample_step: sampling rows are never reordered");
+  T5D_REQUIRE(s->S > 2 && s->topk >= 0 && s->topp >= 0.f &&
+                  (s->gumbel == nullptr || s->noise_ring > 0),
+              T5D_EINVAL,
+              "t5d_temperature_sample_step: S=%d topk=%d topp=%f ring=%d", s->S,
+              s->topk, (double)s->topp, s->noise_ring);
+  T5D_REQUIRE(!(s->topk > 0 && s->topp > 0.f), T5D_EINVAL,
+              "At most one of `topp` or `topk` may be non-zero.");
+  T5D_TRY(decoder_step_impl(stream, m, s->cur_token, nullptr, nullptr, 0,
+                            false));
+  GateScope gate(s->keep_going);
+  return launch_sample_step(as_stream(stream), m->logits, s, m->R, m->V,
+                            m->cache_index, m->NL);
+}
+
 // ---- HIP graph capture --------------------------------------------------------
 
 extern "C" int t5d_graph_begin(void* stream) {

@@ -290,7 +290,18 @@ def temperature_sample(
     max_decode_steps = np.minimum(max_decode_steps,
                                   max_decode_steps_hard_limit)
   inputs = _dev(inputs, torch.int32)
-  if num_decodes > 1:
+  # A step function that can run whole iterations on the device exposes
+  # `fused_sample_step(...)`; it then owns the caches of all rows (the incoming
+  # cache must be the untouched zero cache, which is then not even expanded).
+  use_fused = (getattr(tokens_to_logits, 'fused_sample_step', None) is not None
+               and getattr(cache, 'fresh', False) and initial_index is None and
+               cache_offset == 0 and state_callback_fn is None and
+               logit_callback_fn is None)
+  if use_fused:
+    expanded_inputs = (flat_batch_beam_expand(inputs, num_decodes)
+                       if num_decodes > 1 else inputs)
+    expanded_cache = cache
+  elif num_decodes > 1:
     expanded_inputs = flat_batch_beam_expand(inputs, num_decodes)
     expanded_cache = cache_map(
         functools.partial(flat_batch_beam_expand, beam_size=num_decodes,
@@ -306,7 +317,8 @@ def temperature_sample(
       expanded_inputs, expanded_cache, tokens_to_logits, eos_id, decode_rng,
       num_decodes, temperature, topk, topp, initial_index=initial_index,
       max_decode_steps=max_decode_steps, rescale_log_probs=rescale_log_probs,
-      state_callback_fn=state_callback_fn, logit_callback_fn=logit_callback_fn)
+      state_callback_fn=state_callback_fn, logit_callback_fn=logit_callback_fn,
+      use_fused=use_fused)
 
   batch_size = inputs.shape[0]
   decodes = unflatten_beam_dim(expanded_decodes, batch_size, num_decodes)
@@ -327,6 +339,7 @@ def _temperature_sample_single_trial(
     max_decode_steps=None, rescale_log_probs: bool = True,
     state_callback_fn: Optional[Callable] = None,
     logit_callback_fn: Optional[Callable] = None,
+    use_fused: bool = False,
 ):
   """:412-715."""
   if topp and topk:
@@ -374,6 +387,16 @@ def _temperature_sample_single_trial(
   tok_lp = torch.empty((batch_size,), dtype=torch.float32, device=dev)
   source = _noise_source(prng_key)
   step = 0
+
+  if use_fused:
+    fused = tokens_to_logits.fused_sample_step(
+        sequences=sequences, cur_index=cur_index, cur_token=cur_token,
+        ended=ended, log_prob=log_prob, max_decode_len=mdl,
+        initial_eos_count=eos0, temperature=temps_dev, all_ended=all_ended,
+        eos_id=eos_id, topk=topk, topp=topp, rescale=rescale_log_probs,
+        noise_source=source if any_sampling else None)
+    fused.run()
+    return sequences[:, 1:-1], log_prob
 
   def loop_state():
     return SamplingLoopState(

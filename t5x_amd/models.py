@@ -32,7 +32,7 @@ class Vocabulary:
 class StepFunction:
   """`tokens_ids_to_logits` of t5x/models.py:703-715: the bound
   `_compute_logits_from_slice`, as an object so the decode loop can also ask
-  for a fused on-device step (`fused_beam_step`)."""
+  for a fused on-device step (`fused_beam_step`, `fused_sample_step`)."""
 
   def __init__(self, model, params, encoded_inputs, raw_inputs,
                max_decode_length):
@@ -43,6 +43,9 @@ class StepFunction:
     if hasattr(module, 'make_fused_beam_step'):
       self.fused_beam_step = lambda loop: module.make_fused_beam_step(
           loop, params, encoded_inputs, raw_inputs)
+    if hasattr(module, 'make_fused_sample_step'):
+      self.fused_sample_step = lambda **kw: module.make_fused_sample_step(
+          params, encoded_inputs, raw_inputs, **kw)
 
   def __call__(self, decoding_state):
     return self.model._compute_logits_from_slice(

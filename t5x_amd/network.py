@@ -490,6 +490,152 @@ class Transformer:
     return FusedBeamStep(self, loop, params, encoded, enc_tokens)
 
 
+  # -- fused sampling: one graph replay per loop iteration --------------------------
+  def make_fused_sample_step(self, params, encoded, enc_tokens, **kw):
+    """Returns a FusedSampleStep (see there for the arguments)."""
+    beams = encoded.beams if isinstance(encoded, BeamShared) else 1
+    rows = kw['sequences'].shape[0]
+    enc_rows = (encoded.x if isinstance(encoded, BeamShared) else
+                encoded).shape[0]
+    if rows != enc_rows * beams:
+      raise ValueError(f'{rows} decoder rows vs {enc_rows} x {beams} encoder '
+                       'rows')
+    return FusedSampleStep(self, params, encoded, enc_tokens, **kw)
+
+
+class FusedSampleStep:
+  """Whole temperature_sample iterations as replays of one captured HIP graph
+  (decoder step on the current tokens, token choice, bookkeeping, loop flag).
+  Owns the self-attention caches of its rows as one block
+  [layers, 2, rows, H, 64, L].  The host refills a ring of Gumbel noise for
+  the next `ring` steps, enqueues that many replays, and only then reads the
+  flag back; replays enqueued after the last row ended change nothing."""
+
+  def __init__(self, module, params, encoded, enc_tokens, *, sequences,
+               cur_index, cur_token, ended, log_prob, max_decode_len,
+               initial_eos_count, temperature, all_ended, eos_id, topk, topp,
+               rescale, noise_source=None, ring=8):
+    from t5x_amd import _lib
+    self._lib = _lib
+    cfg, dev = module.config, module._dev()
+    self.module, self.device = module, dev
+    w = module.decoder_weights(params)
+    if isinstance(encoded, BeamShared):
+      beams, enc, enc_tok = encoded.beams, encoded.x, enc_tokens.x
+    else:
+      beams, enc, enc_tok = 1, encoded, enc_tokens
+    enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
+        enc_tok, torch.Tensor) else enc_tok.to(dev)
+    cross = module._cross_kv(w, enc, enc_tok, beams)
+    R, S = sequences.shape
+    act = w.act_dtype
+    el = 16 // torch.empty((), dtype=act).element_size()
+    self.L = L = (S - 2 + el - 1) // el * el
+    nl = cfg.num_decoder_layers
+    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
+                          dtype=act, device=dev)
+    self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
+    self.bufs = _StepBuffers(cfg, R, dev, act)
+    self.keep_going = torch.ones((), dtype=torch.int32, device=dev)
+    self.step_count = torch.zeros((), dtype=torch.int32, device=dev)
+    self.tokens = torch.empty((R,), dtype=torch.int32, device=dev)
+    self.tok_lp = torch.empty((R,), dtype=torch.float32, device=dev)
+    self.all_ended = all_ended
+    self.noise_source, self.ring = noise_source, int(ring)
+    # A row ends at the latest in the iteration that writes its last position,
+    # so no more than max(max_decode_len) iterations ever run (and no noise is
+    # asked for beyond them).
+    self.max_steps = int(max_decode_len.max().item())
+    self.noise = None
+    if noise_source is not None:
+      self.noise = torch.empty((self.ring, R, cfg.vocab_size),
+                               dtype=torch.float32, device=dev)
+    layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
+    self.model = module._model_step(w, cross, self.bufs, layer_caches,
+                                    self.cache_index, R, beams, L,
+                                    gate=self.keep_going)
+    P = _lib.ptr
+    st = _lib.SampleStep()
+    st.sequences, st.cur_index, st.cur_token = (P(sequences), P(cur_index),
+                                                P(cur_token))
+    st.ended, st.log_prob = P(ended), P(log_prob)
+    st.max_decode_len, st.initial_eos_count = (P(max_decode_len),
+                                               P(initial_eos_count))
+    st.temperature, st.gumbel = P(temperature), P(self.noise)
+    st.noise_ring = self.ring
+    st.step_count, st.tokens, st.token_logprobs = (
+        P(self.step_count), P(self.tokens), P(self.tok_lp))
+    st.all_ended, st.keep_going = P(all_ended), P(self.keep_going)
+    st.S, st.eos_id, st.topk = S, int(eos_id), int(topk)
+    st.rescale, st.topp = int(bool(rescale)), float(topp)
+    self.sample = st
+    self._keepalive = (sequences, cur_index, cur_token, ended, log_prob,
+                       max_decode_len, initial_eos_count, temperature)
+    self.stream = torch.cuda.Stream(device=dev)
+    self.graph = None
+    self.step = 0
+    self._capture()
+
+  def _enqueue(self):
+    self._lib.call('t5d_temperature_sample_step', self.stream.cuda_stream,
+                   self.model, self.sample)
+
+  def _capture(self):
+    lib = self._lib
+    self.stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(self.stream):
+      # First launches load the code objects; with the gate closed they
+      # compute nothing.
+      self.keep_going.zero_()
+      self._enqueue()
+      self.stream.synchronize()
+      lib.call('t5d_graph_begin', self.stream.cuda_stream)
+      try:
+        self._enqueue()
+      finally:
+        handle = ctypes_void_p()
+        lib.call('t5d_graph_end', self.stream.cuda_stream, handle_ref(handle))
+      self.graph = handle
+      self.keep_going.fill_(1)
+    self.stream.synchronize()
+
+  def run(self):
+    """Runs the loop to its end (every row ended)."""
+    lib = self._lib
+    with torch.cuda.stream(self.stream):
+      while self.step < self.max_steps:
+        n = min(self.ring, self.max_steps - self.step)
+        if self.noise is not None:
+          for step in range(self.step, self.step + n):
+            g = self.noise_source.noise(step, tuple(self.noise.shape[1:]))
+            self.noise[step % self.ring].copy_(
+                torch.as_tensor(g, device=self.device).to(torch.float32))
+        for _ in range(n):
+          lib.call('t5d_graph_launch', self.graph, self.stream.cuda_stream)
+        self.step += n
+        self.stream.synchronize()
+        if int(self.all_ended.item()):
+          break
+    torch.cuda.current_stream().wait_stream(self.stream)
+    return int(self.step_count.item())
+
+  def cache_tree(self):
+    """The caches in the reference's tree layout."""
+    self.stream.synchronize()
+    nl = self.kv.shape[0]
+    return {'decoder': {
+        f'layers_{i}': {'self_attention': {
+            'cached_key': self.kv[i, 0], 'cached_value': self.kv[i, 1],
+            'cache_index': self.cache_index[i]}} for i in range(nl)}}
+
+  def __del__(self):
+    try:
+      if self.graph is not None:
+        self._lib.call('t5d_graph_destroy', self.graph)
+    except Exception:  # pylint: disable=broad-except
+      pass
+
+
 class _BeamLane:
   """One independent slice [b0, b1) of the batch: its own caches, activations,
   loop flag, position counter, stream and captured graph."""

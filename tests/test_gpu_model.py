@@ -423,6 +423,54 @@ def test_fused_loop_early_stop_is_independent_of_check_interval(check_every,
   assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
 
 
+class _SuppliedNoise:
+  """Pre-generated Gumbel noise [steps, rows, vocab], one slice per step."""
+
+  def __init__(self, g):
+    self.g = g
+
+  def noise(self, step, shape):
+    assert tuple(self.g.shape[1:]) == tuple(shape)
+    return self.g[step]
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+@pytest.mark.parametrize('eos_bias,kw', [
+    (0.0, dict(temperature=0.0)),
+    (0.0, dict(temperature=0.7, topk=40)),
+    (6.0, dict(temperature=0.7, topk=40)),
+    (0.0, dict(temperature=1.0, topk=0, topp=0.8)),
+    (6.0, dict(temperature=0.9, topk=5, num_decodes=3)),
+    (0.0, dict(temperature=0.0, max_decode_steps=5)),
+    (0.0, dict(temperature=np.array([0.0, 0.5, 1.0], np.float32), topk=7,
+               rescale_log_probs=False)),
+])
+def test_fused_sampling_loop_equals_generic_loop(dtype, eos_bias, kw):
+  """temperature_sample as replays of the captured step (fresh zero cache)
+  against the kernel-per-call loop (a plain dict cache), same noise: sequences
+  and log-probs must be identical, also when rows end long before the last
+  replay that was enqueued."""
+  from t5x_amd import decoding
+  B, L = 3, 21
+  K = kw.get('num_decodes', 1)
+  module, fn = _decode_setup(dtype, B, K, 16, L, seed=5, eos_bias=eos_bias)
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(17)
+  u = torch.rand((L + 2, B * K, module.config.vocab_size), generator=gen,
+                 device='cuda').clamp_min(1e-30)
+  noise = _SuppliedNoise(-torch.log(-torch.log(u)))
+  inputs = np.zeros((B, L), np.int32)
+  want, wlp = decoding.temperature_sample(
+      inputs, dict(module.init_cache(B, L)), fn, 1, decode_rng=noise, **kw)
+  got, glp = decoding.temperature_sample(
+      inputs, module.init_cache(B, L), fn, 1, decode_rng=noise, **kw)
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp))
+  if eos_bias and K == 1:
+    lens = (host(want) != 0).sum(-1)
+    assert lens.max() < L - 8, lens  # the case does stop early
+
+
 def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
   """The reference's host loop (get_infer_fn) around predict_batch_with_aux:
   5 examples at batch 2 (one pad), float32 so tokens are exact."""
