@@ -28,12 +28,17 @@ import numpy as np
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor peak
 
 CONFIGS = {
-    # name: (size, batch, beams, enc_len, enc_min_len, max_decode_len, dtype,
-    #        weight_dtype)
-    'base-beam4': ('base', 32, 4, 512, 128, 128, 'bfloat16', None),
-    'xl-int8-beam4': ('xl', 16, 4, 512, 512, 128, 'bfloat16', 'int8'),
-    'large-greedy': ('large', 64, 1, 512, 512, 256, 'bfloat16', None),
+    # name: (size, batch, decodes per item, enc_len, enc_min_len,
+    #        max_decode_len, dtype, weight_dtype, loop)
+    # loop: 'beam' or ('sample', temperature, topk)
+    'base-beam4': ('base', 32, 4, 512, 128, 128, 'bfloat16', None, 'beam'),
+    'xl-int8-beam4': ('xl', 16, 4, 512, 512, 128, 'bfloat16', 'int8', 'beam'),
+    'large-sample': ('large', 64, 1, 512, 512, 256, 'bfloat16', None,
+                     ('sample', 0.7, 40)),
+    'xxl-greedy': ('xxl', 128, 1, 1024, 1024, 256, 'bfloat16', None,
+                   ('sample', 0.0, 0)),
 }
+DEFAULT_CONFIG = 'base-beam4'
 
 
 def parse_args():
@@ -41,7 +46,7 @@ def parse_args():
   ap.add_argument('--gpus', type=int, default=1)
   ap.add_argument('--steps', type=int, default=256)
   ap.add_argument('--warmup', type=int, default=128)
-  ap.add_argument('--config', default='base-beam4', choices=sorted(CONFIGS))
+  ap.add_argument('--config', default=DEFAULT_CONFIG, choices=sorted(CONFIGS))
   ap.add_argument('--seed', type=int, default=0)
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--lanes', type=int, default=None,
@@ -61,8 +66,9 @@ class Workload:
     import torch
     from t5x_amd import decoding, models, network
     self.torch, self.decoding = torch, decoding
-    size, B, K, E, Emin, L, dtype, wdt = CONFIGS[name]
+    size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[name]
     self.name, self.B, self.K, self.E, self.L = name, B, K, E, L
+    self.loop_kind, self.seed = loop, seed
     self.cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
     dev = torch.device('cuda')
     self.params = network.init_params(self.cfg, seed, dev, with_encoder=False)
@@ -94,7 +100,31 @@ class Workload:
         self.inputs, cache, self.tokens_to_logits, eos_id=1,
         num_decodes=self.K, alpha=0.6)
 
+  def run_sample_steps(self, n):
+    """Exactly n temperature_sample iterations: whole decodes of L steps, then
+    one decode limited to the remainder by max_decode_steps.  A decode that
+    ended early (every row hit EOS) would make the count wrong and raises."""
+    torch = self.torch
+    _, temperature, topk = self.loop_kind
+    done = 0
+    while done < n:
+      take = min(n - done, self.L)
+      cache = self.module.init_cache(self.B, self.L)
+      seqs, _ = self.decoding.temperature_sample(
+          self.inputs, cache, self.tokens_to_logits, 1,
+          decode_rng=self.seed + done, num_decodes=self.K,
+          temperature=temperature, topk=topk,
+          max_decode_steps=take if take < self.L else None)
+      if not bool((seqs[:, :, take - 1] != 0).any()):
+        raise RuntimeError(f'sampling decode ended before step {take}')
+      done += take
+
   def run_steps(self, n):
+    if self.loop_kind != 'beam':
+      return self.run_sample_steps(n)
+    return self.run_beam_steps(n)
+
+  def run_beam_steps(self, n):
     """Runs exactly n loop iterations, starting a new decode whenever the
     current one has produced its max_decode_len tokens.  The loop condition is
     evaluated on the device after every iteration; it is read back once per
@@ -122,15 +152,18 @@ class Workload:
                          'step count of this run would be wrong')
 
   # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
-  def cross_attention_bytes(self):
-    """Valid K and V rows once per batch item, the residual-stream rows and
-    layer-norm scale in, the query kernel once, the attention output out."""
+  def cross_attention_bytes(self, fused=True):
+    """Valid K and V rows once per batch item and the attention output out;
+    in: the residual-stream rows, the layer-norm scale and the query kernel
+    (fused projection), or the projected queries."""
     s = 2  # bf16
     hd = self.cfg.num_heads * self.cfg.head_dim
     d = self.cfg.emb_dim
     R = self.B * self.K
-    return (int(self.enc_lens.sum()) * hd * 2 * s + R * d * s + d * s +
-            d * hd * s + R * hd * s)
+    kv = int(self.enc_lens.sum()) * hd * 2 * s
+    if fused:
+      return kv + R * d * s + d * s + d * hd * s + R * hd * s
+    return kv + 2 * R * hd * s
 
   def self_attention_bytes(self, t):
     s = 2
@@ -191,31 +224,46 @@ def measured_traffic(name):
 
 def roofline_cross_attention(w, reps_per_layer=4):
   """The step's largest single stream of HBM bytes per launch: the
-  cross-attention kernel (pre-attention layer norm and query projection fused
-  in) over the encoder K/V, one launch per layer per step, same shape every
-  step.  Replayed here back to back, walking the layers so no launch finds its
-  K/V in a cache, and timed with HIP events on the launch stream."""
+  cross-attention kernel over the encoder K/V (with the pre-attention layer
+  norm and the query projection fused in where the model width allows), one
+  launch per layer per step, same shape every step.  Replayed here back to
+  back, walking the layers so no launch finds its K/V in a cache, and timed
+  with HIP events on the launch stream."""
   from t5x_amd import ops
   torch = w.torch
   cross = w.module._cross[1]
   R = w.B * w.K
-  hd = w.cfg.num_heads * w.cfg.head_dim
-  x = torch.randn((R, w.cfg.emb_dim), device='cuda').to(w.encoded.dtype)
-  out = torch.empty((R, hd), dtype=x.dtype, device='cuda')
+  cfg = w.cfg
+  hd = cfg.num_heads * cfg.head_dim
+  act = w.encoded.dtype
+  x = torch.randn((R, cfg.emb_dim), device='cuda').to(act)
+  q = torch.randn((R, hd), device='cuda').to(act)
+  out = torch.empty((R, hd), dtype=act, device='cuda')
   layers = w.weights.layers
   nl = len(cross['k'])
+  fused = (w.weights.layers[0]['cross_q'].w_dtype == 1 and cross['E'] <= 512
+           and cfg.emb_dim <= 1024)
   state = {'i': 0}
 
   def launch():
     i = state['i'] = (state['i'] + 1) % nl  # walk the layers: no cache reuse
-    ops.cross_attention_step_norm_q(x, layers[i]['ln_cross'],
-                                    layers[i]['cross_q'], cross['k'][i],
-                                    cross['v'][i], cross['enc_len'], w.K, out)
+    if fused:
+      ops.cross_attention_step_norm_q(x, layers[i]['ln_cross'],
+                                      layers[i]['cross_q'], cross['k'][i],
+                                      cross['v'][i], cross['enc_len'], w.K, out)
+    else:
+      ops.cross_attention_step(q, cross['k'][i], cross['v'][i],
+                               cross['enc_len'], w.K, out)
 
-  sec = time_kernel(torch, launch, reps_per_layer * nl)
-  nbytes = w.cross_attention_bytes()
+  reps = max(1, min(reps_per_layer, 96 // nl))
+  sec = time_kernel(torch, launch, reps * nl)
+  nbytes = w.cross_attention_bytes(fused)
   achieved = nbytes / sec / 1e9
-  return {'kernel': 'cross_attn_mfma_kernel<4,4,3>', 'bound': 'hbm',
+  if fused:
+    name = 'cross_attn_mfma_kernel<4,4,%d>' % ((cfg.emb_dim // 64 + 3) // 4)
+  else:
+    name = 'cross_attn_mfma_kernel (query projected separately)'
+  return {'kernel': name, 'bound': 'hbm',
           'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS,
           'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBPS, 4),
           'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes,
@@ -239,7 +287,7 @@ def cpu_baseline(name, steps, seed):
   shape (decoder only, cross K/V hoisted as in the GPU path)."""
   from oracle import decoding as odec
   from oracle import t5 as ot5
-  size, B, K, E, Emin, L, dtype, wdt = CONFIGS[name]
+  size, B, K, E, Emin, L, dtype, wdt, _ = CONFIGS[name]
   from t5x_amd import network
   kw = dict(network.T5_1_1[size])
   kw['num_encoder_layers'] = 0
@@ -306,9 +354,18 @@ def main():
   torch.cuda.synchronize()
   elapsed = time.perf_counter() - t0
 
-  size, B, K, E, Emin, L, dtype, wdt = CONFIGS[args.config]
+  size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[args.config]
+  if loop == 'beam':
+    what = f'beam_search decode loop: batch {B} x {K} beams'
+  elif loop[1] > 0:
+    what = (f'temperature_sample decode loop (temperature {loop[1]}, top-k '
+            f'{loop[2]}): batch {B}')
+  else:
+    what = f'temperature_sample decode loop (greedy): batch {B}'
   out = {
-      'metric': 'decoded tokens/sec, T5.1.1-base beam=4 on 1 GPU',
+      'metric': ('decoded tokens/sec, T5.1.1-base beam=4 on 1 GPU'
+                 if args.config == DEFAULT_CONFIG else
+                 f'decoded tokens/sec, {args.config} on 1 GPU'),
       'value': round(B * args.steps / elapsed, 1),
       'unit': 'tokens/s',
       'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -316,14 +373,13 @@ def main():
       'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
       'dtype': 'bf16' if wdt is None else f'bf16 act / {wdt} weights',
       'data': 'synthetic',
-      'config': {'workload': f'T5.1.1-{size} beam_search decode loop: batch '
-                             f'{B} x {K} beams, encoder {E} ({Emin}..{E} '
+      'config': {'workload': f'T5.1.1-{size} {what}, encoder {E} ({Emin}..{E} '
                              f'valid), max decode length {L}',
                  'name': args.config, 'beam_rows': B * K,
                  'rows_x_steps_per_s': round(B * K * args.steps / elapsed, 1)},
       'roofline': roofline_cross_attention(w),
   }
-  if not args.no_cpu_baseline:
+  if not args.no_cpu_baseline and loop == 'beam':
     out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
   print(json.dumps(out))
 

@@ -95,7 +95,8 @@ __device__ long long t5d_probe_buf[64 * 16];
 // bits as the stand-alone dense layer given the same row statistics.  NJ is
 // the number of k-tile pairs per wavefront (d / 256, rounded up).
 template <int NQP, int WM, int NJ>
-__global__ void __launch_bounds__(64 * WM, NJ > 0 ? 2 : 1)  // fused: 2 WGs per CU
+// fused, d <= 768: 2 workgroups per CU (256 registers hold both streams)
+__global__ void __launch_bounds__(64 * WM, NJ > 0 && NJ <= 3 ? 2 : 1)
 cross_attn_mfma_kernel(AttnMfmaArgs a) {
   constexpr int REP = 16 / NQP;   // copies of each query column
   constexpr int TPL = 8 / REP;    // score tiles a lane keeps
@@ -191,7 +192,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   // B operand of K·Q^T: lane (col n16 -> query q, g) holds Q[q][32c + 8g .. +8].
   Frag16 qb[2];
   if constexpr (!FQ) {
-    load_v();
+    // 16 wavefronts leave 128 registers each: V follows once K is consumed
+    if constexpr (WM <= 8) load_v();
     const bool qrow = q < a.nq;
     const bf16_t* qp = a.q + (size_t)(b * a.nq + (qrow ? q : 0)) * a.q_stride +
                        h * kHeadDim + 8 * g;
@@ -299,6 +301,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       }
     }
 
+  if constexpr (!FQ && WM > 8) load_v();
   T5D_STAMP(2);
   // Softmax over all positions of the workgroup for query q.  The 16 lanes
   // that share q differ in lane bits {2,3 (if REP == 4) | 3 (REP == 2)} and

@@ -927,6 +927,302 @@ sample_tokens_kernel(SampleArgs a) {
   }
 }
 
+// Fast path of sample_tokens_kernel for 16-byte aligned rows of at most 32768
+// elements with V % 4 == 0: 1024 threads per row, the scaled row lives in
+// registers (8 float4 per thread), so logits and noise are read once.
+// The top-k cutoff (the k-th largest scaled logit, ties kept) is found by
+// threshold: with m = ceil(k / 16), the smallest over the 16 wavefronts of the
+// m-th largest per-thread maximum of a wavefront is a bound that at least k
+// elements reach; the few elements at or above it go to a list in LDS, where
+// the k-th largest is read off by counting.  More than kTopkCap such elements
+// (long runs of equal values) fall back to the radix select, on registers.
+__device__ __forceinline__ float kth_largest_by_radix(const float4 (&y)[8],
+                                                      int nvec, int tid, int k,
+                                                      unsigned* hist,
+                                                      int* iscratch) {
+  uint32_t prefix = 0, mask = 0;
+  int want = k;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u * 1024 + tid < nvec) {
+        const float e[4] = {y[u].x, y[u].y, y[u].z, y[u].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t key = order_key(e[c]);
+          if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xFF], 1u);
+        }
+      }
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int digit = 255, acc = 0;
+      for (; digit > 0; --digit) {
+        if (acc + (int)hist[digit] >= want) break;
+        acc += hist[digit];
+      }
+      iscratch[0] = digit;
+      iscratch[1] = want - acc;
+    }
+    __syncthreads();
+    prefix |= ((uint32_t)iscratch[0]) << shift;
+    mask |= 0xFFu << shift;
+    want = iscratch[1];
+    __syncthreads();
+  }
+  return key_to_float(prefix);
+}
+
+__global__ void __launch_bounds__(1024)
+sample_tokens_fast_kernel(SampleArgs a) {
+  __shared__ Cand cscratch[16];
+  __shared__ float fscratch[16];
+  __shared__ double dscratch[16];
+  __shared__ int iscratch[4];
+  __shared__ unsigned hist[256];
+  __shared__ float s_lv[kTopkCap];
+  __shared__ int s_count;
+  __shared__ float s_cut;
+  T5D_GATED(a.gate);
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int V = a.V, nvec = V >> 2;
+  const float4 kPad = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  const float4* x4 = reinterpret_cast<const float4*>(a.logits + (size_t)r * V);
+  float4 y[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int vi = u * 1024 + tid;
+    y[u] = vi < nvec ? x4[vi] : kPad;
+  }
+  const float T = a.temperature[r];
+  const float kMinT = 1e-4f;
+  if (tid == 0) s_count = 0;
+
+  if (!(T > kMinT)) {  // greedy (t5x/decoding.py:575-592)
+    Cand best = {-INFINITY, 0x7FFFFFFF};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int j = 4 * (u * 1024 + tid);  // ascending within the thread
+      if (y[u].x > best.v) { best.v = y[u].x; best.i = j; }
+      if (y[u].y > best.v) { best.v = y[u].y; best.i = j + 1; }
+      if (y[u].z > best.v) { best.v = y[u].z; best.i = j + 2; }
+      if (y[u].w > best.v) { best.v = y[u].w; best.i = j + 3; }
+    }
+    best = block_best(best, cscratch);
+    float lp = 0.f;
+    if (!a.rescale) {
+      double sum = 0.0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        sum += (double)expf(y[u].x - best.v);
+        sum += (double)expf(y[u].y - best.v);
+        sum += (double)expf(y[u].z - best.v);
+        sum += (double)expf(y[u].w - best.v);
+      }
+      sum = block_sum_f64(sum, dscratch);
+      lp = (best.v - best.v) - (float)log(sum);
+    }
+    if (tid == 0) { a.tokens[r] = best.i; a.logprobs[r] = lp; }
+    return;
+  }
+
+  const float Tm = fmaxf(T, kMinT);
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    y[u].x /= Tm; y[u].y /= Tm; y[u].z /= Tm; y[u].w /= Tm;
+  }
+
+  float cutoff = -INFINITY;  // keep scaled >= cutoff
+  if (a.topk > 0 && a.topk < V) {
+    const int m = (a.topk + 15) >> 4;
+    bool counted = false;
+    if (m <= 8) {
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        tmax = fmaxf(fmaxf(tmax, fmaxf(y[u].x, y[u].y)), fmaxf(y[u].z, y[u].w));
+      // m-th largest per-thread maximum of this wavefront
+      float rest = tmax, wm = -INFINITY;
+      for (int it = 0; it < m; ++it) {
+        wm = wave_max(rest);
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(rest == wm);
+        if (lane == (int)__builtin_ctzll(hit | (1ull << 63))) rest = -INFINITY;
+      }
+      if (lane == 0) fscratch[wave] = wm;
+      __syncthreads();
+      float bound = fscratch[0];
+      for (int w = 1; w < 16; ++w) bound = fminf(bound, fscratch[w]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float top = fmaxf(fmaxf(y[u].x, y[u].y), fmaxf(y[u].z, y[u].w));
+        if (u * 1024 + tid < nvec && top >= bound) {
+          const float e[4] = {y[u].x, y[u].y, y[u].z, y[u].w};
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            if (e[c] >= bound) {
+              const int p = atomicAdd(&s_count, 1);
+              if (p < kTopkCap) s_lv[p] = e[c];
+            }
+          }
+        }
+      }
+      __syncthreads();
+      const int ncand = s_count;
+      if (ncand >= a.topk && ncand <= kTopkCap) {
+        if (tid < ncand) {
+          const float v = s_lv[tid];
+          int gt = 0, ge = 0;
+          for (int c = 0; c < ncand; ++c) {
+            const float o = s_lv[c];
+            gt += o > v ? 1 : 0;
+            ge += o >= v ? 1 : 0;
+          }
+          // the k-th largest value; equal candidates all write the same bits
+          if (gt < a.topk && a.topk <= ge) s_cut = v;
+        }
+        __syncthreads();
+        cutoff = s_cut;
+        counted = true;
+      }
+    }
+    if (!counted)
+      cutoff = kth_largest_by_radix(y, nvec, tid, a.topk, hist, iscratch);
+  }
+  // apply the top-k mask in place (t5x/decoding.py:556-562: others = -1e7)
+  if (cutoff > -INFINITY) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u * 1024 + tid < nvec) {
+        y[u].x = y[u].x >= cutoff ? y[u].x : kNegInf;
+        y[u].y = y[u].y >= cutoff ? y[u].y : kNegInf;
+        y[u].z = y[u].z >= cutoff ? y[u].z : kNegInf;
+        y[u].w = y[u].w >= cutoff ? y[u].w : kNegInf;
+      }
+    }
+  }
+
+  if (a.topp > 0.f) {
+    // t5x/binary_search.py:230-299 — largest threshold whose kept mass >= p,
+    // found by the same 32-step search over float bit patterns.
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      mx = fmaxf(fmaxf(mx, fmaxf(y[u].x, y[u].y)), fmaxf(y[u].z, y[u].w));
+    const float smax = block_max_f32(mx, fscratch);
+    double sum = 0.0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      sum += (double)expf(y[u].x - smax);
+      sum += (double)expf(y[u].y - smax);
+      sum += (double)expf(y[u].z - smax);
+      sum += (double)expf(y[u].w - smax);
+    }
+    const float ssum = (float)block_sum_f64(sum, dscratch);
+    float4 pr[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      pr[u].x = expf(y[u].x - smax) / ssum;
+      pr[u].y = expf(y[u].y - smax) / ssum;
+      pr[u].z = expf(y[u].z - smax) / ssum;
+      pr[u].w = expf(y[u].w - smax) / ssum;
+    }
+    int32_t bits = 0;
+    for (int it = 0; it < 32; ++it) {
+      const int32_t mid = it == 0 ? bits : (bits | (int32_t)(1u << (31 - it)));
+      const int32_t pat = mid ^ (mid < 0 ? 0x7FFFFFFF : 0);
+      const bool finite = (pat & 0x7F800000) != 0x7F800000;
+      bool pred;
+      if (finite) {
+        const float thr = __int_as_float(pat);
+        double mass = 0.0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (pr[u].x >= thr) mass += (double)pr[u].x;
+          if (pr[u].y >= thr) mass += (double)pr[u].y;
+          if (pr[u].z >= thr) mass += (double)pr[u].z;
+          if (pr[u].w >= thr) mass += (double)pr[u].w;
+        }
+        mass = block_sum_f64(mass, dscratch);
+        pred = (float)mass < a.topp;
+      } else {
+        pred = pat >= 0;
+      }
+      if (it == 0) {
+        if (pred) bits |= (int32_t)0x80000000u;
+      } else if (!pred) {
+        bits |= (int32_t)(1u << (31 - it));
+      }
+    }
+    const int32_t pat = bits ^ (bits < 0 ? 0x7FFFFFFF : 0);
+    const float pcut = __int_as_float(pat);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u * 1024 + tid < nvec) {
+        y[u].x = pr[u].x >= pcut ? y[u].x : kNegInf;
+        y[u].y = pr[u].y >= pcut ? y[u].y : kNegInf;
+        y[u].z = pr[u].z >= pcut ? y[u].z : kNegInf;
+        y[u].w = pr[u].w >= pcut ? y[u].w : kNegInf;
+      }
+    }
+  }
+
+  // argmax(masked + gumbel), and log-softmax statistics of the masked row (or
+  // of the raw logits when log-probs are not rescaled).
+  const int slot = a.noise_step ? *a.noise_step % a.noise_ring : 0;
+  const float4* g4 = reinterpret_cast<const float4*>(
+      a.gumbel + ((size_t)slot * a.R + r) * V);
+  Cand best = {-INFINITY, 0x7FFFFFFF};
+  float mx = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int vi = u * 1024 + tid;
+    if (vi < nvec) {
+      const float4 g = g4[vi];
+      const int j = 4 * vi;
+      const float z0 = y[u].x + g.x, z1 = y[u].y + g.y;
+      const float z2 = y[u].z + g.z, z3 = y[u].w + g.w;
+      if (z0 > best.v) { best.v = z0; best.i = j; }
+      if (z1 > best.v) { best.v = z1; best.i = j + 1; }
+      if (z2 > best.v) { best.v = z2; best.i = j + 2; }
+      if (z3 > best.v) { best.v = z3; best.i = j + 3; }
+    }
+    // without rescaling the log-probs are those of the raw logits, read again
+    const float4 w = a.rescale ? y[u] : (vi < nvec ? x4[vi] : kPad);
+    mx = fmaxf(fmaxf(mx, fmaxf(w.x, w.y)), fmaxf(w.z, w.w));
+  }
+  best = block_best(best, cscratch);
+  mx = block_max_f32(mx, fscratch);
+  double sum = 0.0;
+  float wtok = 0.f;
+  bool mine = false;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const float4 w =
+        a.rescale ? y[u] : (u * 1024 + tid < nvec ? x4[u * 1024 + tid] : kPad);
+    sum += (double)expf(w.x - mx);
+    sum += (double)expf(w.y - mx);
+    sum += (double)expf(w.z - mx);
+    sum += (double)expf(w.w - mx);
+    const int j = 4 * (u * 1024 + tid);
+    if (best.i == j) { wtok = w.x; mine = true; }
+    if (best.i == j + 1) { wtok = w.y; mine = true; }
+    if (best.i == j + 2) { wtok = w.z; mine = true; }
+    if (best.i == j + 3) { wtok = w.w; mine = true; }
+  }
+  sum = block_sum_f64(sum, dscratch);
+  __syncthreads();
+  if (mine) fscratch[0] = wtok;  // exactly one thread holds the token
+  __syncthreads();
+  wtok = fscratch[0];
+  if (tid == 0) {
+    a.tokens[r] = best.i;
+    a.logprobs[r] = (wtok - mx) - (float)log(sum);
+  }
+}
+
 struct SampleUpdateArgs {
   const int32_t* tokens;
   const float* token_logprobs;
@@ -949,12 +1245,16 @@ struct SampleUpdateArgs {
   const int32_t* gate;
 };
 
-__global__ void __launch_bounds__(256)
+// One workgroup; a wavefront per row (rows are dealt round-robin), its lanes
+// count the row's EOS tokens in parallel.
+constexpr int kSampleUpdateThreads = 1024;
+__global__ void __launch_bounds__(kSampleUpdateThreads)
 sample_update_kernel(SampleUpdateArgs a) {
-  __shared__ int iscratch[4];
+  __shared__ int iscratch[kSampleUpdateThreads / 64];
   T5D_GATED(a.gate);
-  int not_ended = 0;
-  for (int r = threadIdx.x; r < a.R; r += 256) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int not_ended = 0;  // rows of this wavefront still running (all lanes agree)
+  for (int r = wave; r < a.R; r += kSampleUpdateThreads / 64) {
     int32_t* seq = a.sequences + (size_t)r * a.S;
     const int mdl = a.max_decode_len[r];
     const int i = min(a.cur_index[r], mdl);
@@ -962,24 +1262,34 @@ sample_update_kernel(SampleUpdateArgs a) {
     const bool oop = next_input == 0;
     const bool was_ended = a.ended[r] != 0;
     const int tok = oop ? a.tokens[r] : next_input;
-    if (oop && !was_ended) a.log_prob[r] = a.log_prob[r] + a.token_logprobs[r];
     const int out_tok = was_ended ? 0 : tok;
-    seq[i + 1] = out_tok;
+    // EOS count of the row with position i + 1 already holding out_tok
     int eos = 0;
-    for (int j = 0; j < a.S; ++j) eos += (seq[j] == a.eos_id);
+    for (int j = lane; j < a.S; j += 64)
+      eos += ((j == i + 1 ? out_tok : seq[j]) == a.eos_id) ? 1 : 0;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) eos += __shfl_xor(eos, o, 64);
     const bool ended = was_ended || (eos > a.initial_eos_count[r]) ||
                        (i >= mdl - 1);
-    a.ended[r] = ended ? 1 : 0;
-    a.cur_index[r] = i + 1;
-    a.cur_token[r] = out_tok;
+    if (lane == 0) {
+      if (oop && !was_ended)
+        a.log_prob[r] = a.log_prob[r] + a.token_logprobs[r];
+      seq[i + 1] = out_tok;
+      a.ended[r] = ended ? 1 : 0;
+      a.cur_index[r] = i + 1;
+      a.cur_token[r] = out_tok;
+    }
     if (!ended) ++not_ended;
   }
-  not_ended = block_sum_i32(not_ended, iscratch);
+  if (lane == 0) iscratch[wave] = not_ended;
+  __syncthreads();
   if (threadIdx.x == 0) {
-    *a.all_ended = not_ended == 0 ? 1 : 0;
+    int total = 0;
+    for (int w = 0; w < kSampleUpdateThreads / 64; ++w) total += iscratch[w];
+    *a.all_ended = total == 0 ? 1 : 0;
     if (a.step_count) *a.step_count += 1;
-    // the gate was read by every thread before the reduction's barriers
-    if (a.keep_going) *a.keep_going = not_ended == 0 ? 0 : 1;
+    // the gate was read by every thread before the barrier above
+    if (a.keep_going) *a.keep_going = total == 0 ? 0 : 1;
   }
   if ((int)threadIdx.x < a.n_counters) a.counters[threadIdx.x] += 1;
 }
@@ -1187,6 +1497,15 @@ int t5d::launch_beam_tail(hipStream_t s, const t5d_beam_state* state, int B,
   return T5D_OK;
 }
 
+static void launch_sample_tokens(hipStream_t s, const SampleArgs& a, int R) {
+  const bool aligned = ((uintptr_t)a.logits % 16) == 0 &&
+                       (a.gumbel == nullptr || ((uintptr_t)a.gumbel % 16) == 0);
+  if (a.V % 4 == 0 && a.V <= 32768 && aligned)
+    hipLaunchKernelGGL(sample_tokens_fast_kernel, dim3(R), dim3(1024), 0, s, a);
+  else
+    hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0, s, a);
+}
+
 extern "C" int t5d_sample_tokens(void* stream, const float* logits,
                                  const float* gumbel, const float* temperature,
                                  int32_t* tokens, float* logprobs, int R,
@@ -1203,8 +1522,7 @@ extern "C" int t5d_sample_tokens(void* stream, const float* logits,
   a.tokens = tokens; a.logprobs = logprobs;
   a.V = V; a.topk = topk; a.rescale = rescale; a.topp = topp;
   a.noise_step = nullptr; a.noise_ring = 1; a.R = R; a.gate = tls_gate;
-  hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0,
-                     as_stream(stream), a);
+  launch_sample_tokens(as_stream(stream), a, R);
   T5D_CHECK_LAUNCH("t5d_sample_tokens");
   return T5D_OK;
 }
@@ -1218,7 +1536,7 @@ int t5d::launch_sample_step(hipStream_t s, const float* logits,
   a.V = V; a.topk = st->topk; a.rescale = st->rescale; a.topp = st->topp;
   a.noise_step = st->step_count; a.noise_ring = st->noise_ring; a.R = R;
   a.gate = tls_gate;
-  hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0, s, a);
+  launch_sample_tokens(s, a, R);
   T5D_CHECK_LAUNCH("sample step (tokens)");
   SampleUpdateArgs u;
   u.tokens = st->tokens; u.token_logprobs = st->token_logprobs;
@@ -1229,7 +1547,8 @@ int t5d::launch_sample_step(hipStream_t s, const float* logits,
   u.R = R; u.S = st->S; u.eos_id = st->eos_id;
   u.keep_going = st->keep_going; u.step_count = st->step_count;
   u.counters = counters; u.n_counters = n_counters; u.gate = tls_gate;
-  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(256), 0, s, u);
+  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(kSampleUpdateThreads),
+                     0, s, u);
   T5D_CHECK_LAUNCH("sample step (update)");
   return T5D_OK;
 }
@@ -1254,8 +1573,8 @@ extern "C" int t5d_sample_update(void* stream, const int32_t* tokens,
   a.R = R; a.S = S; a.eos_id = eos_id;
   a.keep_going = nullptr; a.step_count = nullptr; a.counters = nullptr;
   a.n_counters = 0; a.gate = tls_gate;
-  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(256), 0,
-                     as_stream(stream), a);
+  hipLaunchKernelGGL(sample_update_kernel, dim3(1), dim3(kSampleUpdateThreads),
+                     0, as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_sample_update");
   return T5D_OK;
 }

@@ -513,6 +513,51 @@ def test_sample_tokens_topk(ops, V, topk, temp, rescale):
   np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize('V', [1000, 32128, 32127])
+@pytest.mark.parametrize('topp', [0.3, 0.9])
+@pytest.mark.parametrize('rescale', [True, False])
+def test_sample_tokens_topp_vocab(ops, V, topp, rescale):
+  """Top-p at vocabulary width against the oracle's mask; probabilities near
+  the threshold can fall either side of it by a rounding of the softmax, so
+  rows whose oracle mask has an element within 1e-6 (relative) of the
+  threshold probability are skipped (none with these seeds).  V = 32127 takes
+  the generic kernel (rows not 16-byte aligned)."""
+  rs = np.random.RandomState(V + int(10 * topp))
+  R = 5
+  logits = (3 * rs.randn(R, V)).astype(np.float32)
+  g = odec.GumbelNoise(seed=5).noise(0, (R, V))
+  temp = np.float32(0.8)
+  temps = np.full((R,), temp, np.float32)
+  tok, lp = ops.sample_tokens(dev(logits), dev(g), dev(temps), 0, topp, rescale)
+  scaled = (logits / temp).astype(np.float32)
+  masked = obs.topp_mask(scaled, np.float32(topp), np.float32(-1e7))
+  want_tok = np.argmax(masked + g, axis=-1)
+  src = masked if rescale else logits
+  want_lp = odec.log_softmax(src)[np.arange(R), want_tok]
+  np.testing.assert_array_equal(host(tok), want_tok)
+  np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize('k', [1, 16, 17, 40, 128, 129, 1000])
+def test_sample_tokens_topk_cutoff_with_ties(ops, k):
+  """The k-th largest as cutoff when it sits inside a run of equal values, for
+  k on both sides of the per-wavefront bound's limits and of the candidate
+  list's capacity: the kept set is everything >= the k-th largest."""
+  V, R = 32128, 3
+  rs = np.random.RandomState(k)
+  logits = rs.randn(R, V).astype(np.float32)
+  logits[0, rs.permutation(V)[:600]] = 5.0     # 600 equal maxima
+  logits[1] = np.round(logits[1] * 4) / 4       # heavy ties everywhere
+  g = odec.GumbelNoise(seed=k).noise(0, (R, V))
+  temps = np.ones((R,), np.float32)
+  tok, lp = ops.sample_tokens(dev(logits), dev(g), dev(temps), k, 0.0, True)
+  masked = obs.topk_mask(logits, k, np.float32(-1e7))
+  want_tok = np.argmax(masked + g, axis=-1)
+  want_lp = odec.log_softmax(masked)[np.arange(R), want_tok]
+  np.testing.assert_array_equal(host(tok), want_tok)
+  np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
+
+
 def test_sample_tokens_topp_table(ops):
   # t5x/binary_search_test.py:143-209 through the kernel: with a huge Gumbel
   # bonus on one index the sampled token reveals whether it survived the mask.
