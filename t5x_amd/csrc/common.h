@@ -99,6 +99,10 @@ __device__ __forceinline__ float dpp_move(float v) {
   return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(
       0, (int)__float_as_uint(v), CTRL, 0xF, 0xF, true));
 }
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
 constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i within 8

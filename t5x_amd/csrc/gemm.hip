@@ -17,6 +17,8 @@
 //     slice comes from HBM once and from that XCD's L2 afterwards.
 // The activation operand is read from L2 in full 128-byte lines (a pair of
 // k-tiles is 64 contiguous bf16 per row).
+#include <cstdlib>
+
 #include "common.h"
 
 namespace t5d {
@@ -499,6 +501,13 @@ static GemmPlan plan_gemm(int M, int K, int N) {
   const int n_tiles = N / 16;
   GemmPlan best = {1, 1, 1, 1};
   double best_cost = 1e30;
+#ifdef T5D_PROBE  // tuning runs force a tile: T5D_GEMM_TILE="mp,nt"
+  if (const char* force = getenv("T5D_GEMM_TILE")) {
+    int mp = 1, nt = 1;
+    if (sscanf(force, "%d,%d", &mp, &nt) == 2)
+      return {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt};
+  }
+#endif
   const int mps[4] = {1, 2, 4, 8};
   const int nts[3] = {1, 2, 4};
   for (int mi = 0; mi < 4; ++mi)

@@ -1245,16 +1245,21 @@ struct SampleUpdateArgs {
   const int32_t* gate;
 };
 
-// One workgroup; a wavefront per row (rows are dealt round-robin), its lanes
-// count the row's EOS tokens in parallel.
+// One workgroup; 16 lanes per row (rows are dealt round-robin to the 64 groups
+// of 16 lanes), which count the row's EOS tokens in parallel.
 constexpr int kSampleUpdateThreads = 1024;
 __global__ void __launch_bounds__(kSampleUpdateThreads)
 sample_update_kernel(SampleUpdateArgs a) {
   __shared__ int iscratch[kSampleUpdateThreads / 64];
   T5D_GATED(a.gate);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int not_ended = 0;  // rows of this wavefront still running (all lanes agree)
-  for (int r = wave; r < a.R; r += kSampleUpdateThreads / 64) {
+  const int group = threadIdx.x >> 4, gl = threadIdx.x & 15;
+  int not_ended = 0;  // rows of this group still running (its 16 lanes agree)
+  for (int r0 = 0; r0 < a.R; r0 += kSampleUpdateThreads / 16) {
+    // whole wavefronts stay in the loop (the reduction below is wave-wide);
+    // groups past the last row work on row 0 and discard the result
+    const bool real = r0 + group < a.R;
+    const int r = real ? r0 + group : 0;
     int32_t* seq = a.sequences + (size_t)r * a.S;
     const int mdl = a.max_decode_len[r];
     const int i = min(a.cur_index[r], mdl);
@@ -1265,13 +1270,12 @@ sample_update_kernel(SampleUpdateArgs a) {
     const int out_tok = was_ended ? 0 : tok;
     // EOS count of the row with position i + 1 already holding out_tok
     int eos = 0;
-    for (int j = lane; j < a.S; j += 64)
+    for (int j = gl; j < a.S; j += 16)
       eos += ((j == i + 1 ? out_tok : seq[j]) == a.eos_id) ? 1 : 0;
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) eos += __shfl_xor(eos, o, 64);
+    eos = lanes16_sum(eos);
     const bool ended = was_ended || (eos > a.initial_eos_count[r]) ||
                        (i >= mdl - 1);
-    if (lane == 0) {
+    if (real && gl == 0) {
       if (oop && !was_ended)
         a.log_prob[r] = a.log_prob[r] + a.token_logprobs[r];
       seq[i + 1] = out_tok;
@@ -1279,8 +1283,11 @@ sample_update_kernel(SampleUpdateArgs a) {
       a.cur_index[r] = i + 1;
       a.cur_token[r] = out_tok;
     }
-    if (!ended) ++not_ended;
+    if (real && gl == 0 && !ended) ++not_ended;
   }
+  // lanes 0, 16, 32, 48 hold their groups' counts
+  not_ended += __shfl_xor(not_ended, 16, 64);
+  not_ended += __shfl_xor(not_ended, 32, 64);
   if (lane == 0) iscratch[wave] = not_ended;
   __syncthreads();
   if (threadIdx.x == 0) {
