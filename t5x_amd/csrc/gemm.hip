@@ -18,6 +18,7 @@
 // The activation operand is read from L2 in full 128-byte lines (a pair of
 // k-tiles is 64 contiguous bf16 per row).
 #include <cstdlib>
+#include <cstring>
 
 #include "common.h"
 
@@ -501,11 +502,17 @@ static GemmPlan plan_gemm(int M, int K, int N) {
   const int n_tiles = N / 16;
   GemmPlan best = {1, 1, 1, 1};
   double best_cost = 1e30;
-#ifdef T5D_PROBE  // tuning runs force a tile: T5D_GEMM_TILE="mp,nt"
+#ifdef T5D_PROBE  // tuning runs force tiles: T5D_GEMM_TILE="K,N,mp,nt;K,N,mp,nt"
   if (const char* force = getenv("T5D_GEMM_TILE")) {
-    int mp = 1, nt = 1;
-    if (sscanf(force, "%d,%d", &mp, &nt) == 2)
-      return {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt};
+    const char* p = force;
+    while (p && *p) {
+      int k = 0, n = 0, mp = 1, nt = 1;
+      if (sscanf(p, "%d,%d,%d,%d", &k, &n, &mp, &nt) == 4 &&
+          (k == 0 || k == K) && (n == 0 || n == N))
+        return {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt};
+      p = strchr(p, ';');
+      if (p) ++p;
+    }
   }
 #endif
   const int mps[4] = {1, 2, 4, 8};
