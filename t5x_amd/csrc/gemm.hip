@@ -34,24 +34,38 @@ union Frag {
 
 __device__ __forceinline__ uint32_t pack_i8x2_to_bf16x2(int a, int b) {
   // int8 values are exactly representable in bfloat16.
-  uint32_t fa = __float_as_uint((float)a) >> 16;
-  uint32_t fb = __float_as_uint((float)b) & 0xFFFF0000u;
-  return fa | fb;
+  return pack_bf16x2((float)a, (float)b);
 }
 
+// A packed weight tile as it travels from memory (`Raw`, kept in registers
+// while the load is in flight) and as the matrix cores take it (`Frag`).
+// int8 tiles are half the bytes, so twice as many can be in flight (kDepth);
+// they are widened only when consumed — converting at load time would put a
+// wait for the load right behind it.
 template <typename WT> struct WeightTile;
 template <> struct WeightTile<bf16_t> {
   static constexpr int kTileBytes = 1024;
-  __device__ static __forceinline__ Frag load(const void* tile, int lane) {
+  static constexpr int kDepth = 1;
+  typedef uint4 Raw;
+  __device__ static __forceinline__ Raw load(const void* tile, int lane) {
+    return reinterpret_cast<const uint4*>(tile)[lane];
+  }
+  __device__ static __forceinline__ Raw zero() { return make_uint4(0, 0, 0, 0); }
+  __device__ static __forceinline__ Frag frag(const Raw& r) {
     Frag f;
-    f.u = reinterpret_cast<const uint4*>(tile)[lane];
+    f.u = r;
     return f;
   }
 };
 template <> struct WeightTile<int8_t> {
   static constexpr int kTileBytes = 512;
-  __device__ static __forceinline__ Frag load(const void* tile, int lane) {
-    uint2 q = reinterpret_cast<const uint2*>(tile)[lane];
+  static constexpr int kDepth = 2;
+  typedef uint2 Raw;
+  __device__ static __forceinline__ Raw load(const void* tile, int lane) {
+    return reinterpret_cast<const uint2*>(tile)[lane];
+  }
+  __device__ static __forceinline__ Raw zero() { return make_uint2(0, 0); }
+  __device__ static __forceinline__ Frag frag(const Raw& q) {
     Frag f;
     f.u.x = pack_i8x2_to_bf16x2((int8_t)(q.x), (int8_t)(q.x >> 8));
     f.u.y = pack_i8x2_to_bf16x2((int8_t)(q.x >> 16), (int8_t)(q.x >> 24));
@@ -102,7 +116,9 @@ __global__ void __launch_bounds__(256)
 gemm_mfma_kernel(GemmArgs g) {
   constexpr int ACC = MP * NT;
   constexpr int TN = NT * 16;
-  constexpr int PF = (NT >= 4) ? 2 : (NT == 2 ? 3 : 4);  // pairs in flight
+  // k-tile pairs in flight per wavefront
+  constexpr int PF =
+      ((NT >= 4) ? 2 : (NT == 2 ? 3 : 4)) * WeightTile<WT>::kDepth;
   static_assert(ACC <= 16, "accumulator tile budget");
   // Small tiles: every wavefront parks its partial sums and one barrier
   // suffices; large tiles: two buffers and a tree (LDS budget).
@@ -135,7 +151,7 @@ gemm_mfma_kernel(GemmArgs g) {
   const char* wbase = reinterpret_cast<const char*>(g.W);
   constexpr int TB = WeightTile<WT>::kTileBytes;
 
-  Frag bq[PF][2][NT];
+  typename WeightTile<WT>::Raw bq[PF][2][NT];
   auto load_b = [&](int slot_, int j) {
     const int kt = (wave + 4 * j) * 2;
 #pragma unroll
@@ -147,7 +163,7 @@ gemm_mfma_kernel(GemmArgs g) {
           bq[slot_][h][nn] = WeightTile<WT>::load(
               wbase + ((size_t)nt * KT + kt + h) * TB, lane);
         else
-          bq[slot_][h][nn].u = make_uint4(0, 0, 0, 0);
+          bq[slot_][h][nn] = WeightTile<WT>::zero();
       }
   };
 #pragma unroll
@@ -193,7 +209,8 @@ gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int nn = 0; nn < NT; ++nn)
               acc[mt * NT + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  a[h][mt].v, bq[p][h][nn].v, acc[mt * NT + nn], 0, 0, 0);
+                  a[h][mt].v, WeightTile<WT>::frag(bq[p][h][nn]).v,
+                  acc[mt * NT + nn], 0, 0, 0);
         if (j + PF < nj) load_b(p, j + PF);
       }
     }
