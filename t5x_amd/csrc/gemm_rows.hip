@@ -1,16 +1,21 @@
 // Dense layers over many rows (the encoder side: M = batch x encoder length).
 //
 // Unlike the decode-step GEMMs these are compute-bound.  A workgroup (4
-// wavefronts, 2 x 2) owns a 128 x 128 output tile, each wavefront a 64 x 64
-// sub-tile = 4 x 4 MFMA tiles (v_mfma_f32_16x16x32_bf16).  Both operands go
-// straight from memory into MFMA operand registers, double-buffered over k:
-// the weights are the same pre-packed 32 x 16 lane-major tiles the decode
-// GEMMs use (one contiguous 1 KB load per tile), an activation fragment is 16
-// rows x 64 contiguous bytes.  A packed weight tile has the same lane layout
-// as either MFMA operand, so the product can be formed as C (activations as A)
-// or as C^T (weights as A); C^T leaves every lane with 4 consecutive output
-// COLUMNS of one row, C with 4 consecutive ROWS of one column — whichever makes
-// the 8-byte stores contiguous in the requested output layout.
+// wavefronts, 2 x 2) owns a 256 x 128 output tile, each wavefront a 128 x 64
+// sub-tile = 8 x 4 MFMA tiles (v_mfma_f32_16x16x32_bf16).  Per k-tile of 32 the
+// workgroup needs 16 activation fragments (16 rows x 64 bytes each) and 8
+// packed weight tiles, 1 KB apiece in MFMA operand layout; every wavefront
+// fetches 6 of them from memory, parks them in LDS exactly as loaded (lane l
+// at byte 16 l: conflict-free both ways), and after one barrier reads the 12
+// it multiplies.  Global loads for k + 1 are in flight while k is multiplied;
+// two LDS buffers, one barrier per k-tile.  Sharing through LDS cuts the
+// operand traffic per matrix instruction to 3/8 of what loading every
+// operand per wavefront costs, which is what bounds this shape.
+// A packed weight tile has the same lane layout as either MFMA operand, so the
+// product can be formed as C (activations as A) or as C^T (weights as A); C^T
+// leaves every lane with 4 consecutive output COLUMNS of one row, C with 4
+// consecutive ROWS of one column — whichever makes the 8-byte stores
+// contiguous in the requested output layout.
 #include "common.h"
 
 namespace t5d {
@@ -29,24 +34,28 @@ __device__ __forceinline__ uint32_t i8x2_to_bf16x2(int a, int b) {
          (__float_as_uint((float)b) & 0xFFFF0000u);
 }
 
+// A packed weight tile as loaded (`Raw`) and widened to bfloat16 (`frag`).
 template <typename WT> struct RowsWeightTile;
 template <> struct RowsWeightTile<bf16_t> {
   static constexpr int kTileBytes = 1024;
-  __device__ static __forceinline__ FragR load(const char* tile, int lane) {
-    FragR f;
-    f.u = reinterpret_cast<const uint4*>(tile)[lane];
-    return f;
+  typedef uint4 Raw;
+  __device__ static __forceinline__ Raw load(const char* tile, int lane) {
+    return reinterpret_cast<const uint4*>(tile)[lane];
   }
+  __device__ static __forceinline__ uint4 frag(const Raw& r) { return r; }
 };
 template <> struct RowsWeightTile<int8_t> {
   static constexpr int kTileBytes = 512;
-  __device__ static __forceinline__ FragR load(const char* tile, int lane) {
-    const uint2 q = reinterpret_cast<const uint2*>(tile)[lane];
-    FragR f;
-    f.u.x = i8x2_to_bf16x2((int8_t)(q.x), (int8_t)(q.x >> 8));
-    f.u.y = i8x2_to_bf16x2((int8_t)(q.x >> 16), (int8_t)(q.x >> 24));
-    f.u.z = i8x2_to_bf16x2((int8_t)(q.y), (int8_t)(q.y >> 8));
-    f.u.w = i8x2_to_bf16x2((int8_t)(q.y >> 16), (int8_t)(q.y >> 24));
+  typedef uint2 Raw;
+  __device__ static __forceinline__ Raw load(const char* tile, int lane) {
+    return reinterpret_cast<const uint2*>(tile)[lane];
+  }
+  __device__ static __forceinline__ uint4 frag(const Raw& q) {
+    uint4 f;
+    f.x = i8x2_to_bf16x2((int8_t)(q.x), (int8_t)(q.x >> 8));
+    f.y = i8x2_to_bf16x2((int8_t)(q.x >> 16), (int8_t)(q.x >> 24));
+    f.z = i8x2_to_bf16x2((int8_t)(q.y), (int8_t)(q.y >> 8));
+    f.w = i8x2_to_bf16x2((int8_t)(q.y >> 16), (int8_t)(q.y >> 24));
     return f;
   }
 };
@@ -70,73 +79,108 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
   return p;
 }
 
+constexpr int kRowsBM = 256, kRowsBN = 128;  // workgroup tile
+constexpr int kRowsMT = 8, kRowsNT = 4;        // MFMA tiles per wavefront
+
 // SWAP: weights are the MFMA A operand (C^T is formed).
 template <typename WT, bool SWAP>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 rows_gemm_kernel(RowsGemmArgs g) {
   constexpr int TB = RowsWeightTile<WT>::kTileBytes;
+  constexpr int MT = kRowsMT, NT = kRowsNT;
+  // [buffer][tile][lane]: tiles 0..15 activations (rows 16 t ..), 16..23 weights
+  __shared__ uint4 s_t[2][24][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, gq = lane >> 4;
-  const int m_blocks = (g.M + 127) >> 7;
+  const int m_blocks = (g.M + kRowsBM - 1) / kRowsBM;
   const int m_blk = blockIdx.x % m_blocks, n_blk = blockIdx.x / m_blocks;
-  const int m0 = m_blk * 128 + (wave >> 1) * 64;
-  const int nt0 = n_blk * 8 + (wave & 1) * 4;  // first 16-column tile
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = m_blk * kRowsBM + wm * (16 * MT);
+  const int nt0 = n_blk * (kRowsBN / 16) + wn * NT;  // first 16-column tile
   const int KT = g.K >> 5, n_tiles = g.N >> 4;
-  if (m0 >= g.M || nt0 >= n_tiles) return;
 
+  // The 6 tiles this wavefront fetches: activation tiles wave + 4 i (i < 4),
+  // weight tiles wave + 4 i (i < 2).  Out-of-range rows / tiles are clamped
+  // (their products are discarded in the epilogue).
   const bf16_t* arow[4];
-  const char* wtile[4];
+  const char* wtile[2];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    arow[t] = g.A + (size_t)min(m0 + 16 * t + l16, g.M - 1) * g.K + 8 * gq;
-    wtile[t] = g.W + (size_t)min(nt0 + t, n_tiles - 1) * KT * TB;
-  }
-  f32x4_r acc[4][4];
+  for (int i = 0; i < 4; ++i)
+    arow[i] = g.A +
+              (size_t)min(m_blk * kRowsBM + 16 * (wave + 4 * i) + l16, g.M - 1) *
+                  g.K + 8 * gq;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = (f32x4_r){0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < 2; ++i)
+    wtile[i] = g.W + (size_t)min(n_blk * (kRowsBN / 16) + wave + 4 * i,
+                                 n_tiles - 1) * KT * TB;
 
-  FragR xa[2][4], wb[2][4];
-  auto load = [&](int buf, int kt) {
+  f32x4_r acc[MT][NT];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      xa[buf][t].u = *reinterpret_cast<const uint4*>(arow[t] + 32 * kt);
-      wb[buf][t] = RowsWeightTile<WT>::load(wtile[t] + (size_t)kt * TB, lane);
-    }
-  };
-  auto mma = [&](int buf) {
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = (f32x4_r){0.f, 0.f, 0.f, 0.f};
+
+  // Staging registers of the 6 tiles in flight (named, not an array: they
+  // must stay in registers across the loop).
+  typedef typename RowsWeightTile<WT>::Raw RawW;
+  uint4 sa0, sa1, sa2, sa3;
+  RawW sw0, sw1;
+#define T5D_ROWS_FETCH(kt_)                                                    \
+  do {                                                                         \
+    sa0 = *reinterpret_cast<const uint4*>(arow[0] + 32 * (kt_));               \
+    sa1 = *reinterpret_cast<const uint4*>(arow[1] + 32 * (kt_));               \
+    sa2 = *reinterpret_cast<const uint4*>(arow[2] + 32 * (kt_));               \
+    sa3 = *reinterpret_cast<const uint4*>(arow[3] + 32 * (kt_));               \
+    sw0 = RowsWeightTile<WT>::load(wtile[0] + (size_t)(kt_) * TB, lane);       \
+    sw1 = RowsWeightTile<WT>::load(wtile[1] + (size_t)(kt_) * TB, lane);       \
+  } while (0)
+#define T5D_ROWS_PARK(buf_)                                                    \
+  do {                                                                         \
+    s_t[buf_][wave][lane] = sa0;                                               \
+    s_t[buf_][wave + 4][lane] = sa1;                                           \
+    s_t[buf_][wave + 8][lane] = sa2;                                           \
+    s_t[buf_][wave + 12][lane] = sa3;                                          \
+    s_t[buf_][16 + wave][lane] = RowsWeightTile<WT>::frag(sw0);                \
+    s_t[buf_][20 + wave][lane] = RowsWeightTile<WT>::frag(sw1);                \
+  } while (0)
+  T5D_ROWS_FETCH(0);
+  T5D_ROWS_PARK(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) T5D_ROWS_FETCH(kt + 1);
+    FragR wb[NT];
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) wb[nt].u = s_t[buf][16 + wn * NT + nt][lane];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      FragR xa;
+      xa.u = s_t[buf][wm * MT + mt][lane];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
         if (SWAP)
           acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              wb[buf][nt].v, xa[buf][mt].v, acc[mt][nt], 0, 0, 0);
+              wb[nt].v, xa.v, acc[mt][nt], 0, 0, 0);
         else
           acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              xa[buf][mt].v, wb[buf][nt].v, acc[mt][nt], 0, 0, 0);
+              xa.v, wb[nt].v, acc[mt][nt], 0, 0, 0);
       }
-  };
-  load(0, 0);
-  for (int kt = 0; kt < KT; kt += 2) {
-    if (kt + 1 < KT) load(1, kt + 1);
-    mma(0);
-    if (kt + 1 < KT) {
-      if (kt + 2 < KT) load(0, kt + 2);
-      mma(1);
     }
+    if (kt + 1 < KT) T5D_ROWS_PARK(buf ^ 1);
+    __syncthreads();
   }
+#undef T5D_ROWS_FETCH
+#undef T5D_ROWS_PARK
 
   // ---- epilogue ---------------------------------------------------------------
   if (SWAP) {
     // acc[mt][nt][i]: row m = m0 + 16 mt + l16, column n = 16 (nt0 + nt) + 4 gq + i
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int m = m0 + 16 * mt + l16;
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
+      for (int nt = 0; nt < NT; ++nt) {
         if (nt0 + nt >= n_tiles) continue;
         const int n = 16 * (nt0 + nt) + 4 * gq;
         float v[4];
@@ -188,12 +232,12 @@ rows_gemm_kernel(RowsGemmArgs g) {
     // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
     // (values layout [B, H, 64, Ep]: 4 consecutive positions per store)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int m = m0 + 16 * mt + 4 * gq;
       if (m >= g.M) continue;
       const int b = m / g.E, e = m - b * g.E;
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
+      for (int nt = 0; nt < NT; ++nt) {
         if (nt0 + nt >= n_tiles) continue;
         const int n = 16 * (nt0 + nt) + l16;
         float s = g.scales ? g.scales[n] : 1.f;
@@ -250,7 +294,8 @@ extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
   g.M = (int)M; g.K = K; g.N = N;
   g.epilogue = epilogue; g.layout = out_layout;
   g.E = E; g.Ep = Ep; g.H = H;
-  const int m_blocks = ((int)M + 127) / 128, n_blocks = (N / 16 + 7) / 8;
+  const int m_blocks = ((int)M + kRowsBM - 1) / kRowsBM;
+  const int n_blocks = (N + kRowsBN - 1) / kRowsBN;
   dim3 grid((unsigned)m_blocks * n_blocks), block(256);
   hipStream_t s = as_stream(stream);
   const bool swap = out_layout != T5D_OUT_HEADS_VALUE;
