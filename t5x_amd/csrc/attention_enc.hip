@@ -39,16 +39,22 @@ struct EncAttnArgs {
   int H, E, Ep, q_stride, k_stride;
 };
 
+constexpr int kMaxEncLen = 2048;
+
 __global__ void __launch_bounds__(256)
 enc_attn_kernel(EncAttnArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t s_p[4][16][32];
+  __shared__ float s_bias[2 * kMaxEncLen];  // this head's bias by distance
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, gq = lane >> 4;
   const int h = blockIdx.y, b = blockIdx.z;
   const int q0 = blockIdx.x * 64 + wave * 16;
-  if (q0 >= a.E) return;
   const int E = a.E;
+  for (int i = threadIdx.x; i < 2 * E - 1; i += 256)
+    s_bias[i] = bf16_to_f32(a.bias[(size_t)h * (2 * E - 1) + i]);
+  __syncthreads();
+  if (q0 >= E) return;
   int n = a.len[b];
   n = n < 0 ? 0 : (n > E ? E : n);
   const float kMasked = -9.9857e9f;  // bf16(-1e10), layers.py:309-311
@@ -62,26 +68,36 @@ enc_attn_kernel(EncAttnArgs a) {
     qb[c].u = *reinterpret_cast<const uint4*>(
         a.q + (row0 + qi) * a.q_stride + h * 64 + 32 * c + 8 * gq);
   const bool q_valid = (q0 + l16) < n;
-  const bf16_t* bias_row = a.bias + (size_t)h * (2 * E - 1) + (E - 1) - qi;
+  const float* bias_row = s_bias + (E - 1) - qi;
 
-  // scores of key tile kt for this lane: keys 16 kt + 4 g + i of query l16
-  auto score_tile = [&](int kt, float (&s)[4]) {
+  // Keys past the valid length get -1e10, whose exp underflows to exactly 0
+  // next to any valid key: when all 16 queries of this wavefront are valid,
+  // the key tiles that hold only padding are skipped.  (A padded query attends
+  // uniformly over ALL keys, so a wavefront with one walks them all.)
+  const int n_tiles =
+      (q0 + 15 < n) ? (n + 15) >> 4 : (E + 15) >> 4;
+
+  // K tile kt as the A operand: lane (row = key l16, g) holds K[key][32c + 8g .. +8]
+  auto load_k = [&](int kt, FragE (&ka)[2]) {
     const int key_row = min(16 * kt + l16, E - 1);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      ka[c].u = *reinterpret_cast<const uint4*>(
+          a.k + (row0 + key_row) * a.k_stride + h * 64 + 32 * c + 8 * gq);
+  };
+  // scores of key tile kt for this lane: keys 16 kt + 4 g + i of query l16
+  auto score_tile = [&](int kt, const FragE (&ka)[2], float (&s)[4]) {
     f32x4_e acc = (f32x4_e){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      FragE ka;
-      ka.u = *reinterpret_cast<const uint4*>(
-          a.k + (row0 + key_row) * a.k_stride + h * 64 + 32 * c + 8 * gq);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qb[c].v, acc, 0, 0, 0);
-    }
+    for (int c = 0; c < 2; ++c)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c].v, qb[c].v, acc, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = 16 * kt + 4 * gq + i;
       float x = round_bf16(acc[i]);
       if (key < E) {
         const bool ok = q_valid && key < n;
-        x = ok ? round_bf16(x + bf16_to_f32(bias_row[key])) : kMasked;
+        x = ok ? round_bf16(x + bias_row[key]) : kMasked;
       } else {
         x = -INFINITY;
       }
@@ -89,18 +105,24 @@ enc_attn_kernel(EncAttnArgs a) {
     }
   };
 
-  const int n_tiles = (E + 15) >> 4;
   float m = -INFINITY, l = 0.f;
-  for (int kt = 0; kt < n_tiles; ++kt) {
-    float s[4];
-    score_tile(kt, s);
-    const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-    const float nm = fmaxf(m, tm);
-    float add = 0.f;
+  {
+    FragE kcur[2], knext[2];
+    load_k(0, kcur);
+    for (int kt = 0; kt < n_tiles; ++kt) {
+      if (kt + 1 < n_tiles) load_k(kt + 1, knext);  // in flight during this tile
+      float s[4];
+      score_tile(kt, kcur, s);
+      const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+      const float nm = fmaxf(m, tm);
+      float add = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) add += __expf(s[i] - nm);
-    l = l * __expf(m - nm) + add;  // exp(-inf - finite) == 0 on the first tile
-    m = nm;
+      for (int i = 0; i < 4; ++i) add += __expf(s[i] - nm);
+      l = l * __expf(m - nm) + add;  // exp(-inf - finite) == 0 on the first tile
+      m = nm;
+      kcur[0] = knext[0];
+      kcur[1] = knext[1];
+    }
   }
   // combine the 4 lanes (g) that share a query
 #pragma unroll
@@ -116,11 +138,29 @@ enc_attn_kernel(EncAttnArgs a) {
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_e){0.f, 0.f, 0.f, 0.f};
   const bf16_t* vbase = a.vt + ((size_t)b * a.H + h) * 64 * (size_t)a.Ep;
+  // V^T fragments of a 32-key step: lane (row = d l16, g) holds
+  // V^T[16 dt + l16][key0 .. +8]
+  auto load_v = [&](int kb, FragE (&va)[4]) {
+    const int key0 = min(16 * kb + 8 * gq, a.Ep - 8);
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+      va[dt].u = *reinterpret_cast<const uint4*>(
+          vbase + (size_t)(16 * dt + l16) * a.Ep + key0);
+  };
+  FragE kcur[2][2], knext[2][2], vcur[4], vnext[4];
+  load_k(0, kcur[0]);
+  if (1 < n_tiles) load_k(1, kcur[1]);
+  load_v(0, vcur);
   for (int kb = 0; kb < n_tiles; kb += 2) {  // 32 keys per step
+    if (kb + 2 < n_tiles) {
+      load_k(kb + 2, knext[0]);
+      if (kb + 3 < n_tiles) load_k(kb + 3, knext[1]);
+      load_v(kb + 2, vnext);
+    }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       float s[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-      if (kb + t < n_tiles) score_tile(kb + t, s);
+      if (kb + t < n_tiles) score_tile(kb + t, kcur[t], s);
       uint2 pk;
       pk.x = pack_bf16x2(__expf(s[0] - m) * inv, __expf(s[1] - m) * inv);
       pk.y = pack_bf16x2(__expf(s[2] - m) * inv, __expf(s[3] - m) * inv);
@@ -132,16 +172,18 @@ enc_attn_kernel(EncAttnArgs a) {
     __builtin_amdgcn_wave_barrier();
     FragE pb;  // B: lane (col = query l16, g) holds P[q][8g .. +8] of the 32
     pb.u = *reinterpret_cast<const uint4*>(&s_p[wave][l16][8 * gq]);
-    const int key0 = min(16 * kb + 8 * gq, a.Ep - 8);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
-      FragE va;  // A: lane (row = d l16, g) holds V^T[16 dt + l16][key0 .. +8]
-      va.u = *reinterpret_cast<const uint4*>(
-          vbase + (size_t)(16 * dt + l16) * a.Ep + key0);
-      oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, oc[dt], 0, 0,
-                                                       0);
-    }
+    for (int dt = 0; dt < 4; ++dt)
+      oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vcur[dt].v, pb.v, oc[dt],
+                                                       0, 0, 0);
     __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      kcur[t][0] = knext[t][0];
+      kcur[t][1] = knext[t][1];
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) vcur[dt] = vnext[dt];
   }
   // oc[dt][i]: out[q = l16][d = 16 dt + 4 g + i]
   if (q0 + l16 < E) {
@@ -177,6 +219,8 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
   T5D_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 &&
                   ((uintptr_t)v_t % 16) == 0 && ((uintptr_t)out % 8) == 0,
               T5D_EINVAL, "t5d_encoder_attention: operand alignment");
+  T5D_REQUIRE(E <= kMaxEncLen, T5D_ELIMIT,
+              "t5d_encoder_attention: E=%d beyond %d", E, kMaxEncLen);
   T5D_REQUIRE(H <= 65535 && B <= 65535, T5D_ELIMIT,
               "t5d_encoder_attention: H=%d B=%d beyond the launch grid", H, B);
   EncAttnArgs a;
