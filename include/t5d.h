@@ -51,8 +51,8 @@ enum {
 /* Output layouts of t5d_gemm_rows. */
 enum {
   T5D_OUT_ROWS = 0,        /* row-major [M, N] */
-  T5D_OUT_HEADS_KEY = 1,   /* [B, H, Ep, 64]: cross-attention keys */
-  T5D_OUT_HEADS_VALUE = 2  /* [B, H, 64, Ep]: cross-attention values */
+  T5D_OUT_HEADS_KEY = 1,   /* [B, H, 2, Ep, 32]: cross-attention keys */
+  T5D_OUT_HEADS_VALUE = 2  /* [B, H, Ep/32, 64, 32]: cross-attention values */
 };
 
 int t5d_version(void);
@@ -159,10 +159,15 @@ int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
 /* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
  * mask :366-370).  The reference re-projects K/V from the beam-expanded
  * encoder output every step; here they are projected once per batch item:
- *   cross_key [B, H, E, 64] (head dim contiguous) and cross_value
- *   [B, H, 64, E] (positions contiguous), shared by the item's `beams` rows
- *   (<= 8); these are the layouts in which a 16-byte chunk is directly an MFMA
- *   operand of Q.K^T and P.V respectively.  E a multiple of 8 (bf16) / 4 (f32).
+ *   float32: cross_key [B, H, E, 64] (head dim contiguous) and cross_value
+ *   [B, H, 64, E] (positions contiguous), E a multiple of 4.
+ *   bfloat16: cross_key [B, H, 2, E, 32] (dims 32 c .. 32 c + 31 of key e at
+ *   [b, h, c, e, :]) and cross_value [B, H, E/32, 64, 32] (dim d of key
+ *   32 j + p at [b, h, j, d, p]), E a multiple of 32: a 16-byte chunk is
+ *   directly an MFMA operand of Q.K^T and P.V respectively, and the 64 chunks
+ *   one wavefront load instruction fetches are 1 KB of consecutive memory.
+ *   t5d_gemm_rows writes both (T5D_OUT_HEADS_KEY / T5D_OUT_HEADS_VALUE).
+ *   K/V are shared by the item's `beams` rows (<= 8).
  *   enc_len [B]: number of leading valid (non-padding) encoder positions.
  *   q [B*beams, H*64] -> out [B*beams, H*64]. */
 int t5d_cross_attention_step(void* stream, int dtype, const void* q,
@@ -176,8 +181,8 @@ int t5d_cross_attention_step(void* stream, int dtype, const void* q,
  * normalises its batch item's rows of x and multiplies them with its head's
  * 64 columns of the packed query kernel while its K stream is in flight.
  *   x [B*beams, d] residual stream; ln_scale [d]; query_kernel: packed
- *   (t5d_pack_weight) [d, H*64] bfloat16 kernel.  bfloat16 only; E <= 512;
- *   d a multiple of 64, <= 1024. */
+ *   (t5d_pack_weight) [d, H*64] bfloat16 kernel.  bfloat16 only (K/V in the
+ *   bfloat16 layouts above); E <= 512; d a multiple of 64, <= 1024. */
 int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
                                     const void* x, const void* ln_scale,
                                     float eps, const void* query_kernel,
@@ -192,7 +197,8 @@ int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
  * bidirectional relative-position bias and padding mask,
  * t5x/examples/t5/network.py:47-96,325-328).
  *   q, k [B*E, *_stride]: head h in columns h*64 .. h*64+63 (row-major
- *   projections); v_t [B, H, 64, Ep] (t5d_gemm_rows, T5D_OUT_HEADS_VALUE);
+ *   projections); v_t [B, H, Ep/32, 64, 32] (t5d_gemm_rows,
+ *   T5D_OUT_HEADS_VALUE), Ep a multiple of 32;
  *   rel_bias [H, 2E-1] bfloat16 indexed by (key - query + E - 1);
  *   enc_len [B]: keys and queries at positions >= enc_len[b] are padding
  *   (masked with -1e10 as in the reference); out [B*E, H*64]. */
@@ -322,8 +328,8 @@ typedef struct {
   const float *qkv_scales, *self_out_scales, *cross_q_scales,
       *cross_out_scales, *wi_scales, *wo_scales;
   void *cached_key, *cached_value;        /* [R, H, 64, L] */
-  const void *cross_key;                  /* [B, H, E, 64] */
-  const void *cross_value;                /* [B, H, 64, E] */
+  const void *cross_key;    /* as t5d_cross_attention_step takes them */
+  const void *cross_value;
 } t5d_layer;
 
 typedef struct {

@@ -523,6 +523,9 @@ extern "C" int t5d_cross_attention_step(void* stream, int dtype, const void* q,
                 kMaxWaves * 64);
     launch_cross_f32(a, B, as_stream(stream));
   } else {
+    T5D_REQUIRE(E % 32 == 0, T5D_EINVAL,
+                "t5d_cross_attention_step: bfloat16 K/V are stored in blocks of "
+                "32 positions, E=%d", E);
     launch_cross_attention_bf16(as_stream(stream), q, cross_key, cross_value,
                                 enc_len, out, B, beams, H, E, nullptr, nullptr,
                                 nullptr, 0, 0.f);
@@ -548,9 +551,10 @@ extern "C" int t5d_cross_attention_step_norm_q(
   T5D_REQUIRE(beams >= 1 && beams <= 8, T5D_ELIMIT,
               "t5d_cross_attention_step_norm_q: beams=%d (supported: 1..8)",
               beams);
-  T5D_REQUIRE(E <= 512 && d >= 64 && d % 64 == 0 && d <= 1024, T5D_ELIMIT,
-              "t5d_cross_attention_step_norm_q: E=%d (<= 512), d=%d (multiple "
-              "of 64, <= 1024)", E, d);
+  T5D_REQUIRE(E <= 512 && E % 32 == 0 && d >= 64 && d % 64 == 0 && d <= 1024,
+              T5D_ELIMIT,
+              "t5d_cross_attention_step_norm_q: E=%d (multiple of 32, <= 512), "
+              "d=%d (multiple of 64, <= 1024)", E, d);
   T5D_REQUIRE(((uintptr_t)cross_key % 16) == 0 &&
                   ((uintptr_t)cross_value % 16) == 0 &&
                   ((uintptr_t)x % 16) == 0 && ((uintptr_t)ln_scale % 16) == 0 &&

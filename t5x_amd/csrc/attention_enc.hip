@@ -10,9 +10,9 @@
 //           rounds them, running max / sum per lane, combined at the end;
 //   pass 2: S^T again, P = bf16(exp(s - max) / sum) written 4 keys at a time
 //           into a small LDS tile, read back as the B operand of
-//           out^T = V^T P^T, 32 keys per step.  V is given transposed
-//           ([B, H, 64, Ep], what t5d_gemm_rows' value layout writes), so its
-//           fragments are contiguous 16-byte loads.
+//           out^T = V^T P^T, 32 keys per step.  V is given transposed in
+//           32-key blocks ([B, H, Ep / 32, 64, 32], what t5d_gemm_rows' value
+//           layout writes), so a fragment is one contiguous 1 KB.
 // Masked keys get the reference's -1e10 (so a padded query attends uniformly,
 // as it does there); keys beyond E do not exist and get -inf.
 #include <math.h>
@@ -32,7 +32,7 @@ union FragE {
 struct EncAttnArgs {
   const bf16_t* q;    // [B*E, q_stride]: head h at columns h*64 .. +64
   const bf16_t* k;    // same layout as q
-  const bf16_t* vt;   // [B, H, 64, Ep]
+  const bf16_t* vt;   // [B, H, Ep / 32, 64, 32]: 32-key blocks
   const bf16_t* bias; // [H, 2E-1]: by (key - query + E - 1)
   const int32_t* len; // [B] valid prefix length
   bf16_t* out;        // [B*E, H*64]
@@ -139,13 +139,12 @@ enc_attn_kernel(EncAttnArgs a) {
   for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_e){0.f, 0.f, 0.f, 0.f};
   const bf16_t* vbase = a.vt + ((size_t)b * a.H + h) * 64 * (size_t)a.Ep;
   // V^T fragments of a 32-key step: lane (row = d l16, g) holds
-  // V^T[16 dt + l16][key0 .. +8]
-  auto load_v = [&](int kb, FragE (&va)[4]) {
-    const int key0 = min(16 * kb + 8 * gq, a.Ep - 8);
+  // V^T[16 dt + l16][32 (kb / 2) + 8 g .. +8], 1 KB contiguous per fragment
+  auto load_v = [&](int kb, FragE (&va)[4]) {  // kb even: block kb / 2
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
       va[dt].u = *reinterpret_cast<const uint4*>(
-          vbase + (size_t)(16 * dt + l16) * a.Ep + key0);
+          vbase + ((size_t)(kb >> 1) * 64 + 16 * dt + l16) * 32 + 8 * gq);
   };
   FragE kcur[2][2], knext[2][2], vcur[4], vnext[4];
   load_k(0, kcur[0]);
@@ -209,7 +208,7 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
                                      int k_stride) {
   T5D_REQUIRE(q && k && v_t && rel_bias && enc_len && out, T5D_EINVAL,
               "t5d_encoder_attention: null pointer");
-  T5D_REQUIRE(B > 0 && H > 0 && E > 0 && Ep >= E && Ep % 8 == 0 && Ep >= 8,
+  T5D_REQUIRE(B > 0 && H > 0 && E > 0 && Ep >= E && Ep % 32 == 0,
               T5D_EINVAL, "t5d_encoder_attention: B=%d H=%d E=%d Ep=%d", B, H,
               E, Ep);
   T5D_REQUIRE(q_stride >= H * 64 && k_stride >= H * 64 && q_stride % 8 == 0 &&

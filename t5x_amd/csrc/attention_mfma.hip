@@ -127,6 +127,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   if (n == 0) { uniform = true; n = a.S; }
 
   const int jw = wave * kBlockJ;  // first position of this wavefront
+  // K [B, H, 2, S, 32] (the head dim's two halves as planes) and
+  // V [B, H, S / 32, 64, 32] (32-position blocks): every fragment load of a
+  // wavefront below is one contiguous 1 KB.
   const bf16_t* kbase = a.k + ((size_t)b * a.H + h) * (size_t)a.S * kHeadDim;
   const bf16_t* vbase = a.v + ((size_t)b * a.H + h) * (size_t)kHeadDim * a.S;
   const int nw = n - jw;  // valid positions of this wavefront (may be <= 0)
@@ -168,8 +171,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
 #pragma unroll
       for (int c = 0; c < 2; ++c)
         kb[jt][c].u = *reinterpret_cast<const uint4*>(
-            kbase + (size_t)min(jw + 16 * jt + n16, a.S - 1) * kHeadDim +
-            32 * c + 8 * g);
+            kbase + ((size_t)c * a.S + min(jw + 16 * jt + n16, a.S - 1)) * 32 +
+            8 * g);
     } else {
       kb[jt][0].u = kb[jt][1].u = make_uint4(0, 0, 0, 0);
     }
@@ -181,8 +184,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
           vb[jb][dt].u = *reinterpret_cast<const uint4*>(
-              vbase + (size_t)(16 * dt + n16) * a.S +
-              min(jw + 32 * jb + 8 * g, a.S - 8));
+              vbase + ((size_t)(wave * (kBlockJ / 32) + jb) * kHeadDim +
+                       16 * dt + n16) * 32 + 8 * g);
       } else {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);

@@ -211,9 +211,10 @@ rows_gemm_kernel(RowsGemmArgs g) {
         if (m >= g.M) continue;
         size_t o;
         if (g.layout == T5D_OUT_HEADS_KEY) {
+          // [B, H, 2, Ep, 32]: the two 32-wide halves of the head dim as planes
           const int b = m / g.E, e = m - b * g.E;
-          const int hh = n >> 6, d = n & 63;
-          o = (((size_t)b * g.H + hh) * g.Ep + e) * 64 + d;
+          const int hh = n >> 6, c = (n >> 5) & 1, j = n & 31;
+          o = ((((size_t)b * g.H + hh) * 2 + c) * g.Ep + e) * 32 + j;
         } else {
           o = (size_t)m * g.N + n;
         }
@@ -230,7 +231,7 @@ rows_gemm_kernel(RowsGemmArgs g) {
     }
   } else {
     // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
-    // (values layout [B, H, 64, Ep]: 4 consecutive positions per store)
+    // (values layout [B, H, Ep / 32, 64, 32]: 4 consecutive positions per store)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = m0 + 16 * mt + 4 * gq;
@@ -242,7 +243,9 @@ rows_gemm_kernel(RowsGemmArgs g) {
         const int n = 16 * (nt0 + nt) + l16;
         float s = g.scales ? g.scales[n] : 1.f;
         const int hh = n >> 6, d = n & 63;
-        const size_t o = (((size_t)b * g.H + hh) * 64 + d) * g.Ep + e;
+        const size_t o =
+            ((((size_t)b * g.H + hh) * (g.Ep >> 5) + (e >> 5)) * 64 + d) * 32 +
+            (e & 31);
         *reinterpret_cast<uint2*>(g.C + o) =
             pack4(acc[mt][nt][0] * s, acc[mt][nt][1] * s, acc[mt][nt][2] * s,
                   acc[mt][nt][3] * s);
@@ -281,10 +284,11 @@ extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
   int H = 0;
   if (out_layout != T5D_OUT_ROWS) {
     T5D_REQUIRE(epilogue == T5D_EPI_NONE && N % 64 == 0 && E > 0 && Ep >= E &&
-                    M % E == 0 && E % 4 == 0 && Ep % 4 == 0,
+                    M % E == 0 && E % 4 == 0 && Ep % 32 == 0,
                 T5D_EINVAL,
                 "t5d_gemm_rows: heads layout needs epilogue none, N %% 64 == 0,"
-                " M %% E == 0, E %% 4 == 0 (N=%d E=%d Ep=%d)", N, E, Ep);
+                " M %% E == 0, E %% 4 == 0, Ep %% 32 == 0 (N=%d E=%d Ep=%d)", N,
+                E, Ep);
     H = N / 64;
   }
   RowsGemmArgs g;

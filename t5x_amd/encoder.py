@@ -120,12 +120,12 @@ def _encode_hip(module, params, tokens):
   if not bool((prefix == valid).all()):
     raise ValueError('encoder padding must be a suffix of zeros')
   lens = lens.contiguous()
-  Ep = (E + 7) // 8 * 8
+  Ep = (E + 31) // 32 * 32  # values are stored in blocks of 32 positions
   bias = w.rel_bias(E)
   ids = tokens.reshape(-1).to(torch.int32).contiguous()
   x = ops.embed(w.embedding, ids)
   M = B * E
-  v_t = torch.zeros((B, H, 64, Ep), dtype=x.dtype, device=dev)
+  v_t = torch.zeros((B, H, Ep // 32, 64, 32), dtype=x.dtype, device=dev)
   for l in w.layers:
     xn = ops.rmsnorm(x, l['ln_attn'])
     qk = ops.gemm_rows(xn, l['qk'])                       # [M, q | k]

@@ -325,15 +325,18 @@ class Transformer:
     cfg = self.config
     B, E, d = encoded.shape
     H, D = cfg.num_heads, cfg.head_dim
-    el = 16 // encoded.element_size()
-    Ep = (E + el - 1) // el * el  # rows padded to 16-byte multiples
+    bf16 = encoded.dtype == torch.bfloat16
+    # float32: [B, H, Ep, 64] / [B, H, 64, Ep], rows padded to 16 bytes;
+    # bfloat16: [B, H, 2, Ep, 32] / [B, H, Ep/32, 64, 32] (blocks of 32
+    # positions).  Padding positions e >= E stay zero.
+    pad = 32 if bf16 else 16 // encoded.element_size()
+    Ep = (E + pad - 1) // pad * pad
     x = encoded.reshape(B * E, d).contiguous()
     ks, vs = [], []
-    hip = x.dtype == torch.bfloat16 and E % 4 == 0
+    hip = bf16 and E % 4 == 0
     for l in w.layers:
       if hip:
-        # [B, H, Ep, 64] keys and [B, H, 64, Ep] values straight from the
-        # dense kernel's epilogue; the padding rows e >= E stay zero
+        # straight from the dense kernel's epilogue
         from t5x_amd import _lib
         ks.append(ops.gemm_rows(x, l['cross_k_packed'],
                                 layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep))
@@ -348,10 +351,11 @@ class Transformer:
         if dst is ks:  # keys: [B, H, E, D], head dim contiguous
           buf = torch.zeros((B, H, Ep, D), dtype=x.dtype, device=x.device)
           buf[:, :, :E] = y.permute(0, 2, 1, 3)
+          dst.append(ops.tile_cross_key(buf) if bf16 else buf)
         else:  # values: [B, H, D, E], positions contiguous
           buf = torch.zeros((B, H, D, Ep), dtype=x.dtype, device=x.device)
           buf[..., :E] = y.permute(0, 2, 3, 1)
-        dst.append(buf)
+          dst.append(ops.tile_cross_value(buf) if bf16 else buf)
     tok = enc_tokens.reshape(B, E)
     valid = tok > 0
     # The mask keeps exactly the positions with token > 0 (network.py:366-370).

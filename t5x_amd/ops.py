@@ -254,18 +254,50 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
   return out
 
 
+def tile_cross_key(k):
+  """[B, H, E, 64] keys -> the bfloat16 kernels' [B, H, 2, E, 32] (the two
+  halves of the head dim as planes).  E must be a multiple of 32."""
+  B, H, E, D = k.shape
+  return k.reshape(B, H, E, 2, 32).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def tile_cross_value(v):
+  """[B, H, 64, E] values -> the bfloat16 kernels' [B, H, E/32, 64, 32]
+  (blocks of 32 positions).  E must be a multiple of 32."""
+  B, H, D, E = v.shape
+  return v.reshape(B, H, D, E // 32, 32).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def _cross_kv_dims(cross_key, cross_value):
+  """(B, H, E) of a cross K/V pair in the layout of its dtype: float32
+  [B, H, E, 64] / [B, H, 64, E]; bfloat16 [B, H, 2, E, 32] /
+  [B, H, E/32, 64, 32]."""
+  if cross_key.dtype == torch.float32:
+    _chk(cross_key, 'cross_key', torch.float32, 4)
+    _chk(cross_value, 'cross_value', torch.float32, 4)
+    B, H, E, D = cross_key.shape
+    if D != 64 or tuple(cross_value.shape) != (B, H, D, E):
+      raise ValueError(f'float32 cross_key must be [B, H, E, 64] and '
+                       f'cross_value [B, H, 64, E], got '
+                       f'{tuple(cross_key.shape)} / {tuple(cross_value.shape)}')
+    return B, H, E
+  _chk(cross_key, 'cross_key', torch.bfloat16, 5)
+  _chk(cross_value, 'cross_value', torch.bfloat16, 5)
+  B, H, two, E, w = cross_key.shape
+  if (two, w) != (2, 32) or E % 32 or tuple(cross_value.shape) != (
+      B, H, E // 32, 64, 32):
+    raise ValueError(f'bfloat16 cross_key must be [B, H, 2, E, 32] and '
+                     f'cross_value [B, H, E/32, 64, 32] (E %% 32 == 0), got '
+                     f'{tuple(cross_key.shape)} / {tuple(cross_value.shape)}')
+  return B, H, E
+
+
 def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
   _chk(q, 'q', ndim=2)
-  _chk(cross_key, 'cross_key', q.dtype, 4)
-  _chk(cross_value, 'cross_value', q.dtype, 4)
+  _chk(cross_key, 'cross_key', q.dtype)
   _chk(enc_len, 'enc_len', torch.int32, 1)
-  B, H, E, D = cross_key.shape
-  if D != 64:
-    raise ValueError('head_dim must be 64')
-  if tuple(cross_value.shape) != (B, H, D, E):
-    raise ValueError(f'cross_key {tuple(cross_key.shape)} is [B, H, E, 64]; '
-                     f'cross_value must be [B, H, 64, E], got '
-                     f'{tuple(cross_value.shape)}')
+  B, H, E = _cross_kv_dims(cross_key, cross_value)
+  D = 64
   if tuple(q.shape) != (B * beams, H * D):
     raise ValueError(f'q shape {tuple(q.shape)} != {(B * beams, H * D)}')
   if enc_len.shape[0] != B:
@@ -285,13 +317,11 @@ def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
   """rmsnorm(x, ln_scale) @ wq followed by cross_attention_step, one kernel."""
   _chk(x, 'x', torch.bfloat16, 2)
   _chk(ln_scale, 'ln_scale', torch.bfloat16, 1)
-  _chk(cross_key, 'cross_key', x.dtype, 4)
-  _chk(cross_value, 'cross_value', x.dtype, 4)
+  _chk(cross_key, 'cross_key', x.dtype)
   _chk(enc_len, 'enc_len', torch.int32, 1)
-  B, H, E, D = cross_key.shape
+  B, H, E = _cross_kv_dims(cross_key, cross_value)
+  D = 64
   R, d = x.shape
-  if D != 64 or tuple(cross_value.shape) != (B, H, D, E):
-    raise ValueError('cross_key must be [B, H, E, 64], cross_value [B, H, 64, E]')
   if R != B * beams or ln_scale.shape[0] != d or enc_len.shape[0] != B:
     raise ValueError('x / ln_scale / enc_len do not match the batch')
   if wq.K != d or wq.N != H * D or wq.geglu:
@@ -309,7 +339,8 @@ def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
 def gemm_rows(a, w: PackedWeight, out=None, residual=None,
               layout=_lib.OUT_ROWS, E=0, Ep=0):
   """Dense layer over any number of rows (bfloat16).  layout OUT_HEADS_KEY /
-  OUT_HEADS_VALUE writes [B, H, Ep, 64] / [B, H, 64, Ep] (rows m = b*E + e)."""
+  OUT_HEADS_VALUE writes [B, H, 2, Ep, 32] / [B, H, Ep/32, 64, 32] (rows
+  m = b*E + e; Ep a multiple of 32, positions e >= E stay zero)."""
   _chk(a, 'a', torch.bfloat16, 2)
   M, K = a.shape
   if K != w.K or w.w_dtype == F32:
@@ -323,7 +354,8 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
       raise ValueError(f'out shape {tuple(out.shape)}')
   else:
     B, H = M // max(E, 1), w.N // 64
-    want = (B, H, Ep, 64) if layout == _lib.OUT_HEADS_KEY else (B, H, 64, Ep)
+    want = ((B, H, 2, Ep, 32) if layout == _lib.OUT_HEADS_KEY else
+            (B, H, Ep // 32, 64, 32))
     if out is None:
       out = torch.zeros(want, dtype=a.dtype, device=a.device)
     if tuple(out.shape) != want:
@@ -341,11 +373,15 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
 
 def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
   """q, k: [B*E, >= H*64] row-major views (row stride = stride(0)); v_t
-  [B, H, 64, Ep]; rel_bias [H, 2E-1]; enc_len [B] -> out [B*E, H*64]."""
-  _chk(v_t, 'v_t', torch.bfloat16, 4)
+  [B, H, Ep/32, 64, 32] (tile_cross_value of [B, H, 64, Ep]); rel_bias
+  [H, 2E-1]; enc_len [B] -> out [B*E, H*64]."""
+  _chk(v_t, 'v_t', torch.bfloat16, 5)
   _chk(rel_bias, 'rel_bias', torch.bfloat16, 2)
   _chk(enc_len, 'enc_len', torch.int32, 1)
-  B, H, D, Ep = v_t.shape
+  B, H, blocks, D, w = v_t.shape
+  if w != 32:
+    raise ValueError('v_t must be [B, H, Ep/32, 64, 32]')
+  Ep = blocks * 32
   E = (rel_bias.shape[1] + 1) // 2
   for name, t in (('q', q), ('k', k)):
     if (not t.is_cuda or t.dtype != torch.bfloat16 or t.dim() != 2 or
@@ -353,7 +389,8 @@ def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
       raise ValueError(f'{name} must be a [B*E, H*64] bfloat16 view with unit '
                        f'column stride, got {tuple(t.shape)}')
   if D != 64 or rel_bias.shape[0] != H or enc_len.shape[0] != B:
-    raise ValueError('v_t [B, H, 64, Ep], rel_bias [H, 2E-1], enc_len [B]')
+    raise ValueError('v_t [B, H, Ep/32, 64, 32], rel_bias [H, 2E-1], '
+                     'enc_len [B]')
   if out is None:
     out = torch.empty((B * E, H * 64), dtype=torch.bfloat16, device=v_t.device)
   _chk(out, 'out', torch.bfloat16, 2)

@@ -63,12 +63,14 @@ def test_gemm_rows(ops, M, K, N, mode):
     np.testing.assert_allclose(host(out), host(small), atol=2e-2, rtol=2**-7)
 
 
-@pytest.mark.parametrize('B,E,Ep,H,d', [(2, 16, 16, 1, 64), (3, 40, 40, 2, 128),
-                                        (2, 100, 104, 3, 256),
+@pytest.mark.parametrize('B,E,Ep,H,d', [(2, 16, 32, 1, 64), (3, 40, 64, 2, 128),
+                                        (2, 100, 128, 3, 256),
                                         (4, 512, 512, 12, 768)])
 def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
-  """Key layout [B, H, Ep, 64] and value layout [B, H, 64, Ep] hold exactly the
-  row-major result, re-arranged; padding rows stay untouched (zero)."""
+  """Key layout [B, H, 2, Ep, 32] and value layout [B, H, Ep/32, 64, 32] hold
+  exactly the row-major result, re-arranged (tile_cross_key / tile_cross_value
+  of [B, H, Ep, 64] / [B, H, 64, Ep]); padding positions stay untouched
+  (zero)."""
   rs = np.random.RandomState(B + E + H)
   x = dev(rs.randn(B * E, d).astype(np.float32), torch.bfloat16)
   w = dev((rs.randn(d, H * 64) / np.sqrt(d)).astype(np.float32))
@@ -77,9 +79,14 @@ def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
   rows = ops.gemm_rows(x, pw).view(B, E, H, 64)
   keys = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep)
   vals = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep)
-  assert torch.equal(keys[:, :, :E], rows.permute(0, 2, 1, 3))
-  assert torch.equal(vals[..., :E], rows.permute(0, 2, 3, 1))
-  assert not keys[:, :, E:].any() and not vals[..., E:].any()
+  plain_k = torch.zeros((B, H, Ep, 64), dtype=rows.dtype, device='cuda')
+  plain_k[:, :, :E] = rows.permute(0, 2, 1, 3)
+  plain_v = torch.zeros((B, H, 64, Ep), dtype=rows.dtype, device='cuda')
+  plain_v[..., :E] = rows.permute(0, 2, 3, 1)
+  assert tuple(keys.shape) == (B, H, 2, Ep, 32)
+  assert tuple(vals.shape) == (B, H, Ep // 32, 64, 32)
+  assert torch.equal(keys, ops.tile_cross_key(plain_k))
+  assert torch.equal(vals, ops.tile_cross_value(plain_v))
 
 
 def _enc_attn_oracle(q, k, v, rel_emb, lens):
@@ -110,12 +117,13 @@ def test_encoder_attention(ops, B, E, H):
   lens[0] = E
   want = _enc_attn_oracle(q, k, v, rel_emb, lens)
 
-  Ep = (E + 7) // 8 * 8
+  Ep = (E + 31) // 32 * 32
   bucket = network.relative_position_bucket(
       np.arange(-(E - 1), E), bidirectional=True)        # key - query
   rel_bias = dev(ot5.bf16_round(rel_emb)[:, bucket], torch.bfloat16).contiguous()
   v_t = torch.zeros((B, H, 64, Ep), dtype=torch.bfloat16, device='cuda')
   v_t[..., :E] = dev(v, torch.bfloat16).permute(0, 2, 3, 1)
+  v_t = ops.tile_cross_value(v_t)
   qk = torch.stack([dev(q, torch.bfloat16).reshape(B * E, H * 64),
                     dev(k, torch.bfloat16).reshape(B * E, H * 64)], dim=1)
   qk = qk.reshape(B * E, 2 * H * 64)                      # strided q | k views
@@ -175,8 +183,16 @@ def test_cross_kv_projection_layouts_match_oracle():
   w = module.decoder_weights(params)
   cross = module._cross_kv(w, dev(encoded, torch.bfloat16), dev(tok), K)
   assert cross['enc_len'].tolist() == [24, 10, 24]
+  Ep = cross['E']
+  assert Ep == 32
   for (wk, wv), gk, gv in zip(want, cross['k'], cross['v']):
-    np.testing.assert_allclose(host(gk)[:, :, :E].transpose(0, 2, 1, 3), wk,
+    Bk, H = gk.shape[:2]
+    # undo the blocking: [B, H, 2, Ep, 32] -> [B, H, Ep, 64],
+    # [B, H, Ep/32, 64, 32] -> [B, H, 64, Ep]
+    pk = host(gk.permute(0, 1, 3, 2, 4).reshape(Bk, H, Ep, 64))
+    pv = host(gv.permute(0, 1, 3, 2, 4).reshape(Bk, H, 64, Ep))
+    np.testing.assert_allclose(pk[:, :, :E].transpose(0, 2, 1, 3), wk,
                                atol=2e-2, rtol=2**-7)
-    np.testing.assert_allclose(host(gv)[..., :E].transpose(0, 3, 1, 2), wv,
+    np.testing.assert_allclose(pv[..., :E].transpose(0, 3, 1, 2), wv,
                                atol=2e-2, rtol=2**-7)
+    assert not pk[:, :, E:].any() and not pv[..., E:].any()

@@ -327,6 +327,11 @@ def test_cross_attention_step(ops, dt, B, beams, H, E):
                               np.repeat(v, beams, axis=0)))
   kd = dev(np.ascontiguousarray(k.transpose(0, 2, 1, 3)), dt)  # [B,H,E,D]
   vd = dev(np.ascontiguousarray(v.transpose(0, 2, 3, 1)), dt)  # [B,H,D,E]
+  if dt == torch.bfloat16:
+    # blocks of 32 positions: zero-pad E (the padding is beyond every length)
+    Ep = (E + 31) // 32 * 32
+    kd = ops.tile_cross_key(torch.nn.functional.pad(kd, (0, 0, 0, Ep - E)))
+    vd = ops.tile_cross_value(torch.nn.functional.pad(vd, (0, Ep - E)))
   out = ops.cross_attention_step(dev(q, dt), kd, vd, dev(lens), beams)
   np.testing.assert_allclose(host(out), want[:, 0], atol=TOL[dt],
                              rtol=TOL[dt])
@@ -374,7 +379,7 @@ def test_beam_topk(ops, B, beams, V):
 
 
 @pytest.mark.parametrize('B,beams,H,E,d', [(3, 4, 2, 512, 768),
-                                           (2, 8, 3, 264, 256),
+                                           (2, 8, 3, 288, 256),
                                            (32, 4, 12, 512, 768),
                                            (2, 1, 2, 64, 1024),
                                            (2, 3, 2, 128, 64),
@@ -393,7 +398,8 @@ def test_cross_attention_with_fused_norm_and_query_projection(ops, B, beams, H,
   x = (2 * rnd(R, d)).to(bf)
   scale = (1 + 0.1 * rnd(d)).to(bf)
   wq = ops.pack_weight(rnd(d, HD) / (8 * d ** 0.5), bf)
-  ck, cv = rnd(B, H, E, 64).to(bf), rnd(B, H, 64, E).to(bf)
+  ck = ops.tile_cross_key(rnd(B, H, E, 64).to(bf))
+  cv = ops.tile_cross_value(rnd(B, H, 64, E).to(bf))
   lens = torch.randint(1, E + 1, (B,), generator=gen, device='cuda',
                        dtype=torch.int32)
   lens[0] = E
