@@ -148,13 +148,20 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
  * (cache_gather_beams, t5x/decoding.py:1449-1457): row (b, e) attends over the
  * cache of row (b, pending_src[b, e]) and, if the item's beams were permuted,
  * that cache is written into slot (b, e).  After the call the caches equal
- * gather-then-step.  bfloat16 only; beams * ceil(L/128) <= 16. */
+ * gather-then-step.  bfloat16 only; beams * ceil(L/128) <= 16.
+ * pending_src may be NULL (no gather: plain t5d_self_attention_step).
+ * value_blocked != 0: cached_value is stored per (row, head) as
+ * [L/32][64][32] (blocks of 32 positions, L a multiple of 32) instead of the
+ * reference's [64][L]; a caller that owns its caches (a decode loop) gets
+ * loads of consecutive memory for them and converts when it hands the cache
+ * tree out. */
 int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
                                    void* cached_key, void* cached_value,
                                    const void* rel_bias,
                                    const int32_t* cache_index, void* out,
                                    int B, int beams, int H, int L,
-                                   const int32_t* pending_src);
+                                   const int32_t* pending_src,
+                                   int value_blocked);
 
 /* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
  * mask :366-370).  The reference re-projects K/V from the beam-expanded
@@ -355,6 +362,9 @@ typedef struct {
   /* optional [B, beams] source-beam indices of a deferred cache gather, applied
    * inside the self-attention kernels (t5d_self_attention_step_gather) */
   const int32_t* pending_src;
+  /* non-zero: the layers' cached_value are in the blocked layout of
+   * t5d_self_attention_step_gather (bfloat16, L a multiple of 32) */
+  int value_blocked;
 } t5d_model_step;
 
 /* One decoder step for R rows (Decoder.__call__ with decode=True,

@@ -42,7 +42,8 @@ class ModelStep(Structure):
           'embedding', 'rel_bias', 'ln_final', 'logits_w', 'logits_scales')] +
               [('layers', POINTER(Layer))] + [(n, c_void_p) for n in (
                   'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
-                  'ao', 'h', 'logits', 'gate', 'pending_src')])
+                  'ao', 'h', 'logits', 'gate', 'pending_src')] +
+              [('value_blocked', c_int)])
 
 
 class BeamStep(Structure):
@@ -100,7 +101,7 @@ _SIGNATURES = {
                                         c_int, c_int, c_int]),
     't5d_self_attention_step_gather': (c_int, [_P, c_int, _P, _P, _P, _P, _P,
                                                _P, c_int, c_int, c_int, c_int,
-                                               _P]),
+                                               _P, c_int]),
     't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
                                          c_int, c_int, c_int]),
     't5d_cross_attention_step_norm_q': (c_int, [_P, c_int, c_int, _P, _P,

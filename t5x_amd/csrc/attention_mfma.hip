@@ -54,6 +54,7 @@ struct AttnMfmaArgs {
   const void* wq;          // packed [d, H*64] query kernel (bf16 tiles)
   int d;
   float eps;
+  int v_blocked;  // self-attention: value cache stored as [S/32][64][32] per head
 };
 
 constexpr int kHeadDim = 64;
@@ -524,10 +525,18 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       kc[i] = *reinterpret_cast<const uint4*>(
           reinterpret_cast<const char*>(ksrc + (size_t)i * S) + koff);
   }
+  // Byte offset of this lane's chunk of V tile (jb, dt) inside the head's
+  // slot.  Reference layout [64][S]: row 16 dt + n16, positions 32 jb + 8 g ..;
+  // blocked layout [S/32][64][32] (S a multiple of 32): the same chunk sits in
+  // block blk * 4 + jb, and the 64 chunks of a tile are 1 KB of consecutive
+  // memory instead of 16 separate half cache lines.
   uint32_t voff[4];
 #pragma unroll
   for (int jb = 0; jb < 4; ++jb)
-    voff[jb] = (uint32_t)(n16 * S + min(jw + 32 * jb + 8 * g, S - 8)) * 2u;
+    voff[jb] = a.v_blocked
+                   ? (uint32_t)(((blk * 4 + jb) * kHeadDim + n16) * 32 + 8 * g) * 2u
+                   : (uint32_t)(n16 * S + min(jw + 32 * jb + 8 * g, S - 8)) * 2u;
+  const uint32_t vdt = (a.v_blocked ? 16u * 32u : 16u * (uint32_t)S) * 2u;
   Frag16 vb[4][4];
 #pragma unroll
   for (int jb = 0; jb < 4; ++jb) {
@@ -535,8 +544,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
         vb[jb][dt].u = *reinterpret_cast<const uint4*>(
-            reinterpret_cast<const char*>(vsrc + (size_t)(16 * dt) * S) +
-            voff[jb]);
+            reinterpret_cast<const char*>(vsrc) + dt * vdt + voff[jb]);
     }
   }
   // Query: this lane's 16 head dims.  New key / value / query element of
@@ -586,9 +594,8 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
         if (32 * jb < nw) {
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt)
-            *reinterpret_cast<uint4*>(
-                reinterpret_cast<char*>(vdst + (size_t)(16 * dt) * S) +
-                voff[jb]) = vb[jb][dt].u;
+            *reinterpret_cast<uint4*>(reinterpret_cast<char*>(vdst) + dt * vdt +
+                                      voff[jb]) = vb[jb][dt].u;
         }
       }
     }
@@ -602,7 +609,8 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     if (wave_has_t) {
       if (r != rs) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       kdst[(size_t)lane * S + t] = knew_d;
-      vdst[(size_t)lane * S + t] = vnew_d;
+      vdst[a.v_blocked ? ((size_t)(t >> 5) * kHeadDim + lane) * 32 + (t & 31)
+                       : (size_t)lane * S + t] = vnew_d;
     }
   };
 
@@ -745,6 +753,7 @@ int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 const void* x, const void* ln, const void* wq,
                                 int d, float eps) {
   AttnMfmaArgs a;
+  a.v_blocked = 0;
   a.x = (const bf16_t*)x; a.ln = (const bf16_t*)ln; a.wq = wq;
   a.d = d; a.eps = eps;
   a.q = (const bf16_t*)q; a.k = (bf16_t*)k; a.v = (bf16_t*)v;
@@ -760,8 +769,9 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                void* cv, const void* rel_bias,
                                const int32_t* cache_index, void* out, int R,
                                int H, int L, const int32_t* pending,
-                               int beams) {
+                               int beams, int value_blocked) {
   AttnMfmaArgs a;
+  a.v_blocked = value_blocked;
   a.q = (const bf16_t*)qkv; a.k = (bf16_t*)ck; a.v = (bf16_t*)cv;
   a.rel_bias = (const bf16_t*)rel_bias; a.index = cache_index;
   a.out = (bf16_t*)out;

@@ -78,11 +78,11 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
       T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
                        m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
     }
-    if (m->pending_src)
+    if (m->pending_src || m->value_blocked)
       T5D_TRY(t5d_self_attention_step_gather(
           stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
           m->cache_index + l, m->ao, m->B, m->beams, m->H, m->L,
-          m->pending_src));
+          m->pending_src, m->value_blocked));
     else
       T5D_TRY(t5d_self_attention_step(stream, dt, m->qkv, w.cached_key,
                                       w.cached_value, m->rel_bias,

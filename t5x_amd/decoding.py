@@ -545,7 +545,7 @@ class BeamLoop:
     use_fused = (factory is not None and initial_index is None and
                  getattr(cache, 'fresh', False))
     self.fused = None
-    self.cur, self.beam_cache = beam_init(
+    self.cur, self._beam_cache = beam_init(
         batch_size, beam_size, max_decode_len, {} if use_fused else cache,
         cache_offset, live_seqs=live_seqs, initial_index=initial_index_np)
     self.nxt = (self.cur if use_fused else
@@ -568,11 +568,17 @@ class BeamLoop:
     if use_fused:
       self.fused = factory(self)
       if self.fused is None:  # configuration not covered: generic path
-        self.cur, self.beam_cache = beam_init(
+        self.cur, self._beam_cache = beam_init(
             batch_size, beam_size, max_decode_len, cache, cache_offset)
         self.nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)
-      else:
-        self.beam_cache = self.fused.cache_tree()
+
+  @property
+  def beam_cache(self):
+    """The beam-expanded caches in the reference's tree layout (with the fused
+    loop: copies made on request)."""
+    if self.fused is not None:
+      return self.fused.cache_tree()
+    return self._beam_cache
 
   def cond(self) -> bool:
     """:1250-1300 (reads one flag back from the device)."""
@@ -630,7 +636,7 @@ class BeamLoop:
                     self.init_idx_dev, self.brevity, self.top_alive,
                     self.vocab_size, self.eos_id)
     # :1449-1457.  After this step the caches hold step + 1 valid columns.
-    self.beam_cache = cache_gather_beams(new_cache, self.top_alive, B, K, K,
+    self._beam_cache = cache_gather_beams(new_cache, self.top_alive, B, K, K,
                                          True, off)
     self.cur, self.nxt = nxt, cur
     self.step += 1

@@ -371,7 +371,7 @@ class Transformer:
 
   # -- the decode step -------------------------------------------------------------
   def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
-                  L, gate=None, pending_src=None):
+                  L, gate=None, pending_src=None, value_blocked=False):
     """Fills a t5d_model_step for one call of t5d_decoder_step."""
     from t5x_amd import _lib
     cfg = self.config
@@ -403,6 +403,7 @@ class Transformer:
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
     m.pending_src = P(pending_src)
+    m.value_blocked = int(bool(value_blocked))
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
                     pending_src)
     return m
@@ -533,7 +534,11 @@ class FusedSampleStep:
     cross = module._cross_kv(w, enc, enc_tok, beams)
     R, S = sequences.shape
     act = w.act_dtype
-    el = 16 // torch.empty((), dtype=act).element_size()
+    # bfloat16: the value caches are kept in blocks of 32 positions (loads of
+    # consecutive memory); cache_tree() converts back.
+    self.value_blocked = act == torch.bfloat16
+    el = 32 if self.value_blocked else 16 // torch.empty(
+        (), dtype=act).element_size()
     self.L = L = (S - 2 + el - 1) // el * el
     nl = cfg.num_decoder_layers
     self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
@@ -557,7 +562,8 @@ class FusedSampleStep:
     layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
     self.model = module._model_step(w, cross, self.bufs, layer_caches,
                                     self.cache_index, R, beams, L,
-                                    gate=self.keep_going)
+                                    gate=self.keep_going,
+                                    value_blocked=self.value_blocked)
     P = _lib.ptr
     st = _lib.SampleStep()
     st.sequences, st.cur_index, st.cur_token = (P(sequences), P(cur_index),
@@ -626,10 +632,12 @@ class FusedSampleStep:
   def cache_tree(self):
     """The caches in the reference's tree layout."""
     self.stream.synchronize()
+    from t5x_amd import ops
     nl = self.kv.shape[0]
+    value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
     return {'decoder': {
         f'layers_{i}': {'self_attention': {
-            'cached_key': self.kv[i, 0], 'cached_value': self.kv[i, 1],
+            'cached_key': self.kv[i, 0], 'cached_value': value(self.kv[i, 1]),
             'cache_index': self.cache_index[i]}} for i in range(nl)}}
 
   def __del__(self):
@@ -675,7 +683,8 @@ class _BeamLane:
     self.model = module._model_step(
         w, lane_cross, self.bufs, layer_caches, self.cache_index, R, K, L,
         gate=self.keep_going,
-        pending_src=self.top_alive if owner.deferred_gather else None)
+        pending_src=self.top_alive if owner.deferred_gather else None,
+        value_blocked=owner.value_blocked)
     st = loop.cur
     P = _lib.ptr
     ptrs = _lib.BeamStatePtrs()
@@ -740,12 +749,24 @@ class FusedBeamStep:
     S = loop.max_decode_len
     act = w.act_dtype
     el = 16 // torch.empty((), dtype=act).element_size()
-    self.L = L = (S - 1 + el - 1) // el * el
+    L = (S - 1 + el - 1) // el * el
     # With bfloat16 caches the reorder of a step is deferred into the next
     # step's self-attention kernels, which read each row's cache from its
     # source beam anyway; the permutation in flight lives in loop.top_alive.
     self.deferred_gather = (K > 1 and act == torch.bfloat16 and
                             K * ((L + 127) // 128) <= 16)
+    # The value caches are then kept in blocks of 32 positions (loads of
+    # consecutive memory); cache_tree() converts back.  (The stand-alone
+    # reorder kernel of the other path copies row prefixes, which only the
+    # reference layout has.)
+    self.value_blocked = self.deferred_gather or (K == 1 and
+                                                  act == torch.bfloat16)
+    if self.value_blocked:
+      L = (L + 31) // 32 * 32
+      if K * ((L + 127) // 128) > 16:
+        self.value_blocked = self.deferred_gather = False
+        L = (S - 1 + el - 1) // el * el
+    self.L = L
     loop.top_alive.copy_(torch.arange(K, dtype=torch.int32,
                                       device=dev).expand(B, K))
     if lanes is None:
@@ -853,9 +874,10 @@ class FusedBeamStep:
     nl = self.lanes[0].kv.shape[0]
     kv = torch.cat([lane.kv for lane in self.lanes], dim=2)
     idx = self.lanes[0].cache_index
+    value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
     return {'decoder': {
         f'layers_{i}': {'self_attention': {
-            'cached_key': kv[i, 0], 'cached_value': kv[i, 1],
+            'cached_key': kv[i, 0], 'cached_value': value(kv[i, 1]),
             'cache_index': idx[i]}} for i in range(nl)}}
 
   def __del__(self):

@@ -213,10 +213,28 @@ def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
   return out
 
 
+def block_cached_value(v):
+  """[R, H, 64, L] value cache -> the blocked [R, H, L/32, 64, 32] layout
+  (same bytes count; L a multiple of 32)."""
+  R, H, D, L = v.shape
+  return v.reshape(R, H, D, L // 32, 32).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def unblock_cached_value(v):
+  """Inverse of block_cached_value: [R, H, L/32, 64, 32] (or the same memory
+  viewed as [R, H, 64, L]) -> [R, H, 64, L]."""
+  R, H = v.shape[:2]
+  L = v.numel() // (R * H * 64)
+  return v.reshape(R, H, L // 32, 64, 32).permute(0, 1, 3, 2, 4).reshape(
+      R, H, 64, L)
+
+
 def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
-                        out=None, pending_src=None):
+                        out=None, pending_src=None, value_blocked=False):
   """One cached self-attention step; with pending_src [B, beams] the rows'
-  caches are first gathered from their source beams inside the kernel."""
+  caches are first gathered from their source beams inside the kernel.
+  value_blocked: cached_value holds the blocked layout (see
+  block_cached_value) in a tensor of the usual [R, H, 64, L] shape."""
   _chk(qkv, 'qkv', ndim=2)
   _chk(cached_key, 'cached_key', qkv.dtype, 4)
   _chk(cached_value, 'cached_value', qkv.dtype, 4)
@@ -236,16 +254,18 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
   if out is None:
     out = torch.empty((R, H * D), dtype=qkv.dtype, device=qkv.device)
   _chk(out, 'out', qkv.dtype, 2)
-  if pending_src is not None:
-    _chk(pending_src, 'pending_src', torch.int32, 2)
-    B, beams = pending_src.shape
-    if B * beams != R:
-      raise ValueError(f'pending_src {(B, beams)} does not cover {R} rows')
+  if pending_src is not None or value_blocked:
+    B, beams = R, 1
+    if pending_src is not None:
+      _chk(pending_src, 'pending_src', torch.int32, 2)
+      B, beams = pending_src.shape
+      if B * beams != R:
+        raise ValueError(f'pending_src {(B, beams)} does not cover {R} rows')
     _lib.call('t5d_self_attention_step_gather', _s(),
               _lib.dtype_code(qkv.dtype), qkv.data_ptr(),
               cached_key.data_ptr(), cached_value.data_ptr(),
               rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), B,
-              beams, H, L, pending_src.data_ptr())
+              beams, H, L, _lib.ptr(pending_src), int(bool(value_blocked)))
     return out
   _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
             qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),

@@ -299,6 +299,28 @@ def test_self_attention_step_with_pending_gather(ops, B, beams, H, L, t):
   assert torch.equal(ck_b[..., :t + 1], ck_a[..., :t + 1])
   assert torch.equal(cv_b[..., :t + 1], cv_a[..., :t + 1])
 
+  # The same step with the value cache in blocks of 32 positions
+  # ([R, H, L/32, 64, 32]), with the deferred reorder and without: identical
+  # outputs and, converted back, identical caches.
+  ck_c = ck.clone()
+  cv_c = ops.block_cached_value(cv).view(R, H, D, L)
+  got_c = ops.self_attention_step(qkv, ck_c, cv_c, rel_bias, idx,
+                                  pending_src=src, value_blocked=True)
+  assert torch.equal(got_c, want)
+  assert torch.equal(ck_c[..., :t + 1], ck_a[..., :t + 1])
+  assert torch.equal(ops.unblock_cached_value(cv_c)[..., :t + 1],
+                     cv_a[..., :t + 1])
+  cv_plain = cv.clone()
+  ops.cache_gather_beams(cv_plain.view(B, beams, H, D, L), src, valid_len=valid)
+  cv_d = ops.block_cached_value(cv_plain).view(R, H, D, L)
+  ck_e = ck.clone()
+  ops.cache_gather_beams(ck_e.view(B, beams, H, D, L), src, valid_len=valid)
+  got_d = ops.self_attention_step(qkv, ck_e, cv_d, rel_bias, idx,
+                                  value_blocked=True)
+  assert torch.equal(got_d, want)
+  assert torch.equal(ops.unblock_cached_value(cv_d)[..., :t + 1],
+                     cv_a[..., :t + 1])
+
 
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('B,beams,H,E', [(2, 1, 3, 64), (3, 4, 2, 512),
