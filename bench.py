@@ -141,8 +141,7 @@ class Workload:
         if not self.loop.cond():
           raise RuntimeError('fresh decode terminated immediately')
       take = min(n - done, self.L - self.loop.step)
-      for _ in range(take):
-        self.loop.body()
+      self.loop.advance(take)
       done += take
 
   def check_full_decode(self):

@@ -600,6 +600,16 @@ class BeamLoop:
       self.fused.launch(check_every)
       self.step += check_every
 
+  def advance(self, n: int):
+    """n loop iterations without looking at the condition in between (with the
+    fused loop: iterations past its end change nothing)."""
+    if self.fused is not None:
+      self.fused.launch(n)
+      self.step += n
+      return
+    for _ in range(n):
+      self.body()
+
   def body(self):
     """:1302-1506."""
     if self.fused is not None:

@@ -248,6 +248,7 @@ class Transformer:
     self._bufs = {}
     self._cross = None
     self._step_cache = None
+    self._beam_ctx = {}
 
   # -- plumbing ---------------------------------------------------------------
   def _dev(self):
@@ -317,11 +318,22 @@ class Transformer:
         'initialisation) are implemented')
 
   # -- cross-attention K/V, once per batch ---------------------------------------
-  def _cross_kv(self, w: DecoderWeights, encoded, enc_tokens, beams):
+  def _cross_kv(self, w: DecoderWeights, encoded, enc_tokens, beams, out=None):
+    """Projects the encoder output to every decoder layer's cross-attention
+    K/V, once per batch.  `out`: a result of an earlier call with the same
+    shapes whose tensors are to be (re)used — a decode context that has their
+    addresses recorded in a captured graph passes its own."""
     key = (encoded.data_ptr(), tuple(encoded.shape), enc_tokens.data_ptr(),
            id(w), encoded._version)
     if self._cross is not None and self._cross[0] == key:
-      return self._cross[1]
+      res = self._cross[1]
+      if out is None or res is out:
+        return res
+      for dst, src in zip(out['k'] + out['v'], res['k'] + res['v']):
+        dst.copy_(src)
+      out['enc_len'].copy_(res['enc_len'])
+      self._cross = (key, out, encoded)
+      return out
     cfg = self.config
     B, E, d = encoded.shape
     H, D = cfg.num_heads, cfg.head_dim
@@ -331,16 +343,20 @@ class Transformer:
     # positions).  Padding positions e >= E stay zero.
     pad = 32 if bf16 else 16 // encoded.element_size()
     Ep = (E + pad - 1) // pad * pad
+    if out is not None and (out['B'], out['E']) != (B, Ep):
+      raise ValueError('cross K/V buffers of another shape')
     x = encoded.reshape(B * E, d).contiguous()
     ks, vs = [], []
     hip = bf16 and E % 4 == 0
-    for l in w.layers:
+    for i, l in enumerate(w.layers):
       if hip:
         # straight from the dense kernel's epilogue
         from t5x_amd import _lib
         ks.append(ops.gemm_rows(x, l['cross_k_packed'],
+                                out=out['k'][i] if out else None,
                                 layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep))
         vs.append(ops.gemm_rows(x, l['cross_v_packed'],
+                                out=out['v'][i] if out else None,
                                 layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep))
         continue
       for (kern, scale), dst in ((l['cross_k'], ks), (l['cross_v'], vs)):
@@ -351,11 +367,14 @@ class Transformer:
         if dst is ks:  # keys: [B, H, E, D], head dim contiguous
           buf = torch.zeros((B, H, Ep, D), dtype=x.dtype, device=x.device)
           buf[:, :, :E] = y.permute(0, 2, 1, 3)
-          dst.append(ops.tile_cross_key(buf) if bf16 else buf)
+          buf = ops.tile_cross_key(buf) if bf16 else buf
         else:  # values: [B, H, D, E], positions contiguous
           buf = torch.zeros((B, H, D, Ep), dtype=x.dtype, device=x.device)
           buf[..., :E] = y.permute(0, 2, 3, 1)
-          dst.append(ops.tile_cross_value(buf) if bf16 else buf)
+          buf = ops.tile_cross_value(buf) if bf16 else buf
+        if out is not None:
+          buf = (out['k'] if dst is ks else out['v'])[i].copy_(buf)
+        dst.append(buf)
     tok = enc_tokens.reshape(B, E)
     valid = tok > 0
     # The mask keeps exactly the positions with token > 0 (network.py:366-370).
@@ -365,9 +384,14 @@ class Transformer:
               lens[:, None])
     if not bool((prefix == valid).all()):
       raise ValueError('encoder padding must be a suffix of zeros')
-    out = dict(k=ks, v=vs, enc_len=lens.contiguous(), B=B, beams=beams, E=Ep)
-    self._cross = (key, out, encoded)
-    return out
+    if out is not None:
+      out['enc_len'].copy_(lens)
+      res = out
+    else:
+      res = dict(k=ks, v=vs, enc_len=lens.contiguous(), B=B, beams=beams,
+                 E=Ep)
+    self._cross = (key, res, encoded)
+    return res
 
   # -- the decode step -------------------------------------------------------------
   def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
@@ -487,12 +511,30 @@ class Transformer:
   # -- fused beam search: one graph replay per loop iteration ------------------------
   def make_fused_beam_step(self, loop, params, encoded, enc_tokens):
     """Returns a FusedBeamStep driving `loop` (a decoding.BeamLoop), or None
-    when this configuration has to use the generic per-call path."""
+    when this configuration has to use the generic per-call path.  The step
+    object (caches, cross K/V buffers, state, captured graphs) is kept and
+    re-bound to the next loop of the same shape and options, so a stream of
+    batches pays for allocation and graph capture once."""
     if not isinstance(encoded, BeamShared) or loop.cache_offset != 0:
       return None
     if loop.beam_size > 8:
       return None
-    return FusedBeamStep(self, loop, params, encoded, enc_tokens)
+    w = self.decoder_weights(params)
+    key = (id(w), tuple(encoded.x.shape), encoded.x.dtype, encoded.beams,
+           loop.batch_size, loop.beam_size, loop.max_decode_len,
+           tuple(loop.inputs_dev.shape), tuple(loop.brevity.shape),
+           int(loop.eos_id), float(loop.min_brevity), float(loop.min_log_prob),
+           int(loop.max_decode_step), int(loop.min_initial),
+           int(self.decode_lanes))
+    ctx = self._beam_ctx.get(key)
+    if ctx is not None:
+      ctx.rebind(loop, encoded, enc_tokens)
+      return ctx
+    ctx = FusedBeamStep(self, loop, params, encoded, enc_tokens)
+    if len(self._beam_ctx) >= 2:  # a context holds the caches: keep few
+      self._beam_ctx.pop(next(iter(self._beam_ctx)))
+    self._beam_ctx[key] = ctx
+    return ctx
 
 
   # -- fused sampling: one graph replay per loop iteration --------------------------
@@ -716,6 +758,7 @@ class _BeamLane:
     self.stream = torch.cuda.Stream(device=dev)
     self.event = torch.cuda.Event()
     self.graph = None
+    self.graph_long = None
 
 
 class FusedBeamStep:
@@ -776,9 +819,57 @@ class FusedBeamStep:
     bounds = [B * i // n for i in range(n + 1)]
     self.lane_cur_index = loop.cur.cur_index.to(torch.int32).reshape(1).repeat(n)
     self.cond_event = torch.cuda.Event()
+    # What the captured graphs hold addresses of, beyond the lanes' own
+    # buffers: the loop's state.  A later loop is re-bound onto these.
+    self.w, self.cross = w, cross
+    self.state = loop.cur
+    self.inputs_dev, self.init_idx_dev = loop.inputs_dev, loop.init_idx_dev
+    self.brevity, self.flag = loop.brevity, loop.keep_going
+    self.top_alive = loop.top_alive
     self.lanes = [_BeamLane(self, i, bounds[i], bounds[i + 1], w, cross)
                   for i in range(n)]
     self._capture()
+
+  _STATE_FIELDS = ('cur_index', 'live_logprobs', 'finished_scores', 'live_seqs',
+                   'finished_seqs', 'finished_flags')
+
+  def rebind(self, loop, encoded, enc_tokens):
+    """Takes over a freshly initialised loop of the same shape and options:
+    its initial state is copied into the buffers the captured graphs address
+    (which the loop then uses as its own), the new encoder output is projected
+    into the same cross K/V buffers, caches and counters start from zero."""
+    module, dev = self.module, self.device
+    cur = torch.cuda.current_stream()
+    for lane in self.lanes:  # whatever the previous loop left in flight
+      cur.wait_stream(lane.stream)
+    enc_tok = enc_tokens.x
+    enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
+        enc_tok, torch.Tensor) else enc_tok.to(dev)
+    cross = module._cross_kv(self.w, encoded.x, enc_tok, encoded.beams,
+                             out=self.cross)
+    assert cross is self.cross
+    for name in self._STATE_FIELDS:
+      getattr(self.state, name).copy_(getattr(loop.cur, name))
+    self.inputs_dev.copy_(loop.inputs_dev)
+    self.init_idx_dev.copy_(loop.init_idx_dev)
+    self.brevity.copy_(loop.brevity)
+    K = loop.beam_size
+    self.top_alive.copy_(torch.arange(K, dtype=torch.int32, device=dev).expand(
+        loop.batch_size, K))
+    self.lane_cur_index.copy_(
+        loop.cur.cur_index.to(torch.int32).reshape(1).expand(self.n_lanes))
+    for lane in self.lanes:
+      lane.kv.zero_()
+      lane.cache_index.zero_()
+    loop.cur = loop.nxt = self.state
+    loop.inputs_dev, loop.init_idx_dev = self.inputs_dev, self.init_idx_dev
+    loop.brevity, loop.keep_going = self.brevity, self.flag
+    loop.top_alive = self.top_alive
+    self.loop = loop
+    for lane in self.lanes:
+      lane.stream.wait_stream(cur)
+    self._cond(self.lanes[0].stream)
+    self.lanes[0].stream.synchronize()
 
   def _enqueue(self, lane):
     self._lib.call('t5d_beam_search_step', lane.stream.cuda_stream,
@@ -801,8 +892,23 @@ class FusedBeamStep:
                    int(loop.max_decode_step), int(loop.min_initial),
                    loop.keep_going.data_ptr())
 
+  # Iterations recorded in the long graph of a single-lane loop: one launch
+  # (and one gap between launches) per that many iterations.
+  GRAPH_STEPS = 8
+
+  def _record(self, lane, steps):
+    lib = self._lib
+    lib.call('t5d_graph_begin', lane.stream.cuda_stream)
+    try:
+      for _ in range(steps):
+        self._enqueue(lane)
+    finally:
+      handle = ctypes_void_p()
+      lib.call('t5d_graph_end', lane.stream.cuda_stream, handle_ref(handle))
+    return handle
+
   def _capture(self):
-    lib, loop = self._lib, self.loop
+    loop = self.loop
     cur = torch.cuda.current_stream()
     for lane in self.lanes:
       lane.stream.wait_stream(cur)
@@ -812,14 +918,9 @@ class FusedBeamStep:
         loop.keep_going.zero_()
         self._enqueue(lane)
         lane.stream.synchronize()
-        lib.call('t5d_graph_begin', lane.stream.cuda_stream)
-        try:
-          self._enqueue(lane)
-        finally:
-          handle = ctypes_void_p()
-          lib.call('t5d_graph_end', lane.stream.cuda_stream,
-                   handle_ref(handle))
-        lane.graph = handle
+        lane.graph = self._record(lane, 1)
+        if self.n_lanes == 1:
+          lane.graph_long = self._record(lane, self.GRAPH_STEPS)
       lane.stream.synchronize()
     self._cond(self.lanes[0].stream)
     self.lanes[0].stream.synchronize()
@@ -827,18 +928,25 @@ class FusedBeamStep:
   def launch(self, n=1):
     lanes, lib = self.lanes, self._lib
     first = lanes[0].stream
+    if len(lanes) == 1:
+      lane = lanes[0]
+      while n >= self.GRAPH_STEPS:
+        lib.call('t5d_graph_launch', lane.graph_long, first.cuda_stream)
+        n -= self.GRAPH_STEPS
+      for _ in range(n):
+        lib.call('t5d_graph_launch', lane.graph, first.cuda_stream)
+      return
     for _ in range(n):
       for lane in lanes:
         lib.call('t5d_graph_launch', lane.graph, lane.stream.cuda_stream)
-      if len(lanes) > 1:
-        # join -> one condition for the whole batch -> fork
-        for lane in lanes[1:]:
-          lane.event.record(lane.stream)
-          first.wait_event(lane.event)
-        self._cond(first)
-        self.cond_event.record(first)
-        for lane in lanes[1:]:
-          lane.stream.wait_event(self.cond_event)
+      # join -> one condition for the whole batch -> fork
+      for lane in lanes[1:]:
+        lane.event.record(lane.stream)
+        first.wait_event(lane.event)
+      self._cond(first)
+      self.cond_event.record(first)
+      for lane in lanes[1:]:
+        lane.stream.wait_event(self.cond_event)
 
   def synchronize(self):
     for lane in self.lanes:
@@ -883,8 +991,9 @@ class FusedBeamStep:
   def __del__(self):
     try:
       for lane in self.lanes:
-        if lane.graph is not None:
-          self._lib.call('t5d_graph_destroy', lane.graph)
+        for g in (lane.graph, lane.graph_long):
+          if g is not None:
+            self._lib.call('t5d_graph_destroy', g)
     except Exception:  # pylint: disable=broad-except
       pass
 

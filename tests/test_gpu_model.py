@@ -423,6 +423,50 @@ def test_fused_loop_early_stop_is_independent_of_check_interval(check_every,
   assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
 
 
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_fused_loop_context_is_reused_across_batches(dtype):
+  """A second (and third) batch of the same shape on the same module re-binds
+  the first one's decode context — caches, cross K/V buffers, state, captured
+  graphs — instead of building a new one; every batch must still equal the
+  kernel-per-call loop, also after a batch that stopped early and with a
+  decode length that is not a multiple of the long graph's 8 iterations."""
+  from t5x_amd import decoding, models, network
+  B, K, E, L = 3, 4, 16, 21
+  _, gcfg = tiny(dtype)
+  dev = torch.device('cuda')
+  params = network.init_params(gcfg, 3, dev, with_encoder=False)
+  params['decoder']['logits_dense']['kernel'][:, 1] *= 3.0  # some early EOS
+  module = network.Transformer(gcfg, dev)
+  model = models.EncoderDecoderModel(module, decode_fn=decoding.beam_search)
+  inputs = np.zeros((B, L), np.int32)
+  first = None
+  for batch in range(3):
+    rs = np.random.RandomState(100 + batch)
+    tok = torch.as_tensor(ragged_tokens(rs, B, E, gcfg.vocab_size, 3),
+                          device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(200 + batch)
+    encoded = torch.randn((B, E, gcfg.emb_dim), generator=gen,
+                          device=dev).to(network._TORCH_DTYPE[dtype])
+    fn = models.StepFunction(model, params, network.BeamShared(encoded, K),
+                             network.BeamShared(tok, K), L)
+    plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
+                              eos_id=1, num_decodes=K)
+    plain.run()
+    want, ws = plain.finish()
+    fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                              num_decodes=K)
+    assert fused.fused is not None
+    if first is None:
+      first = fused.fused
+    assert fused.fused is first and len(module._beam_ctx) == 1
+    fused.run()
+    got, gs = fused.finish()
+    assert int(fused.cur.cur_index.item()) == int(plain.cur.cur_index.item())
+    assert torch.equal(torch.as_tensor(got), torch.as_tensor(want)), batch
+    assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws)), batch
+
+
 class _SuppliedNoise:
   """Pre-generated Gumbel noise [steps, rows, vocab], one slice per step."""
 
