@@ -241,7 +241,7 @@ def roofline_cross_attention(w, reps_per_layer=4):
   layers = w.weights.layers
   nl = len(cross['k'])
   fused = (w.weights.layers[0]['cross_q'].w_dtype == 1 and cross['E'] <= 512
-           and cfg.emb_dim <= 1024)
+           and cfg.emb_dim <= 768)  # as t5d_decoder_step chooses
   state = {'i': 0}
 
   def launch():
