@@ -31,6 +31,8 @@ CONFIGS = {
     # name: (size, batch, decodes per item, enc_len, enc_min_len,
     #        max_decode_len, dtype, weight_dtype, loop)
     # loop: 'beam' or ('sample', temperature, topk)
+    'small-fp32-greedy': ('small', 8, 1, 64, 64, 32, 'float32', None,
+                          ('sample', 0.0, 0)),
     'base-beam4': ('base', 32, 4, 512, 128, 128, 'bfloat16', None, 'beam'),
     'xl-int8-beam4': ('xl', 16, 4, 512, 512, 128, 'bfloat16', 'int8', 'beam'),
     'large-sample': ('large', 64, 1, 512, 512, 256, 'bfloat16', None,
@@ -155,7 +157,7 @@ class Workload:
     """Valid K and V rows once per batch item and the attention output out;
     in: the residual-stream rows, the layer-norm scale and the query kernel
     (fused projection), or the projected queries."""
-    s = 2  # bf16
+    s = self.encoded.element_size()
     hd = self.cfg.num_heads * self.cfg.head_dim
     d = self.cfg.emb_dim
     R = self.B * self.K
@@ -370,7 +372,8 @@ def main():
       'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
       'ms_per_step': round(elapsed / args.steps * 1e3, 4),
       'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-      'dtype': 'bf16' if wdt is None else f'bf16 act / {wdt} weights',
+      'dtype': ({'bfloat16': 'bf16', 'float32': 'f32'}[dtype] if wdt is None
+                else f'bf16 act / {wdt} weights'),
       'data': 'synthetic',
       'config': {'workload': f'T5.1.1-{size} {what}, encoder {E} ({Emin}..{E} '
                              f'valid), max decode length {L}',

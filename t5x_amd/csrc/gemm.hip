@@ -444,7 +444,40 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
   const int kq = (K + 3) / 4;
   const int kb = wave * kq, ke = min(K, kb + kq);
-  for (int k = kb; k < ke; ++k) {
+  int k = kb;
+  if ((K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
+    // 8 k per pass, all loads of a pass in flight together; the products are
+    // still accumulated in ascending k, one fma each.
+    for (; k + 8 <= ke; k += 8) {
+      float w0[8], w1[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        w0[u] = active ? W[(size_t)(k + u) * N + n] : 0.f;
+        w1[u] = (active && geglu) ? W[(size_t)(k + u) * N + F + n] : 0.f;
+      }
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        const int row = m0 + m;
+        float a[8];
+        if (row < M) {
+          const float4* ap =
+              reinterpret_cast<const float4*>(A + (size_t)row * K + k);
+          const float4 x = ap[0], y = ap[1];
+          a[0] = x.x; a[1] = x.y; a[2] = x.z; a[3] = x.w;
+          a[4] = y.x; a[5] = y.y; a[6] = y.z; a[7] = y.w;
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) a[u] = 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          acc0[m] = fmaf(a[u], w0[u], acc0[m]);
+          acc1[m] = fmaf(a[u], w1[u], acc1[m]);
+        }
+      }
+    }
+  }
+  for (; k < ke; ++k) {
     const float w0 = active ? W[(size_t)k * N + n] : 0.f;
     const float w1 = (active && geglu) ? W[(size_t)k * N + F + n] : 0.f;
 #pragma unroll
