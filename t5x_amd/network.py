@@ -527,6 +527,9 @@ class Transformer:
            int(loop.max_decode_step), int(loop.min_initial),
            int(self.decode_lanes))
     ctx = self._beam_ctx.get(key)
+    if ctx is not None and ctx.w is not w:  # an id reused by other weights
+      del self._beam_ctx[key]
+      ctx = None
     if ctx is not None:
       ctx.rebind(loop, encoded, enc_tokens)
       return ctx
