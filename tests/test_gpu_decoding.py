@@ -24,8 +24,10 @@ def decoding():
 
 
 def host(t):
-  return t.detach().cpu().numpy() if isinstance(t, torch.Tensor) else \
-      np.asarray(t)
+  if isinstance(t, torch.Tensor):
+    t = t.detach()
+    return (t.float() if t.dtype == torch.bfloat16 else t).cpu().numpy()
+  return np.asarray(t)
 
 
 def const_logits(logits, calls=None):
@@ -179,6 +181,42 @@ def test_beam_dim_helpers(decoding):
   np.testing.assert_array_equal(
       [[0, 5, 1, 0], [0, 5, 1, 0], [0, 8, 6, 9], [0, 8, 6, 9]],
       host(decoding.flat_batch_beam_expand(x, beam_size=2)))
+
+
+@pytest.mark.parametrize('dt,L', [(torch.bfloat16, 16), (torch.float32, 8),
+                                  (torch.float32, 5)])
+def test_beam_dim_helpers_with_a_leading_layer_axis(decoding, dt, L):
+  """offset=1 (caches of scanned layers, [layers, batch, ...]) against the
+  oracle's helpers; the gather runs in place on rows of 16-byte multiples and
+  out of place otherwise (L=5)."""
+  from oracle import decoding as odec
+  rs = np.random.RandomState(L)
+  layers, B, K, H = 3, 2, 4, 2
+  x = rs.randn(layers, B, H, 64, L).astype(np.float32)
+  xd = torch.as_tensor(x, device='cuda').to(dt)
+  xr = host(xd)
+  y = decoding.add_beam_dim(xd, K, offset=1)
+  np.testing.assert_array_equal(host(y), odec.add_beam_dim(xr, K, offset=1))
+  flat = decoding.flatten_beam_dim(y, offset=1)
+  np.testing.assert_array_equal(
+      host(flat), odec.flatten_beam_dim(odec.add_beam_dim(xr, K, 1), 1))
+  np.testing.assert_array_equal(
+      host(decoding.unflatten_beam_dim(flat, B, K, offset=1)), host(y))
+  z = rs.randn(layers, B, K, H, 64, L).astype(np.float32)
+  zd = torch.as_tensor(z, device='cuda').to(dt)
+  zr = host(zd).copy()
+  idx = rs.randint(0, K, size=(B, K)).astype(np.int32)
+  tree = {'decoder': {'layers': {'cached_key': zd,
+                                 'cache_index': torch.zeros((), dtype=torch.int32,
+                                                            device='cuda')}}}
+  got = decoding.cache_gather_beams(tree, idx, B, K, K, offset=1)
+  want = odec.cache_gather_beams(
+      {'decoder': {'layers': {'cached_key': zr,
+                              'cache_index': np.int32(0)}}}, idx, B, K, K,
+      offset=1)
+  np.testing.assert_array_equal(
+      host(got['decoder']['layers']['cached_key']),
+      want['decoder']['layers']['cached_key'])
 
 
 @pytest.mark.parametrize('batch,k', [(1, 16), (8, 16), (9, 11), (32, 11)])

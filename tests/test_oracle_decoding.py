@@ -188,6 +188,30 @@ def test_add_beam_dim_and_expand():
       decoding.flat_batch_beam_expand(x, beam_size=2))
 
 
+def test_beam_dim_helpers_with_a_leading_layer_axis():
+  """offset=1 (caches of scanned layers, [layers, batch, ...],
+  t5x/decoding.py:773-870): the beam axis goes after the batch axis, which is
+  then axis 1.  Closed form: plain NumPy indexing."""
+  rs = np.random.RandomState(0)
+  x = rs.randn(2, 3, 5).astype(np.float32)            # [layers, batch, d]
+  y = decoding.add_beam_dim(x, 4, offset=1)
+  assert y.shape == (2, 3, 4, 5)
+  np.testing.assert_array_equal(y, np.broadcast_to(x[:, :, None], y.shape))
+  flat = decoding.flatten_beam_dim(y, offset=1)
+  assert flat.shape == (2, 12, 5)
+  np.testing.assert_array_equal(flat, np.repeat(x, 4, axis=1))
+  np.testing.assert_array_equal(
+      decoding.unflatten_beam_dim(flat, 3, 4, offset=1), y)
+  np.testing.assert_array_equal(
+      decoding.flat_batch_beam_expand(x, 4, offset=1), flat)
+  z = rs.randn(2, 3, 4, 5).astype(np.float32)
+  idx = rs.randint(0, 4, size=(3, 4))
+  got = decoding.cache_gather_beams({'k': z, 'cache_index': np.int32(7)}, idx,
+                                    3, 4, 4, offset=1)
+  np.testing.assert_array_equal(got['k'], z[:, np.arange(3)[:, None], idx])
+  assert got['cache_index'] == 7
+
+
 @pytest.mark.parametrize('batch,k', [(1, 16), (8, 16), (9, 11), (32, 11)])
 def test_top_k_two_stage_equals_plain_top_k(batch, k):
   # decoding_test.py:825-843
