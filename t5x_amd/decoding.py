@@ -396,7 +396,8 @@ def _temperature_sample_single_trial(
         eos_id=eos_id, topk=topk, topp=topp, rescale=rescale_log_probs,
         noise_source=source if any_sampling else None)
     fused.run()
-    return sequences[:, 1:-1], log_prob
+    # the context's buffers serve the next call too: hand out copies
+    return fused.sequences[:, 1:-1].clone(), fused.log_prob.clone()
 
   def loop_state():
     return SamplingLoopState(

@@ -542,15 +542,32 @@ class Transformer:
 
   # -- fused sampling: one graph replay per loop iteration --------------------------
   def make_fused_sample_step(self, params, encoded, enc_tokens, **kw):
-    """Returns a FusedSampleStep (see there for the arguments)."""
+    """Returns a FusedSampleStep (see there for the arguments).  Like the beam
+    contexts, the step object is kept per (weights, shapes, options) and
+    re-bound to the next call's state."""
     beams = encoded.beams if isinstance(encoded, BeamShared) else 1
+    enc = encoded.x if isinstance(encoded, BeamShared) else encoded
     rows = kw['sequences'].shape[0]
-    enc_rows = (encoded.x if isinstance(encoded, BeamShared) else
-                encoded).shape[0]
-    if rows != enc_rows * beams:
-      raise ValueError(f'{rows} decoder rows vs {enc_rows} x {beams} encoder '
-                       'rows')
-    return FusedSampleStep(self, params, encoded, enc_tokens, **kw)
+    if rows != enc.shape[0] * beams:
+      raise ValueError(f'{rows} decoder rows vs {enc.shape[0]} x {beams} '
+                       'encoder rows')
+    w = self.decoder_weights(params)
+    key = ('sample', id(w), tuple(enc.shape), enc.dtype, beams,
+           tuple(kw['sequences'].shape), int(kw['eos_id']), int(kw['topk']),
+           float(kw['topp']), bool(kw['rescale']),
+           kw.get('noise_source') is not None)
+    ctx = self._beam_ctx.get(key)
+    if ctx is not None and ctx.w is not w:
+      del self._beam_ctx[key]
+      ctx = None
+    if ctx is not None:
+      ctx.rebind(encoded, enc_tokens, **kw)
+      return ctx
+    ctx = FusedSampleStep(self, params, encoded, enc_tokens, **kw)
+    if len(self._beam_ctx) >= 2:
+      self._beam_ctx.pop(next(iter(self._beam_ctx)))
+    self._beam_ctx[key] = ctx
+    return ctx
 
 
 class FusedSampleStep:
@@ -577,6 +594,15 @@ class FusedSampleStep:
     enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
         enc_tok, torch.Tensor) else enc_tok.to(dev)
     cross = module._cross_kv(w, enc, enc_tok, beams)
+    self.w, self.cross = w, cross
+    # The state the captured graph addresses; a later call is re-bound onto it
+    # and reads its results (sequences, log_prob) from here.
+    self.sequences, self.cur_index, self.cur_token = (sequences, cur_index,
+                                                      cur_token)
+    self.ended, self.log_prob = ended, log_prob
+    self.max_decode_len, self.initial_eos_count = (max_decode_len,
+                                                   initial_eos_count)
+    self.temperature = temperature
     R, S = sequences.shape
     act = w.act_dtype
     # bfloat16: the value caches are kept in blocks of 32 positions (loads of
@@ -630,6 +656,37 @@ class FusedSampleStep:
     self.graph = None
     self.step = 0
     self._capture()
+
+  _STATE = ('sequences', 'cur_index', 'cur_token', 'ended', 'log_prob',
+            'max_decode_len', 'initial_eos_count', 'temperature')
+
+  def rebind(self, encoded, enc_tokens, *, noise_source=None, **state):
+    """Starts another call of the same shape and options on this context: the
+    new state is copied into the buffers the graph addresses, the new encoder
+    output is projected into the same cross K/V buffers, caches and counters
+    restart."""
+    module, dev = self.module, self.device
+    cur = torch.cuda.current_stream()
+    cur.wait_stream(self.stream)
+    if isinstance(encoded, BeamShared):
+      beams, enc, enc_tok = encoded.beams, encoded.x, enc_tokens.x
+    else:
+      beams, enc, enc_tok = 1, encoded, enc_tokens
+    enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
+        enc_tok, torch.Tensor) else enc_tok.to(dev)
+    cross = module._cross_kv(self.w, enc, enc_tok, beams, out=self.cross)
+    assert cross is self.cross
+    for name in self._STATE:
+      getattr(self, name).copy_(state[name])
+    self.all_ended.zero_()
+    self.keep_going.fill_(1)
+    self.step_count.zero_()
+    self.kv.zero_()
+    self.cache_index.zero_()
+    self.noise_source = noise_source
+    self.max_steps = int(self.max_decode_len.max().item())
+    self.step = 0
+    self.stream.wait_stream(cur)
 
   def _enqueue(self):
     self._lib.call('t5d_temperature_sample_step', self.stream.cuda_stream,

@@ -515,6 +515,44 @@ def test_fused_sampling_loop_equals_generic_loop(dtype, eos_bias, kw):
     assert lens.max() < L - 8, lens  # the case does stop early
 
 
+@pytest.mark.parametrize('kw', [dict(temperature=0.0),
+                                dict(temperature=0.8, topk=10, num_decodes=2)])
+def test_fused_sampling_context_is_reused_across_batches(kw):
+  """Three batches of the same shape on one module share one sampling context;
+  each must equal the kernel-per-call loop on its own inputs and noise."""
+  from t5x_amd import decoding, models, network
+  B, E, L = 3, 16, 19
+  K = kw.get('num_decodes', 1)
+  _, gcfg = tiny('bfloat16')
+  dev = torch.device('cuda')
+  params = network.init_params(gcfg, 4, dev, with_encoder=False)
+  params['decoder']['logits_dense']['kernel'][:, 1] *= 3.0  # some early EOS
+  module = network.Transformer(gcfg, dev)
+  model = models.EncoderDecoderModel(module,
+                                     decode_fn=decoding.temperature_sample)
+  inputs = np.zeros((B, L), np.int32)
+  for batch in range(3):
+    rs = np.random.RandomState(300 + batch)
+    tok = torch.as_tensor(ragged_tokens(rs, B, E, gcfg.vocab_size, 3),
+                          device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(400 + batch)
+    encoded = torch.randn((B, E, gcfg.emb_dim), generator=gen,
+                          device=dev).to(torch.bfloat16)
+    u = torch.rand((L + 2, B * K, gcfg.vocab_size), generator=gen,
+                   device=dev).clamp_min(1e-30)
+    noise = _SuppliedNoise(-torch.log(-torch.log(u)))
+    fn = models.StepFunction(model, params, network.BeamShared(encoded, K),
+                             network.BeamShared(tok, K), L)
+    want, wlp = decoding.temperature_sample(
+        inputs, dict(module.init_cache(B, L)), fn, 1, decode_rng=noise, **kw)
+    got, glp = decoding.temperature_sample(
+        inputs, module.init_cache(B, L), fn, 1, decode_rng=noise, **kw)
+    assert len(module._beam_ctx) == 1
+    assert torch.equal(torch.as_tensor(got), torch.as_tensor(want)), batch
+    assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp)), batch
+
+
 def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
   """The reference's host loop (get_infer_fn) around predict_batch_with_aux:
   5 examples at batch 2 (one pad), float32 so tokens are exact."""
