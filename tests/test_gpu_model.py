@@ -553,6 +553,80 @@ def test_fused_sampling_context_is_reused_across_batches(kw):
     assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp)), batch
 
 
+def _full_size_setup(size, B, K, E, Emin, L, decode_fn):
+  from t5x_amd import decoding, models, network
+  cfg = network.t5_1_1_config(size, dtype='bfloat16')
+  dev = torch.device('cuda')
+  params = network.init_params(cfg, 0, dev, with_encoder=False)
+  module = network.Transformer(cfg, dev)
+  model = models.EncoderDecoderModel(module, decode_fn=decode_fn)
+  rs = np.random.Generator(np.random.PCG64(1))
+  tok = rs.integers(2, 32128, size=(B, E)).astype(np.int32)
+  lens = rs.integers(Emin, E + 1, size=(B,))
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  tok = torch.as_tensor(tok, device=dev)
+  gen = torch.Generator(device=dev)
+  gen.manual_seed(2)
+  encoded = torch.randn((B, E, cfg.emb_dim), generator=gen,
+                        device=dev).to(torch.bfloat16)
+  fn = models.StepFunction(model, params, network.BeamShared(encoded, K),
+                           network.BeamShared(tok, K), L)
+  return module, fn
+
+
+def test_full_size_base_beam4_fused_loop_equals_generic_loop():
+  """The benchmark workload itself (T5.1.1-base, batch 32 x 4 beams, encoder
+  512 with 128..512 valid, 128 positions): the graph-replay loop (deferred
+  reorder, blocked caches, fused kernels) against the kernel-per-call loop,
+  bit for bit, plus the invariants of the result (scores ascending along the
+  beam axis, t5x/decoding_test.py:1103; every sequence as long as the loop
+  ran)."""
+  from t5x_amd import decoding
+  B, K, E, L = 32, 4, 512, 128
+  module, fn = _full_size_setup('base', B, K, E, 128, L, decoding.beam_search)
+  inputs = np.zeros((B, L), np.int32)
+  plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
+                            eos_id=1, num_decodes=K, alpha=0.6)
+  plain.run()
+  want, ws = plain.finish()
+  fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                            num_decodes=K, alpha=0.6)
+  assert fused.fused is not None and fused.fused.deferred_gather
+  fused.run()
+  got, gs = fused.finish()
+  assert int(fused.cur.cur_index.item()) == int(plain.cur.cur_index.item())
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
+  scores = host(gs)
+  assert (np.diff(scores, axis=1) >= 0).all()
+  assert np.isfinite(scores).all()
+
+
+def test_full_size_large_sampling_fused_loop_equals_generic_loop():
+  """T5.1.1-large, batch 64, temperature 0.7, top-k 40, encoder 512, with the
+  Gumbel noise supplied to both loops; 64 of the 256 positions (the full decode
+  only repeats the same step)."""
+  from t5x_amd import decoding
+  B, E, L, steps = 64, 512, 256, 64
+  module, fn = _full_size_setup('large', B, 1, E, 512, L,
+                                decoding.temperature_sample)
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(9)
+  u = torch.rand((steps + 2, B, 32128), generator=gen,
+                 device='cuda').clamp_min(1e-30)
+  noise = _SuppliedNoise(-torch.log(-torch.log(u)))
+  inputs = np.zeros((B, L), np.int32)
+  kw = dict(temperature=0.7, topk=40, max_decode_steps=steps)
+  want, wlp = decoding.temperature_sample(
+      inputs, dict(module.init_cache(B, L)), fn, 1, decode_rng=noise, **kw)
+  got, glp = decoding.temperature_sample(
+      inputs, module.init_cache(B, L), fn, 1, decode_rng=noise, **kw)
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp))
+  seqs = host(got)[:, 0]
+  assert (seqs[:, steps:] == 0).all() and (seqs[:, :steps] != 0).mean() > 0.9
+
+
 def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
   """The reference's host loop (get_infer_fn) around predict_batch_with_aux:
   5 examples at batch 2 (one pad), float32 so tokens are exact."""
