@@ -53,11 +53,16 @@ def parse_args():
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--lanes', type=int, default=None,
                   help='batch slices stepped concurrently (default: library)')
+  ap.add_argument('--stage', default='decode', choices=['decode', 'encoder'],
+                  help="'encoder': the once-per-batch stage before the decode "
+                       'loop (encoder forward + cross K/V projection); a step '
+                       'is one batch')
   ap.add_argument('--roofline-only', action='store_true',
                   help='only the dominant-kernel replay plus a plain copy of '
                        'known size (for counter runs under rocprofv3 --pmc)')
   ap.add_argument('--cpu-steps', type=int, default=3,
-                  help='decode steps of the CPU oracle sample')
+                  help='size of the CPU oracle sample: decode steps (batch '
+                       'rows with --stage encoder)')
   return ap.parse_args()
 
 
@@ -333,15 +338,145 @@ def cpu_baseline(name, steps, seed):
   odec.beam_search(inputs, ot5.init_cache(cfg, B, L), tokens_to_logits, 1,
                    num_decodes=K, alpha=0.6, max_decode_step=steps)
   sec = time.perf_counter() - calls['t0']
-  try:
-    from threadpoolctl import threadpool_info
-    threads = max([p.get('num_threads', 1) for p in threadpool_info()] or [1])
-  except Exception:  # pylint: disable=broad-except
-    threads = os.cpu_count() or 1
   return {'value': round(B * calls['n'] / sec, 2), 'unit': 'tokens/s',
-          'cores': int(threads), 'kind': 'port',
+          'cores': host_threads(), 'kind': 'port',
           'sample': f'{calls["n"]} beam-search steps of {name} (NumPy oracle, '
                     f'decoder only, {sec:.1f} s)'}
+
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
+
+
+class EncoderStage:
+  """What runs once per batch before the decode loop: the encoder forward over
+  the [B, E] tokens and the projection of its output to every decoder layer's
+  cross-attention K/V.  Same synthetic batch as the decode workload."""
+
+  def __init__(self, name, seed):
+    import torch
+    from t5x_amd import network
+    self.torch = torch
+    size, B, K, E, Emin, L, dtype, wdt, _ = CONFIGS[name]
+    if dtype != 'bfloat16':
+      raise SystemExit('bench.py --stage encoder: the HIP encoder is bfloat16; '
+                       f'{name} is {dtype}')
+    self.size, self.B, self.K, self.E = size, B, K, E
+    self.cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
+    dev = torch.device('cuda')
+    self.params = network.init_params(self.cfg, seed, dev, with_encoder=True)
+    self.module = network.Transformer(self.cfg, dev)
+    rs = np.random.Generator(np.random.PCG64(seed + 1))
+    tok = rs.integers(2, 32128, size=(B, E)).astype(np.int32)
+    lens = rs.integers(Emin, E + 1, size=(B,))
+    tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+    self.tok_host, self.lens = tok, lens
+    self.tokens = torch.as_tensor(tok, device=dev)
+    self.weights = self.module.decoder_weights(self.params)
+
+  def run_steps(self, n):
+    for _ in range(n):
+      encoded = self.module.apply({'params': self.params}, self.tokens,
+                                  enable_dropout=False,
+                                  method=self.module.encode)
+      # a fresh encoder output every pass: nothing is served from a cache
+      self.module._cross_kv(self.weights, encoded, self.tokens, self.K)
+
+  def flops(self):
+    """Dense-equivalent multiply-adds x 2 of one pass (padding included)."""
+    c = self.cfg
+    M, d, F = self.B * self.E, c.emb_dim, c.mlp_dim
+    hd = c.num_heads * c.head_dim
+    enc = c.num_encoder_layers * (2 * M * d * (3 * hd) + 2 * M * hd * d +
+                                  2 * M * d * 2 * F + 2 * M * F * d +
+                                  4 * self.B * c.num_heads * self.E * self.E *
+                                  c.head_dim)
+    cross = c.num_decoder_layers * 2 * (2 * M * d * hd)
+    return enc + cross
+
+  def roofline(self):
+    """The stage's dominant kernel: rows_gemm_kernel on the gated MLP input
+    projection ([B*E, d] x [d, 2F], GELU gate in the epilogue), one launch per
+    encoder layer; replayed over the layers' kernels and timed with HIP events
+    on the launch stream."""
+    from t5x_amd import ops
+    torch, c = self.torch, self.cfg
+    layers = self.module._enc_weights[('hip', id(self.params))][1].layers
+    M = self.B * self.E
+    y = torch.randn((M, c.emb_dim), device='cuda').to(torch.bfloat16)
+    out = torch.empty((M, c.mlp_dim), dtype=torch.bfloat16, device='cuda')
+    state = {'i': 0}
+
+    def launch():
+      i = state['i'] = (state['i'] + 1) % len(layers)
+      ops.gemm_rows(y, layers[i]['wi'], out=out)
+
+    sec = time_kernel(torch, launch, 2 * len(layers))
+    flops = 2.0 * M * c.emb_dim * 2 * c.mlp_dim
+    achieved = flops / sec / 1e12
+    return {'kernel': 'rows_gemm_kernel (gated MLP input projection)',
+            'bound': 'mfma', 'achieved': round(achieved, 1),
+            'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s',
+            'frac': round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+            'traffic': None, 'flops_per_launch': flops,
+            'avg_launch_us': round(sec * 1e6, 2)}
+
+  def cpu_baseline(self, rows, seed):
+    """NumPy oracle on this host: encoder forward + cross K/V projection of the
+    first `rows` batch items."""
+    from oracle import t5 as ot5
+    from t5x_amd import network
+    cfg = ot5.T5Config(dtype='bfloat16', **network.T5_1_1[self.size])
+    params = ot5.init_params(cfg, seed, with_encoder=True)
+    tok = self.tok_host[:rows]
+    t0 = time.perf_counter()
+    encoded = ot5.encode(params, cfg, tok)
+    ot5.project_cross_kv(params, cfg, encoded)
+    sec = time.perf_counter() - t0
+    return {'value': round(rows * self.E / sec, 1), 'unit': 'tokens/s',
+            'cores': host_threads(), 'kind': 'port',
+            'sample': f'{rows} of the {self.B} batch rows, one pass'}
+
+
+def host_threads():
+  try:
+    from threadpoolctl import threadpool_info
+    return int(max([p.get('num_threads', 1) for p in threadpool_info()] or [1]))
+  except Exception:  # pylint: disable=broad-except
+    return os.cpu_count() or 1
+
+
+def main_encoder(args):
+  import torch
+  w = EncoderStage(args.config, args.seed)
+  w.run_steps(max(1, args.warmup))
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  w.run_steps(args.steps)
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+  size = CONFIGS[args.config][0]
+  out = {
+      'metric': f'encoder tokens/sec, T5.1.1-{size} encoder forward + cross '
+                'K/V projection on 1 GPU',
+      'value': round(w.B * w.E * args.steps / elapsed, 1),
+      'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps,
+      'warmup': max(1, args.warmup),
+      'ms_per_step': round(elapsed / args.steps * 1e3, 4),
+      'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+      'dtype': 'bf16', 'data': 'synthetic',
+      'config': {'workload': f'T5.1.1-{size} encoder forward over batch {w.B} x '
+                             f'{w.E} tokens ({int(w.lens.min())}..'
+                             f'{int(w.lens.max())} valid) + cross K/V '
+                             f'projection for {w.cfg.num_decoder_layers} '
+                             'decoder layers',
+                 'name': args.config, 'stage': 'encoder',
+                 'tflops_whole_stage': round(
+                     w.flops() * args.steps / elapsed / 1e12, 1)},
+      'roofline': w.roofline(),
+  }
+  if not args.no_cpu_baseline:
+    out['cpu_baseline'] = w.cpu_baseline(args.cpu_steps, args.seed)
+  print(json.dumps(out))
 
 
 def main():
@@ -355,6 +490,8 @@ def main():
   if not torch.cuda.is_available():
     print('bench.py: no GPU visible', file=sys.stderr)
     sys.exit(3)
+  if args.stage == 'encoder':
+    return main_encoder(args)
   w = Workload(args.config, args.seed, args.lanes)
   if args.roofline_only:
     w.new_decode()  # builds the cross-attention K/V
