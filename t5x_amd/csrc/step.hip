@@ -95,10 +95,15 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
           stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
           w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d));
     } else {
-      T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
-      T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q, w.cross_q_scales,
-                       nullptr, m->q, R, d, HD, T5D_EPI_NONE, nullptr,
-                       nullptr));
+      if (fuse_norm) {
+        T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, m->x1, w.ln_cross, 1e-6f,
+                              w.cross_q, m->q, R, d, HD, T5D_EPI_NONE));
+      } else {
+        T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
+        T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q,
+                         w.cross_q_scales, nullptr, m->q, R, d, HD,
+                         T5D_EPI_NONE, nullptr, nullptr));
+      }
       T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
                                        w.cross_value, m->enc_len, m->ao, m->B,
                                        m->beams, m->H, m->E));
