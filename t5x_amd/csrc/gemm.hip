@@ -544,10 +544,18 @@ struct GemmPlan {
   int mp, nt, m_parts, n_groups;
 };
 
-// Pick the workgroup tile.  Model: all workgroups run in ceil(wgs / 512)
-// rounds (two resident per CU); a round costs a fixed latency plus the time
-// one workgroup needs to pull its A and B bytes.
-static GemmPlan plan_gemm(int M, int K, int N) {
+// Pick the workgroup tile.  Model: the workgroups run in rounds of as many
+// as are resident at once (256 CUs x the tile's occupancy, which its register
+// count sets); a round costs a fixed latency plus the time one workgroup needs
+// to pull its A and B bytes; all bytes entering the CUs share one aggregate
+// rate.  w_bytes: bytes per weight element.
+static int tile_occupancy(int mp, int nt) {
+  // workgroups per CU = wavefronts per SIMD of gemm_mfma_kernel<mp, nt>
+  const int acc = mp * nt;
+  return acc == 1 ? 8 : acc == 2 ? 5 : acc == 4 ? 4 : acc == 8 && mp < 8 ? 3 : 2;
+}
+
+static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
   const int mt_total = (M + 15) / 16;
   const int n_tiles = N / 16;
   GemmPlan best = {1, 1, 1, 1};
@@ -575,9 +583,10 @@ static GemmPlan plan_gemm(int M, int K, int N) {
       const int m_parts = (mt_total + mp - 1) / mp;
       const int n_groups = (n_tiles + nt - 1) / nt;
       const double wgs = (double)m_parts * n_groups;
-      const double rounds = (double)(long)((wgs + 511) / 512);
-      const double bytes = (double)K * 2.0 * (mp * 16 + nt * 16);
-      const double cost = rounds * (3.0 + bytes / 40e3) + wgs * bytes / 30e6;
+      const double slots = 256.0 * tile_occupancy(mp, nt);
+      const double rounds = (double)(long)((wgs + slots - 1) / slots);
+      const double bytes = (double)K * (2.0 * mp * 16 + (double)w_bytes * nt * 16);
+      const double cost = rounds * (3.0 + bytes / 40e3) + wgs * bytes / 40e6;
       if (cost < best_cost) {
         best_cost = cost;
         best = {mp, nt, m_parts, n_groups};
@@ -695,7 +704,7 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
   T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
               "t5d_gemm: A/W must be 16-byte aligned");
   (void)workspace; (void)counters;
-  GemmPlan p = plan_gemm(M, K, N);
+  GemmPlan p = plan_gemm(M, K, N, w_dtype == T5D_I8 ? 1 : 2);
   GemmArgs g;
   g.A = (const bf16_t*)A;
   g.W = W;
