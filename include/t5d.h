@@ -106,12 +106,13 @@ int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
  * LayerNorm feeding its dense layer, t5x/examples/t5/network.py:134-139,
  * 166-171): the rows of A are normalised on their way into the matrix product,
  * with the same two roundings to bfloat16 as t5d_rmsnorm and the same
- * summation order of the product as t5d_gemm.  bfloat16 activations and
- * packed bfloat16 weights; K a multiple of 64, <= 1024; epilogue NONE or
- * GEGLU. */
+ * summation order of the product as t5d_gemm.  bfloat16 activations; packed
+ * bfloat16 or int8 weights (scales: per-output-channel float32 [N] for int8,
+ * else NULL); K a multiple of 64, <= 2048; epilogue NONE or GEGLU. */
 int t5d_norm_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
                   const void* A, const void* norm_scale, float eps,
-                  const void* W, void* C, int M, int K, int N, int epilogue);
+                  const void* W, const float* scales, void* C, int M, int K,
+                  int N, int epilogue);
 
 /* Bias-free dense layer over any number of rows (the encoder's DenseGeneral /
  * MlpBlock layers, t5x/examples/t5/layers.py:364-414,434-487, residual adds of

@@ -302,13 +302,15 @@ gemm_mfma_kernel(GemmArgs g) {
 // y = bf16(bf16(x / rms(x)) * scale) feeds the matrix cores directly.  A
 // workgroup owns 16 rows and NT column tiles; its 4 wavefronts split K in
 // k-tile pairs exactly like gemm_mfma_kernel (same accumulation and summation
-// order) and hold ALL their operand fragments in registers (K <= 256 * NJ), so
+// order) and hold ALL their operand fragments in registers (K <= 256 * NJ;
+// int8 weight tiles stay raw until they are multiplied), so
 // the row statistics come from the fragments already loaded for the product:
 // one exchange through LDS, no second pass over x, and only 16 rows per
 // workgroup to normalise.
-template <int NT, int NJ>
+template <int NT, int NJ, typename WT>
 __global__ void __launch_bounds__(256)
 norm_gemm_kernel(GemmArgs g) {
+  constexpr int TB = WeightTile<WT>::kTileBytes;
   constexpr int TN = NT * 16;
   __shared__ float red[4][NT * 4][64];
   __shared__ float s_ss[4][16];
@@ -327,7 +329,8 @@ norm_gemm_kernel(GemmArgs g) {
   const int row = m0 + n16;
   const bool row_ok = row < g.M;
 
-  Frag xa[NJ][2], wt[NJ][2][NT];
+  Frag xa[NJ][2];
+  typename WeightTile<WT>::Raw wt[NJ][2][NT];
   uint4 lnv[NJ][2];
   {
     const bf16_t* xrow = g.A + (size_t)(row_ok ? row : g.M - 1) * g.K + 8 * gq;
@@ -342,9 +345,9 @@ norm_gemm_kernel(GemmArgs g) {
             *reinterpret_cast<const uint4*>(g.norm_scale + 32 * kt + 8 * gq);
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn)
-          wt[j][hh][nn].u = reinterpret_cast<const uint4*>(
-              wbase + ((size_t)min(nt0 + nn, n_tiles_total - 1) * KT + kt) *
-                          1024)[lane];
+          wt[j][hh][nn] = WeightTile<WT>::load(
+              wbase + ((size_t)min(nt0 + nn, n_tiles_total - 1) * KT + kt) * TB,
+              lane);
       }
   }
   T5D_GATE_TEST();
@@ -392,7 +395,7 @@ norm_gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn)
           acc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              an.v, wt[j][hh][nn].v, acc[nn], 0, 0, 0);
+              an.v, WeightTile<WT>::frag(wt[j][hh][nn]).v, acc[nn], 0, 0, 0);
       }
     }
   }
@@ -416,8 +419,12 @@ norm_gemm_kernel(GemmArgs g) {
     const int m = m0 + ml, n = nt0 * 16 + nl;
     if (m >= g.M || n >= g.N) continue;
     if (geglu && (nl & 8)) continue;
-    const float v = tile_sum(ml, nl);
-    const float vg = geglu ? tile_sum(ml, nl + 8) : 0.f;
+    float v = tile_sum(ml, nl);
+    float vg = geglu ? tile_sum(ml, nl + 8) : 0.f;
+    if (g.scales) {
+      v *= g.scales[n];
+      if (geglu) vg *= g.scales[n + 8];
+    }
     store_result(g, m, n, v, vg, 0.f);
   }
 }
@@ -727,11 +734,16 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
 extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
                              int out_dtype, const void* A,
                              const void* norm_scale, float eps, const void* W,
-                             void* C, int M, int K, int N, int epilogue) {
+                             const float* scales, void* C, int M, int K, int N,
+                             int epilogue) {
   T5D_REQUIRE(A && norm_scale && W && C, T5D_EINVAL,
               "t5d_norm_gemm: null pointer");
-  T5D_REQUIRE(dtype == T5D_BF16 && w_dtype == T5D_BF16, T5D_EINVAL,
-              "t5d_norm_gemm: bfloat16 activations and weights only");
+  T5D_REQUIRE(dtype == T5D_BF16 && (w_dtype == T5D_BF16 || w_dtype == T5D_I8),
+              T5D_EINVAL,
+              "t5d_norm_gemm: bfloat16 activations, packed bfloat16 or int8 "
+              "weights only");
+  T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
+              "t5d_norm_gemm: int8 weights need scales");
   T5D_REQUIRE(out_dtype == T5D_BF16 ||
                   (out_dtype == T5D_F32 && epilogue == T5D_EPI_NONE),
               T5D_EINVAL, "t5d_norm_gemm: out_dtype %d with epilogue %d",
@@ -739,15 +751,17 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
   T5D_REQUIRE(epilogue == T5D_EPI_NONE || epilogue == T5D_EPI_GEGLU, T5D_EINVAL,
               "t5d_norm_gemm: epilogue %d (none or geglu)", epilogue);
   T5D_REQUIRE(M > 0 && M <= 128, T5D_ELIMIT, "t5d_norm_gemm: M=%d (1..128)", M);
-  T5D_REQUIRE(K >= 64 && K % 64 == 0 && K <= 1024 && N > 0 && N % 16 == 0,
+  T5D_REQUIRE(K >= 64 && K % 64 == 0 && K <= 2048 && N > 0 && N % 16 == 0,
               T5D_ELIMIT,
-              "t5d_norm_gemm: K=%d (multiple of 64, <= 1024), N=%d (multiple "
+              "t5d_norm_gemm: K=%d (multiple of 64, <= 2048), N=%d (multiple "
               "of 16)", K, N);
   T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 &&
                   ((uintptr_t)norm_scale % 16) == 0,
               T5D_EINVAL, "t5d_norm_gemm: operands must be 16-byte aligned");
   GemmArgs g;
-  g.A = (const bf16_t*)A; g.W = W; g.scales = nullptr; g.residual = nullptr;
+  g.A = (const bf16_t*)A; g.W = W;
+  g.scales = w_dtype == T5D_I8 ? scales : nullptr;
+  g.residual = nullptr;
   g.C = C; g.M = M; g.K = K; g.N = N;
   g.m_parts = (M + 15) / 16;
   g.gate = tls_gate;
@@ -756,21 +770,32 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
   g.norm_scale = (const bf16_t*)norm_scale;
   g.eps = eps;
   const int n_tiles = N / 16;
-  // 64-column tiles unless that leaves too few workgroups to fill the chip
-  const int nt = (n_tiles / 4) * g.m_parts >= 256 ? 4 : (n_tiles >= 64 ? 2 : 1);
+  const int nj = (K / 64 + 3) / 4;  // k-tile pairs per wavefront
+  // 64-column tiles unless that leaves too few workgroups to fill the chip;
+  // beyond K = 1024 the fragments of fewer column tiles fit the registers
+  // (bfloat16 weights: one, int8: two).
+  int nt = (n_tiles / 4) * g.m_parts >= 256 ? 4 : (n_tiles >= 64 ? 2 : 1);
+  if (nj > 4) nt = min(nt, w_dtype == T5D_I8 ? 2 : 1);
   const int n_groups = (n_tiles + nt - 1) / nt;
   dim3 grid((n_groups + 7) / 8 * 8 * g.m_parts), block(256);
   hipStream_t s = as_stream(stream);
-  const int nj = (K / 64 + 3) / 4;
-#define T5D_NG_CASE(NT_)                                                     \
-  if (nt == NT_) {                                                           \
-    if (nj <= 3)                                                             \
-      hipLaunchKernelGGL((norm_gemm_kernel<NT_, 3>), grid, block, 0, s, g);  \
-    else                                                                     \
-      hipLaunchKernelGGL((norm_gemm_kernel<NT_, 4>), grid, block, 0, s, g);  \
+#define T5D_NG_LAUNCH(NT_, NJ_, WT_)                                          \
+  hipLaunchKernelGGL((norm_gemm_kernel<NT_, NJ_, WT_>), grid, block, 0, s, g)
+#define T5D_NG_CASE(NT_, WT_)                                                 \
+  if (nt == NT_) {                                                            \
+    if (nj <= 3) T5D_NG_LAUNCH(NT_, 3, WT_);                                  \
+    else if (nj <= 4) T5D_NG_LAUNCH(NT_, 4, WT_);                             \
   }
-  T5D_NG_CASE(1) T5D_NG_CASE(2) T5D_NG_CASE(4)
+  if (w_dtype == T5D_BF16) {
+    if (nj > 4) T5D_NG_LAUNCH(1, 8, bf16_t);
+    T5D_NG_CASE(1, bf16_t) T5D_NG_CASE(2, bf16_t) T5D_NG_CASE(4, bf16_t)
+  } else {
+    if (nj > 4 && nt == 1) T5D_NG_LAUNCH(1, 8, int8_t);
+    if (nj > 4 && nt == 2) T5D_NG_LAUNCH(2, 8, int8_t);
+    T5D_NG_CASE(1, int8_t) T5D_NG_CASE(2, int8_t) T5D_NG_CASE(4, int8_t)
+  }
 #undef T5D_NG_CASE
+#undef T5D_NG_LAUNCH
   T5D_CHECK_LAUNCH("t5d_norm_gemm");
   return T5D_OK;
 }

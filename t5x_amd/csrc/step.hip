@@ -65,14 +65,21 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
   // (measured at d = 1024: 56 us fused against 41 us for the three kernels).
   const bool fuse_cross_q = dt == T5D_BF16 && wd == T5D_BF16 && m->E <= 512 &&
                             d % 64 == 0 && d <= 768;
-  // Likewise the pre-attention / pre-MLP norms ride inside their dense layers.
-  const bool fuse_norm = dt == T5D_BF16 && wd == T5D_BF16 && d % 64 == 0 &&
-                         d <= 1024;
+  // Likewise the pre-attention / pre-MLP norms ride inside their dense layers
+  // where that was measured to pay: up to d = 1024 for every layer (all
+  // fragments of a row tile fit the registers with room to spare); with int8
+  // weights up to d = 2048 for a layer of at most 2048 columns (wider ones
+  // lose more to the single resident workgroup per CU than the launch saves:
+  // 23.8 us against 15.3 us for 6144 columns).
+  auto norm_rides = [&](int n_out) {
+    return dt == T5D_BF16 && d % 64 == 0 &&
+           (d <= 1024 || (wd == T5D_I8 && d <= 2048 && n_out <= 2048));
+  };
   for (int l = 0; l < m->NL; ++l) {
     const t5d_layer& w = m->layers[l];
-    if (fuse_norm) {
+    if (norm_rides(3 * HD)) {
       T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, x, w.ln_self, 1e-6f, w.qkv,
-                            m->qkv, R, d, 3 * HD, T5D_EPI_NONE));
+                            w.qkv_scales, m->qkv, R, d, 3 * HD, T5D_EPI_NONE));
     } else {
       T5D_TRY(t5d_rmsnorm(stream, dt, x, w.ln_self, m->xn, R, d, 1e-6f));
       T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
@@ -95,9 +102,10 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
           stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
           w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d));
     } else {
-      if (fuse_norm) {
+      if (norm_rides(HD)) {
         T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, m->x1, w.ln_cross, 1e-6f,
-                              w.cross_q, m->q, R, d, HD, T5D_EPI_NONE));
+                              w.cross_q, w.cross_q_scales, m->q, R, d, HD,
+                              T5D_EPI_NONE));
       } else {
         T5D_TRY(t5d_rmsnorm(stream, dt, m->x1, w.ln_cross, m->xn, R, d, 1e-6f));
         T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.cross_q,
@@ -111,9 +119,9 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
                      w.cross_out_scales, m->x1, m->x2, R, HD, d,
                      T5D_EPI_RESIDUAL, nullptr, nullptr));
-    if (fuse_norm) {
+    if (norm_rides(2 * F)) {
       T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, m->x2, w.ln_mlp, 1e-6f, w.wi,
-                            m->h, R, d, 2 * F, T5D_EPI_GEGLU));
+                            w.wi_scales, m->h, R, d, 2 * F, T5D_EPI_GEGLU));
     } else {
       T5D_TRY(t5d_rmsnorm(stream, dt, m->x2, w.ln_mlp, m->xn, R, d, 1e-6f));
       T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.wi, w.wi_scales, nullptr,

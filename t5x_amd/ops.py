@@ -196,7 +196,8 @@ def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
       raise ValueError('norm_scale must be [K]; no residual with a fused norm')
     _lib.call('t5d_norm_gemm', _s(), dt, w.w_dtype,
               _lib.dtype_code(out_dtype), a.data_ptr(), norm_scale.data_ptr(),
-              float(eps), w.data.data_ptr(), out.data_ptr(), M, K, w.N, epi)
+              float(eps), w.data.data_ptr(), _lib.ptr(w.scales),
+              out.data_ptr(), M, K, w.N, epi)
     return out
   ws_bytes = _lib.load().t5d_gemm_workspace_bytes(dt, w.w_dtype, M, K, w.N)
   ws = cnt = None

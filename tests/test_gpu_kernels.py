@@ -96,7 +96,8 @@ def test_gemm_bf16(ops, M, K, N, epi):
 @pytest.mark.parametrize('M,K,N', [(1, 768, 768), (5, 256, 512), (32, 768, 2304),
                                    (128, 768, 768), (128, 768, 4096),
                                    (100, 1024, 1024), (128, 64, 48),
-                                   (128, 832, 2304)])
+                                   (128, 832, 2304), (20, 1536, 768),
+                                   (64, 2048, 2048), (128, 2048, 6144)])
 @pytest.mark.parametrize('mode', ['none', 'geglu', 'f32out'])
 def test_norm_gemm_equals_rmsnorm_then_gemm(ops, M, K, N, mode):
   """The layer norm fused into the dense kernel against the two-kernel
@@ -135,15 +136,48 @@ def test_norm_gemm_equals_rmsnorm_then_gemm(ops, M, K, N, mode):
   np.testing.assert_allclose(host(one), want, atol=2e-2, rtol=2**-7)
 
 
+@pytest.mark.parametrize('M,K,N', [(16, 768, 768), (5, 256, 48),
+                                   (64, 1024, 3072), (64, 2048, 2048),
+                                   (64, 2048, 6144), (128, 1280, 512)])
+@pytest.mark.parametrize('geglu', [False, True])
+def test_norm_gemm_int8_weights(ops, M, K, N, geglu):
+  """The fused layer norm with int8 weights (per-channel scales applied after
+  the product, as in the plain kernel): against the two-kernel sequence and
+  against the oracle's layer_norm + dense over the dequantised kernel."""
+  rs = np.random.RandomState(M + K + N + 1)
+  x = dev(rs.randn(M, K).astype(np.float32) * 3, torch.bfloat16)
+  scale = dev(1 + 0.1 * rs.randn(K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  q0 = ot5.quantize_int8(w0)
+  xn = ot5.layer_norm(host(x), host(scale), 'bfloat16')
+  if geglu:
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    q1 = ot5.quantize_int8(w1)
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, torch.int8,
+                         gate_kernel=dev(w1))
+    want = ot5.mlp_block({'wi_0': {'kernel': q0}, 'wi_1': {'kernel': q1},
+                          'wo': {'kernel': np.eye(N, dtype=np.float32)}},
+                         xn, ('gelu', 'linear'), 'bfloat16')
+  else:
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, torch.int8)
+    want = ot5.dense_general(xn, q0, 'bfloat16')
+  two = ops.gemm(ops.rmsnorm(x, scale), pw)
+  one = ops.gemm(x, pw, norm_scale=scale)
+  diff = (one.float() - two.float()).abs()
+  assert float((diff > 0).float().mean()) < 0.02, float((diff > 0).float().mean())
+  assert float(diff.max()) <= 2e-2
+  np.testing.assert_allclose(host(one), want, atol=2e-2, rtol=2**-7)
+
+
 def test_norm_gemm_rejects_what_it_does_not_cover(ops):
   x = dev(np.zeros((4, 64), np.float32))
   pw = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.float32)
   with pytest.raises(ValueError, match='bfloat16'):
     ops.gemm(x, pw, norm_scale=dev(np.ones(64, np.float32)))
-  xb = dev(np.zeros((4, 2048), np.float32), torch.bfloat16)
-  pwb = ops.pack_weight(dev(np.zeros((2048, 32), np.float32)), torch.bfloat16)
-  with pytest.raises(Exception, match='1024'):
-    ops.gemm(xb, pwb, norm_scale=dev(np.ones(2048, np.float32), torch.bfloat16))
+  xb = dev(np.zeros((4, 2112), np.float32), torch.bfloat16)
+  pwb = ops.pack_weight(dev(np.zeros((2112, 32), np.float32)), torch.bfloat16)
+  with pytest.raises(Exception, match='2048'):
+    ops.gemm(xb, pwb, norm_scale=dev(np.ones(2112, np.float32), torch.bfloat16))
 
 
 @pytest.mark.parametrize('M', [8, 128])
