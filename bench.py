@@ -484,7 +484,8 @@ def main():
   if args.gpus != 1:
     print('bench.py: this build measures ONE GPU; --gpus must be 1 '
           f'(got {args.gpus}). The decode path shards over batch with no '
-          'exchange; see DESIGN.md.', file=sys.stderr)
+          'exchange: each GPU would run this program on its share of the '
+          'batch.', file=sys.stderr)
     sys.exit(2)
   import torch
   if not torch.cuda.is_available():
