@@ -553,9 +553,9 @@ def test_fused_sampling_context_is_reused_across_batches(kw):
     assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp)), batch
 
 
-def _full_size_setup(size, B, K, E, Emin, L, decode_fn):
+def _full_size_setup(size, B, K, E, Emin, L, decode_fn, weight_dtype=None):
   from t5x_amd import decoding, models, network
-  cfg = network.t5_1_1_config(size, dtype='bfloat16')
+  cfg = network.t5_1_1_config(size, dtype='bfloat16', weight_dtype=weight_dtype)
   dev = torch.device('cuda')
   params = network.init_params(cfg, 0, dev, with_encoder=False)
   module = network.Transformer(cfg, dev)
@@ -584,6 +584,34 @@ def test_full_size_base_beam4_fused_loop_equals_generic_loop():
   from t5x_amd import decoding
   B, K, E, L = 32, 4, 512, 128
   module, fn = _full_size_setup('base', B, K, E, 128, L, decoding.beam_search)
+  inputs = np.zeros((B, L), np.int32)
+  plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
+                            eos_id=1, num_decodes=K, alpha=0.6)
+  plain.run()
+  want, ws = plain.finish()
+  fused = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                            num_decodes=K, alpha=0.6)
+  assert fused.fused is not None and fused.fused.deferred_gather
+  fused.run()
+  got, gs = fused.finish()
+  assert int(fused.cur.cur_index.item()) == int(plain.cur.cur_index.item())
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
+  scores = host(gs)
+  assert (np.diff(scores, axis=1) >= 0).all()
+  assert np.isfinite(scores).all()
+
+
+def test_full_size_xl_int8_beam4_fused_loop_equals_generic_loop():
+  """T5.1.1-XL with int8 weights (per-output-channel scales), batch 16 x 4
+  beams, encoder 512, 128 positions: the graph-replay loop against the
+  kernel-per-call loop, bit for bit (d = 2048: stand-alone layer norms except
+  in front of the cross-attention query projection, int8 tiles widened at the
+  matrix instruction)."""
+  from t5x_amd import decoding
+  B, K, E, L = 16, 4, 512, 128
+  module, fn = _full_size_setup('xl', B, K, E, 512, L, decoding.beam_search,
+                                weight_dtype='int8')
   inputs = np.zeros((B, L), np.int32)
   plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn,
                             eos_id=1, num_decodes=K, alpha=0.6)
