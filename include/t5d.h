@@ -151,6 +151,11 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
  * that cache is written into slot (b, e).  After the call the caches equal
  * gather-then-step.  bfloat16 only; beams * ceil(L/128) <= 16.
  * pending_src may be NULL (no gather: plain t5d_self_attention_step).
+ * pending_dst (optional, needs pending_src): row (b, e) keeps its cache in
+ * slot (b, pending_dst[b, e]) instead of (b, e): what it read is copied there
+ * unless that is where it read it, and the new column goes there.  Per item
+ * pending_dst must be a permutation of 0..beams-1 and no slot that some row
+ * writes without reading it may be read by another row.
  * value_blocked != 0: cached_value is stored per (row, head) as
  * [L/32][64][32] (blocks of 32 positions, L a multiple of 32) instead of the
  * reference's [64][L]; a caller that owns its caches (a decode loop) gets
@@ -162,6 +167,7 @@ int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
                                    const int32_t* cache_index, void* out,
                                    int B, int beams, int H, int L,
                                    const int32_t* pending_src,
+                                   const int32_t* pending_dst,
                                    int value_blocked);
 
 /* One step of encoder-decoder attention (t5x/examples/t5/network.py:149-159,
@@ -360,9 +366,11 @@ typedef struct {
   /* optional device flag: when non-NULL and 0, every kernel of the step
    * returns immediately (the step becomes a no-op) */
   const int32_t* gate;
-  /* optional [B, beams] source-beam indices of a deferred cache gather, applied
-   * inside the self-attention kernels (t5d_self_attention_step_gather) */
+  /* optional [B, beams] source slots of a deferred cache gather, applied
+   * inside the self-attention kernels (t5d_self_attention_step_gather), and
+   * optional destination slots (NULL: row e keeps slot e) */
   const int32_t* pending_src;
+  const int32_t* pending_dst;
   /* non-zero: the layers' cached_value are in the blocked layout of
    * t5d_self_attention_step_gather (bfloat16, L a multiple of 32) */
   int value_blocked;
@@ -397,13 +405,24 @@ typedef struct {
    * t5d_beam_cond itself, e.g. once over all slices of a batch that it steps
    * on separate streams */
   int skip_cond;
+  /* optional, all three or none, [B, K] each: where the beams' cache rows
+   * live.  cache_slot[b, e] = slot of beam e (identity before the first
+   * iteration; updated in place).  Every iteration writes, for the next reader
+   * of the cache, cache_src[b, e] = slot holding the rows of new beam e's
+   * parent and cache_dst[b, e] = slot of new beam e: the first child of a
+   * parent inherits its slot (a re-ranking of the beams moves nothing), further
+   * children are copied into slots that no new beam reads.  With these set the
+   * model's pending_src / pending_dst must be cache_src / cache_dst; beam e's
+   * cache is then NOT in row e but in row cache_slot[b, e]. */
+  int32_t *cache_slot, *cache_src, *cache_dst;
 } t5d_beam_step;
 
 /* One iteration of the beam_search loop body plus the loop condition
  * (t5x/decoding.py:1250-1506): gather ids, decoder step, log_softmax + top-2K,
  * bookkeeping, cache reorder over the valid prefix (done here, or deferred to
- * the next step's self-attention when model->pending_src == beam->top_alive;
- * top_alive must then start as the identity), condition -> *keep_going.
+ * the next step's self-attention when model->pending_src == beam->top_alive,
+ * which must then start as the identity, or == beam->cache_src with the slot
+ * bookkeeping above), condition -> *keep_going.
  * Every kernel is gated on *keep_going, so iterations enqueued after the
  * condition turned false leave all state untouched. */
 int t5d_beam_search_step(void* stream, const t5d_model_step* model,

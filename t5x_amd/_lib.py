@@ -42,7 +42,8 @@ class ModelStep(Structure):
           'embedding', 'rel_bias', 'ln_final', 'logits_w', 'logits_scales')] +
               [('layers', POINTER(Layer))] + [(n, c_void_p) for n in (
                   'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
-                  'ao', 'h', 'logits', 'gate', 'pending_src')] +
+                  'ao', 'h', 'logits', 'gate', 'pending_src',
+                  'pending_dst')] +
               [('value_blocked', c_int)])
 
 
@@ -55,7 +56,9 @@ class BeamStep(Structure):
                ('min_brevity', c_float), ('min_log_prob', c_float),
                ('max_decode_step', c_int), ('min_initial_index', c_int),
                ('kv_base', c_void_p), ('kv_tensor_stride_bytes', c_int64),
-               ('n_kv_tensors', c_int), ('skip_cond', c_int)])
+               ('n_kv_tensors', c_int), ('skip_cond', c_int),
+               ('cache_slot', c_void_p), ('cache_src', c_void_p),
+               ('cache_dst', c_void_p)])
 
 
 class SampleStep(Structure):
@@ -101,7 +104,7 @@ _SIGNATURES = {
                                         c_int, c_int, c_int]),
     't5d_self_attention_step_gather': (c_int, [_P, c_int, _P, _P, _P, _P, _P,
                                                _P, c_int, c_int, c_int, c_int,
-                                               _P, c_int]),
+                                               _P, _P, c_int]),
     't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
                                          c_int, c_int, c_int]),
     't5d_cross_attention_step_norm_q': (c_int, [_P, c_int, c_int, _P, _P,

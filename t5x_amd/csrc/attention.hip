@@ -424,7 +424,8 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                void* cv, const void* rel_bias,
                                const int32_t* cache_index, void* out, int R,
                                int H, int L, const int32_t* pending,
-                               int beams, int value_blocked);
+                               const int32_t* pending_dst, int beams,
+                               int value_blocked);
 
 static int check_common(const char* name, int dtype, int H, int S) {
   T5D_REQUIRE(dtype == T5D_F32 || dtype == T5D_BF16, T5D_EINVAL, "%s: dtype %d",
@@ -465,8 +466,8 @@ extern "C" int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
     launch_attn_nq<float, 1, true>(a, R, as_stream(stream));
   else
     launch_self_attention_bf16(as_stream(stream), qkv, cached_key, cached_value,
-                               rel_bias, cache_index, out, R, H, L, nullptr, 1,
-                               0);
+                               rel_bias, cache_index, out, R, H, L, nullptr,
+                               nullptr, 1, 0);
   T5D_CHECK_LAUNCH("t5d_self_attention_step");
   return T5D_OK;
 }
@@ -475,7 +476,7 @@ extern "C" int t5d_self_attention_step_gather(
     void* stream, int dtype, const void* qkv, void* cached_key,
     void* cached_value, const void* rel_bias, const int32_t* cache_index,
     void* out, int B, int beams, int H, int L, const int32_t* pending_src,
-    int value_blocked) {
+    const int32_t* pending_dst, int value_blocked) {
   int rc = check_common("t5d_self_attention_step_gather", dtype, H, L);
   if (rc) return rc;
   T5D_REQUIRE(dtype == T5D_BF16, T5D_EINVAL,
@@ -490,6 +491,8 @@ extern "C" int t5d_self_attention_step_gather(
               T5D_ELIMIT,
               "t5d_self_attention_step_gather: beams=%d x L=%d needs more than "
               "%d wavefronts per workgroup", beams, L, kMaxWaves);
+  T5D_REQUIRE(pending_dst == nullptr || pending_src != nullptr, T5D_EINVAL,
+              "t5d_self_attention_step_gather: pending_dst without pending_src");
   T5D_REQUIRE(!value_blocked || L % 32 == 0, T5D_EINVAL,
               "t5d_self_attention_step_gather: blocked values need L %% 32 == 0 "
               "(L=%d)", L);
@@ -499,7 +502,8 @@ extern "C" int t5d_self_attention_step_gather(
               "t5d_self_attention_step_gather: cache not 16-byte aligned");
   launch_self_attention_bf16(as_stream(stream), qkv, cached_key, cached_value,
                              rel_bias, cache_index, out, B * beams, H, L,
-                             pending_src, beams, value_blocked ? 1 : 0);
+                             pending_src, pending_dst, beams,
+                             value_blocked ? 1 : 0);
   T5D_CHECK_LAUNCH("t5d_self_attention_step_gather");
   return T5D_OK;
 }

@@ -46,7 +46,8 @@ struct AttnMfmaArgs {
   int H, S, nq, q_stride;
   const int32_t* gate;
   // self-attention only
-  const int32_t* pending;  // [B, beams] source beam per row, or null
+  const int32_t* pending;  // [B, beams] source slot per row, or null
+  const int32_t* pending_dst;  // [B, beams] slot per row (null: row e, slot e)
   int beams, nblk;         // rows per workgroup, wavefronts per row
   // cross-attention with the query projection fused in (q == nullptr)
   const bf16_t* x;         // [R, d] residual stream
@@ -443,6 +444,9 @@ __device__ __forceinline__ void reduce_scatter_8(const float (&s)[8],
 // writes what it read into its own slot after a workgroup barrier (all reads
 // are in registers by then, so the in-place permutation is safe).  This
 // replaces a separate read+write pass over every cache by the writes alone.
+// With `pending_dst` the row's own slot is pending_dst[b, e] rather than e: a
+// caller that lets beams inherit their parents' slots writes only the rows
+// of beams whose parent has another child.
 //
 //   scores: vector ALU.  Lane (dg = lane / 16, jc = lane % 16) multiplies head
 //     dims 16 dg .. +16 of the query with positions 8 jc .. +8 of the key
@@ -476,18 +480,20 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   const int HD = a.H * kHeadDim;
   const int S = a.S;
 
-  int r, rs;             // own row (slot) and source row
-  bool permuted = false; // does this batch item need its beams moved?
+  int r, rs, rw;         // row of the step; cache slot it reads; its own slot
+  bool permuted = false; // does this batch item need cache rows moved?
   if (a.pending != nullptr) {
     const int b = blockIdx.y, e = wave / nblk;
+    auto in_range = [&](int v) { return v < 0 ? 0 : (v >= a.beams ? a.beams - 1 : v); };
     r = b * a.beams + e;
-    int src = a.pending[r];
-    src = src < 0 ? 0 : (src >= a.beams ? a.beams - 1 : src);
-    rs = b * a.beams + src;
+    rs = b * a.beams + in_range(a.pending[r]);
+    rw = a.pending_dst ? b * a.beams + in_range(a.pending_dst[r]) : r;
     for (int q = 0; q < a.beams; ++q)
-      permuted = permuted || (a.pending[b * a.beams + q] != q);
+      permuted = permuted ||
+                 (a.pending[b * a.beams + q] !=
+                  (a.pending_dst ? a.pending_dst[b * a.beams + q] : q));
   } else {
-    r = rs = blockIdx.y;
+    r = rs = rw = blockIdx.y;
   }
 
   T5D_STAMP_SELF(8);
@@ -501,8 +507,8 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   const size_t slot = (size_t)kHeadDim * S;
   const bf16_t* ksrc = a.k + ((size_t)rs * a.H + h) * slot;
   const bf16_t* vsrc = a.v + ((size_t)rs * a.H + h) * slot;
-  bf16_t* kdst = a.k + ((size_t)r * a.H + h) * slot;
-  bf16_t* vdst = a.v + ((size_t)r * a.H + h) * slot;
+  bf16_t* kdst = a.k + ((size_t)rw * a.H + h) * slot;
+  bf16_t* vdst = a.v + ((size_t)rw * a.H + h) * slot;
   const bf16_t* qrow = a.q + (size_t)r * a.q_stride + h * kHeadDim;
 
   // Relative-position bias of this head, by distance, for the softmax below.
@@ -582,7 +588,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     // before any slot is written.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (r != rs) {
+    if (rw != rs) {
       if (live) {
 #pragma unroll
         for (int i = 0; i < 16; ++i)
@@ -607,7 +613,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   // it is issued last, when waiting for those stores costs nothing.
   auto store_column = [&]() {
     if (wave_has_t) {
-      if (r != rs) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (rw != rs) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       kdst[(size_t)lane * S + t] = knew_d;
       vdst[a.v_blocked ? ((size_t)(t >> 5) * kHeadDim + lane) * 32 + (t & 31)
                        : (size_t)lane * S + t] = vnew_d;
@@ -769,7 +775,8 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                void* cv, const void* rel_bias,
                                const int32_t* cache_index, void* out, int R,
                                int H, int L, const int32_t* pending,
-                               int beams, int value_blocked) {
+                               const int32_t* pending_dst, int beams,
+                               int value_blocked) {
   AttnMfmaArgs a;
   a.v_blocked = value_blocked;
   a.q = (const bf16_t*)qkv; a.k = (bf16_t*)ck; a.v = (bf16_t*)cv;
@@ -780,6 +787,7 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
   a.x = nullptr; a.ln = nullptr; a.wq = nullptr; a.d = 0; a.eps = 0.f;
   a.nblk = (L + kBlockJ - 1) / kBlockJ;
   a.pending = pending;
+  a.pending_dst = pending ? pending_dst : nullptr;
   a.beams = pending ? beams : 1;
   const int waves = a.nblk * a.beams;
   dim3 grid(H, pending ? R / beams : R), block(64 * waves);

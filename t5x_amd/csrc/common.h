@@ -215,7 +215,8 @@ int launch_beam_select(hipStream_t s, const float* logits,
                        void* scratch, const int32_t* inputs,
                        const int32_t* initial_index, const float* brevity,
                        int32_t* top_alive, int B, int K, int S, int Lin, int V,
-                       int eos_id);
+                       int eos_id, int32_t* cache_slot, int32_t* cache_src,
+                       int32_t* cache_dst);
 // End of a beam-search iteration in one single-workgroup kernel: advance
 // *state.cur_index, add 1 to `counters[0..n_counters)` (the layers' cache
 // indices), and, if do_cond, evaluate the loop condition into *keep_going.

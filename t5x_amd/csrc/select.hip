@@ -492,7 +492,52 @@ struct BeamUpdateArgs {
   const int32_t* cand_idx;
   float* topk_vals_out;
   int32_t* topk_idx_out;
+  // optional bookkeeping of where each beam's cache rows live (all [B, K]):
+  // cache_slot[b, e] is the slot of beam e (in: before, out: after this
+  // iteration); cache_src / cache_dst (out) tell the next reader of the cache
+  // where new beam e finds its parent's rows and where its own go.
+  int32_t* cache_slot;
+  int32_t* cache_src;
+  int32_t* cache_dst;
 };
+
+// Slots for the K new beams of one item, given their parents' slots rd[0..K):
+// the first child of a parent (lowest e) inherits the parent's slot, so a
+// mere re-ranking of the beams moves no cache row at all; every further child
+// takes the n-th slot that no new beam reads (n counted over such children in
+// order of e), which it must fill with a copy.  The result is a permutation
+// of 0..K-1 and no slot that is written is also read.
+__device__ __forceinline__ int new_beam_slot(const int (&rd)[kMaxBeams], int K,
+                                             int e) {
+  unsigned seen = 0, all = 0;
+  int later = 0;  // children before e that also need a free slot
+#pragma unroll
+  for (int o = 0; o < kMaxBeams; ++o) {
+    if (o < K) {
+      const unsigned bit = 1u << rd[o];
+      if (o < e) {
+        later += (seen & bit) ? 1 : 0;
+        seen |= bit;
+      }
+      all |= bit;
+    }
+  }
+  int mine = 0;
+#pragma unroll
+  for (int o = 0; o < kMaxBeams; ++o) mine = o == e ? rd[o] : mine;
+  if (!(seen & (1u << mine))) return mine;
+  int found = mine;  // K reads of fewer than K slots always leave one free
+#pragma unroll
+  for (int slot = kMaxBeams - 1; slot >= 0; --slot) {
+    if (slot < K && !(all & (1u << slot))) {
+      // free slots below `slot`: this is the later-th free slot if that count
+      // equals `later`
+      const unsigned below = ~all & ((1u << slot) - 1u);
+      if (__popc(below) == later) found = slot;
+    }
+  }
+  return found;
+}
 
 // Stable descending order of n values (ties keep index order).
 __device__ __forceinline__ void stable_order_desc(const float* v, int n,
@@ -520,6 +565,7 @@ constexpr int kUpdateThreads = 256;
 __global__ void __launch_bounds__(kUpdateThreads)
 beam_update_kernel(BeamUpdateArgs a) {
   __shared__ int s_src_live[kMaxBeams];       // source live beam of new live e
+  __shared__ int s_slot_of[kMaxBeams];        // cache slot of old beam e
   __shared__ int s_tok_live[kMaxBeams];
   __shared__ int s_fin_from[kMaxBeams];       // <K: old finished; else K+cand
   __shared__ int s_cand_beam[2 * kMaxBeams];
@@ -548,9 +594,11 @@ beam_update_kernel(BeamUpdateArgs a) {
   }
   float old_score = 0.f;
   int old_flag = 0;
+  int old_slot = 0;
   if (lane < K) {
     old_score = a.cur.finished_scores[(size_t)b * K + lane];
     old_flag = a.cur.finished_flags[(size_t)b * K + lane];
+    if (a.cache_slot) old_slot = a.cache_slot[(size_t)b * K + lane];
   }
   const int first = a.initial_index[b];
   const int cur = *a.cur.cur_index;
@@ -642,8 +690,22 @@ beam_update_kernel(BeamUpdateArgs a) {
     a.top_alive_indices[(size_t)b * K + e] = s_src_live[e];
     a.next.finished_scores[(size_t)b * K + e] = s_fin_score[e];
     a.next.finished_flags[(size_t)b * K + e] = (uint8_t)s_fin_flag[e];
+    s_slot_of[e] = old_slot < 0 ? 0 : (old_slot >= K ? K - 1 : old_slot);
   }
   __syncthreads();
+  // (the last wavefront does this: it has the fewest sequence columns below)
+  const int slot_lane = lane - (kUpdateThreads - 64);
+  if (a.cache_slot && slot_lane >= 0 && slot_lane < K) {
+    const int e = slot_lane;
+    int rd[kMaxBeams];
+#pragma unroll
+    for (int o = 0; o < kMaxBeams; ++o)
+      rd[o] = o < K ? s_slot_of[s_src_live[o]] : 0;
+    const int dst = new_beam_slot(rd, K, e);
+    a.cache_src[(size_t)b * K + e] = s_slot_of[s_src_live[e]];
+    a.cache_dst[(size_t)b * K + e] = dst;
+    a.cache_slot[(size_t)b * K + e] = dst;
+  }
 
   for (int j = lane; j < S; j += kUpdateThreads) {
     if (j != lane) {
@@ -1427,6 +1489,7 @@ extern "C" int t5d_beam_update(void* stream, const t5d_beam_state* cur,
   a.gate = tls_gate;
   a.cand_vals = nullptr; a.cand_idx = nullptr;
   a.topk_vals_out = nullptr; a.topk_idx_out = nullptr;
+  a.cache_slot = a.cache_src = a.cache_dst = nullptr;
   hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(kUpdateThreads), 0,
                      as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_beam_update");
@@ -1459,7 +1522,8 @@ int t5d::launch_beam_select(hipStream_t s, const float* logits,
                             void* scratch, const int32_t* inputs,
                             const int32_t* initial_index, const float* brevity,
                             int32_t* top_alive, int B, int K, int S, int Lin,
-                            int V, int eos_id) {
+                            int V, int eos_id, int32_t* cache_slot,
+                            int32_t* cache_src, int32_t* cache_dst) {
   int rc = check_state("beam select", st);
   if (rc) return rc;
   T5D_REQUIRE(K <= kMaxBeams, T5D_ELIMIT, "beam select: K=%d > %d", K,
@@ -1479,6 +1543,7 @@ int t5d::launch_beam_select(hipStream_t s, const float* logits,
   a.gate = tls_gate;
   a.cand_vals = cand_vals; a.cand_idx = cand_idx;
   a.topk_vals_out = topk_vals; a.topk_idx_out = topk_idx;
+  a.cache_slot = cache_slot; a.cache_src = cache_src; a.cache_dst = cache_dst;
   hipLaunchKernelGGL(beam_update_kernel, dim3(B), dim3(kUpdateThreads), 0, s, a);
   T5D_CHECK_LAUNCH("beam select");
   return T5D_OK;

@@ -89,7 +89,7 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
       T5D_TRY(t5d_self_attention_step_gather(
           stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
           m->cache_index + l, m->ao, m->B, m->beams, m->H, m->L,
-          m->pending_src, m->value_blocked));
+          m->pending_src, m->pending_dst, m->value_blocked));
     else
       T5D_TRY(t5d_self_attention_step(stream, dt, m->qkv, w.cached_key,
                                       w.cached_value, m->rel_bias,
@@ -156,9 +156,21 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
               T5D_EINVAL, "t5d_beam_search_step: null buffer");
   T5D_REQUIRE(m->gate == b->keep_going, T5D_EINVAL,
               "t5d_beam_search_step: the model gate must be the loop flag");
-  T5D_REQUIRE(m->pending_src == nullptr || m->pending_src == b->top_alive,
-              T5D_EINVAL,
-              "t5d_beam_search_step: pending_src must be the top_alive buffer");
+  const bool slots = b->cache_slot || b->cache_src || b->cache_dst;
+  if (slots) {
+    T5D_REQUIRE(b->cache_slot && b->cache_src && b->cache_dst, T5D_EINVAL,
+                "t5d_beam_search_step: cache_slot / cache_src / cache_dst go "
+                "together");
+    T5D_REQUIRE(m->pending_src == b->cache_src && m->pending_dst == b->cache_dst,
+                T5D_EINVAL,
+                "t5d_beam_search_step: with cache slots the model's pending_src "
+                "/ pending_dst must be cache_src / cache_dst");
+  } else {
+    T5D_REQUIRE(m->pending_dst == nullptr &&
+                    (m->pending_src == nullptr || m->pending_src == b->top_alive),
+                T5D_EINVAL,
+                "t5d_beam_search_step: pending_src must be the top_alive buffer");
+  }
   const int K = m->beams, B = m->B;
   T5D_TRY(decoder_step_impl(stream, m, nullptr, b->state.live_seqs,
                             b->state.cur_index, b->S, false));
@@ -168,7 +180,8 @@ extern "C" int t5d_beam_search_step(void* stream, const t5d_model_step* m,
                              b->topk_idx, b->row_max, b->row_lse, b->scratch,
                              b->inputs, b->initial_index, b->brevity,
                              b->top_alive, B, K, b->S, b->Lin, m->V,
-                             b->eos_id));
+                             b->eos_id, b->cache_slot, b->cache_src,
+                             b->cache_dst));
   // When the model applies pending gathers inside its self-attention
   // (pending_src == top_alive) the reorder happens there, on the next step.
   // Otherwise reorder now: cur_index + 1 columns are valid.

@@ -395,7 +395,8 @@ class Transformer:
 
   # -- the decode step -------------------------------------------------------------
   def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
-                  L, gate=None, pending_src=None, value_blocked=False):
+                  L, gate=None, pending_src=None, value_blocked=False,
+                  pending_dst=None):
     """Fills a t5d_model_step for one call of t5d_decoder_step."""
     from t5x_amd import _lib
     cfg = self.config
@@ -426,10 +427,10 @@ class Transformer:
     for name in ('x', 'x1', 'x2', 'xn', 'qkv', 'q', 'ao', 'h', 'logits'):
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
-    m.pending_src = P(pending_src)
+    m.pending_src, m.pending_dst = P(pending_src), P(pending_dst)
     m.value_blocked = int(bool(value_blocked))
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
-                    pending_src)
+                    pending_src, pending_dst)
     return m
 
   def _step_buffers(self, R, w):
@@ -777,6 +778,10 @@ class _BeamLane:
     self.row_lse = torch.empty((R,), dtype=f32, device=dev)
     self.scratch = torch.empty((2 * R * k2,), dtype=i32, device=dev)
     self.top_alive = loop.top_alive[b0:b1]
+    # where the beams' cache rows live: slot of beam e, and for the reorder in
+    # flight the slot each new beam reads and the slot it keeps
+    self.cache_slot, self.cache_src, self.cache_dst = (
+        owner.cache_slots[i, b0:b1] for i in range(3))
     lane_cross = dict(k=[t[b0:b1] for t in cross['k']],
                       v=[t[b0:b1] for t in cross['v']],
                       enc_len=cross['enc_len'][b0:b1], B=B, beams=K,
@@ -785,7 +790,8 @@ class _BeamLane:
     self.model = module._model_step(
         w, lane_cross, self.bufs, layer_caches, self.cache_index, R, K, L,
         gate=self.keep_going,
-        pending_src=self.top_alive if owner.deferred_gather else None,
+        pending_src=self.cache_src if owner.deferred_gather else None,
+        pending_dst=self.cache_dst if owner.deferred_gather else None,
         value_blocked=owner.value_blocked)
     st = loop.cur
     P = _lib.ptr
@@ -814,6 +820,9 @@ class _BeamLane:
     bs.kv_tensor_stride_bytes = self.kv[0, 0].numel() * self.kv.element_size()
     bs.n_kv_tensors = 2 * nl
     bs.skip_cond = 1 if owner.n_lanes > 1 else 0
+    if owner.deferred_gather:
+      bs.cache_slot, bs.cache_src, bs.cache_dst = (
+          P(self.cache_slot), P(self.cache_src), P(self.cache_dst))
     self.beam = bs
     self.stream = torch.cuda.Stream(device=dev)
     self.event = torch.cuda.Event()
@@ -855,7 +864,9 @@ class FusedBeamStep:
     L = (S - 1 + el - 1) // el * el
     # With bfloat16 caches the reorder of a step is deferred into the next
     # step's self-attention kernels, which read each row's cache from its
-    # source beam anyway; the permutation in flight lives in loop.top_alive.
+    # source beam anyway.  Beams do not own fixed cache rows: a new beam
+    # inherits the slot of its parent (only a parent's further children are
+    # copied), so the reorder in flight is a pair of slot maps, cache_slots.
     self.deferred_gather = (K > 1 and act == torch.bfloat16 and
                             K * ((L + 127) // 128) <= 16)
     # The value caches are then kept in blocks of 32 positions (loads of
@@ -872,6 +883,9 @@ class FusedBeamStep:
     self.L = L
     loop.top_alive.copy_(torch.arange(K, dtype=torch.int32,
                                       device=dev).expand(B, K))
+    # [0]: slot of beam e; [1], [2]: source / destination slots in flight
+    self.cache_slots = torch.arange(K, dtype=torch.int32, device=dev).expand(
+        3, B, K).contiguous()
     if lanes is None:
       lanes = module.decode_lanes
     n = max(1, min(int(lanes), B))
@@ -916,6 +930,8 @@ class FusedBeamStep:
     K = loop.beam_size
     self.top_alive.copy_(torch.arange(K, dtype=torch.int32, device=dev).expand(
         loop.batch_size, K))
+    self.cache_slots.copy_(torch.arange(K, dtype=torch.int32,
+                                        device=dev).expand_as(self.cache_slots))
     self.lane_cur_index.copy_(
         loop.cur.cur_index.to(torch.int32).reshape(1).expand(self.n_lanes))
     for lane in self.lanes:
@@ -1029,15 +1045,20 @@ class FusedBeamStep:
     K = self.loop.beam_size
     for lane in self.lanes:
       if self.deferred_gather:
-        # Apply the reorder still in flight, then mark it done.
+        # Beam e's rows are in slot cache_src[b, e] (the copy into its own
+        # slot is still in flight): bring every beam to slot e, then mark all
+        # of it done.
         nl = lane.kv.shape[0]
         B = lane.b1 - lane.b0
         ops.cache_gather_beams(
-            lane.kv[0, 0].view(B, K, *lane.kv.shape[3:]), lane.top_alive,
+            lane.kv[0, 0].view(B, K, *lane.kv.shape[3:]), lane.cache_src,
             n_tensors=2 * nl,
             tensor_stride_bytes=lane.kv[0, 0].numel() * lane.kv.element_size())
-        lane.top_alive.copy_(torch.arange(
-            K, dtype=torch.int32, device=self.device).expand(B, K))
+        identity = torch.arange(K, dtype=torch.int32,
+                                device=self.device).expand(B, K)
+        for t in (lane.top_alive, lane.cache_slot, lane.cache_src,
+                  lane.cache_dst):
+          t.copy_(identity)
     torch.cuda.synchronize()
     nl = self.lanes[0].kv.shape[0]
     kv = torch.cat([lane.kv for lane in self.lanes], dim=2)

@@ -231,11 +231,13 @@ def unblock_cached_value(v):
 
 
 def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
-                        out=None, pending_src=None, value_blocked=False):
+                        out=None, pending_src=None, value_blocked=False,
+                        pending_dst=None):
   """One cached self-attention step; with pending_src [B, beams] the rows'
-  caches are first gathered from their source beams inside the kernel.
-  value_blocked: cached_value holds the blocked layout (see
-  block_cached_value) in a tensor of the usual [R, H, 64, L] shape."""
+  caches are first gathered from their source beams inside the kernel, into
+  slot e of row (b, e) or, with pending_dst [B, beams], into slot
+  pending_dst[b, e].  value_blocked: cached_value holds the blocked layout
+  (see block_cached_value) in a tensor of the usual [R, H, 64, L] shape."""
   _chk(qkv, 'qkv', ndim=2)
   _chk(cached_key, 'cached_key', qkv.dtype, 4)
   _chk(cached_value, 'cached_value', qkv.dtype, 4)
@@ -262,11 +264,16 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
       B, beams = pending_src.shape
       if B * beams != R:
         raise ValueError(f'pending_src {(B, beams)} does not cover {R} rows')
+    if pending_dst is not None:
+      _chk(pending_dst, 'pending_dst', torch.int32, 2)
+      if pending_src is None or pending_dst.shape != pending_src.shape:
+        raise ValueError('pending_dst goes with a pending_src of its shape')
     _lib.call('t5d_self_attention_step_gather', _s(),
               _lib.dtype_code(qkv.dtype), qkv.data_ptr(),
               cached_key.data_ptr(), cached_value.data_ptr(),
               rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), B,
-              beams, H, L, _lib.ptr(pending_src), int(bool(value_blocked)))
+              beams, H, L, _lib.ptr(pending_src), _lib.ptr(pending_dst),
+              int(bool(value_blocked)))
     return out
   _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
             qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),

@@ -356,6 +356,89 @@ def test_self_attention_step_with_pending_gather(ops, B, beams, H, L, t):
                      cv_a[..., :t + 1])
 
 
+def inherit_slots(slot_of, parents):
+  """Host model of the slot rule: slot_of[e] = slot of old beam e, parents[e] =
+  old beam that new beam e continues.  Returns (src, dst): the first child of
+  a parent keeps the parent's slot, further children take, in order, the slots
+  that no new beam reads."""
+  K = len(parents)
+  src = [int(slot_of[p]) for p in parents]
+  dst, taken = [None] * K, set()
+  for e in range(K):
+    if src[e] not in taken:
+      dst[e] = src[e]
+      taken.add(src[e])
+  free = [x for x in range(K) if x not in set(src)]
+  for e in range(K):
+    if dst[e] is None:
+      dst[e] = free.pop(0)
+  return src, dst
+
+
+@pytest.mark.parametrize('B,beams,H,L,t', [(3, 4, 2, 128, 0), (3, 4, 3, 128, 77),
+                                           (2, 2, 2, 32, 9), (2, 8, 2, 256, 200),
+                                           (32, 4, 12, 128, 64)])
+@pytest.mark.parametrize('blocked', [False, True])
+def test_self_attention_step_with_destination_slots(ops, B, beams, H, L, t,
+                                                     blocked):
+  """Beams that inherit their parents' slots: with the caches of the old beams
+  scattered over the slots (slot_of), the step over (src, dst) slot maps gives
+  the outputs of gather-then-step and leaves new beam e's cache in slot
+  dst[e]; rows whose slot is inherited are not rewritten (their columns beyond
+  t keep the old content), only further children of a parent are copied."""
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(B * 71 + beams * 13 + L + t)
+  rs = np.random.RandomState(B + beams + t)
+  R, D, dt = B * beams, 64, torch.bfloat16
+  ck = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  cv = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  qkv = torch.randn((R, 3 * H * D), generator=gen, device='cuda').to(dt)
+  rel_bias = torch.randn((H, L), generator=gen, device='cuda').to(dt)
+  idx = torch.tensor(t, dtype=torch.int32, device='cuda')
+  slot_of = np.stack([rs.permutation(beams) for _ in range(B)])
+  parents = rs.randint(0, beams, size=(B, beams))
+  parents[0] = np.arange(beams)           # nothing moves
+  parents[1] = rs.permutation(beams)      # a re-ranking: nothing is copied
+  if B > 2:
+    parents[2] = 0                        # one parent, beams - 1 copies
+  maps = [inherit_slots(slot_of[b], parents[b]) for b in range(B)]
+  src = torch.tensor([m[0] for m in maps], dtype=torch.int32, device='cuda')
+  dst = torch.tensor([m[1] for m in maps], dtype=torch.int32, device='cuda')
+  for b in range(B):
+    s_, d_ = maps[b]
+    assert sorted(d_) == list(range(beams))
+    assert not ({d for s0, d in zip(s_, d_) if d != s0} & set(s_))
+    if b == 1:
+      assert s_ == d_
+
+  # reference: caches in beam order, gathered by parent, then the plain step
+  so = torch.as_tensor(slot_of, device='cuda').long()
+  pa = torch.as_tensor(parents, device='cuda').long()
+  rows = (torch.arange(B, device='cuda')[:, None] * beams)
+  logical_k = ck[(rows + so).reshape(-1)]   # cache of old beam e
+  logical_v = cv[(rows + so).reshape(-1)]
+  ck_a = logical_k[(rows + pa).reshape(-1)].clone()
+  cv_a = logical_v[(rows + pa).reshape(-1)].clone()
+  want = ops.self_attention_step(qkv, ck_a, cv_a, rel_bias, idx)
+
+  ck_b = ck.clone()
+  cv_b = (ops.block_cached_value(cv).view(R, H, D, L) if blocked
+          else cv.clone())
+  got = ops.self_attention_step(qkv, ck_b, cv_b, rel_bias, idx,
+                                pending_src=src, pending_dst=dst,
+                                value_blocked=blocked)
+  assert torch.equal(got, want)
+  cv_out = ops.unblock_cached_value(cv_b) if blocked else cv_b
+  at = (rows + dst.long()).reshape(-1)      # where new beam e's cache is now
+  assert torch.equal(ck_b[at][..., :t + 1], ck_a[..., :t + 1])
+  assert torch.equal(cv_out[at][..., :t + 1], cv_a[..., :t + 1])
+  # inherited slots were not rewritten beyond the new column
+  keep = (src == dst).reshape(-1)
+  if t + 1 < L and bool(keep.any()):
+    assert torch.equal(ck_b[at][keep][..., t + 1:],
+                       ck[(rows + src.long()).reshape(-1)][keep][..., t + 1:])
+
+
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('B,beams,H,E', [(2, 1, 3, 64), (3, 4, 2, 512),
                                          (2, 2, 2, 128), (1, 8, 2, 264),

@@ -602,6 +602,38 @@ def test_full_size_base_beam4_fused_loop_equals_generic_loop():
   assert np.isfinite(scores).all()
 
 
+def test_fused_beam_loop_slot_maps_follow_the_inheritance_rule():
+  """Where the graph-replay loop keeps the beams' cache rows: after every
+  iteration the slot maps written on the device equal the host model of the
+  rule (first child inherits, further children take the unread slots) applied
+  to the parents the iteration chose, and stay permutations."""
+  from t5x_amd import decoding
+  from tests.test_gpu_kernels import inherit_slots
+  B, K, E, L = 6, 4, 64, 24
+  module, fn = _full_size_setup('small', B, K, E, 16, L, decoding.beam_search)
+  inputs = np.zeros((B, L), np.int32)
+  loop = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
+                           num_decodes=K, alpha=0.6)
+  fused = loop.fused
+  assert fused is not None and fused.deferred_gather
+  slot_of = np.tile(np.arange(K), (B, 1))
+  moved = 0
+  for _ in range(L - 2):
+    if not loop.cond():
+      break
+    loop.advance(1)
+    torch.cuda.synchronize()
+    parents = host(loop.top_alive)
+    slots = host(fused.cache_slots)
+    for b in range(B):
+      src, dst = inherit_slots(slot_of[b], parents[b])
+      assert list(slots[1, b]) == src and list(slots[2, b]) == dst
+      assert list(slots[0, b]) == dst
+      moved += sum(int(a != c) for a, c in zip(src, dst))
+    slot_of = slots[0].copy()
+  assert moved > 0  # random-init weights do duplicate parents
+
+
 def test_full_size_xl_int8_beam4_fused_loop_equals_generic_loop():
   """T5.1.1-XL with int8 weights (per-output-channel scales), batch 16 x 4
   beams, encoder 512, 128 positions: the graph-replay loop against the
