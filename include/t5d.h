@@ -412,8 +412,10 @@ typedef struct {
    * parent and cache_dst[b, e] = slot of new beam e: the first child of a
    * parent inherits its slot (a re-ranking of the beams moves nothing), further
    * children are copied into slots that no new beam reads.  With these set the
-   * model's pending_src / pending_dst must be cache_src / cache_dst; beam e's
-   * cache is then NOT in row e but in row cache_slot[b, e]. */
+   * model's pending_src / pending_dst must be cache_src / cache_dst.  Beam
+   * e's cache is then NOT in row e: after an iteration it is in row
+   * cache_src[b, e], and from the next iteration's self-attention on in row
+   * cache_dst[b, e] = cache_slot[b, e]. */
   int32_t *cache_slot, *cache_src, *cache_dst;
 } t5d_beam_step;
 
