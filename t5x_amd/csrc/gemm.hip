@@ -430,13 +430,18 @@ norm_gemm_kernel(GemmArgs g) {
 }
 
 // ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
-// Lane = output column, the 4 wavefronts split K, MB rows per pass.
-template <int MB>
-__global__ void __launch_bounds__(256)
+// Lane = output column, the WV wavefronts split K, MB rows per pass.  With a
+// handful of rows and 64 columns per workgroup there are few workgroups, so
+// the length of a wavefront's chain of loads sets the time: 16 wavefronts
+// keep it to K / 16 steps.
+template <int MB, int WV>
+__global__ void __launch_bounds__(64 * WV)
 gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
                 const float* __restrict__ residual, float* __restrict__ C,
                 int M, int K, int N, int epilogue, const int32_t* gate) {
-  __shared__ float red[4][2 * MB][64];
+  static_assert(WV == 4 || WV == 16, "wavefronts per workgroup");
+  constexpr int RW = WV == 4 ? 4 : 8;  // partial sums held in LDS at once
+  __shared__ float red[RW][2 * MB][64];
   T5D_GATED(gate);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -449,8 +454,9 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   float acc0[MB], acc1[MB];
 #pragma unroll
   for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
-  const int kq = (K + 3) / 4;
-  const int kb = wave * kq, ke = min(K, kb + kq);
+  // contiguous K ranges, multiples of 8 so that the 8-wide passes apply
+  const int kq = ((K + WV - 1) / WV + 7) & ~7;
+  const int kb = min(K, wave * kq), ke = min(K, kb + kq);
   int k = kb;
   if ((K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
     // 8 k per pass, all loads of a pass in flight together; the products are
@@ -495,21 +501,47 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       acc1[m] = fmaf(a, w1, acc1[m]);
     }
   }
+  if constexpr (WV == 16) {
+    // wavefronts 8..15 hand their sums to 0..7 first (LDS budget)
+    if (wave >= 8) {
 #pragma unroll
-  for (int m = 0; m < MB; ++m) {
-    red[wave][m][lane] = acc0[m];
-    red[wave][MB + m][lane] = acc1[m];
+      for (int m = 0; m < MB; ++m) {
+        red[wave - 8][m][lane] = acc0[m];
+        red[wave - 8][MB + m][lane] = acc1[m];
+      }
+    }
+    __syncthreads();
+    if (wave < 8) {
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        acc0[m] += red[wave][m][lane];
+        acc1[m] += red[wave][MB + m][lane];
+      }
+    }
+    __syncthreads();
+  }
+  if (wave < RW) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      red[wave][m][lane] = acc0[m];
+      red[wave][MB + m][lane] = acc1[m];
+    }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < MB * 64; e += 256) {
+  auto total = [&](int i, int l) -> float {
+    float v = (red[0][i][l] + red[1][i][l]) + (red[2][i][l] + red[3][i][l]);
+    if constexpr (RW == 8)
+      v += (red[4][i][l] + red[5][i][l]) + (red[6][i][l] + red[7][i][l]);
+    return v;
+  };
+  for (int e = threadIdx.x; e < MB * 64; e += 64 * WV) {
     const int m = e >> 6, l = e & 63;
     const int col = blockIdx.x * 64 + l;
     const int row = m0 + m;
     if (row >= M || col >= ncols) continue;
-    float v = (red[0][m][l] + red[1][m][l]) + (red[2][m][l] + red[3][m][l]);
+    float v = total(m, l);
     if (geglu) {
-      float vg = (red[0][MB + m][l] + red[1][MB + m][l]) +
-                 (red[2][MB + m][l] + red[3][MB + m][l]);
+      float vg = total(MB + m, l);
       C[(size_t)row * F + col] = gelu_tanh(v) * vg;
     } else {
       if (epilogue == T5D_EPI_RESIDUAL) v += residual[(size_t)row * N + col];
@@ -680,19 +712,20 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
     T5D_REQUIRE(w_dtype == T5D_F32 && out_dtype == T5D_F32, T5D_EINVAL,
                 "t5d_gemm: float32 activations need float32 weights/outputs");
     const int ncols = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
-    if (M <= 8) {
-      dim3 grid((ncols + 63) / 64, 1);
-      hipLaunchKernelGGL(gemm_f32_kernel<8>, grid, dim3(256), 0, s,
+    // One kernel shape for every M (rows in groups of 8 along grid.y), so the
+    // summation order, and with it every bit of the result, does not depend
+    // on how many rows a call carries.
+    dim3 grid((ncols + 63) / 64, (M + 7) / 8);
+    if (K >= 128)
+      hipLaunchKernelGGL((gemm_f32_kernel<8, 16>), grid, dim3(1024), 0, s,
                          (const float*)A, (const float*)W,
                          (const float*)residual, (float*)C, M, K, N, epilogue,
                          tls_gate);
-    } else {
-      dim3 grid((ncols + 63) / 64, (M + 15) / 16);
-      hipLaunchKernelGGL(gemm_f32_kernel<16>, grid, dim3(256), 0, s,
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<8, 4>), grid, dim3(256), 0, s,
                          (const float*)A, (const float*)W,
                          (const float*)residual, (float*)C, M, K, N, epilogue,
                          tls_gate);
-    }
     T5D_CHECK_LAUNCH("t5d_gemm(f32)");
     return T5D_OK;
   }
