@@ -454,10 +454,52 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   float acc0[MB], acc1[MB];
 #pragma unroll
   for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
-  // contiguous K ranges, multiples of 8 so that the 8-wide passes apply
-  const int kq = ((K + WV - 1) / WV + 7) & ~7;
+  // contiguous K ranges, multiples of 32 so that the 32-wide passes apply
+  const int kq = ((K + WV - 1) / WV + 31) & ~31;
   const int kb = min(K, wave * kq), ke = min(K, kb + kq);
   int k = kb;
+  if (MB == 8 && (K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
+    // 32 k per pass with every load of the pass in flight at once: 32 weight
+    // rows per lane, and the 8 x 32 activations as ONE load (lane l holds row
+    // l / 8, columns 4 (l % 8) .. +4), broadcast from there when multiplied.
+    // Products are accumulated in ascending k, one fma each.
+    const int arow = m0 + (lane >> 3);
+    for (; k + 32 <= ke; k += 32) {
+      float w0[32], w1[32];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) {
+        w0[u] = active ? W[(size_t)(k + u) * N + n] : 0.f;
+        w1[u] = (active && geglu) ? W[(size_t)(k + u) * N + F + n] : 0.f;
+      }
+      float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (arow < M)
+        av = *reinterpret_cast<const float4*>(A + (size_t)arow * K + k +
+                                              4 * (lane & 7));
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int src = m * 8 + q;  // lane holding columns 4 q .. 4 q + 3
+          const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+              __builtin_bit_cast(int, av.x), src));
+          const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+              __builtin_bit_cast(int, av.y), src));
+          const float a2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+              __builtin_bit_cast(int, av.z), src));
+          const float a3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+              __builtin_bit_cast(int, av.w), src));
+          acc0[m] = fmaf(a0, w0[4 * q + 0], acc0[m]);
+          acc1[m] = fmaf(a0, w1[4 * q + 0], acc1[m]);
+          acc0[m] = fmaf(a1, w0[4 * q + 1], acc0[m]);
+          acc1[m] = fmaf(a1, w1[4 * q + 1], acc1[m]);
+          acc0[m] = fmaf(a2, w0[4 * q + 2], acc0[m]);
+          acc1[m] = fmaf(a2, w1[4 * q + 2], acc1[m]);
+          acc0[m] = fmaf(a3, w0[4 * q + 3], acc0[m]);
+          acc1[m] = fmaf(a3, w1[4 * q + 3], acc1[m]);
+        }
+      }
+    }
+  }
   if ((K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
     // 8 k per pass, all loads of a pass in flight together; the products are
     // still accumulated in ascending k, one fma each.
