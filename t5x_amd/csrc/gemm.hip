@@ -430,25 +430,33 @@ norm_gemm_kernel(GemmArgs g) {
 }
 
 // ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
-// Lane = output column, the WV wavefronts split K, MB rows per pass.  With a
-// handful of rows and 64 columns per workgroup there are few workgroups, so
-// the length of a wavefront's chain of loads sets the time: 16 wavefronts
-// keep it to K / 16 steps.
-template <int MB, int WV>
+// A workgroup owns 8 rows x 16 output columns: with a handful of rows the
+// kernel is a stream of the weight matrix, and narrow column tiles are what
+// spreads that stream over enough CUs (N / 16 workgroups).  Lane (c, s) =
+// (column c of 16, k-subrange s of 4): per pass of 32 k it multiplies the 8 k
+// of subrange s, every load of the pass in flight at once; the WV wavefronts
+// split K in contiguous ranges.  Sums: ascending k inside a lane, then over
+// the 4 subranges (rows_sum), then over the wavefronts in a fixed tree, so
+// the result does not depend on how many rows a call carries.
+constexpr int kF32Rows = 8, kF32Cols = 16;
+
+template <int WV>
 __global__ void __launch_bounds__(64 * WV)
 gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
                 const float* __restrict__ residual, float* __restrict__ C,
                 int M, int K, int N, int epilogue, const int32_t* gate) {
   static_assert(WV == 4 || WV == 16, "wavefronts per workgroup");
+  constexpr int MB = kF32Rows;
   constexpr int RW = WV == 4 ? 4 : 8;  // partial sums held in LDS at once
-  __shared__ float red[RW][2 * MB][64];
+  __shared__ float red[RW][2 * MB][kF32Cols];
   T5D_GATED(gate);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, sub = lane >> 4;
   const bool geglu = epilogue == T5D_EPI_GEGLU;
   const int F = N >> 1;
   const int ncols = geglu ? F : N;  // columns of work
-  const int n = blockIdx.x * 64 + lane;
+  const int n = blockIdx.x * kF32Cols + c;
   const int m0 = blockIdx.y * MB;
   const bool active = n < ncols;
   float acc0[MB], acc1[MB];
@@ -458,72 +466,31 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   const int kq = ((K + WV - 1) / WV + 31) & ~31;
   const int kb = min(K, wave * kq), ke = min(K, kb + kq);
   int k = kb;
-  if (MB == 8 && (K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
-    // 32 k per pass with every load of the pass in flight at once: 32 weight
-    // rows per lane, and the 8 x 32 activations as ONE load (lane l holds row
-    // l / 8, columns 4 (l % 8) .. +4), broadcast from there when multiplied.
-    // Products are accumulated in ascending k, one fma each.
-    const int arow = m0 + (lane >> 3);
-    for (; k + 32 <= ke; k += 32) {
-      float w0[32], w1[32];
-#pragma unroll
-      for (int u = 0; u < 32; ++u) {
-        w0[u] = active ? W[(size_t)(k + u) * N + n] : 0.f;
-        w1[u] = (active && geglu) ? W[(size_t)(k + u) * N + F + n] : 0.f;
-      }
-      float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (arow < M)
-        av = *reinterpret_cast<const float4*>(A + (size_t)arow * K + k +
-                                              4 * (lane & 7));
-#pragma unroll
-      for (int m = 0; m < MB; ++m) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const int src = m * 8 + q;  // lane holding columns 4 q .. 4 q + 3
-          const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
-              __builtin_bit_cast(int, av.x), src));
-          const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
-              __builtin_bit_cast(int, av.y), src));
-          const float a2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
-              __builtin_bit_cast(int, av.z), src));
-          const float a3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
-              __builtin_bit_cast(int, av.w), src));
-          acc0[m] = fmaf(a0, w0[4 * q + 0], acc0[m]);
-          acc1[m] = fmaf(a0, w1[4 * q + 0], acc1[m]);
-          acc0[m] = fmaf(a1, w0[4 * q + 1], acc0[m]);
-          acc1[m] = fmaf(a1, w1[4 * q + 1], acc1[m]);
-          acc0[m] = fmaf(a2, w0[4 * q + 2], acc0[m]);
-          acc1[m] = fmaf(a2, w1[4 * q + 2], acc1[m]);
-          acc0[m] = fmaf(a3, w0[4 * q + 3], acc0[m]);
-          acc1[m] = fmaf(a3, w1[4 * q + 3], acc1[m]);
-        }
-      }
-    }
-  }
   if ((K & 31) == 0 && ((uintptr_t)A & 15) == 0) {
-    // 8 k per pass, all loads of a pass in flight together; the products are
-    // still accumulated in ascending k, one fma each.
-    for (; k + 8 <= ke; k += 8) {
+    for (; k + 32 <= ke; k += 32) {
+      const int kk = k + 8 * sub;
       float w0[8], w1[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        w0[u] = active ? W[(size_t)(k + u) * N + n] : 0.f;
-        w1[u] = (active && geglu) ? W[(size_t)(k + u) * N + F + n] : 0.f;
+        w0[u] = active ? W[(size_t)(kk + u) * N + n] : 0.f;
+        w1[u] = (active && geglu) ? W[(size_t)(kk + u) * N + F + n] : 0.f;
       }
+      float4 ax[MB], ay[MB];
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
         const int row = m0 + m;
-        float a[8];
+        ax[m] = ay[m] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (row < M) {
           const float4* ap =
-              reinterpret_cast<const float4*>(A + (size_t)row * K + k);
-          const float4 x = ap[0], y = ap[1];
-          a[0] = x.x; a[1] = x.y; a[2] = x.z; a[3] = x.w;
-          a[4] = y.x; a[5] = y.y; a[6] = y.z; a[7] = y.w;
-        } else {
-#pragma unroll
-          for (int u = 0; u < 8; ++u) a[u] = 0.f;
+              reinterpret_cast<const float4*>(A + (size_t)row * K + kk);
+          ax[m] = ap[0];
+          ay[m] = ap[1];
         }
+      }
+#pragma unroll
+      for (int m = 0; m < MB; ++m) {
+        const float a[8] = {ax[m].x, ax[m].y, ax[m].z, ax[m].w,
+                            ay[m].x, ay[m].y, ay[m].z, ay[m].w};
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           acc0[m] = fmaf(a[u], w0[u], acc0[m]);
@@ -532,7 +499,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       }
     }
   }
-  for (; k < ke; ++k) {
+  for (k += sub; k < ke; k += 4) {  // any K: one k per lane subrange
     const float w0 = active ? W[(size_t)k * N + n] : 0.f;
     const float w1 = (active && geglu) ? W[(size_t)k * N + F + n] : 0.f;
 #pragma unroll
@@ -543,30 +510,35 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       acc1[m] = fmaf(a, w1, acc1[m]);
     }
   }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    acc0[m] = rows_sum(acc0[m]);
+    acc1[m] = rows_sum(acc1[m]);
+  }
   if constexpr (WV == 16) {
-    // wavefronts 8..15 hand their sums to 0..7 first (LDS budget)
-    if (wave >= 8) {
+    // wavefronts 8..15 hand their sums to 0..7 first
+    if (wave >= 8 && sub == 0) {
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        red[wave - 8][m][lane] = acc0[m];
-        red[wave - 8][MB + m][lane] = acc1[m];
+        red[wave - 8][m][c] = acc0[m];
+        red[wave - 8][MB + m][c] = acc1[m];
       }
     }
     __syncthreads();
     if (wave < 8) {
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
-        acc0[m] += red[wave][m][lane];
-        acc1[m] += red[wave][MB + m][lane];
+        acc0[m] += red[wave][m][c];
+        acc1[m] += red[wave][MB + m][c];
       }
     }
     __syncthreads();
   }
-  if (wave < RW) {
+  if (wave < RW && sub == 0) {
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
-      red[wave][m][lane] = acc0[m];
-      red[wave][MB + m][lane] = acc1[m];
+      red[wave][m][c] = acc0[m];
+      red[wave][MB + m][c] = acc1[m];
     }
   }
   __syncthreads();
@@ -576,9 +548,9 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       v += (red[4][i][l] + red[5][i][l]) + (red[6][i][l] + red[7][i][l]);
     return v;
   };
-  for (int e = threadIdx.x; e < MB * 64; e += 64 * WV) {
-    const int m = e >> 6, l = e & 63;
-    const int col = blockIdx.x * 64 + l;
+  for (int e = threadIdx.x; e < MB * kF32Cols; e += 64 * WV) {
+    const int m = e / kF32Cols, l = e % kF32Cols;
+    const int col = blockIdx.x * kF32Cols + l;
     const int row = m0 + m;
     if (row >= M || col >= ncols) continue;
     float v = total(m, l);
@@ -757,14 +729,14 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
     // One kernel shape for every M (rows in groups of 8 along grid.y), so the
     // summation order, and with it every bit of the result, does not depend
     // on how many rows a call carries.
-    dim3 grid((ncols + 63) / 64, (M + 7) / 8);
+    dim3 grid((ncols + kF32Cols - 1) / kF32Cols, (M + kF32Rows - 1) / kF32Rows);
     if (K >= 128)
-      hipLaunchKernelGGL((gemm_f32_kernel<8, 16>), grid, dim3(1024), 0, s,
+      hipLaunchKernelGGL((gemm_f32_kernel<16>), grid, dim3(1024), 0, s,
                          (const float*)A, (const float*)W,
                          (const float*)residual, (float*)C, M, K, N, epilogue,
                          tls_gate);
     else
-      hipLaunchKernelGGL((gemm_f32_kernel<8, 4>), grid, dim3(256), 0, s,
+      hipLaunchKernelGGL((gemm_f32_kernel<4>), grid, dim3(256), 0, s,
                          (const float*)A, (const float*)W,
                          (const float*)residual, (float*)C, M, K, N, epilogue,
                          tls_gate);
