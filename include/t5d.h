@@ -108,7 +108,10 @@ int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
  * with the same two roundings to bfloat16 as t5d_rmsnorm and the same
  * summation order of the product as t5d_gemm.  bfloat16 activations; packed
  * bfloat16 or int8 weights (scales: per-output-channel float32 [N] for int8,
- * else NULL); K a multiple of 64, <= 2048; epilogue NONE or GEGLU. */
+ * else NULL); K a multiple of 64, <= 2048; epilogue NONE or GEGLU.
+ * float32 (activations, row-major [K, N] weights and outputs): any M, K, N;
+ * the norm scale multiplies the weights as they are loaded and 1/rms the
+ * finished sums, which differs from normalising first by a few float32 ulps. */
 int t5d_norm_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
                   const void* A, const void* norm_scale, float eps,
                   const void* W, const float* scales, void* C, int M, int K,

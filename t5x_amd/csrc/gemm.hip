@@ -438,17 +438,22 @@ norm_gemm_kernel(GemmArgs g) {
 // split K in contiguous ranges.  Sums: ascending k inside a lane, then over
 // the 4 subranges (rows_sum), then over the wavefronts in a fixed tree, so
 // the result does not depend on how many rows a call carries.
+// With `norm_scale` the rows are RMS-normalised on the way (T5 LayerNorm in
+// front of the dense layer): the scale g_k multiplies the weights w_kn as they
+// are loaded, the sum of squares of the row rides along with the products, and
+// 1/rms, which is common to the whole row, multiplies the finished sum.
 constexpr int kF32Rows = 8, kF32Cols = 16;
 
-template <int WV>
+template <int WV, bool NORMED>
 __global__ void __launch_bounds__(64 * WV)
 gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
                 const float* __restrict__ residual, float* __restrict__ C,
-                int M, int K, int N, int epilogue, const int32_t* gate) {
+                int M, int K, int N, int epilogue, const int32_t* gate,
+                const float* __restrict__ norm_scale, float eps) {
   static_assert(WV == 4 || WV == 16, "wavefronts per workgroup");
   constexpr int MB = kF32Rows;
   constexpr int RW = WV == 4 ? 4 : 8;  // partial sums held in LDS at once
-  __shared__ float red[RW][2 * MB][kF32Cols];
+  __shared__ float red[RW][3 * MB][kF32Cols];
   T5D_GATED(gate);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -459,9 +464,10 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   const int n = blockIdx.x * kF32Cols + c;
   const int m0 = blockIdx.y * MB;
   const bool active = n < ncols;
-  float acc0[MB], acc1[MB];
+  float acc0[MB], acc1[MB], ssq[MB];
 #pragma unroll
-  for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
+  for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = ssq[m] = 0.f;
+  constexpr bool normed = NORMED;
   // contiguous K ranges, multiples of 32 so that the 32-wide passes apply
   const int kq = ((K + WV - 1) / WV + 31) & ~31;
   const int kb = min(K, wave * kq), ke = min(K, kb + kq);
@@ -487,12 +493,23 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
           ay[m] = ap[1];
         }
       }
+      if constexpr (normed) {
+        const float4* gp = reinterpret_cast<const float4*>(norm_scale + kk);
+        const float4 x = gp[0], y = gp[1];
+        const float g[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          w0[u] *= g[u];
+          w1[u] *= g[u];
+        }
+      }
 #pragma unroll
       for (int m = 0; m < MB; ++m) {
         const float a[8] = {ax[m].x, ax[m].y, ax[m].z, ax[m].w,
                             ay[m].x, ay[m].y, ay[m].z, ay[m].w};
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
+          if constexpr (normed) ssq[m] = fmaf(a[u], a[u], ssq[m]);
           acc0[m] = fmaf(a[u], w0[u], acc0[m]);
           acc1[m] = fmaf(a[u], w1[u], acc1[m]);
         }
@@ -500,12 +517,17 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
     }
   }
   for (k += sub; k < ke; k += 4) {  // any K: one k per lane subrange
-    const float w0 = active ? W[(size_t)k * N + n] : 0.f;
-    const float w1 = (active && geglu) ? W[(size_t)k * N + F + n] : 0.f;
+    float w0 = active ? W[(size_t)k * N + n] : 0.f;
+    float w1 = (active && geglu) ? W[(size_t)k * N + F + n] : 0.f;
+    if constexpr (normed) {
+      w0 *= norm_scale[k];
+      w1 *= norm_scale[k];
+    }
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
       const int row = m0 + m;
       const float a = row < M ? A[(size_t)row * K + k] : 0.f;
+      if constexpr (normed) ssq[m] = fmaf(a, a, ssq[m]);
       acc0[m] = fmaf(a, w0, acc0[m]);
       acc1[m] = fmaf(a, w1, acc1[m]);
     }
@@ -514,6 +536,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
   for (int m = 0; m < MB; ++m) {
     acc0[m] = rows_sum(acc0[m]);
     acc1[m] = rows_sum(acc1[m]);
+    if constexpr (normed) ssq[m] = rows_sum(ssq[m]);
   }
   if constexpr (WV == 16) {
     // wavefronts 8..15 hand their sums to 0..7 first
@@ -522,6 +545,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       for (int m = 0; m < MB; ++m) {
         red[wave - 8][m][c] = acc0[m];
         red[wave - 8][MB + m][c] = acc1[m];
+        red[wave - 8][2 * MB + m][c] = ssq[m];
       }
     }
     __syncthreads();
@@ -530,6 +554,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
       for (int m = 0; m < MB; ++m) {
         acc0[m] += red[wave][m][c];
         acc1[m] += red[wave][MB + m][c];
+        ssq[m] += red[wave][2 * MB + m][c];
       }
     }
     __syncthreads();
@@ -539,6 +564,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
     for (int m = 0; m < MB; ++m) {
       red[wave][m][c] = acc0[m];
       red[wave][MB + m][c] = acc1[m];
+      red[wave][2 * MB + m][c] = ssq[m];
     }
   }
   __syncthreads();
@@ -554,8 +580,12 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
     const int row = m0 + m;
     if (row >= M || col >= ncols) continue;
     float v = total(m, l);
+    // every lane subrange saw its own k of the row: the total is the row's
+    const float inv =
+        normed ? 1.0f / sqrtf(total(2 * MB + m, l) / (float)K + eps) : 1.f;
+    v *= inv;
     if (geglu) {
-      float vg = total(MB + m, l);
+      float vg = total(MB + m, l) * inv;
       C[(size_t)row * F + col] = gelu_tanh(v) * vg;
     } else {
       if (epilogue == T5D_EPI_RESIDUAL) v += residual[(size_t)row * N + col];
@@ -669,6 +699,29 @@ static void launch_mfma(const GemmPlan& p, GemmArgs g, hipStream_t s) {
 
 using namespace t5d;
 
+// One kernel shape for every M (rows in groups of 8 along grid.y), so the
+// summation order, and with it every bit of the result, does not depend on
+// how many rows a call carries.
+static void launch_gemm_f32(hipStream_t s, const float* A, const float* W,
+                            const float* residual, float* C, int M, int K,
+                            int N, int epilogue, const float* norm_scale,
+                            float eps) {
+  const int ncols = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
+  dim3 grid((ncols + kF32Cols - 1) / kF32Cols, (M + kF32Rows - 1) / kF32Rows);
+#define T5D_F32_LAUNCH(WV_, NORMED_)                                          \
+  hipLaunchKernelGGL((gemm_f32_kernel<WV_, NORMED_>), grid, dim3(64 * WV_), 0, \
+                     s, A, W, residual, C, M, K, N, epilogue, tls_gate,       \
+                     norm_scale, eps)
+  if (K >= 128) {
+    if (norm_scale) T5D_F32_LAUNCH(16, true);
+    else T5D_F32_LAUNCH(16, false);
+  } else {
+    if (norm_scale) T5D_F32_LAUNCH(4, true);
+    else T5D_F32_LAUNCH(4, false);
+  }
+#undef T5D_F32_LAUNCH
+}
+
 extern "C" int64_t t5d_packed_weight_bytes(int w_dtype, int K, int N) {
   if (K <= 0 || N <= 0 || K % 32 || N % 16) return -1;
   if (w_dtype == T5D_BF16) return (int64_t)K * N * 2;
@@ -725,21 +778,8 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
   if (dtype == T5D_F32) {
     T5D_REQUIRE(w_dtype == T5D_F32 && out_dtype == T5D_F32, T5D_EINVAL,
                 "t5d_gemm: float32 activations need float32 weights/outputs");
-    const int ncols = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
-    // One kernel shape for every M (rows in groups of 8 along grid.y), so the
-    // summation order, and with it every bit of the result, does not depend
-    // on how many rows a call carries.
-    dim3 grid((ncols + kF32Cols - 1) / kF32Cols, (M + kF32Rows - 1) / kF32Rows);
-    if (K >= 128)
-      hipLaunchKernelGGL((gemm_f32_kernel<16>), grid, dim3(1024), 0, s,
-                         (const float*)A, (const float*)W,
-                         (const float*)residual, (float*)C, M, K, N, epilogue,
-                         tls_gate);
-    else
-      hipLaunchKernelGGL((gemm_f32_kernel<4>), grid, dim3(256), 0, s,
-                         (const float*)A, (const float*)W,
-                         (const float*)residual, (float*)C, M, K, N, epilogue,
-                         tls_gate);
+    launch_gemm_f32(s, (const float*)A, (const float*)W, (const float*)residual,
+                    (float*)C, M, K, N, epilogue, nullptr, 0.f);
     T5D_CHECK_LAUNCH("t5d_gemm(f32)");
     return T5D_OK;
   }
@@ -785,10 +825,28 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
                              int epilogue) {
   T5D_REQUIRE(A && norm_scale && W && C, T5D_EINVAL,
               "t5d_norm_gemm: null pointer");
+  if (dtype == T5D_F32) {
+    T5D_REQUIRE(w_dtype == T5D_F32 && out_dtype == T5D_F32, T5D_EINVAL,
+                "t5d_norm_gemm: float32 activations need float32 weights / "
+                "outputs");
+    T5D_REQUIRE(epilogue == T5D_EPI_NONE ||
+                    (epilogue == T5D_EPI_GEGLU && N % 2 == 0),
+                T5D_EINVAL, "t5d_norm_gemm: epilogue %d (none or geglu), N=%d",
+                epilogue, N);
+    T5D_REQUIRE(M > 0 && K > 0 && N > 0, T5D_EINVAL,
+                "t5d_norm_gemm: M=%d K=%d N=%d", M, K, N);
+    T5D_REQUIRE(K % 32 != 0 || ((uintptr_t)norm_scale % 16) == 0, T5D_EINVAL,
+                "t5d_norm_gemm: norm_scale must be 16-byte aligned");
+    launch_gemm_f32(as_stream(stream), (const float*)A, (const float*)W,
+                    nullptr, (float*)C, M, K, N, epilogue,
+                    (const float*)norm_scale, eps);
+    T5D_CHECK_LAUNCH("t5d_norm_gemm(f32)");
+    return T5D_OK;
+  }
   T5D_REQUIRE(dtype == T5D_BF16 && (w_dtype == T5D_BF16 || w_dtype == T5D_I8),
               T5D_EINVAL,
-              "t5d_norm_gemm: bfloat16 activations, packed bfloat16 or int8 "
-              "weights only");
+              "t5d_norm_gemm: bfloat16 activations with packed bfloat16 or int8 "
+              "weights, or float32 with float32");
   T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
               "t5d_norm_gemm: int8 weights need scales");
   T5D_REQUIRE(out_dtype == T5D_BF16 ||

@@ -71,7 +71,9 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
   // weights up to d = 2048 for a layer of at most 2048 columns (wider ones
   // lose more to the single resident workgroup per CU than the launch saves:
   // 23.8 us against 15.3 us for 6144 columns).
+  // float32: always (the kernel carries the row statistics along for free).
   auto norm_rides = [&](int n_out) {
+    if (dt == T5D_F32) return true;
     return dt == T5D_BF16 && d % 64 == 0 &&
            (d <= 1024 || (wd == T5D_I8 && d <= 2048 && n_out <= 2048));
   };

@@ -169,11 +169,41 @@ def test_norm_gemm_int8_weights(ops, M, K, N, geglu):
   np.testing.assert_allclose(host(one), want, atol=2e-2, rtol=2**-7)
 
 
+@pytest.mark.parametrize('M,K,N', [(8, 512, 384), (3, 100, 70), (20, 64, 128),
+                                   (8, 512, 1024), (33, 384, 512),
+                                   (8, 512, 32128)])
+@pytest.mark.parametrize('geglu', [False, True])
+def test_norm_gemm_f32(ops, M, K, N, geglu):
+  """float32: the layer norm inside the dense kernel (scale folded into the
+  activations, 1/rms applied to the finished sums) against the two-kernel
+  sequence and against the oracle's layer_norm + dense."""
+  if geglu and N > 4096:
+    pytest.skip('the logits layer has no gate')
+  rs = np.random.RandomState(M + K + N + 5)
+  x = rs.randn(M, K).astype(np.float32) * 3
+  scale = (1 + 0.1 * rs.randn(K)).astype(np.float32)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  xn = ot5.layer_norm(x, scale, 'float32')
+  if geglu:
+    w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    pw = ops.pack_weight(dev(w0), torch.float32, gate_kernel=dev(w1))
+    want = ot5.mlp_block({'wi_0': {'kernel': w0}, 'wi_1': {'kernel': w1},
+                          'wo': {'kernel': np.eye(N, dtype=np.float32)}},
+                         xn, ('gelu', 'linear'), 'float32')
+  else:
+    pw = ops.pack_weight(dev(w0), torch.float32)
+    want = ot5.dense_general(xn, w0, 'float32')
+  two = ops.gemm(ops.rmsnorm(dev(x), dev(scale)), pw)
+  one = ops.gemm(dev(x), pw, norm_scale=dev(scale))
+  np.testing.assert_allclose(host(one), host(two), atol=2e-5, rtol=2e-5)
+  np.testing.assert_allclose(host(one), want, atol=1e-4, rtol=1e-4)
+
+
 def test_norm_gemm_rejects_what_it_does_not_cover(ops):
   x = dev(np.zeros((4, 64), np.float32))
-  pw = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.float32)
-  with pytest.raises(ValueError, match='bfloat16'):
-    ops.gemm(x, pw, norm_scale=dev(np.ones(64, np.float32)))
+  pwq = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.bfloat16)
+  with pytest.raises(Exception, match='float32'):
+    _lib_call_norm_gemm_mixed(ops, x, pwq)
   xb = dev(np.zeros((4, 2112), np.float32), torch.bfloat16)
   pwb = ops.pack_weight(dev(np.zeros((2112, 32), np.float32)), torch.bfloat16)
   with pytest.raises(Exception, match='2048'):
@@ -354,6 +384,17 @@ def test_self_attention_step_with_pending_gather(ops, B, beams, H, L, t):
   assert torch.equal(got_d, want)
   assert torch.equal(ops.unblock_cached_value(cv_d)[..., :t + 1],
                      cv_a[..., :t + 1])
+
+
+def _lib_call_norm_gemm_mixed(ops, x, pw):
+  """float32 activations with packed bfloat16 weights, straight at the C entry
+  (the Python wrapper has no such combination)."""
+  from t5x_amd import _lib
+  scale = dev(np.ones(x.shape[1], np.float32))
+  out = torch.empty((x.shape[0], pw.N), dtype=torch.float32, device='cuda')
+  _lib.call('t5d_norm_gemm', _lib.stream_handle(), _lib.F32, pw.w_dtype,
+            _lib.F32, x.data_ptr(), scale.data_ptr(), 1e-6, pw.data.data_ptr(),
+            None, out.data_ptr(), x.shape[0], x.shape[1], pw.N, 0)
 
 
 def inherit_slots(slot_of, parents):
