@@ -224,6 +224,13 @@ int t5d_encoder_attention(void* stream, const void* q, const void* k,
                           const int32_t* enc_len, void* out, int B, int H,
                           int E, int Ep, int q_stride, int k_stride);
 
+/* The same attention in float32 (the dtype of the exactness tests), straight
+ * from the fused projection: qkv [B*E, 3*H*64] holds q | k | v per row;
+ * rel_bias [H, 2E-1] float32; out [B*E, H*64].  E <= 2048. */
+int t5d_encoder_attention_f32(void* stream, const float* qkv,
+                              const float* rel_bias, const int32_t* enc_len,
+                              float* out, int B, int H, int E);
+
 /* Add `delta` to n int32 values (cache_index += 1, layers.py:275). */
 int t5d_add_i32(void* stream, int32_t* x, int n, int delta);
 

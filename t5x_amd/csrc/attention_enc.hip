@@ -197,6 +197,75 @@ enc_attn_kernel(EncAttnArgs a) {
   }
 }
 
+// ---- float32 -------------------------------------------------------------------
+// The exactness-test dtype: plain vector arithmetic, one wavefront per query
+// row.  Scores (lane = key, ascending head dim), bias and mask summed first and
+// added to the score as the reference does (a masked pair ends at exactly
+// -1e10, so a padded query attends uniformly), softmax over all E keys, then
+// lane = head dim accumulates the normalised weights times V in ascending key
+// order.  qkv rows hold q | k | v (H*64 columns each).
+struct EncAttnF32Args {
+  const float* qkv;   // [B*E, 3*H*64]
+  const float* bias;  // [H, 2E-1], by (key - query + E - 1)
+  const int32_t* len; // [B]
+  float* out;         // [B*E, H*64]
+  int H, E;
+};
+
+constexpr int kEncF32Rows = 4;  // query rows (wavefronts) per workgroup
+constexpr int kHeadDim = 64;
+
+__global__ void __launch_bounds__(64 * kEncF32Rows)
+enc_attn_f32_kernel(EncAttnF32Args a) {
+  __shared__ float s_w[kEncF32Rows][kMaxEncLen];
+  __shared__ __attribute__((aligned(16))) float s_q[kEncF32Rows][kHeadDim];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int e = blockIdx.x * kEncF32Rows + wave;
+  const int h = blockIdx.y, b = blockIdx.z;
+  if (e >= a.E) return;  // whole wavefronts; no workgroup barrier below
+  const int HD = a.H * kHeadDim, row_stride = 3 * HD;
+  const int n = min(max(a.len[b], 0), a.E);
+  const float* base = a.qkv + (size_t)b * a.E * row_stride + h * kHeadDim;
+  s_q[wave][lane] = base[(size_t)e * row_stride + lane];
+  const float* bias = a.bias + (size_t)h * (2 * a.E - 1) + (a.E - 1) - e;
+  const bool q_valid = e < n;
+
+  float m = -INFINITY;
+  for (int j = lane; j < a.E; j += 64) {
+    const float4* kr =
+        reinterpret_cast<const float4*>(base + (size_t)j * row_stride + HD);
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < kHeadDim / 4; ++c) {
+      const float4 kv = kr[c];
+      const float4 qv = *reinterpret_cast<const float4*>(&s_q[wave][4 * c]);
+      s = fmaf(qv.x, kv.x, s);
+      s = fmaf(qv.y, kv.y, s);
+      s = fmaf(qv.z, kv.z, s);
+      s = fmaf(qv.w, kv.w, s);
+    }
+    const float mask = (q_valid && j < n) ? 0.f : -1e10f;
+    const float x = s + (mask + bias[j]);
+    s_w[wave][j] = x;
+    m = fmaxf(m, x);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int j = lane; j < a.E; j += 64) {
+    const float p = expf(s_w[wave][j] - m);
+    s_w[wave][j] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  // s_w[wave] is written and read by this wavefront only
+  float acc = 0.f;
+  const float* vr = base + 2 * HD + lane;
+  for (int j = 0; j < a.E; ++j)
+    acc = fmaf(s_w[wave][j] / sum, vr[(size_t)j * row_stride], acc);
+  a.out[((size_t)b * a.E + e) * HD + h * kHeadDim + lane] = acc;
+}
+
 }  // namespace t5d
 
 using namespace t5d;
@@ -229,5 +298,30 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
   dim3 grid((E + 63) / 64, H, B), block(256);
   hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_encoder_attention");
+  return T5D_OK;
+}
+
+extern "C" int t5d_encoder_attention_f32(void* stream, const float* qkv,
+                                         const float* rel_bias,
+                                         const int32_t* enc_len, float* out,
+                                         int B, int H, int E) {
+  T5D_REQUIRE(qkv && rel_bias && enc_len && out, T5D_EINVAL,
+              "t5d_encoder_attention_f32: null pointer");
+  T5D_REQUIRE(B > 0 && H > 0 && E > 0, T5D_EINVAL,
+              "t5d_encoder_attention_f32: B=%d H=%d E=%d", B, H, E);
+  T5D_REQUIRE(E <= kMaxEncLen, T5D_ELIMIT,
+              "t5d_encoder_attention_f32: E=%d beyond %d", E, kMaxEncLen);
+  T5D_REQUIRE(H <= 65535 && B <= 65535, T5D_ELIMIT,
+              "t5d_encoder_attention_f32: H=%d B=%d beyond the launch grid", H,
+              B);
+  T5D_REQUIRE(((uintptr_t)qkv % 16) == 0, T5D_EINVAL,
+              "t5d_encoder_attention_f32: qkv must be 16-byte aligned");
+  EncAttnF32Args a;
+  a.qkv = qkv; a.bias = rel_bias; a.len = enc_len; a.out = out;
+  a.H = H; a.E = E;
+  dim3 grid((E + kEncF32Rows - 1) / kEncF32Rows, H, B);
+  hipLaunchKernelGGL(enc_attn_f32_kernel, grid, dim3(64 * kEncF32Rows), 0,
+                     as_stream(stream), a);
+  T5D_CHECK_LAUNCH("t5d_encoder_attention_f32");
   return T5D_OK;
 }

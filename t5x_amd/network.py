@@ -155,31 +155,17 @@ class DecoderWeights:
           wi=ops.pack_weight(g(n, mlp, 'wi_0', 'kernel'), act, wdt,
                              gate_kernel=g(n, mlp, 'wi_1', 'kernel')),
           wo=ops.pack_weight(g(n, mlp, 'wo', 'kernel'), act, wdt),
-          # once-per-batch cross K/V projection: packed for t5d_gemm_rows
-          # (bfloat16 activations), library layout for the float32 path
-          cross_k=self._dense_for_library(g(n, ca, 'key', 'kernel'), act, wdt),
-          cross_v=self._dense_for_library(g(n, ca, 'value', 'kernel'), act,
-                                          wdt),
+          # once-per-batch cross K/V projection (t5d_gemm_rows / t5d_gemm)
+          cross_k_packed=ops.pack_weight(g(n, ca, 'key', 'kernel'), act, wdt),
+          cross_v_packed=ops.pack_weight(g(n, ca, 'value', 'kernel'), act,
+                                         wdt),
       )
-      if act == torch.bfloat16:
-        layer['cross_k_packed'] = ops.pack_weight(g(n, ca, 'key', 'kernel'),
-                                                  act, wdt)
-        layer['cross_v_packed'] = ops.pack_weight(g(n, ca, 'value', 'kernel'),
-                                                  act, wdt)
       self.layers.append(layer)
     self.ln_final = g('decoder_norm', 'scale').to(act)
     # Logits layer: float32 in the reference; bf16 configs stream it as bf16
     # (or int8) with float32 accumulation and float32 output.
     self.logits = ops.pack_weight(g('logits_dense', 'kernel'), act, wdt)
     self._rel_bias = {}
-
-  @staticmethod
-  def _dense_for_library(kernel, act, wdt):
-    if wdt == torch.int8:
-      scale = kernel.abs().amax(dim=0).clamp_min(1e-30) / 127.0
-      q = torch.clamp(torch.round(kernel / scale), -127, 127)
-      return (q.to(act), scale.to(torch.float32))
-    return (kernel.to(act), None)
 
   def rel_bias(self, length: int):
     """[H, L] table: bias for distance n = query_pos - key_pos >= 0
@@ -359,10 +345,10 @@ class Transformer:
                                 out=out['v'][i] if out else None,
                                 layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep))
         continue
-      for (kern, scale), dst in ((l['cross_k'], ks), (l['cross_v'], vs)):
-        y = torch.matmul(x, kern)  # float32 accumulate, one rounding
-        if scale is not None:
-          y = (torch.matmul(x.float(), kern.float()) * scale).to(x.dtype)
+      # float32, or an encoder length the head-layout epilogue does not take:
+      # rows from the dense kernel, brought into the head layouts by copies
+      for packed, dst in ((l['cross_k_packed'], ks), (l['cross_v_packed'], vs)):
+        y = (ops.gemm_rows(x, packed) if bf16 else ops.gemm(x, packed))
         y = y.view(B, E, H, D)
         if dst is ks:  # keys: [B, H, E, D], head dim contiguous
           buf = torch.zeros((B, H, Ep, D), dtype=x.dtype, device=x.device)

@@ -428,6 +428,26 @@ def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
   return out
 
 
+def encoder_attention_f32(qkv, rel_bias, enc_len, H, out=None):
+  """float32 encoder self-attention from the fused projection: qkv
+  [B*E, 3*H*64] (q | k | v), rel_bias [H, 2E-1], enc_len [B] -> [B*E, H*64]."""
+  _chk(qkv, 'qkv', torch.float32, 2)
+  _chk(rel_bias, 'rel_bias', torch.float32, 2)
+  _chk(enc_len, 'enc_len', torch.int32, 1)
+  B = enc_len.shape[0]
+  E = (rel_bias.shape[1] + 1) // 2
+  if (tuple(qkv.shape) != (B * E, 3 * H * 64) or rel_bias.shape[0] != H or
+      rel_bias.shape[1] != 2 * E - 1):
+    raise ValueError(f'qkv {tuple(qkv.shape)} / rel_bias {tuple(rel_bias.shape)}'
+                     f' do not match B={B}, E={E}, H={H}')
+  if out is None:
+    out = torch.empty((B * E, H * 64), dtype=torch.float32, device=qkv.device)
+  _chk(out, 'out', torch.float32, 2)
+  _lib.call('t5d_encoder_attention_f32', _s(), qkv.data_ptr(),
+            rel_bias.data_ptr(), enc_len.data_ptr(), out.data_ptr(), B, H, E)
+  return out
+
+
 def add_i32(x, delta):
   _chk(x, 'x', torch.int32)
   _lib.call('t5d_add_i32', _s(), x.data_ptr(), x.numel(), int(delta))

@@ -169,6 +169,108 @@ def test_encoder_forward_matches_oracle(B, E):
   assert err.max() < 0.25, err.max()
 
 
+@pytest.mark.parametrize('B,E', [(2, 18), (3, 41)])
+def test_encoder_forward_at_lengths_off_the_tile_matches_oracle(B, E):
+  """bf16 encoder at lengths that are not a multiple of 4 (the rows are padded
+  with padding tokens for the kernels and dropped again)."""
+  from t5x_amd import network
+  ocfg, gcfg = _tiny_cfgs()
+  params = ot5.init_params(ocfg, seed=E)
+  rs = np.random.RandomState(E)
+  tok = rs.randint(2, ocfg.vocab_size, size=(B, E)).astype(np.int32)
+  lens = rs.randint(3, E + 1, size=(B,))
+  lens[0] = E
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  want = ot5.encode(params, ocfg, tok)
+  module = network.Transformer(gcfg, torch.device('cuda'))
+  got = host(module.apply({'params': params}, tok, enable_dropout=False,
+                          method=module.encode))
+  assert got.shape == want.shape
+  valid = np.arange(E)[None, :] < lens[:, None]
+  err = np.abs(got - want)[valid]
+  assert (err >= 4e-2).mean() < 0.01, (err >= 4e-2).mean()
+  assert err.mean() < 1e-2, err.mean()
+
+
+@pytest.mark.parametrize('B,E,H', [(2, 16, 1), (3, 41, 2), (2, 130, 3)])
+def test_encoder_attention_f32(ops, B, E, H):
+  """float32 encoder self-attention against the closed form (softmax of
+  q.k + bias + mask, times v), ragged lengths; padded query rows attend
+  uniformly over all E keys, as the reference's arithmetic makes them."""
+  rs = np.random.RandomState(B * 31 + E + H)
+  HD = H * 64
+  qkv = rs.randn(B * E, 3 * HD).astype(np.float32)
+  rel = rs.randn(H, 2 * E - 1).astype(np.float32)
+  lens = rs.randint(1, E + 1, size=(B,)).astype(np.int32)
+  lens[0] = E
+  got = host(ops.encoder_attention_f32(dev(qkv), dev(rel), dev(lens), H))
+  q, k, v = (qkv[:, i * HD:(i + 1) * HD].reshape(B, E, H, 64) for i in range(3))
+  idx = np.arange(E)[None, :] - np.arange(E)[:, None] + E - 1   # [query, key]
+  valid = np.arange(E)[None, :] < lens[:, None]
+  mask = valid[:, :, None] & valid[:, None, :]                  # [B, q, k]
+  bias = np.where(mask, 0.0, -1e10).astype(np.float32)[:, None] + rel[:, idx][None]
+  scores = np.einsum('bqhd,bkhd->bhqk', q, k).astype(np.float32) + bias
+  scores = scores - scores.max(-1, keepdims=True)
+  p = np.exp(scores)
+  p = p / p.sum(-1, keepdims=True)
+  want = np.einsum('bhqk,bkhd->bqhd', p, v).reshape(B * E, HD)
+  np.testing.assert_allclose(got, want, atol=2e-5, rtol=2e-5)
+
+
+@pytest.mark.parametrize('B,E', [(2, 16), (3, 41)])
+def test_encoder_forward_f32_matches_oracle(B, E):
+  """Whole float32 encoder on the HIP kernels (dense kernel with the layer
+  norms inside, vector-ALU attention) against the oracle."""
+  from t5x_amd import network
+  ocfg, gcfg = _tiny_cfgs(dtype='float32')
+  params = ot5.init_params(ocfg, seed=E)
+  rs = np.random.RandomState(E)
+  tok = rs.randint(2, ocfg.vocab_size, size=(B, E)).astype(np.int32)
+  lens = rs.randint(3, E + 1, size=(B,))
+  lens[0] = E
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  want = ot5.encode(params, ocfg, tok)
+  module = network.Transformer(gcfg, torch.device('cuda'))
+  got = host(module.apply({'params': params}, tok, enable_dropout=False,
+                          method=module.encode))
+  valid = np.arange(E)[None, :] < lens[:, None]
+  np.testing.assert_allclose(got[valid], want[valid], atol=1e-4, rtol=1e-4)
+
+
+def test_cross_kv_projection_f32_and_odd_length_match_oracle():
+  """The projection through the row-output dense kernels (float32, and
+  bfloat16 at a length the head-layout epilogue does not take)."""
+  from t5x_amd import network
+  rs = np.random.RandomState(2)
+  B, E, K = 2, 18, 2
+  tok = np.ones((B, E), np.int32)
+  tok[1, 7:] = 0
+  for dtype, tol in (('float32', 1e-4), ('bfloat16', 2e-2)):
+    ocfg, gcfg = _tiny_cfgs(dtype=dtype)
+    params = ot5.init_params(ocfg, seed=6)
+    encoded = rs.randn(B, E, ocfg.emb_dim).astype(np.float32)
+    if dtype == 'bfloat16':
+      encoded = ot5.bf16_round(encoded)
+    want = ot5.project_cross_kv(params, ocfg, encoded)
+    module = network.Transformer(gcfg, torch.device('cuda'))
+    w = module.decoder_weights(params)
+    tdt = torch.bfloat16 if dtype == 'bfloat16' else torch.float32
+    cross = module._cross_kv(w, dev(encoded, tdt), dev(tok), K)
+    assert cross['enc_len'].tolist() == [18, 7]
+    Ep = cross['E']
+    for (wk, wv), gk, gv in zip(want, cross['k'], cross['v']):
+      Bk, H = gk.shape[:2]
+      if dtype == 'bfloat16':
+        pk = host(gk.permute(0, 1, 3, 2, 4).reshape(Bk, H, Ep, 64))
+        pv = host(gv.permute(0, 1, 3, 2, 4).reshape(Bk, H, 64, Ep))
+      else:
+        pk, pv = host(gk), host(gv)
+      np.testing.assert_allclose(pk[:, :, :E].transpose(0, 2, 1, 3), wk,
+                                 atol=tol, rtol=2**-7)
+      np.testing.assert_allclose(pv[..., :E].transpose(0, 3, 1, 2), wv,
+                                 atol=tol, rtol=2**-7)
+
+
 def test_cross_kv_projection_layouts_match_oracle():
   from t5x_amd import network
   ocfg, gcfg = _tiny_cfgs()
