@@ -358,8 +358,8 @@ class EncoderStage:
     self.torch = torch
     size, B, K, E, Emin, L, dtype, wdt, _ = CONFIGS[name]
     if dtype != 'bfloat16':
-      raise SystemExit('bench.py --stage encoder: the HIP encoder is bfloat16; '
-                       f'{name} is {dtype}')
+      raise SystemExit('bench.py --stage encoder measures the bfloat16 '
+                       f'encoder (matrix-core kernels); {name} is {dtype}')
     self.size, self.B, self.K, self.E = size, B, K, E
     self.cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
     dev = torch.device('cuda')
