@@ -307,7 +307,9 @@ def cpu_baseline(name, steps, seed):
   shape (decoder only, cross K/V hoisted as in the GPU path)."""
   from oracle import decoding as odec
   from oracle import t5 as ot5
-  size, B, K, E, Emin, L, dtype, wdt, _ = CONFIGS[name]
+  size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[name]
+  if size == 'small':
+    steps = max(steps, L - 2)  # a few steps of this one are over in a blink
   from t5x_amd import network
   kw = dict(network.T5_1_1[size])
   kw['num_encoder_layers'] = 0
@@ -335,12 +337,20 @@ def cpu_baseline(name, steps, seed):
     return logits[:, 0], cache
 
   inputs = np.zeros((B, L), np.int32)
-  odec.beam_search(inputs, ot5.init_cache(cfg, B, L), tokens_to_logits, 1,
-                   num_decodes=K, alpha=0.6, max_decode_step=steps)
+  if loop == 'beam':
+    odec.beam_search(inputs, ot5.init_cache(cfg, B, L), tokens_to_logits, 1,
+                     num_decodes=K, alpha=0.6, max_decode_step=steps)
+    what = 'beam-search'
+  else:
+    odec.temperature_sample(inputs, ot5.init_cache(cfg, B, L), tokens_to_logits,
+                            1, decode_rng=seed, num_decodes=K,
+                            temperature=loop[1], topk=loop[2],
+                            max_decode_steps=steps)
+    what = 'temperature_sample'
   sec = time.perf_counter() - calls['t0']
   return {'value': round(B * calls['n'] / sec, 2), 'unit': 'tokens/s',
           'cores': host_threads(), 'kind': 'port',
-          'sample': f'{calls["n"]} beam-search steps of {name} (NumPy oracle, '
+          'sample': f'{calls["n"]} {what} steps of {name} (NumPy oracle, '
                     f'decoder only, {sec:.1f} s)'}
 
 
@@ -534,7 +544,9 @@ def main():
                  'rows_x_steps_per_s': round(B * K * args.steps / elapsed, 1)},
       'roofline': roofline_cross_attention(w),
   }
-  if not args.no_cpu_baseline and loop == 'beam':
+  # (the oracle's float32 copy of the XXL weights alone is 45 GB and minutes
+  # of initialisation: no CPU figure for that shape)
+  if not args.no_cpu_baseline and size != 'xxl':
     out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
   print(json.dumps(out))
 
