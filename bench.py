@@ -60,7 +60,7 @@ def parse_args():
   ap.add_argument('--roofline-only', action='store_true',
                   help='only the dominant-kernel replay plus a plain copy of '
                        'known size (for counter runs under rocprofv3 --pmc)')
-  ap.add_argument('--cpu-steps', type=int, default=3,
+  ap.add_argument('--cpu-steps', type=int, default=6,
                   help='size of the CPU oracle sample: decode steps (batch '
                        'rows with --stage encoder)')
   return ap.parse_args()
