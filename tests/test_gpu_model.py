@@ -347,7 +347,8 @@ def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
 @pytest.mark.parametrize('B,K,L,lanes', [(3, 4, 12, 1), (3, 4, 12, 2),
                                          (2, 2, 140, 2), (5, 1, 9, 3),
-                                         (5, 3, 20, 8)])
+                                         (5, 3, 20, 8), (3, 8, 30, 1),
+                                         (2, 8, 200, 1)])
 def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L, lanes):
   """The captured whole-iteration graph (in-place state, gated kernels,
   reorder deferred into the next step's attention for bf16) and the
@@ -602,14 +603,15 @@ def test_full_size_base_beam4_fused_loop_equals_generic_loop():
   assert np.isfinite(scores).all()
 
 
-def test_fused_beam_loop_slot_maps_follow_the_inheritance_rule():
+@pytest.mark.parametrize('K', [2, 3, 4, 8])
+def test_fused_beam_loop_slot_maps_follow_the_inheritance_rule(K):
   """Where the graph-replay loop keeps the beams' cache rows: after every
   iteration the slot maps written on the device equal the host model of the
   rule (first child inherits, further children take the unread slots) applied
   to the parents the iteration chose, and stay permutations."""
   from t5x_amd import decoding
   from tests.test_gpu_kernels import inherit_slots
-  B, K, E, L = 6, 4, 64, 24
+  B, E, L = 6, 64, 24
   module, fn = _full_size_setup('small', B, K, E, 16, L, decoding.beam_search)
   inputs = np.zeros((B, L), np.int32)
   loop = decoding.BeamLoop(inputs, module.init_cache(B, L), fn, eos_id=1,
