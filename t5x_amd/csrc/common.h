@@ -201,6 +201,10 @@ extern thread_local const int32_t* tls_gate;
   if (t5d_gate_open_ == 0) return
 
 // ---- internal launches used by the fused step (not part of the C ABI) -------
+// True when t5d_norm_gemm (bfloat16 activations, no epilogue) runs this shape on
+// its kernel for very wide layers, which keeps the rows resident and streams
+// only the weights.
+bool norm_gemm_is_wide(int w_dtype, int K, int N);
 // Embedding rows of the current tokens, read straight from the sequences:
 // ids[r] = seqs[r, *cur_index] (t5d_gather_step_ids + t5d_embed in one kernel).
 int launch_embed_from_seqs(hipStream_t s, int dtype, const void* table,

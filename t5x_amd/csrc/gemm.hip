@@ -429,6 +429,215 @@ norm_gemm_kernel(GemmArgs g) {
   }
 }
 
+// ---- layer norm + dense for a very wide layer (the vocabulary projection) -------
+// With tens of thousands of output columns the kernels above re-read the
+// activation rows once per column group, and those re-reads, not the weights,
+// are most of what enters the CUs.  Here the rows stay put: a workgroup
+// normalises 64 rows once, parks them in LDS in matrix-core operand order
+// ([m-tile][k-tile][lane], read back without bank conflicts) and then walks
+// over column groups of 128 (groups g0, g0 + G, ...), so that only weights
+// stream.  A wavefront owns 2 column tiles of the group over ALL of K — no
+// sum across wavefronts — and every operand it reads from LDS feeds two
+// products.  The weight tiles of a whole group are in flight at once, in
+// chunks of 8 k-tiles; a chunk's registers are refilled with the same chunk of
+// the next group as soon as it is consumed.  The rows and the norm scale are
+// requested BEFORE the weights: loads return in the order they were issued,
+// so the normalisation runs while the weight tiles are still on their way.
+// The two row halves of a 128-row call work on the same groups from the same
+// XCD (block ids 8 apart), so the second read of a weight tile is served by
+// that XCD's L2.  The code is kept small on purpose (one copy of the chunk
+// loop and of the stores): it runs once or twice per workgroup, so every
+// instruction is an instruction-cache miss.
+constexpr int kWideCT = 2;     // column tiles per wavefront
+constexpr int kWideChunk = 8;  // k-tiles per chunk
+constexpr int kWideMinN = 8192;  // columns from which the wide kernel is used
+
+#ifdef T5D_PROBE_WIDE
+__device__ long long t5d_wide_probe_buf[64 * 16];
+#define T5D_WSTAMP(i)                                              \
+  if (lane == 0 && wave == 0 && blockIdx.x % 4 == 0)               \
+    t5d_wide_probe_buf[(blockIdx.x / 4) * 16 + (i)] = wall_clock64()
+#else
+#define T5D_WSTAMP(i)
+#endif
+
+template <int KT>
+__global__ void __launch_bounds__(256)
+norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
+  static_assert(KT % kWideChunk == 0 && KT <= 32, "K of the wide kernel");
+  constexpr int CT = kWideCT, CH = kWideChunk;
+  constexpr int CPG = KT / CH;  // chunks per column group
+  __shared__ uint4 s_a[4 * KT * 64];
+  __shared__ uint4 s_scale[KT * 4];
+  T5D_GATE_READ(g.gate);
+  const int xcd = blockIdx.x & 7, s = blockIdx.x >> 3;
+  const int half = s % halves;
+  const int g0 = (s / halves) * 8 + xcd;
+  const int n_tiles_total = g.N >> 4;
+  const int n_groups = (n_tiles_total + 4 * CT - 1) / (4 * CT);
+  if (g0 >= n_groups) return;
+  const int m0 = half * 64;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n16 = lane & 15, gq = lane >> 4;
+  T5D_WSTAMP(0);
+
+  // Rows of m-tile `wave` and the norm scale first ...
+  const int row = m0 + wave * 16 + n16;
+  const bool row_ok = row < g.M;
+  uint4 xa[KT];
+  {
+    const bf16_t* xrow = g.A + (size_t)(row_ok ? row : g.M - 1) * g.K + 8 * gq;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+      xa[kt] = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+  }
+  uint4 scale_part = make_uint4(0, 0, 0, 0);
+  if (threadIdx.x < KT * 4)
+    scale_part = reinterpret_cast<const uint4*>(g.norm_scale)[threadIdx.x];
+  T5D_GATE_TEST();
+
+  // ... then the weight tiles of the first group.
+  const uint4* wbase = reinterpret_cast<const uint4*>(g.W);
+  uint4 wq[CPG][CH][CT];
+  auto load_chunk = [&](int ci, int grp) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int nt = min((grp * 4 + wave) * CT + ct, n_tiles_total - 1);
+      const uint4* p = wbase + ((size_t)nt * KT + ci * CH) * 64 + lane;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) wq[ci][k][ct] = p[k * 64];
+    }
+  };
+  // (at most three chunks now, the rest once the rows have left the registers)
+  constexpr int PRE = CPG < 2 ? CPG : 2;
+  constexpr int MID = CPG < 3 ? CPG : 3;
+#pragma unroll
+  for (int ci = 0; ci < PRE; ++ci) load_chunk(ci, g0);
+  T5D_WSTAMP(1);
+
+  if (threadIdx.x < KT * 4) s_scale[threadIdx.x] = scale_part;
+  float ss = 0.f;
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt) {
+    float f[8];
+    unpack16(xa[kt], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+  }
+  ss = rows_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)g.K + g.eps);
+  __syncthreads();
+  T5D_WSTAMP(2);
+  // the rows have arrived: a third chunk can follow without delaying them
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int ci = PRE; ci < MID; ++ci) load_chunk(ci, g0);
+  __builtin_amdgcn_sched_barrier(0);
+  // (scale reads in batches of 8 k-tiles: one LDS latency per batch, not one
+  // per k-tile)
+#pragma unroll
+  for (int kb = 0; kb < KT; kb += 8) {
+    uint4 sc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sc[j] = s_scale[(kb + j) * 4 + gq];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kt = kb + j;
+      float xf[8], sf[8];
+      unpack16(xa[kt], xf);
+      unpack16(sc[j], sf);
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float y0 = round_bf16(xf[2 * e] * inv);
+        const float y1 = round_bf16(xf[2 * e + 1] * inv);
+        o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
+      }
+      s_a[(wave * KT + kt) * 64 + lane] =
+          row_ok ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int ci = MID; ci < CPG; ++ci) load_chunk(ci, g0);
+  __syncthreads();
+  T5D_WSTAMP(3);
+
+  for (int grp = g0; grp < n_groups; grp += G) {
+    f32x4_v acc[4][CT];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[mt][ct] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+    const bool more = grp + G < n_groups;
+    // The row operands of k-tile kk + 1 are read from LDS while the products
+    // of k-tile kk run (two register sets, pinned in this order: left alone,
+    // the compiler reads one operand, waits, multiplies, and pays the LDS
+    // latency 4 * KT times per group).
+    Frag af[2][4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) af[0][mt].u = s_a[(mt * KT) * 64 + lane];
+#pragma unroll
+    for (int ci = 0; ci < CPG; ++ci) {
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int kk = ci * CH + k;
+        __builtin_amdgcn_sched_barrier(0);
+        if (kk + 1 < KT) {
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+            af[(kk + 1) & 1][mt].u = s_a[(mt * KT + kk + 1) * 64 + lane];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct) {
+            Frag b;
+            b.u = wq[ci][k][ct];
+            acc[mt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                af[kk & 1][mt].v, b.v, acc[mt][ct], 0, 0, 0);
+          }
+        }
+      }
+      // keep the refill behind the products that read these registers
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) load_chunk(ci, grp + G);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    T5D_WSTAMP(grp == g0 ? 4 : 6);
+    // Accumulator element i of tile (mt, ct) in lane l is
+    // C[16*mt + 4*(l/16) + i][16*ct + l%16].
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int nt = (grp * 4 + wave) * CT + ct;
+      if (nt >= n_tiles_total) continue;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int m = m0 + mt * 16 + 4 * gq + i;
+          if (m >= g.M) continue;
+          const size_t o = (size_t)m * g.N + nt * 16 + n16;
+          if (g.out_f32)
+            reinterpret_cast<float*>(g.C)[o] = acc[mt][ct][i];
+          else
+            reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(acc[mt][ct][i]);
+        }
+    }
+    T5D_WSTAMP(grp == g0 ? 5 : 7);
+  }
+  T5D_WSTAMP(15);
+}
+#ifdef T5D_PROBE_WIDE
+extern "C" int t5d_wide_probe_read(long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t5d_wide_probe_buf),
+                                  sizeof(long long) * 64 * 16);
+}
+#endif
+
 // ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
 // A workgroup owns 8 rows x 16 output columns: with a handful of rows the
 // kernel is a stream of the weight matrix, and narrow column tiles are what
@@ -699,6 +908,11 @@ static void launch_mfma(const GemmPlan& p, GemmArgs g, hipStream_t s) {
 
 using namespace t5d;
 
+bool t5d::norm_gemm_is_wide(int w_dtype, int K, int N) {
+  return w_dtype == T5D_BF16 && N >= kWideMinN && N % 16 == 0 &&
+         (K == 512 || K == 768 || K == 1024);
+}
+
 // One kernel shape for every M (rows in groups of 8 along grid.y), so the
 // summation order, and with it every bit of the result, does not depend on
 // how many rows a call carries.
@@ -875,6 +1089,23 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
   g.norm_scale = (const bf16_t*)norm_scale;
   g.eps = eps;
   const int n_tiles = N / 16;
+  hipStream_t s = as_stream(stream);
+  // Very wide layers (the vocabulary projection): rows resident in LDS, only
+  // the weights stream.
+  if (epilogue == T5D_EPI_NONE && norm_gemm_is_wide(w_dtype, K, N)) {
+    const int halves = (M + 63) / 64;
+    const int n_groups = (n_tiles + 4 * kWideCT - 1) / (4 * kWideCT);
+    const int G = min((n_groups + 7) / 8 * 8, 256 / halves);
+    dim3 grid(G * halves), block(256);
+    if (K == 512)
+      hipLaunchKernelGGL(norm_gemm_wide_kernel<16>, grid, block, 0, s, g, G, halves);
+    else if (K == 768)
+      hipLaunchKernelGGL(norm_gemm_wide_kernel<24>, grid, block, 0, s, g, G, halves);
+    else
+      hipLaunchKernelGGL(norm_gemm_wide_kernel<32>, grid, block, 0, s, g, G, halves);
+    T5D_CHECK_LAUNCH("t5d_norm_gemm(wide)");
+    return T5D_OK;
+  }
   const int nj = (K / 64 + 3) / 4;  // k-tile pairs per wavefront
   // 64-column tiles unless that leaves too few workgroups to fill the chip;
   // beyond K = 1024 the fragments of fewer column tiles fit the registers
@@ -883,7 +1114,6 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
   if (nj > 4) nt = min(nt, w_dtype == T5D_I8 ? 2 : 1);
   const int n_groups = (n_tiles + nt - 1) / nt;
   dim3 grid((n_groups + 7) / 8 * 8 * g.m_parts), block(256);
-  hipStream_t s = as_stream(stream);
 #define T5D_NG_LAUNCH(NT_, NJ_, WT_)                                          \
   hipLaunchKernelGGL((norm_gemm_kernel<NT_, NJ_, WT_>), grid, block, 0, s, g)
 #define T5D_NG_CASE(NT_, WT_)                                                 \

@@ -133,10 +133,19 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
                      R, F, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
     x = m->x;
   }
-  T5D_TRY(t5d_rmsnorm(stream, dt, x, m->ln_final, m->xn, R, d, 1e-6f));
-  T5D_TRY(t5d_gemm(stream, dt, wd, T5D_F32, m->xn, m->logits_w,
-                   m->logits_scales, nullptr, m->logits, R, d, m->V,
-                   T5D_EPI_NONE, nullptr, nullptr));
+  // The final norm rides inside the vocabulary projection where the kernel
+  // for very wide layers covers the shape (34 + 4.7 us as two kernels at
+  // d = 768, V = 32128, 128 rows).
+  if (dt == T5D_BF16 && norm_gemm_is_wide(wd, d, m->V)) {
+    T5D_TRY(t5d_norm_gemm(stream, dt, wd, T5D_F32, x, m->ln_final, 1e-6f,
+                          m->logits_w, nullptr, m->logits, R, d, m->V,
+                          T5D_EPI_NONE));
+  } else {
+    T5D_TRY(t5d_rmsnorm(stream, dt, x, m->ln_final, m->xn, R, d, 1e-6f));
+    T5D_TRY(t5d_gemm(stream, dt, wd, T5D_F32, m->xn, m->logits_w,
+                     m->logits_scales, nullptr, m->logits, R, d, m->V,
+                     T5D_EPI_NONE, nullptr, nullptr));
+  }
   if (bump_index) T5D_TRY(t5d_add_i32(stream, m->cache_index, m->NL, 1));
   return T5D_OK;
 }

@@ -199,6 +199,42 @@ def test_norm_gemm_f32(ops, M, K, N, geglu):
   np.testing.assert_allclose(host(one), want, atol=1e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize('M,K,N', [(128, 768, 32128), (64, 1024, 32128),
+                                   (20, 512, 8192), (100, 768, 8208),
+                                   (1, 768, 32128), (65, 512, 16400)])
+@pytest.mark.parametrize('f32out', [True, False])
+def test_norm_gemm_wide_layer(ops, M, K, N, f32out):
+  """The vocabulary-sized case of the fused layer norm + dense layer (rows
+  resident in LDS, one wavefront sums all of K for its columns): against the
+  two-kernel sequence, against the oracle's layer_norm + dense, and bit for
+  bit against itself."""
+  rs = np.random.RandomState(M + K + N + 9)
+  x = dev(rs.randn(M, K).astype(np.float32) * 3, torch.bfloat16)
+  scale = dev(1 + 0.1 * rs.randn(K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  pw = ops.pack_weight(dev(w0), torch.bfloat16)
+  kw = {'out_dtype': torch.float32} if f32out else {}
+  two = ops.gemm(ops.rmsnorm(x, scale), pw, **kw)
+  one = ops.gemm(x, pw, norm_scale=scale, **kw)
+  assert one.shape == (M, N) and one.dtype == two.dtype
+  xn = ot5.layer_norm(host(x), host(scale), 'bfloat16')
+  if f32out:
+    # float32 sums in a different order agree to 1e-3; a row whose 1/rms
+    # moved by an ulp can flip the bf16 rounding of a normalised element,
+    # which shows as up to 2e-2 in that row's outputs
+    want = xn @ ot5.bf16_round(w0)
+    for ref in (host(two), want):
+      err = np.abs(host(one) - ref)
+      assert float((err > 1e-3 + 1e-4 * np.abs(ref)).mean()) < 2e-3
+      np.testing.assert_allclose(host(one), ref, atol=2e-2, rtol=2**-7)
+  else:
+    want = ot5.dense_general(xn, w0, 'bfloat16')
+    diff = (one.float() - two.float()).abs()
+    assert float((diff > 0).float().mean()) < 0.02
+    np.testing.assert_allclose(host(one), want, atol=2e-2, rtol=2**-7)
+  assert torch.equal(one, ops.gemm(x, pw, norm_scale=scale, **kw))
+
+
 def test_norm_gemm_rejects_what_it_does_not_cover(ops):
   x = dev(np.zeros((4, 64), np.float32))
   pwq = ops.pack_weight(dev(np.zeros((64, 32), np.float32)), torch.bfloat16)
