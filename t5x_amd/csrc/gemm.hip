@@ -75,6 +75,30 @@ template <> struct WeightTile<int8_t> {
   }
 };
 
+// The matrix cores want lane (m, g) = (lane % 16, lane / 16) to hold the 8
+// values k = 8g .. 8g+7 of row m.  Loaded that way, the 16 lanes of a quarter
+// wavefront touch 16 different rows: 64 separate 16-byte requests per load
+// instruction, and the L1's tag lookups (one per request) become the
+// bottleneck of a kernel that reads a few KB.  Instead lane l loads piece
+// l % 4 of row l / 4 — four neighbouring lanes read 64 contiguous bytes — and
+// the 16-byte pieces are moved to the lanes that need them through the LDS
+// crossbar (ds_bpermute: no LDS memory involved).
+struct OperandLanes {
+  int ld_row, ld_piece;  // what this lane loads: row within the tile, 8-k piece
+  int src_addr;          // ds_bpermute address of the lane that loaded my piece
+  __device__ __forceinline__ explicit OperandLanes(int lane)
+      : ld_row(lane >> 2), ld_piece(lane & 3),
+        src_addr((((lane & 15) << 2) | (lane >> 4)) << 2) {}
+  __device__ __forceinline__ uint4 to_operand(const uint4& loaded) const {
+    uint4 r;
+    r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.x);
+    r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.y);
+    r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.z);
+    r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.w);
+    return r;
+  }
+};
+
 struct GemmArgs {
   const bf16_t* A;      // [M, K]
   const void* W;        // packed tiles
@@ -146,8 +170,9 @@ gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
   for (int i = 0; i < ACC; ++i) acc[i] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
 
-  const int arow = lane & 15;
-  const int akoff = (lane >> 4) * 8;
+  const OperandLanes ol(lane);
+  const int arow = ol.ld_row;
+  const int akoff = ol.ld_piece * 8;
   const char* wbase = reinterpret_cast<const char*>(g.W);
   constexpr int TB = WeightTile<WT>::kTileBytes;
 
@@ -202,6 +227,11 @@ gemm_mfma_kernel(GemmArgs g) {
             else
               a[h][mt].u = make_uint4(0, 0, 0, 0);
           }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int mt = 0; mt < MP; ++mt)
+            a[h][mt].u = ol.to_operand(a[h][mt].u);
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -324,7 +354,10 @@ norm_gemm_kernel(GemmArgs g) {
   const int m0 = m_part * 16;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n16 = lane & 15, gq = lane >> 4;
+  // Rows are loaded, measured and normalised in the load layout (lane l: piece
+  // l % 4 of row l / 4) and moved to operand order just before the products.
+  const OperandLanes ol(lane);
+  const int n16 = ol.ld_row, gq = ol.ld_piece;
   const int KT = g.K >> 5, n_pairs = KT >> 1;
   const int row = m0 + n16;
   const bool row_ok = row < g.M;
@@ -365,7 +398,8 @@ norm_gemm_kernel(GemmArgs g) {
       }
     }
   }
-  ss = rows_sum(ss);
+  ss += dpp_move<kDppXor1>(ss);  // over the 4 pieces of the row
+  ss += dpp_move<kDppXor2>(ss);
   if (gq == 0) s_ss[wave][n16] = ss;
   __syncthreads();
   const float tot = (s_ss[0][n16] + s_ss[2][n16]) + (s_ss[1][n16] + s_ss[3][n16]);
@@ -390,8 +424,8 @@ norm_gemm_kernel(GemmArgs g) {
           o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
         }
         Frag an;
-        an.u = row_ok ? make_uint4(o[0], o[1], o[2], o[3])
-                      : make_uint4(0, 0, 0, 0);
+        an.u = ol.to_operand(row_ok ? make_uint4(o[0], o[1], o[2], o[3])
+                                    : make_uint4(0, 0, 0, 0));
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn)
           acc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
