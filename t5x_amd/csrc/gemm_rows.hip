@@ -103,13 +103,23 @@ rows_gemm_kernel(RowsGemmArgs g) {
   // The 6 tiles this wavefront fetches: activation tiles wave + 4 i (i < 4),
   // weight tiles wave + 4 i (i < 2).  Out-of-range rows / tiles are clamped
   // (their products are discarded in the epilogue).
+  // An activation tile is fetched with lane l reading piece l % 4 (8 k) of row
+  // l / 4, so that four neighbouring lanes read 64 contiguous bytes: fetched in
+  // operand order (lane = row + 16 * piece) every lane of a quarter wavefront
+  // touches another row, 64 separate requests per instruction, and the L1's
+  // tag lookups, not the matrix cores, set the pace.  The piece lands in LDS at
+  // its operand slot, XOR-swizzled so that neither the parking writes nor the
+  // operand reads collide on banks.
+  const int ld_row = lane >> 2, ld_piece = lane & 3;
+  const int park_slot = (ld_piece * 16 + ld_row) ^ (ld_piece * 2);
+  const int read_slot = lane ^ (gq * 2);
   const bf16_t* arow[4];
   const char* wtile[2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
     arow[i] = g.A +
-              (size_t)min(m_blk * kRowsBM + 16 * (wave + 4 * i) + l16, g.M - 1) *
-                  g.K + 8 * gq;
+              (size_t)min(m_blk * kRowsBM + 16 * (wave + 4 * i) + ld_row, g.M - 1) *
+                  g.K + 8 * ld_piece;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
     wtile[i] = g.W + (size_t)min(n_blk * (kRowsBN / 16) + wave + 4 * i,
@@ -137,10 +147,10 @@ rows_gemm_kernel(RowsGemmArgs g) {
   } while (0)
 #define T5D_ROWS_PARK(buf_)                                                    \
   do {                                                                         \
-    s_t[buf_][wave][lane] = sa0;                                               \
-    s_t[buf_][wave + 4][lane] = sa1;                                           \
-    s_t[buf_][wave + 8][lane] = sa2;                                           \
-    s_t[buf_][wave + 12][lane] = sa3;                                          \
+    s_t[buf_][wave][park_slot] = sa0;                                          \
+    s_t[buf_][wave + 4][park_slot] = sa1;                                      \
+    s_t[buf_][wave + 8][park_slot] = sa2;                                      \
+    s_t[buf_][wave + 12][park_slot] = sa3;                                     \
     s_t[buf_][16 + wave][lane] = RowsWeightTile<WT>::frag(sw0);                \
     s_t[buf_][20 + wave][lane] = RowsWeightTile<WT>::frag(sw1);                \
   } while (0)
@@ -156,7 +166,7 @@ rows_gemm_kernel(RowsGemmArgs g) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       FragR xa;
-      xa.u = s_t[buf][wm * MT + mt][lane];
+      xa.u = s_t[buf][wm * MT + mt][read_slot];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         if (SWAP)
