@@ -77,20 +77,28 @@ enc_attn_kernel(EncAttnArgs a) {
   const int n_tiles =
       (q0 + 15 < n) ? (n + 15) >> 4 : (E + 15) >> 4;
 
-  // K tile kt as the A operand: lane (row = key l16, g) holds K[key][32c + 8g .. +8]
+  // K tile kt as the A operand: lane (row = key l16, g) holds K[key][32c + 8g .. +8].
+  // It is fetched with four neighbouring lanes on 64 contiguous bytes of one key
+  // (16 requests per instruction instead of 64: this kernel walks every key
+  // tile twice, and fetched in operand order the L1's tag lookups bound it) and
+  // moved to operand order by `operand_k` when it is consumed.
+  const OperandLanes ol(lane);
   auto load_k = [&](int kt, FragE (&ka)[2]) {
-    const int key_row = min(16 * kt + l16, E - 1);
+    const int key_row = min(16 * kt + ol.ld_row, E - 1);
 #pragma unroll
     for (int c = 0; c < 2; ++c)
       ka[c].u = *reinterpret_cast<const uint4*>(
-          a.k + (row0 + key_row) * a.k_stride + h * 64 + 32 * c + 8 * gq);
+          a.k + (row0 + key_row) * a.k_stride + h * 64 + 32 * c + 8 * ol.ld_piece);
   };
   // scores of key tile kt for this lane: keys 16 kt + 4 g + i of query l16
   auto score_tile = [&](int kt, const FragE (&ka)[2], float (&s)[4]) {
     f32x4_e acc = (f32x4_e){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c].v, qb[c].v, acc, 0, 0, 0);
+    for (int c = 0; c < 2; ++c) {
+      FragE kop;
+      kop.u = ol.to_operand(ka[c].u);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qb[c].v, acc, 0, 0, 0);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = 16 * kt + 4 * gq + i;

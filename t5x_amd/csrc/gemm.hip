@@ -75,30 +75,6 @@ template <> struct WeightTile<int8_t> {
   }
 };
 
-// The matrix cores want lane (m, g) = (lane % 16, lane / 16) to hold the 8
-// values k = 8g .. 8g+7 of row m.  Loaded that way, the 16 lanes of a quarter
-// wavefront touch 16 different rows: 64 separate 16-byte requests per load
-// instruction, and the L1's tag lookups (one per request) become the
-// bottleneck of a kernel that reads a few KB.  Instead lane l loads piece
-// l % 4 of row l / 4 — four neighbouring lanes read 64 contiguous bytes — and
-// the 16-byte pieces are moved to the lanes that need them through the LDS
-// crossbar (ds_bpermute: no LDS memory involved).
-struct OperandLanes {
-  int ld_row, ld_piece;  // what this lane loads: row within the tile, 8-k piece
-  int src_addr;          // ds_bpermute address of the lane that loaded my piece
-  __device__ __forceinline__ explicit OperandLanes(int lane)
-      : ld_row(lane >> 2), ld_piece(lane & 3),
-        src_addr((((lane & 15) << 2) | (lane >> 4)) << 2) {}
-  __device__ __forceinline__ uint4 to_operand(const uint4& loaded) const {
-    uint4 r;
-    r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.x);
-    r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.y);
-    r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.z);
-    r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(src_addr, (int)loaded.w);
-    return r;
-  }
-};
-
 struct GemmArgs {
   const bf16_t* A;      // [M, K]
   const void* W;        // packed tiles
