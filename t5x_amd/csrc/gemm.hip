@@ -492,15 +492,22 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
   const int n16 = lane & 15, gq = lane >> 4;
   T5D_WSTAMP(0);
 
-  // Rows of m-tile `wave` and the norm scale first ...
-  const int row = m0 + wave * 16 + n16;
-  const bool row_ok = row < g.M;
-  uint4 xa[KT];
-  {
-    const bf16_t* xrow = g.A + (size_t)(row_ok ? row : g.M - 1) * g.K + 8 * gq;
+  // Rows of m-tile `wave` and the norm scale first ...  Lane l fetches piece
+  // l % 8 (8 k) of a pair of k-tiles for rows l / 8 and 8 + l / 8: eight
+  // neighbouring lanes read one 128-byte line (fetched in operand order, each
+  // lane of a quarter wavefront would touch another row and the L1 would look
+  // up 64 lines per instruction instead of 8).
+  const int ld_r8 = lane >> 3, oct = lane & 7;
+  bool row_ok[2];
+  uint4 xa[2][KT / 2];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt)
-      xa[kt] = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+  for (int i = 0; i < 2; ++i) {
+    const int row = m0 + wave * 16 + 8 * i + ld_r8;
+    row_ok[i] = row < g.M;
+    const bf16_t* xrow = g.A + (size_t)(row_ok[i] ? row : g.M - 1) * g.K + 8 * oct;
+#pragma unroll
+    for (int j = 0; j < KT / 2; ++j)
+      xa[i][j] = *reinterpret_cast<const uint4*>(xrow + 64 * j);
   }
   uint4 scale_part = make_uint4(0, 0, 0, 0);
   if (threadIdx.x < KT * 4)
@@ -527,16 +534,22 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
   T5D_WSTAMP(1);
 
   if (threadIdx.x < KT * 4) s_scale[threadIdx.x] = scale_part;
-  float ss = 0.f;
+  float inv[2];
 #pragma unroll
-  for (int kt = 0; kt < KT; ++kt) {
-    float f[8];
-    unpack16(xa[kt], f);
+  for (int i = 0; i < 2; ++i) {
+    float ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+    for (int j = 0; j < KT / 2; ++j) {
+      float f[8];
+      unpack16(xa[i][j], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+    }
+    ss += dpp_move<kDppXor1>(ss);  // over the 8 lanes that share the row
+    ss += dpp_move<kDppXor2>(ss);
+    ss += lane_xor4(ss);
+    inv[i] = 1.0f / sqrtf(ss / (float)g.K + g.eps);
   }
-  ss = rows_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)g.K + g.eps);
   __syncthreads();
   T5D_WSTAMP(2);
   // the rows have arrived: a third chunk can follow without delaying them
@@ -544,29 +557,39 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
 #pragma unroll
   for (int ci = PRE; ci < MID; ++ci) load_chunk(ci, g0);
   __builtin_amdgcn_sched_barrier(0);
-  // (scale reads in batches of 8 k-tiles: one LDS latency per batch, not one
-  // per k-tile)
+  // Normalised pieces go to their operand slot (lane = row + 16 * piece of
+  // k-tile 2 j + oct / 4), XOR-swizzled so that neither these writes nor the
+  // operand reads below collide on LDS banks.  Scale reads in batches: one LDS
+  // latency per batch, not one per piece.
+  const int kt_lo = oct >> 2, piece = oct & 3;
+  constexpr int JB = 4;
 #pragma unroll
-  for (int kb = 0; kb < KT; kb += 8) {
-    uint4 sc[8];
+  for (int jb = 0; jb < KT / 2; jb += JB) {
+    uint4 sc[JB];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sc[j] = s_scale[(kb + j) * 4 + gq];
+    for (int jj = 0; jj < JB; ++jj) sc[jj] = s_scale[8 * (jb + jj) + oct];
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int kt = kb + j;
-      float xf[8], sf[8];
-      unpack16(xa[kt], xf);
-      unpack16(sc[j], sf);
-      uint32_t o[4];
+    for (int jj = 0; jj < JB; ++jj) {
+      const int j = jb + jj;
+      float sf[8];
+      unpack16(sc[jj], sf);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float y0 = round_bf16(xf[2 * e] * inv);
-        const float y1 = round_bf16(xf[2 * e + 1] * inv);
-        o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
+      for (int i = 0; i < 2; ++i) {
+        float xf[8];
+        unpack16(xa[i][j], xf);
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(xf[2 * e] * inv[i]);
+          const float y1 = round_bf16(xf[2 * e + 1] * inv[i]);
+          o[e] = pack_bf16x2(y0 * sf[2 * e], y1 * sf[2 * e + 1]);
+        }
+        const int slot = (piece * 16 + 8 * i + ld_r8) ^ (2 * piece + kt_lo);
+        s_a[(wave * KT + 2 * j + kt_lo) * 64 + slot] =
+            row_ok[i] ? make_uint4(o[0], o[1], o[2], o[3])
+                      : make_uint4(0, 0, 0, 0);
       }
-      s_a[(wave * KT + kt) * 64 + lane] =
-          row_ok ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -588,7 +611,8 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
     // latency 4 * KT times per group).
     Frag af[2][4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) af[0][mt].u = s_a[(mt * KT) * 64 + lane];
+    for (int mt = 0; mt < 4; ++mt)
+      af[0][mt].u = s_a[(mt * KT) * 64 + (lane ^ (2 * gq))];
 #pragma unroll
     for (int ci = 0; ci < CPG; ++ci) {
 #pragma unroll
@@ -598,7 +622,8 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
         if (kk + 1 < KT) {
 #pragma unroll
           for (int mt = 0; mt < 4; ++mt)
-            af[(kk + 1) & 1][mt].u = s_a[(mt * KT + kk + 1) * 64 + lane];
+            af[(kk + 1) & 1][mt].u =
+                s_a[(mt * KT + kk + 1) * 64 + (lane ^ (2 * gq + ((kk + 1) & 1)))];
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
