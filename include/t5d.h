@@ -109,6 +109,12 @@ int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
  * summation order of the product as t5d_gemm.  bfloat16 activations; packed
  * bfloat16 or int8 weights (scales: per-output-channel float32 [N] for int8,
  * else NULL); K a multiple of 64, <= 2048; epilogue NONE or GEGLU.
+ * Very wide layers (bfloat16 weights, no epilogue, N >= 8192, K = 512, 768 or
+ * 1024: the final LayerNorm + logits layer, t5x/examples/t5/network.py:274-291)
+ * run on a kernel that keeps the normalised rows in LDS and streams only the
+ * weights; there one wavefront sums all of K for its columns, so float32
+ * results differ from t5d_rmsnorm + t5d_gemm by summation order (~1e-6
+ * relative), deterministically.
  * float32 (activations, row-major [K, N] weights and outputs): any M, K, N;
  * the norm scale multiplies the weights as they are loaded and 1/rms the
  * finished sums, which differs from normalising first by a few float32 ulps. */
