@@ -62,6 +62,55 @@ rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
   }
 }
 
+// bfloat16 rows in 16-byte pieces: RPW rows per 256-thread workgroup, 256 / RPW
+// threads per row (a wavefront per row when there are thousands of rows, the
+// whole workgroup on one row when rows are few and long).  Same roundings as
+// above; the row is read a second time for the output, from L1.
+template <int RPW>
+__global__ void __launch_bounds__(256)
+rmsnorm_vec_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ scale,
+                   bf16_t* __restrict__ out, int R, int d, float eps,
+                   const int32_t* gate) {
+  constexpr int TPR = 256 / RPW;  // threads per row
+  static_assert(TPR == 64 || TPR == 256, "a wavefront or the workgroup per row");
+  T5D_GATE_READ(gate);
+  __shared__ float partial[4];
+  const int t = threadIdx.x % TPR;
+  const int r = blockIdx.x * RPW + threadIdx.x / TPR;
+  const bool row_ok = r < R;  // uniform per wavefront
+  const int chunks = d >> 3;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + (size_t)(row_ok ? r : 0) * d);
+  float ss = 0.f;
+  for (int c = t; c < chunks; c += TPR) {
+    float f[8];
+    unpack16(xr[c], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+  }
+  T5D_GATE_TEST();
+  ss = wave_sum(ss);
+  if (TPR == 256) {
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  }
+  if (!row_ok) return;
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  uint4* o = reinterpret_cast<uint4*>(out + (size_t)r * d);
+  const uint4* sv = reinterpret_cast<const uint4*>(scale);
+  for (int c = t; c < chunks; c += TPR) {
+    float xf[8], sf[8];
+    unpack16(xr[c], xf);
+    unpack16(sv[c], sf);
+    uint32_t y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      y[e] = pack_bf16x2(round_bf16(xf[2 * e] * inv) * sf[2 * e],
+                         round_bf16(xf[2 * e + 1] * inv) * sf[2 * e + 1]);
+    o[c] = make_uint4(y[0], y[1], y[2], y[3]);
+  }
+}
+
 __global__ void add_i32_kernel(int32_t* x, int n, int delta,
                                const int32_t* gate) {
   T5D_GATED(gate);
@@ -119,6 +168,14 @@ extern "C" int t5d_rmsnorm(void* stream, int dtype, const void* x,
     hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(R), dim3(256), 0,
                        as_stream(stream), (const float*)x, (const float*)scale,
                        (float*)out, d, eps, tls_gate);
+  else if (d % 8 == 0 && R >= 512 && ((uintptr_t)x | (uintptr_t)scale | (uintptr_t)out) % 16 == 0)
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<4>, dim3((R + 3) / 4), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)x,
+                       (const bf16_t*)scale, (bf16_t*)out, R, d, eps, tls_gate);
+  else if (d % 8 == 0 && d >= 2048 && ((uintptr_t)x | (uintptr_t)scale | (uintptr_t)out) % 16 == 0)
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<1>, dim3(R), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)x,
+                       (const bf16_t*)scale, (bf16_t*)out, R, d, eps, tls_gate);
   else
     hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(R), dim3(256), 0,
                        as_stream(stream), (const bf16_t*)x,

@@ -49,7 +49,8 @@ def test_embed_exact(ops, dt):
 
 
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize('R,d', [(1, 64), (8, 512), (128, 768), (5, 4096)])
+@pytest.mark.parametrize('R,d', [(1, 64), (8, 512), (128, 768), (5, 4096),
+                                 (1001, 768), (514, 1024), (128, 2048)])
 def test_rmsnorm(ops, dt, R, d):
   rs = np.random.RandomState(R + d)
   x = dev(3 * rs.randn(R, d).astype(np.float32), dt)
