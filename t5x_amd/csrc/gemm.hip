@@ -167,9 +167,33 @@ gemm_mfma_kernel(GemmArgs g) {
           bq[slot_][h][nn] = WeightTile<WT>::zero();
       }
   };
+  // The activation rows of a pair travel with its weight tiles (requested
+  // together, PF pairs ahead): requested only when a pair is due, they would be
+  // the newest loads in flight, and since loads return in order, waiting for
+  // them would drain the whole weight queue once per pair.
+  // (at most 64 registers of them: fewer pairs ahead for tall tiles)
+  constexpr int APF = PF * MP <= 8 ? PF : (8 / MP > 0 ? 8 / MP : 1);
+  uint4 aq[APF][2][MP];
+  auto load_a = [&](int slot_, int j) {
+    const int kt = (wave + 4 * j) * 2;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int mt = 0; mt < MP; ++mt) {
+        const int row = m0 + mt * 16 + arow;
+        if (row < g.M && kt + h < KT)
+          aq[slot_][h][mt] = *reinterpret_cast<const uint4*>(
+              g.A + (size_t)row * g.K + (kt + h) * 32 + akoff);
+        else
+          aq[slot_][h][mt] = make_uint4(0, 0, 0, 0);
+      }
+  };
 #pragma unroll
   for (int p = 0; p < PF; ++p)
-    if (p < nj) load_b(p, p);
+    if (p < nj) {
+      load_b(p, p);
+      if (p < APF) load_a(p, p);
+    }
   // The residual elements this thread will need in the epilogue.
   float res[FLAT ? ACC : 1];
   if (FLAT && g.epilogue == T5D_EPI_RESIDUAL) {
@@ -190,24 +214,12 @@ gemm_mfma_kernel(GemmArgs g) {
     for (int p = 0; p < PF; ++p) {
       const int j = j0 + p;
       if (j < nj) {
-        const int kt = (wave + 4 * j) * 2;
         Frag a[2][MP];
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int mt = 0; mt < MP; ++mt) {
-            const int row = m0 + mt * 16 + arow;
-            if (row < g.M && kt + h < KT)
-              a[h][mt].u = *reinterpret_cast<const uint4*>(
-                  g.A + (size_t)row * g.K + (kt + h) * 32 + akoff);
-            else
-              a[h][mt].u = make_uint4(0, 0, 0, 0);
-          }
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
           for (int mt = 0; mt < MP; ++mt)
-            a[h][mt].u = ol.to_operand(a[h][mt].u);
+            a[h][mt].u = ol.to_operand(aq[p % APF][h][mt]);
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -218,6 +230,7 @@ gemm_mfma_kernel(GemmArgs g) {
                   a[h][mt].v, WeightTile<WT>::frag(bq[p][h][nn]).v,
                   acc[mt * NT + nn], 0, 0, 0);
         if (j + PF < nj) load_b(p, j + PF);
+        if (j + APF < nj) load_a(p % APF, j + APF);
       }
     }
   }
@@ -878,8 +891,11 @@ struct GemmPlan {
 // rate.  w_bytes: bytes per weight element.
 static int tile_occupancy(int mp, int nt) {
   // workgroups per CU = wavefronts per SIMD of gemm_mfma_kernel<mp, nt>
+  // (from the registers the compiler reports for the bfloat16 instances)
   const int acc = mp * nt;
-  return acc == 1 ? 8 : acc == 2 ? 5 : acc == 4 ? 4 : acc == 8 && mp < 8 ? 3 : 2;
+  if (acc == 1) return 5;
+  if (acc <= 4) return mp == 1 ? 4 : 3;
+  return acc == 8 && mp == 2 ? 3 : 2;
 }
 
 static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
