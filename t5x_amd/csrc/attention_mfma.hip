@@ -154,13 +154,27 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     const int xr = b * a.nq + (n16 < a.nq ? n16 : 0);
     const bf16_t* xrow = a.x + (size_t)xr * a.d + 8 * g;
     const char* wbase = reinterpret_cast<const char*>(a.wq);
+    // Rows, then the norm scale, then the weight tiles: loads return in the
+    // order they were issued, and the row statistics need only the rows.
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
         xa[j][hh].u = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+      }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
         lnv[j][hh] = *reinterpret_cast<const uint4*>(a.ln + 32 * kt + 8 * g);
+      }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
 #pragma unroll
         for (int nn = 0; nn < 4; ++nn)
           wt[j][hh][nn].u = reinterpret_cast<const uint4*>(

@@ -355,6 +355,9 @@ norm_gemm_kernel(GemmArgs g) {
   typename WeightTile<WT>::Raw wt[NJ][2][NT];
   uint4 lnv[NJ][2];
   {
+    // Rows first, then the norm scale, then the weight tiles: loads return in
+    // the order they were issued, and the row statistics need only the rows —
+    // issued between the weight tiles they would wait for most of those too.
     const bf16_t* xrow = g.A + (size_t)(row_ok ? row : g.M - 1) * g.K + 8 * gq;
     const char* wbase = reinterpret_cast<const char*>(g.W);
 #pragma unroll
@@ -363,8 +366,20 @@ norm_gemm_kernel(GemmArgs g) {
       for (int hh = 0; hh < 2; ++hh) {
         const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
         xa[j][hh].u = *reinterpret_cast<const uint4*>(xrow + 32 * kt);
+      }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
         lnv[j][hh] =
             *reinterpret_cast<const uint4*>(g.norm_scale + 32 * kt + 8 * gq);
+      }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kt = min((wave + 4 * j) * 2 + hh, KT - 1);
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn)
           wt[j][hh][nn] = WeightTile<WT>::load(
