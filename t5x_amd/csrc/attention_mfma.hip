@@ -139,11 +139,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   // Every K and V chunk is requested up front (whole 16 / 32 position tiles,
   // skipped by wave-uniform branches beyond the valid length; inside a tile
   // the tail past the valid length is read and masked, it must be finite).
-  // A skipped tile's registers are left alone — the products that would read
-  // them are skipped by the same conditions: giving them a value here makes the
-  // compiler merge it with the loaded one by a register copy right behind the
-  // load, i.e. a wait for that load (and, loads returning in order, for every
-  // load before it) in the middle of the requests.
   //   K: A operand, lane (row = position n16, g) holds K[j][32c + 8g .. +8];
   //   V: A operand, lane (row = d n16, g) holds V[16dt + n16][32jb + 8g .. +8].
   // S is a multiple of 8 but not of the tile sizes: addresses are clamped to
@@ -194,6 +189,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
         kb[jt][c].u = *reinterpret_cast<const uint4*>(
             kbase + ((size_t)c * a.S + min(jw + 16 * jt + n16, a.S - 1)) * 32 +
             8 * g);
+    } else {
+      kb[jt][0].u = kb[jt][1].u = make_uint4(0, 0, 0, 0);
     }
   }
   auto load_v = [&]() {
@@ -205,6 +202,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
           vb[jb][dt].u = *reinterpret_cast<const uint4*>(
               vbase + ((size_t)(wave * (kBlockJ / 32) + jb) * kHeadDim +
                        16 * dt + n16) * 32 + 8 * g);
+      } else {
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);
       }
     }
   };
