@@ -8,7 +8,11 @@ A "step" is one iteration of the beam-search loop: one decoder forward for the
 reorder and the loop-condition check.  `value` = batch * steps / seconds
 (decoded tokens per second: every batch item emits one token per step).  The
 encoder output is synthetic and the cross-attention K/V projection, weight
-packing and upload happen before the timed region.
+packing and upload happen before the timed region.  An iteration costs more
+the later it comes in a decode (self-attention streams the cache filled so
+far), so the timed iterations are whole decodes plus, for a remainder or a
+step count below the decode length, a window centred on the middle of a fresh
+decode (`config.t_first` / `t_last`); decode starts are outside the clock.
 
 Prints ONE JSON line.  `roofline` describes the dominant HBM-bound kernel of
 the step, timed live with HIP events on the launch stream; `cpu_baseline` is the
@@ -100,34 +104,26 @@ class Workload:
         network.BeamShared(self.enc_tokens, K), L)
     self.weights = self.module.decoder_weights(self.params)
     self.loop = None
+    self.decodes = 0
 
   def new_decode(self):
     # Drop the finished decode first so that its cache buffers go back to the
     # allocator before the new ones are requested: no hipMalloc per decode.
     self.loop = None
     cache = self.module.init_cache(self.B, self.L)
-    self.loop = self.decoding.BeamLoop(
-        self.inputs, cache, self.tokens_to_logits, eos_id=1,
-        num_decodes=self.K, alpha=0.6)
-
-  def run_sample_steps(self, n):
-    """Exactly n temperature_sample iterations: whole decodes of L steps, then
-    one decode limited to the remainder by max_decode_steps.  A decode that
-    ended early (every row hit EOS) would make the count wrong and raises."""
-    torch = self.torch
-    _, temperature, topk = self.loop_kind
-    done = 0
-    while done < n:
-      take = min(n - done, self.L)
-      cache = self.module.init_cache(self.B, self.L)
-      seqs, _ = self.decoding.temperature_sample(
+    if self.loop_kind == 'beam':
+      self.loop = self.decoding.BeamLoop(
+          self.inputs, cache, self.tokens_to_logits, eos_id=1,
+          num_decodes=self.K, alpha=0.6)
+    else:
+      _, temperature, topk = self.loop_kind
+      self.decodes += 1
+      self.loop = self.decoding.SampleLoop(
           self.inputs, cache, self.tokens_to_logits, 1,
-          decode_rng=self.seed + done, num_decodes=self.K,
-          temperature=temperature, topk=topk,
-          max_decode_steps=take if take < self.L else None)
-      if not bool((seqs[:, :, take - 1] != 0).any()):
-        raise RuntimeError(f'sampling decode ended before step {take}')
-      done += take
+          self.seed + self.decodes, self.K, temperature, topk,
+          use_fused=True)
+    if not self.loop.cond():
+      raise RuntimeError('fresh decode terminated immediately')
 
   def prime(self):
     """Set-up, before the warm-up steps: a few iterations of a first decode
@@ -140,36 +136,58 @@ class Workload:
       self.loop = None
     self.torch.cuda.synchronize()
 
-  def run_steps(self, n):
-    if self.loop_kind != 'beam':
-      return self.run_sample_steps(n)
-    return self.run_beam_steps(n)
-
-  def run_beam_steps(self, n):
+  def run_steps(self, n, timed=False):
     """Runs exactly n loop iterations, starting a new decode whenever the
     current one has produced its max_decode_len tokens.  The loop condition is
     evaluated on the device after every iteration; it is read back once per
-    decode (with these random-init weights no batch item ever finishes early,
-    which the read-back at the end of each decode verifies)."""
-    done = 0
+    decode (with these random-init weights no decode ends early, which the
+    read-back at the end of each decode verifies).
+
+    timed: returns (seconds, windows).  The cost of an iteration grows with
+    its position t in the decode (self-attention streams t + 1 cache columns),
+    so the timed iterations are whole decodes (t = 0 .. L-1) and, for what is
+    left over (or all of it when n < L), a window centred on t = (L-1)/2 of a
+    fresh decode, which is advanced to the window's start untimed.  Decode
+    starts (cache clear, state initialisation, cross K/V projection: once per
+    batch, not part of the step loop) and the end-of-decode read-back are
+    outside the clock; every timed segment has a device synchronisation on
+    both sides."""
+    sync = self.torch.cuda.synchronize
+    if timed:
+      self.loop = None
+    done, seconds, windows = 0, 0.0, []
     while done < n:
       if self.loop is None or self.loop.step >= self.L:
         if self.loop is not None:
-          if self.loop.cond():
-            raise RuntimeError('decode did not stop at max_decode_len')
           self.check_full_decode()
         self.new_decode()
-        if not self.loop.cond():
-          raise RuntimeError('fresh decode terminated immediately')
       take = min(n - done, self.L - self.loop.step)
+      if timed and self.loop.step == 0 and take < self.L:
+        self.loop.advance((self.L - take) // 2)
+      first = self.loop.step
+      if timed:
+        sync()
+        t0 = time.perf_counter()
       self.loop.advance(take)
+      if timed:
+        sync()
+        seconds += time.perf_counter() - t0
+        windows.append((first, first + take - 1))
       done += take
+    if timed and self.loop.step >= self.L:
+      self.check_full_decode()
+    return seconds, windows
 
   def check_full_decode(self):
-    cur_index = int(self.loop.cur.cur_index.item())
-    if cur_index != self.L:
-      raise RuntimeError(f'decode stopped early at step {cur_index}; the '
-                         'step count of this run would be wrong')
+    if self.loop.cond():
+      raise RuntimeError('decode did not stop at max_decode_len')
+    if self.loop_kind == 'beam':
+      count = int(self.loop.cur.cur_index.item())
+    else:
+      count = int(self.loop.fused.step_count.item())
+    if count != self.L:
+      raise RuntimeError(f'decode stopped early at step {count}; the step '
+                         'count of this run would be wrong')
 
   # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
   def cross_attention_bytes(self, fused=True):
@@ -513,10 +531,7 @@ def main():
   w.prime()
   w.run_steps(args.warmup)
   torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  w.run_steps(args.steps)
-  torch.cuda.synchronize()
-  elapsed = time.perf_counter() - t0
+  elapsed, windows = w.run_steps(args.steps, timed=True)
 
   size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[args.config]
   if loop == 'beam':
@@ -541,6 +556,10 @@ def main():
       'config': {'workload': f'T5.1.1-{size} {what}, encoder {E} ({Emin}..{E} '
                              f'valid), max decode length {L}',
                  'name': args.config, 'beam_rows': B * K,
+                 # positions t of the decode the timed iterations covered:
+                 # whole decodes, then a window centred on (L-1)/2
+                 't_first': windows[-1][0], 't_last': windows[-1][1],
+                 'timed_windows': [list(x) for x in windows],
                  'rows_x_steps_per_s': round(B * K * args.steps / elapsed, 1)},
       'roofline': roofline_cross_attention(w),
   }

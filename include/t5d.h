@@ -128,10 +128,12 @@ int t5d_norm_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
  * network.py:73,87, and the once-per-batch key / value projections of the
  * decoder's cross-attention, network.py:149-159).  bfloat16 activations;
  * W packed by t5d_pack_weight (bfloat16 or int8 + scales); epilogues as
- * t5d_gemm.  out_layout T5D_OUT_HEADS_*: row m = b * E + e, column
- * n = h * 64 + d is written to [B, H, Ep, 64] / [B, H, 64, Ep] (what
- * t5d_cross_attention_step reads); rows e >= E of those buffers are left
- * untouched. */
+ * t5d_gemm.  out_layout T5D_OUT_HEADS_KEY / T5D_OUT_HEADS_VALUE: row
+ * m = b * E + e, column n = h * 64 + d is written to [B, H, 2, Ep, 32] at
+ * [b, h, d / 32, e, d % 32] / to [B, H, Ep/32, 64, 32] at
+ * [b, h, e / 32, d, e % 32] (the bfloat16 layouts t5d_cross_attention_step
+ * and t5d_encoder_attention read; Ep a multiple of 32); positions e >= E of
+ * those buffers are left untouched. */
 int t5d_gemm_rows(void* stream, int w_dtype, const void* A, const void* W,
                   const float* scales, const void* residual, void* C,
                   int64_t M, int K, int N, int epilogue, int out_layout, int E,

@@ -228,7 +228,11 @@ def multi_head_attention(params, inputs_q, inputs_kv, mask, bias, *,
         mask,
         np.broadcast_to(np.arange(length) <= cur_index, (b, 1, 1, length)))
     if bias is not None:  # :297-303 row `cur_index` of the bias matrix
-      ci = int(cur_index)
+      # lax.dynamic_slice_in_dim (:132-134) clamps a start beyond the last
+      # row to the last row; jax.nn.one_hot above is all zeros there, so a
+      # step past the end of the cache inserts nothing and attends to all of
+      # it.  (No reference test goes there: parity unpinned for that case.)
+      ci = min(max(int(cur_index), 0), bias.shape[2] - 1)
       bias = bias[:, :, ci:ci + 1, :]
 
   if mask is not None:  # :306-314

@@ -59,8 +59,15 @@ attn_step_kernel(AttnArgs a) {
 
   int n, t = 0;
   bool uniform = false;  // no valid key: the masked softmax is uniform
+  // A cache index outside [0, S) (a decode loop longer than its cache) must
+  // not become an address: nothing is inserted then and all S columns are
+  // attended with the bias row of the last position, which is what the
+  // reference's one-hot insert and clamped slices do (layers.py:258-303).
+  bool past_end = false;
   if (SELF) {
     t = *a.index;
+    past_end = t < 0 || t >= a.S;
+    if (past_end) t = a.S - 1;
     n = t + 1;
   } else {
     n = a.index[g];
@@ -92,7 +99,7 @@ attn_step_kernel(AttnArgs a) {
 
   // Self-attention: the lane whose chunk contains column t carries the new
   // key/value, patches its registers and writes the column to the cache.
-  const bool ins = SELF && live && (t >= j0) && (t < j0 + EL);
+  const bool ins = SELF && !past_end && live && (t >= j0) && (t < j0 + EL);
   const int e_t = t - j0;
 
   float s[NQ][EL];

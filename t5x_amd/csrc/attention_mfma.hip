@@ -61,24 +61,6 @@ struct AttnMfmaArgs {
 constexpr int kHeadDim = 64;
 constexpr int kBlockJ = 128;  // positions per wavefront
 
-// Phase timestamps for kernel tuning; compiled out unless T5D_PROBE is set.
-#ifdef T5D_PROBE
-__device__ long long t5d_probe_buf[64 * 16];
-#define T5D_STAMP(i)                                                       \
-  if (lane == 0 && wave == 0 && (blockIdx.x + blockIdx.y * gridDim.x) % 37 == 0 && \
-      (blockIdx.x + blockIdx.y * gridDim.x) / 37 < 64)                      \
-    t5d_probe_buf[((blockIdx.x + blockIdx.y * gridDim.x) / 37) * 16 + (i)] = \
-        wall_clock64()
-#else
-#define T5D_STAMP(i)
-#endif
-#ifdef T5D_PROBE_FQ  // slots 8..15 go to the fused projection instead
-#define T5D_STAMP_SELF(i)
-#define T5D_STAMP_FQ(i) T5D_STAMP(i)
-#else
-#define T5D_STAMP_SELF(i) T5D_STAMP(i)
-#define T5D_STAMP_FQ(i)
-#endif
 
 // ---- cross-attention -----------------------------------------------------------
 // scores^T = K·Q^T with the K tile (16 positions x 32 dims) as the A operand
@@ -120,10 +102,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   const int q = n16 % NQP, rep = n16 / NQP;
   const int HD = a.H * kHeadDim;
 
-  T5D_STAMP(0);
   int n = a.index[b];
   T5D_GATE_TEST();  // after both scalar loads are in flight
-  T5D_STAMP(1);
   n = n < 0 ? 0 : (n > a.S ? a.S : n);
   bool uniform = false;  // no valid key: the masked softmax is uniform
   if (n == 0) { uniform = true; n = a.S; }
@@ -222,7 +202,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       if (!qrow) qb[c].u = make_uint4(0, 0, 0, 0);
     }
   } else {
-    T5D_STAMP_FQ(8);
     // Row statistics: sum of squares of row n16 over this wavefront's k range.
     const int n_pairs = KT >> 1;
     float ss = 0.f;
@@ -239,10 +218,8 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       }
     }
     ss = rows_sum(ss);
-    T5D_STAMP_FQ(9);
     if (g == 0) s_ss[wave][n16] = n16 < a.nq ? ss : 0.f;
     __syncthreads();
-    T5D_STAMP_FQ(10);
     const float tot = (s_ss[0][n16] + s_ss[2][n16]) + (s_ss[1][n16] + s_ss[3][n16]);
     const float inv = 1.0f / sqrtf(tot / (float)a.d + a.eps);
     f32x4_v qacc[4];
@@ -273,7 +250,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
         }
       }
     }
-    T5D_STAMP_FQ(11);
     // qacc[nn][i] in lane (n16, g) is the partial q[row 4g + i][16 nn + n16].
     if (4 * g < NQP) {
 #pragma unroll
@@ -283,9 +259,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
           s_qp[wave][4 * g + i][16 * nn + n16] = qacc[nn][i];
     }
     load_v();  // the V stream follows K while the projection is reduced
-    T5D_STAMP_FQ(12);
     __syncthreads();
-    T5D_STAMP_FQ(13);
     for (int e = threadIdx.x; e < NQP * kHeadDim; e += 64 * WM) {
       const int row = e / kHeadDim, col = e % kHeadDim;
       const float v = (s_qp[0][row][col] + s_qp[2][row][col]) +
@@ -296,7 +270,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
 #pragma unroll
     for (int c = 0; c < 2; ++c)
       qb[c].u = *reinterpret_cast<const uint4*>(&s_qb[q][32 * c + 8 * g]);
-    T5D_STAMP_FQ(14);
   }
 
   // Tile jt: lane (n16, g) gets scores of positions 16 jt + 4g + i, query q.
@@ -321,7 +294,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     }
 
   if constexpr (!FQ && WM > 8) load_v();
-  T5D_STAMP(2);
   // Softmax over all positions of the workgroup for query q.  The 16 lanes
   // that share q differ in lane bits {2,3 (if REP == 4) | 3 (REP == 2)} and
   // in g (bits 4, 5).
@@ -345,7 +317,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     m = s_red[0][0][n16];
     for (int w = 1; w < nwaves; ++w) m = fmaxf(m, s_red[0][w][n16]);
   }
-  T5D_STAMP(3);
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < TPL; ++t)
@@ -364,7 +335,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     sum = s_red[1][0][n16];
     for (int w = 1; w < nwaves; ++w) sum += s_red[1][w][n16];
   }
-  T5D_STAMP(4);
   // Normalise, round to bf16 (where the reference rounds), hand over to the
   // B-operand layout of V·P^T through LDS: 4 consecutive positions per tile.
   {
@@ -378,7 +348,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     }
   }
   __syncthreads();
-  T5D_STAMP(5);
 
   // out^T[d][q] = sum_j V[d][j] P[q][j]; B lane (col n16 -> q, g) holds
   // P[q][32 jb + 8g .. +8].
@@ -396,7 +365,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
                                                          oc[dt], 0, 0, 0);
     }
   }
-  T5D_STAMP(6);
   // oc[dt][i] in lane (n16, g) is out[q][d = 16 dt + 4g + i] (all REP copies).
   if (nwaves == 1) {
     if (rep == 0 && q < a.nq) {
@@ -424,7 +392,6 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int w = 1; w < nwaves; ++w) acc += s_out[w][qq][d];
     a.out[(size_t)(b * a.nq + qq) * HD + h * kHeadDim + d] = f32_to_bf16(acc);
   }
-  T5D_STAMP(7);
 }
 
 // ---- self-attention ------------------------------------------------------------
@@ -510,14 +477,18 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     r = rs = rw = blockIdx.y;
   }
 
-  T5D_STAMP_SELF(8);
-  const int t = *a.index;
+  const int t_in = *a.index;
   T5D_GATE_TEST();  // after the scalar loads above are in flight
-  T5D_STAMP_SELF(9);
+  // A cache index outside [0, S) (a decode loop longer than its cache) must
+  // not become an address: nothing is inserted then and all S columns are
+  // attended with the bias row of the last position, which is what the
+  // reference's one-hot insert and clamped slices do (layers.py:258-303).
+  const bool past_end = t_in < 0 || t_in >= S;
+  const int t = past_end ? S - 1 : t_in;
   const int n = t + 1;
   const int jw = blk * kBlockJ;
   const int nw = n - jw;  // positions of this wavefront in use (may be <= 0)
-  const bool wave_has_t = t >= jw && t < jw + kBlockJ;
+  const bool wave_has_t = !past_end && t >= jw && t < jw + kBlockJ;
   const size_t slot = (size_t)kHeadDim * S;
   const bf16_t* ksrc = a.k + ((size_t)rs * a.H + h) * slot;
   const bf16_t* vsrc = a.v + ((size_t)rs * a.H + h) * slot;
@@ -596,7 +567,6 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     for (int e = 0; e < 8; ++e) s8[e] = fmaf(qv[i], kf[e], s8[e]);
   }
 
-  T5D_STAMP_SELF(10);
   if (permuted) {
     // Every wavefront of the workgroup has its source data in registers
     // before any slot is written.
@@ -634,7 +604,6 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     }
   };
 
-  T5D_STAMP_SELF(11);
   // 2 positions per lane: bias, mask, softmax.
   float sc[2];
   reduce_scatter_8(s8, sc);
@@ -643,7 +612,7 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
     const int j = jp + e;
-    float x = (j == t) ? snew : sc[e];
+    float x = (j == t && !past_end) ? snew : sc[e];
     x = round_bf16(x);
     if (j < n) x = round_bf16(x + s_bias[t - j]);
     else x = -INFINITY;
@@ -657,7 +626,6 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     m = s_red[0][wave0];
     for (int w = 1; w < nblk; ++w) m = fmaxf(m, s_red[0][wave0 + w]);
   }
-  T5D_STAMP_SELF(12);
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
@@ -677,12 +645,11 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
     // column's old content): its probability goes to s_pt instead.
     const float inv = 1.0f / sum;
     float p0 = round_bf16(sc[0] * inv), p1 = round_bf16(sc[1] * inv);
-    if (jp == t) { s_pt[wave] = p0; p0 = 0.f; }
-    if (jp + 1 == t) { s_pt[wave] = p1; p1 = 0.f; }
+    if (jp == t && !past_end) { s_pt[wave] = p0; p0 = 0.f; }
+    if (jp + 1 == t && !past_end) { s_pt[wave] = p1; p1 = 0.f; }
     *reinterpret_cast<uint32_t*>(&s_p[wave][jp - jw]) = pack_bf16x2(p0, p1);
   }
   __syncthreads();
-  T5D_STAMP_SELF(13);
 
   // out^T tile dt: lane (n16, g) gets out[16 dt + 4g + i], i < 4, in every
   // column n16.  B lane (col, g) holds P[32 jb + 8g .. +8].
@@ -712,7 +679,6 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       oc[dt][3] = fmaf(p_t, bf16hi_to_f32(vn.y), oc[dt][3]);
     }
   }
-  T5D_STAMP_SELF(14);
   if (nblk == 1) {
     if (n16 == 0) {
       bf16_t* o = a.out + (size_t)r * HD + h * kHeadDim + 4 * g;
@@ -725,7 +691,6 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       }
     }
     store_column();
-    T5D_STAMP_SELF(15);
     return;
   }
   if (n16 == 0) {
@@ -813,12 +778,5 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
     hipLaunchKernelGGL((self_attn_mfma_kernel<16>), grid, block, 0, s, a);
   return 0;
 }
-
-#ifdef T5D_PROBE
-extern "C" int t5d_probe_read(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t5d_probe_buf),
-                                  sizeof(long long) * 64 * 16);
-}
-#endif
 
 }  // namespace t5d

@@ -490,14 +490,6 @@ constexpr int kWideCT = 2;     // column tiles per wavefront
 constexpr int kWideChunk = 8;  // k-tiles per chunk
 constexpr int kWideMinN = 8192;  // columns from which the wide kernel is used
 
-#ifdef T5D_PROBE_WIDE
-__device__ long long t5d_wide_probe_buf[64 * 16];
-#define T5D_WSTAMP(i)                                              \
-  if (lane == 0 && wave == 0 && blockIdx.x % 4 == 0)               \
-    t5d_wide_probe_buf[(blockIdx.x / 4) * 16 + (i)] = wall_clock64()
-#else
-#define T5D_WSTAMP(i)
-#endif
 
 template <int KT>
 __global__ void __launch_bounds__(256)
@@ -518,7 +510,6 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n16 = lane & 15, gq = lane >> 4;
-  T5D_WSTAMP(0);
 
   // Rows of m-tile `wave` and the norm scale first ...  Lane l fetches piece
   // l % 8 (8 k) of a pair of k-tiles for rows l / 8 and 8 + l / 8: eight
@@ -559,7 +550,6 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
   constexpr int MID = CPG < 3 ? CPG : 3;
 #pragma unroll
   for (int ci = 0; ci < PRE; ++ci) load_chunk(ci, g0);
-  T5D_WSTAMP(1);
 
   if (threadIdx.x < KT * 4) s_scale[threadIdx.x] = scale_part;
   float inv[2];
@@ -579,7 +569,6 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
     inv[i] = 1.0f / sqrtf(ss / (float)g.K + g.eps);
   }
   __syncthreads();
-  T5D_WSTAMP(2);
   // the rows have arrived: a third chunk can follow without delaying them
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -624,7 +613,6 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
 #pragma unroll
   for (int ci = MID; ci < CPG; ++ci) load_chunk(ci, g0);
   __syncthreads();
-  T5D_WSTAMP(3);
 
   for (int grp = g0; grp < n_groups; grp += G) {
     f32x4_v acc[4][CT];
@@ -670,7 +658,6 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
       if (more) load_chunk(ci, grp + G);
       __builtin_amdgcn_sched_barrier(0);
     }
-    T5D_WSTAMP(grp == g0 ? 4 : 6);
     // Accumulator element i of tile (mt, ct) in lane l is
     // C[16*mt + 4*(l/16) + i][16*ct + l%16].
 #pragma unroll
@@ -690,16 +677,8 @@ norm_gemm_wide_kernel(GemmArgs g, int G, int halves) {
             reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(acc[mt][ct][i]);
         }
     }
-    T5D_WSTAMP(grp == g0 ? 5 : 7);
   }
-  T5D_WSTAMP(15);
 }
-#ifdef T5D_PROBE_WIDE
-extern "C" int t5d_wide_probe_read(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t5d_wide_probe_buf),
-                                  sizeof(long long) * 64 * 16);
-}
-#endif
 
 // ---- float32 path (activation dtype float32, unpacked [K, N] kernel) ---------
 // A workgroup owns 8 rows x 16 output columns: with a handful of rows the
@@ -918,19 +897,6 @@ static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
   const int n_tiles = N / 16;
   GemmPlan best = {1, 1, 1, 1};
   double best_cost = 1e30;
-#ifdef T5D_PROBE  // tuning runs force tiles: T5D_GEMM_TILE="K,N,mp,nt;K,N,mp,nt"
-  if (const char* force = getenv("T5D_GEMM_TILE")) {
-    const char* p = force;
-    while (p && *p) {
-      int k = 0, n = 0, mp = 1, nt = 1;
-      if (sscanf(p, "%d,%d,%d,%d", &k, &n, &mp, &nt) == 4 &&
-          (k == 0 || k == K) && (n == 0 || n == N))
-        return {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt};
-      p = strchr(p, ';');
-      if (p) ++p;
-    }
-  }
-#endif
   const int mps[4] = {1, 2, 4, 8};
   const int nts[3] = {1, 2, 4};
   for (int mi = 0; mi < 4; ++mi)

@@ -197,15 +197,6 @@ beam_row_topk_kernel(const float* __restrict__ logits,
 constexpr int kTopkCap = 512;
 constexpr int kFastTopkVec = 8;
 
-// Phase timestamps for kernel tuning; compiled out unless T5D_PROBE is set.
-#ifdef T5D_PROBE
-__device__ long long t5d_select_probe_buf[128 * 8];
-#define T5D_SEL_STAMP(i) \
-  if (tid == 0) t5d_select_probe_buf[blockIdx.x * 8 + (i)] = wall_clock64()
-#else
-#define T5D_SEL_STAMP(i)
-#endif
-
 // exp(x) for x <= 0 to about 1 ulp with the hardware exp2: the rounding error
 // of x * log2(e) is recovered with an fma and folded back in as a first-order
 // correction.  Anything below -1e30 (padding, -inf logits) gives exactly 0.
@@ -249,7 +240,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   constexpr int kNone = 0x7FFFFFFF;
   const int r = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  T5D_SEL_STAMP(0);
   const float4* x4 = reinterpret_cast<const float4*>(logits + (size_t)r * V);
   const int nvec = V >> 2;
   float4 x[kFastTopkVec];
@@ -265,7 +255,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
 #pragma unroll
   for (int u = 0; u < kFastTopkVec; ++u)
     m = fmaxf(fmaxf(m, fmaxf(x[u].x, x[u].y)), fmaxf(x[u].z, x[u].w));
-  T5D_SEL_STAMP(1);
   m = wave_max(m);
   if (lane == 0) s_f[wave] = m;
   if (tid == 0) s_count = 0;
@@ -281,7 +270,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   }
   const unsigned long long whit = __builtin_amdgcn_ballot_w64(wrank == k - 1);
   const float tx = __shfl(wmax, (int)__builtin_ctzll(whit | (1ull << 63)), 64);
-  T5D_SEL_STAMP(2);
 
   double sum = 0.0;
 #pragma unroll
@@ -296,13 +284,11 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   if (lane == 0) s_d[wave] = sum;
   __syncthreads();
   sum = lanes16_sum(s_d[lane & 15]);
-  T5D_SEL_STAMP(3);
   const float lse = (float)log(sum);
   if (tid == 0) {
     row_max[r] = m;
     row_lse[r] = lse;
   }
-  T5D_SEL_STAMP(4);
 
   // f(j) = ((x[j] - max) - lse) + live_logprob, in place; elements at or
   // above the threshold go to the list.
@@ -328,7 +314,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
       }
     }
   }
-  T5D_SEL_STAMP(5);
   __syncthreads();
   const int ncand = s_count;
   if (ncand <= kTopkCap) {
@@ -347,8 +332,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
       cand_vals[(size_t)r * k + tid] = -INFINITY;
       cand_idx[(size_t)r * k + tid] = kNone;
     }
-    T5D_SEL_STAMP(6);
-    T5D_SEL_STAMP(7);
     return;
   }
 
@@ -410,7 +393,6 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
   }
   __syncthreads();
   if (wave != 0) return;
-  T5D_SEL_STAMP(6);
   // Merge the 16 best-first lists: lane w < 16 walks list w.
   int pos = 0;
   for (int out = 0; out < k; ++out) {
@@ -432,15 +414,7 @@ beam_row_topk_fast_kernel(const float* __restrict__ logits,
       cand_idx[(size_t)r * k + out] = best.i;
     }
   }
-  T5D_SEL_STAMP(7);
 }
-
-#ifdef T5D_PROBE
-extern "C" int t5d_select_probe_read(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(t5d_select_probe_buf),
-                                  sizeof(long long) * 128 * 8);
-}
-#endif
 
 // Merge the beams' per-row candidates of one batch item: one candidate per
 // thread (beams*k <= 128), rank by counting better candidates.

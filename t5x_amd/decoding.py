@@ -116,6 +116,33 @@ def cache_map(fn, cache, apply_to_index: bool = False):
   return _unflatten_dict(flat_cache)
 
 
+def _check_cache_room(cache, positions: int, expect_empty: bool):
+  """A decode loop writes one cache column per iteration: a cache shorter than
+  the loop, or one that already holds steps when the loop starts from zero,
+  would push cache_index past the end (the reference silently stops inserting
+  there, layers.py:258-275).  Raises instead.  Only trees with this package's
+  `cached_key` / `cache_index` leaves are looked at; reading the indices back
+  is one host synchronisation per decode."""
+  if not isinstance(cache, Mapping):
+    return
+  flat = _flatten_dict(cache)
+  for path, leaf in flat.items():
+    if path[-1] == 'cached_key' and hasattr(leaf, 'shape'):
+      if leaf.shape[-1] < positions:
+        raise ValueError(
+            f'the decode loop runs up to {positions} steps but the cache '
+            f'{"/".join(map(str, path))} holds {leaf.shape[-1]} positions')
+  if not expect_empty:
+    return
+  idx = [leaf.reshape(-1) for path, leaf in flat.items()
+         if path[-1] == 'cache_index' and isinstance(leaf, torch.Tensor)]
+  if idx and bool((torch.cat(idx) != 0).any()):
+    raise ValueError(
+        'the cache already holds decode steps (cache_index != 0) but no '
+        '`initial_index` was given: start from a cache as the cache '
+        'initialisation returns it')
+
+
 def add_beam_dim(x, beam_size: int, offset: int = 0):
   """:773-780."""
   x = _dev(x).unsqueeze(offset + 1)
@@ -297,6 +324,9 @@ def temperature_sample(
                and getattr(cache, 'fresh', False) and initial_index is None and
                cache_offset == 0 and state_callback_fn is None and
                logit_callback_fn is None)
+  if not use_fused:
+    _check_cache_room(cache, inputs.shape[1],
+                      expect_empty=initial_index is None)
   if use_fused:
     expanded_inputs = (flat_batch_beam_expand(inputs, num_decodes)
                        if num_decodes > 1 else inputs)
@@ -332,6 +362,155 @@ def temperature_sample(
   return decodes, log_prob
 
 
+class SampleLoop:
+  """The loop of _temperature_sample_single_trial (:412-715) as an object:
+  `cond()` / `body()` are the while-loop's condition and body, `finish()` the
+  epilogue; `advance(n)` runs n iterations without reading the condition back
+  (with the fused loop, iterations after every row ended change nothing).
+  Exposing the pieces lets a caller time or single-step the loop."""
+
+  def __init__(self, inputs, cache, tokens_to_logits, eos_id: int, prng_key,
+               num_decodes: int = 1,
+               temperature: Union[float, np.ndarray] = 1.0, topk: int = 20,
+               topp: float = 0.0, initial_index=None, max_decode_steps=None,
+               rescale_log_probs: bool = True,
+               state_callback_fn: Optional[Callable] = None,
+               logit_callback_fn: Optional[Callable] = None,
+               use_fused: bool = False):
+    if topp and topk:
+      raise ValueError('At most one of `topp` or `topk` may be non-zero.')
+    dev = _device()
+    inputs = _dev(inputs, torch.int32)
+    batch_size, length = inputs.shape
+    inputs_np = inputs.cpu().numpy()
+
+    max_decode_len = np.full((batch_size,), length, np.int32)
+    if max_decode_steps is not None:  # :438-455
+      if np.ndim(max_decode_steps) == 0 and max_decode_steps > length:
+        raise ValueError('Cannot decode more steps than the sequence length.')
+      max_decode_len = np.minimum(
+          length, np.sum(inputs_np != 0, axis=1) + max_decode_steps).astype(
+              np.int32)
+
+    sequences_np = np.concatenate(
+        [inputs_np, np.zeros((batch_size, 2), np.int32)], axis=1)  # :465-470
+    if initial_index is None:
+      i0 = np.zeros((batch_size,), np.int32)
+      token0 = np.zeros((batch_size,), np.int32)
+    else:
+      i0 = _dev(initial_index).cpu().numpy().astype(np.int32)
+      token0 = np.take_along_axis(sequences_np, i0[:, None], axis=1)[:, 0]
+    initial_eos = np.sum(sequences_np == eos_id, axis=-1).astype(np.int32)
+
+    temps = np.asarray(temperature, dtype=np.float32)
+    if temps.ndim == 1:  # per-item temperatures (:595-612)
+      temps = np.repeat(temps, num_decodes)
+    else:
+      temps = np.full((batch_size,), float(temps), np.float32)
+    self.any_sampling = bool(np.any(temps > np.float32(MIN_TEMPERATURE)))
+
+    self.tokens_to_logits, self.cache = tokens_to_logits, cache
+    self.eos_id, self.topk, self.topp = eos_id, topk, topp
+    self.rescale_log_probs = rescale_log_probs
+    self.state_callback_fn = state_callback_fn
+    self.logit_callback_fn = logit_callback_fn
+    self.sequences = torch.as_tensor(sequences_np, device=dev).contiguous()
+    self.cur_index = torch.as_tensor(i0, device=dev)
+    self.cur_token = torch.as_tensor(token0.astype(np.int32), device=dev)
+    self.ended = torch.zeros((batch_size,), dtype=torch.uint8, device=dev)
+    self.log_prob = torch.zeros((batch_size,), dtype=torch.float32, device=dev)
+    self.mdl = torch.as_tensor(max_decode_len, device=dev)
+    self.eos0 = torch.as_tensor(initial_eos, device=dev)
+    self.temps_dev = torch.as_tensor(temps, device=dev)
+    self.all_ended = torch.zeros((), dtype=torch.int32, device=dev)
+    self.tokens = torch.empty((batch_size,), dtype=torch.int32, device=dev)
+    self.tok_lp = torch.empty((batch_size,), dtype=torch.float32, device=dev)
+    self.source = _noise_source(prng_key)
+    self.step = 0
+    self.fused = None
+    if use_fused:
+      self.fused = tokens_to_logits.fused_sample_step(
+          sequences=self.sequences, cur_index=self.cur_index,
+          cur_token=self.cur_token, ended=self.ended, log_prob=self.log_prob,
+          max_decode_len=self.mdl, initial_eos_count=self.eos0,
+          temperature=self.temps_dev, all_ended=self.all_ended, eos_id=eos_id,
+          topk=topk, topp=topp, rescale=rescale_log_probs,
+          noise_source=self.source if self.any_sampling else None)
+
+  def _loop_state(self):
+    return SamplingLoopState(
+        torch.tensor(self.step, dtype=torch.int32), self.cur_index,
+        self.sequences, self.cache, self.cur_token[:, None],
+        self.ended.bool()[:, None], _Key(self.source, self.step),
+        self.log_prob)
+
+  def cond(self) -> bool:
+    """:509-515, not every row ended (reads one flag back)."""
+    if self.fused is not None:
+      return self.fused.running()
+    return not bool(self.all_ended.item())
+
+  def body(self):
+    """:517-700."""
+    if self.fused is not None:
+      self.fused.advance(1)
+      self.step += 1
+      return
+    if self.state_callback_fn is not None:
+      st = self.state_callback_fn(self._loop_state())
+      self.sequences = _dev(st.sequences, torch.int32).contiguous()
+      self.cur_index = _dev(st.cur_index, torch.int32).contiguous()
+      self.cache = st.cache
+    decoding_state = DecodingState(cur_index=self.cur_index,
+                                   sequences=self.sequences[:, :-2],
+                                   cur_token=self.cur_token[:, None],
+                                   cache=self.cache)
+    logits, self.cache = self.tokens_to_logits(decoding_state)
+    if self.logit_callback_fn is not None:
+      if not isinstance(logits, torch.Tensor):
+        logits = np.array(logits, dtype=np.float32)
+      logits = self.logit_callback_fn(logits, self._loop_state())
+    logits = _dev(logits, torch.float32).contiguous()
+    gumbel = None
+    if self.any_sampling:
+      gumbel = _dev(self.source.noise(self.step, tuple(logits.shape)),
+                    torch.float32).contiguous()
+    ops.sample_tokens(logits, gumbel, self.temps_dev, self.topk, self.topp,
+                      self.rescale_log_probs, self.tokens, self.tok_lp)
+    ops.sample_update(self.tokens, self.tok_lp, self.sequences, self.cur_index,
+                      self.cur_token, self.ended, self.log_prob, self.mdl,
+                      self.eos0, self.all_ended, self.eos_id)
+    self.step += 1
+
+  def advance(self, n: int):
+    if self.fused is not None:
+      self.fused.advance(n)
+      self.step += n
+      return
+    for _ in range(n):
+      self.body()
+
+  def run(self):
+    if self.fused is not None:
+      self.step = self.fused.run()
+      return
+    while True:  # nothing has ended at step 0
+      self.body()
+      if not self.cond():
+        break
+
+  def finish(self):
+    if self.fused is not None:
+      self.fused.finish()
+      # the context's buffers serve the next call too: hand out copies
+      return (self.fused.sequences[:, 1:-1].clone(),
+              self.fused.log_prob.clone())
+    if self.state_callback_fn is not None:
+      st = self.state_callback_fn(self._loop_state())
+      self.sequences = _dev(st.sequences, torch.int32)
+    return self.sequences[:, 1:-1], self.log_prob
+
+
 def _temperature_sample_single_trial(
     inputs, cache, tokens_to_logits, eos_id: int, prng_key,
     num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
@@ -342,100 +521,12 @@ def _temperature_sample_single_trial(
     use_fused: bool = False,
 ):
   """:412-715."""
-  if topp and topk:
-    raise ValueError('At most one of `topp` or `topk` may be non-zero.')
-  dev = _device()
-  inputs = _dev(inputs, torch.int32)
-  batch_size, length = inputs.shape
-  inputs_np = inputs.cpu().numpy()
-
-  max_decode_len = np.full((batch_size,), length, np.int32)
-  if max_decode_steps is not None:  # :438-455
-    if np.ndim(max_decode_steps) == 0 and max_decode_steps > length:
-      raise ValueError('Cannot decode more steps than the sequence length.')
-    max_decode_len = np.minimum(
-        length, np.sum(inputs_np != 0, axis=1) + max_decode_steps).astype(
-            np.int32)
-
-  sequences_np = np.concatenate(
-      [inputs_np, np.zeros((batch_size, 2), np.int32)], axis=1)  # :465-470
-  if initial_index is None:
-    i0 = np.zeros((batch_size,), np.int32)
-    token0 = np.zeros((batch_size,), np.int32)
-  else:
-    i0 = _dev(initial_index).cpu().numpy().astype(np.int32)
-    token0 = np.take_along_axis(sequences_np, i0[:, None], axis=1)[:, 0]
-  initial_eos = np.sum(sequences_np == eos_id, axis=-1).astype(np.int32)
-
-  temps = np.asarray(temperature, dtype=np.float32)
-  if temps.ndim == 1:  # per-item temperatures (:595-612)
-    temps = np.repeat(temps, num_decodes)
-  else:
-    temps = np.full((batch_size,), float(temps), np.float32)
-  any_sampling = bool(np.any(temps > np.float32(MIN_TEMPERATURE)))
-
-  sequences = torch.as_tensor(sequences_np, device=dev).contiguous()
-  cur_index = torch.as_tensor(i0, device=dev)
-  cur_token = torch.as_tensor(token0.astype(np.int32), device=dev)
-  ended = torch.zeros((batch_size,), dtype=torch.uint8, device=dev)
-  log_prob = torch.zeros((batch_size,), dtype=torch.float32, device=dev)
-  mdl = torch.as_tensor(max_decode_len, device=dev)
-  eos0 = torch.as_tensor(initial_eos, device=dev)
-  temps_dev = torch.as_tensor(temps, device=dev)
-  all_ended = torch.zeros((), dtype=torch.int32, device=dev)
-  tokens = torch.empty((batch_size,), dtype=torch.int32, device=dev)
-  tok_lp = torch.empty((batch_size,), dtype=torch.float32, device=dev)
-  source = _noise_source(prng_key)
-  step = 0
-
-  if use_fused:
-    fused = tokens_to_logits.fused_sample_step(
-        sequences=sequences, cur_index=cur_index, cur_token=cur_token,
-        ended=ended, log_prob=log_prob, max_decode_len=mdl,
-        initial_eos_count=eos0, temperature=temps_dev, all_ended=all_ended,
-        eos_id=eos_id, topk=topk, topp=topp, rescale=rescale_log_probs,
-        noise_source=source if any_sampling else None)
-    fused.run()
-    # the context's buffers serve the next call too: hand out copies
-    return fused.sequences[:, 1:-1].clone(), fused.log_prob.clone()
-
-  def loop_state():
-    return SamplingLoopState(
-        torch.tensor(step, dtype=torch.int32), cur_index, sequences, cache,
-        cur_token[:, None], ended.bool()[:, None], _Key(source, step),
-        log_prob)
-
-  while True:  # cond: not all ended (:509-515); nothing has ended at step 0
-    if state_callback_fn is not None:
-      st = state_callback_fn(loop_state())
-      sequences = _dev(st.sequences, torch.int32).contiguous()
-      cur_index = _dev(st.cur_index, torch.int32).contiguous()
-      cache = st.cache
-    decoding_state = DecodingState(cur_index=cur_index,
-                                   sequences=sequences[:, :-2],
-                                   cur_token=cur_token[:, None], cache=cache)
-    logits, cache = tokens_to_logits(decoding_state)
-    if logit_callback_fn is not None:
-      if not isinstance(logits, torch.Tensor):
-        logits = np.array(logits, dtype=np.float32)
-      logits = logit_callback_fn(logits, loop_state())
-    logits = _dev(logits, torch.float32).contiguous()
-    gumbel = None
-    if any_sampling:
-      gumbel = _dev(source.noise(step, tuple(logits.shape)),
-                    torch.float32).contiguous()
-    ops.sample_tokens(logits, gumbel, temps_dev, topk, topp,
-                      rescale_log_probs, tokens, tok_lp)
-    ops.sample_update(tokens, tok_lp, sequences, cur_index, cur_token, ended,
-                      log_prob, mdl, eos0, all_ended, eos_id)
-    step += 1
-    if int(all_ended.item()):
-      break
-
-  if state_callback_fn is not None:
-    st = state_callback_fn(loop_state())
-    sequences = _dev(st.sequences, torch.int32)
-  return sequences[:, 1:-1], log_prob
+  loop = SampleLoop(inputs, cache, tokens_to_logits, eos_id, prng_key,
+                    num_decodes, temperature, topk, topp, initial_index,
+                    max_decode_steps, rescale_log_probs, state_callback_fn,
+                    logit_callback_fn, use_fused)
+  loop.run()
+  return loop.finish()
 
 
 # ------------------------------------------------------------------------------
@@ -546,6 +637,9 @@ class BeamLoop:
     use_fused = (factory is not None and initial_index is None and
                  getattr(cache, 'fresh', False))
     self.fused = None
+    if not use_fused:
+      _check_cache_room(cache, max_decode_len - 1,
+                        expect_empty=initial_index is None)
     self.cur, self._beam_cache = beam_init(
         batch_size, beam_size, max_decode_len, {} if use_fused else cache,
         cache_offset, live_seqs=live_seqs, initial_index=initial_index_np)
@@ -569,6 +663,7 @@ class BeamLoop:
     if use_fused:
       self.fused = factory(self)
       if self.fused is None:  # configuration not covered: generic path
+        _check_cache_room(cache, max_decode_len - 1, expect_empty=True)
         self.cur, self._beam_cache = beam_init(
             batch_size, beam_size, max_decode_len, cache, cache_offset)
         self.nxt = ops.BeamBuffers(batch_size, beam_size, max_decode_len, dev)

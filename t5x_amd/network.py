@@ -90,10 +90,15 @@ def relative_position_bucket(relative_position, bidirectional=True,
 
 
 class FreshCache(dict):
-  """The zero cache as returned by cache initialisation.  The marker lets a
-  decode loop that owns its (beam-expanded) caches skip expanding this one;
-  any tree derived from it through cache_map is a plain dict again."""
-  fresh = True
+  """The zero cache as returned by cache initialisation.  While `fresh` is set
+  a decode loop that owns its (beam-expanded) caches may skip expanding this
+  one and start from zero caches of its own; the first decode step that writes
+  into the tree clears the flag, and any tree derived from it through
+  cache_map is a plain dict."""
+
+  def __init__(self, *args, **kw):
+    super().__init__(*args, **kw)
+    self.fresh = True
 
 
 class BeamShared:
@@ -435,6 +440,8 @@ class Transformer:
     cfg, dev = self.config, self._dev()
     w = self.decoder_weights(variables['params'])
     cache = variables['cache']
+    if getattr(cache, 'fresh', False):
+      cache.fresh = False  # this step writes into it
     if isinstance(encoded, BeamShared):
       beams, enc = encoded.beams, encoded.x
       enc_tok = encoder_input_tokens.x
@@ -698,24 +705,46 @@ class FusedSampleStep:
       self.keep_going.fill_(1)
     self.stream.synchronize()
 
-  def run(self):
-    """Runs the loop to its end (every row ended)."""
+  def advance(self, n):
+    """Enqueues n more iterations (fewer when the longest row ends sooner),
+    refilling the noise ring for each group of `ring` steps; the host waits
+    for a group only when it has to overwrite its noise."""
     lib = self._lib
     with torch.cuda.stream(self.stream):
-      while self.step < self.max_steps:
-        n = min(self.ring, self.max_steps - self.step)
+      todo = min(int(n), self.max_steps - self.step)
+      while todo > 0:
+        # up to the next multiple of `ring`: a refill never overwrites noise
+        # of a step that is enqueued but not yet executed
+        m = min(todo, self.ring - self.step % self.ring)
         if self.noise is not None:
-          for step in range(self.step, self.step + n):
+          if self.step % self.ring == 0:
+            self.stream.synchronize()
+          for step in range(self.step, self.step + m):
             g = self.noise_source.noise(step, tuple(self.noise.shape[1:]))
             self.noise[step % self.ring].copy_(
                 torch.as_tensor(g, device=self.device).to(torch.float32))
-        for _ in range(n):
+        for _ in range(m):
           lib.call('t5d_graph_launch', self.graph, self.stream.cuda_stream)
-        self.step += n
-        self.stream.synchronize()
-        if int(self.all_ended.item()):
-          break
+        self.step += m
+        todo -= m
+
+  def running(self) -> bool:
+    """The loop condition (not every row ended), read back from the device."""
+    self.stream.synchronize()
+    return not bool(self.all_ended.item())
+
+  def finish(self):
+    self.stream.synchronize()
     torch.cuda.current_stream().wait_stream(self.stream)
+
+  def run(self):
+    """Runs the loop to its end (every row ended); returns the number of
+    iterations executed."""
+    while self.step < self.max_steps:
+      self.advance(self.ring - self.step % self.ring)
+      if not self.running():
+        break
+    self.finish()
     return int(self.step_count.item())
 
   def cache_tree(self):

@@ -362,6 +362,43 @@ def test_self_attention_step(ops, dt, R, H, L, t):
   np.testing.assert_allclose(host(out), want, atol=TOL[dt], rtol=TOL[dt])
 
 
+@pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('R,H,L,over', [(2, 3, 32, 0), (3, 2, 128, 5),
+                                        (2, 2, 256, 1000)])
+def test_self_attention_step_past_the_cache_end(ops, dt, R, H, L, over):
+  """cache_index >= L (a decode loop longer than its cache): the kernels must
+  not turn the index into an address.  Like the reference's one-hot insert and
+  clamped bias slice (layers.py:258-303) they insert nothing, leave the caches
+  as they are and attend to all L columns with the bias row of position L-1."""
+  from t5x_amd import network
+  rs = np.random.RandomState(R + L + over)
+  D, t = 64, L + over
+  od = oracle_dtype(dt)
+  ck = ot5.cast(rs.randn(R, H, D, L).astype(np.float32), od)
+  cv = ot5.cast(rs.randn(R, H, D, L).astype(np.float32), od)
+  qkv = ot5.cast(rs.randn(R, 3 * H * D).astype(np.float32) *
+                 np.concatenate([np.full(H * D, 0.125), np.ones(2 * H * D)]),
+                 od)
+  rel_emb = rs.randn(H, 32).astype(np.float32)
+  want, new = _self_attn_oracle(qkv, ck, cv, rel_emb, t, od)
+  np.testing.assert_array_equal(new['cached_key'], ck)  # nothing inserted
+
+  bucket = network.relative_position_bucket(-np.arange(L), bidirectional=False)
+  rel_bias = dev(ot5.cast(rel_emb, od)[:, bucket], dt)
+  # guard bytes behind both caches: an insert at column t would land there
+  guard = 2 * D * (over + 1) + 64
+  flat_k = torch.zeros(ck.size + guard, dtype=dt, device='cuda')
+  flat_v = torch.zeros(cv.size + guard, dtype=dt, device='cuda')
+  ck_d = flat_k[:ck.size].view(R, H, D, L).copy_(dev(ck, dt))
+  cv_d = flat_v[:cv.size].view(R, H, D, L).copy_(dev(cv, dt))
+  out = ops.self_attention_step(dev(qkv, dt), ck_d, cv_d, rel_bias,
+                                dev(np.array(t, np.int32)))
+  np.testing.assert_array_equal(host(ck_d), ck)
+  np.testing.assert_array_equal(host(cv_d), cv)
+  assert not bool(flat_k[ck.size:].any()) and not bool(flat_v[cv.size:].any())
+  np.testing.assert_allclose(host(out), want, atol=TOL[dt], rtol=TOL[dt])
+
+
 @pytest.mark.parametrize('B,beams,H,L,t', [(3, 4, 2, 128, 0), (3, 4, 2, 128, 1),
                                            (3, 4, 3, 128, 77),
                                            (2, 4, 2, 128, 127),

@@ -739,3 +739,43 @@ def test_predict_batch_with_decoder_prompts_float32_exact(decode_fn_name, kw):
   flat = host(got).reshape(4, -1, 12)
   for i, n in enumerate((0, 3, 5, 1)):
     assert (flat[i, :, :n] == dec[i, 1:1 + n]).all()
+
+
+def test_decode_loop_longer_than_its_cache_raises():
+  """A loop that would run past the end of the cache is refused on the host
+  (the kernels themselves only stay memory-safe there)."""
+  from t5x_amd import decoding
+  B, K, L = 2, 2, 16
+  module, fn = _decode_setup('bfloat16', B, K, 16, L, seed=3)
+  inputs = np.zeros((B, L), np.int32)
+  short = dict(module.init_cache(B, 8))  # a plain dict: the generic loops
+  with pytest.raises(ValueError, match='holds 8 positions'):
+    decoding.beam_search(inputs, short, fn, 1, num_decodes=K)
+  with pytest.raises(ValueError, match='holds 16 positions'):
+    decoding.beam_search(inputs, dict(module.init_cache(B, L)), fn, 1,
+                         num_decodes=K, max_decode_len=40)
+  with pytest.raises(ValueError, match='holds 8 positions'):
+    decoding.temperature_sample(inputs, short, fn, 1, temperature=0.0)
+
+
+def test_used_cache_is_not_taken_for_a_fresh_one():
+  """A cache that a decode step has written into is no longer `fresh`: the
+  fused loops (which start from zero caches of their own) must not take it,
+  and the generic loops refuse to restart a decode on top of it."""
+  from t5x_amd import decoding
+  B, K, L = 2, 1, 8
+  module, fn = _decode_setup('float32', B, K, 16, L, seed=5)
+  cache = module.init_cache(B, L)
+  assert cache.fresh
+  state = decoding.DecodingState(
+      cur_index=torch.zeros((), dtype=torch.int32, device='cuda'),
+      sequences=torch.zeros((B, L), dtype=torch.int32, device='cuda'),
+      cur_token=torch.zeros((B, 1), dtype=torch.int32, device='cuda'),
+      cache=cache)
+  _, new_cache = fn(state)
+  assert new_cache is cache and not cache.fresh
+  inputs = np.zeros((B, L), np.int32)
+  with pytest.raises(ValueError, match='already holds decode steps'):
+    decoding.temperature_sample(inputs, cache, fn, 1, temperature=0.0)
+  with pytest.raises(ValueError, match='already holds decode steps'):
+    decoding.beam_search(inputs, cache, fn, 1, num_decodes=1)

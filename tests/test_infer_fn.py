@@ -122,3 +122,22 @@ def test_structured_inferences_keep_their_structure_per_example():
 def test_unsized_dataset_raises_like_the_reference():
   with pytest.raises(TypeError, match='dataset length is unknown.'):
     infer.get_infer_fn(lambda p, b: b, 2)(iter(_dataset(4)), None)
+
+
+def test_cache_room_check_on_host_tensors():
+  """decoding._check_cache_room looks only at shapes and cache_index values,
+  so it can be exercised without a GPU."""
+  import pytest
+  import torch
+  from t5x_amd import decoding
+  mk = lambda L, idx: {'decoder': {'layers_0': {'self_attention': {
+      'cached_key': torch.zeros((2, 1, 64, L)),
+      'cached_value': torch.zeros((2, 1, 64, L)),
+      'cache_index': torch.tensor(idx, dtype=torch.int32)}}}}
+  decoding._check_cache_room(mk(16, 0), 16, expect_empty=True)
+  decoding._check_cache_room(mk(16, 5), 16, expect_empty=False)
+  decoding._check_cache_room({}, 16, expect_empty=True)
+  with pytest.raises(ValueError, match='holds 16 positions'):
+    decoding._check_cache_room(mk(16, 0), 17, expect_empty=True)
+  with pytest.raises(ValueError, match='already holds decode steps'):
+    decoding._check_cache_room(mk(16, 5), 16, expect_empty=True)
