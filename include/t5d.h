@@ -278,6 +278,23 @@ int t5d_beam_topk(void* stream, const float* logits,
                   int32_t* topk_idx, float* row_max, float* row_lse,
                   void* scratch, int B, int beams, int V, int k);
 
+/* t5d_beam_topk without the `scratch` argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  This entry point has no counterpart in
+ * the reference.  The per-row candidates live in an array built into the
+ * library (128 KiB on every GPU the library runs on, held until the process
+ * ends), so B * beams * k must not exceed 16384; larger calls return
+ * T5D_ELIMIT.  It calls no hipMalloc / hipFree.  The first call on a device
+ * looks the array's address up (not a stream operation; make that call
+ * outside a graph capture).  All calls on one GPU share the array: calls that
+ * overlap on one GPU (different streams) race; the array keeps the previous
+ * call's contents and every call overwrites the part it reads.
+ * Results are bit-identical to t5d_beam_topk. */
+int t5d_beam_topk_static(void* stream, const float* logits,
+                         const float* live_logprobs, float* topk_vals,
+                         int32_t* topk_idx, float* row_max, float* row_lse,
+                         int B, int beams, int V, int k);
+
 /* State of one beam search (t5x/decoding.py:1002-1021), device arrays. */
 typedef struct {
   int32_t* cur_index;        /* scalar */

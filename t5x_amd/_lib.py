@@ -121,6 +121,8 @@ _SIGNATURES = {
     't5d_top_k': (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
     't5d_beam_topk': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int,
                               c_int, c_int]),
+    't5d_beam_topk_static': (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int,
+                                     c_int, c_int]),
     't5d_beam_update': (c_int, [_P, POINTER(BeamStatePtrs),
                                 POINTER(BeamStatePtrs), _P, _P, _P, _P, _P, _P,
                                 c_int, c_int, c_int, c_int, c_int, c_int]),

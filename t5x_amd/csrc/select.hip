@@ -7,6 +7,8 @@
 // rule, so results do not depend on how the work is split over lanes.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace t5d {
@@ -1426,6 +1428,57 @@ extern "C" int t5d_beam_topk(void* stream, const float* logits,
                      cand_idx, topk_vals, topk_idx, beams, k, tls_gate);
   T5D_CHECK_LAUNCH("t5d_beam_topk(merge)");
   return T5D_OK;
+}
+
+// ---- t5d_beam_topk for callers that cannot allocate ---------------------------
+// The per-row candidates (what t5d_beam_topk keeps in its `scratch` argument)
+// live in a file-scope device array instead.  Every GPU the library runs on
+// holds its own copy of the array at its own address; the address is looked up
+// once per device, with that device current, and kept.  The array's name is
+// only a host-side handle: kernels get the looked-up pointer.
+constexpr int kStaticCandPairs = 16384;  // rows * k candidates at most
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char
+    g_topk_scratch[2 * kStaticCandPairs * 4];
+static void* g_topk_scratch_ptr[kMaxDevices];
+static std::mutex g_topk_scratch_mutex;
+
+static int static_topk_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  T5D_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, T5D_EHIP,
+              "t5d_beam_topk_static: hipGetDevice: %s (device %d)",
+              hipGetErrorString(e), dev);
+  std::lock_guard<std::mutex> lock(g_topk_scratch_mutex);
+  if (g_topk_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_topk_scratch));
+    T5D_REQUIRE(e == hipSuccess && p != nullptr, T5D_EHIP,
+                "t5d_beam_topk_static: hipGetSymbolAddress: %s",
+                hipGetErrorString(e));
+    g_topk_scratch_ptr[dev] = p;
+  }
+  *out = g_topk_scratch_ptr[dev];
+  return T5D_OK;
+}
+
+extern "C" int t5d_beam_topk_static(void* stream, const float* logits,
+                                    const float* live_logprobs,
+                                    float* topk_vals, int32_t* topk_idx,
+                                    float* row_max, float* row_lse, int B,
+                                    int beams, int V, int k) {
+  T5D_REQUIRE(B > 0 && beams > 0 && k > 0, T5D_EINVAL,
+              "t5d_beam_topk_static: B=%d beams=%d k=%d", B, beams, k);
+  T5D_REQUIRE((int64_t)B * beams * k <= kStaticCandPairs, T5D_ELIMIT,
+              "t5d_beam_topk_static: B*beams*k = %lld candidates exceed the "
+              "built-in workspace of %d; use t5d_beam_topk with a workspace of "
+              "your own",
+              (long long)B * beams * k, kStaticCandPairs);
+  void* scratch = nullptr;
+  int rc = static_topk_scratch(&scratch);
+  if (rc) return rc;
+  return t5d_beam_topk(stream, logits, live_logprobs, topk_vals, topk_idx,
+                       row_max, row_lse, scratch, B, beams, V, k);
 }
 
 static int check_state(const char* name, const t5d_beam_state* st) {
