@@ -62,8 +62,11 @@ class PackedWeight:
 
 
 def _quantize(w):
-  """Per-output-channel symmetric int8 (scale = max|w| / 127)."""
-  scale = w.abs().amax(dim=0).clamp_min(1e-30) / 127.0
+  """Per-output-channel symmetric int8 (scale = max|w| / 127).  The divisor is
+  a tensor: dividing by a Python scalar multiplies by its rounded reciprocal,
+  which moves some scales by an ulp and with them a few weights by one step."""
+  amax = w.abs().amax(dim=0).clamp_min(1e-30)
+  scale = amax / torch.full_like(amax, 127.0)
   q = torch.clamp(torch.round(w / scale), -127, 127).to(torch.int8)
   return q, scale.to(torch.float32)
 

@@ -254,52 +254,80 @@ def test_predict_batch_mock_module_and_rng_rules():
       "`decoder_params['decode_rng']` (3). Please specify one or the other.")
 
 
-def _step_at_width(name, emb, heads, mlp, B, K, E, Emin, L, t,
-                   weight_dtype=None):
-  """One decode step of a 2-layer decoder at a real model width, in the middle
-  of a decode (position t): caches are pre-filled with the same random prefix
-  on both sides."""
+def step_at_width(emb, heads, mlp, B, K, E, Emin, L, t, weight_dtype=None,
+                  layers=2, round_weights=False, truth=False):
+  """One decode step of a `layers`-deep decoder at a real model width, in the
+  middle of a decode (position t): caches are pre-filled with the same random
+  prefix on both sides.  Returns (hip logits, oracle logits[, truth logits])
+  as [R, V] float32 arrays.
+
+  round_weights: every parameter is rounded to bfloat16 first, so that all
+  sides multiply by exactly the same numbers (the oracle keeps the logits
+  layer's kernel in float32 otherwise, as the reference does).
+  truth: also run the oracle with float32 activations on those parameters."""
   from t5x_amd import network
   kw = dict(vocab_size=32128, dtype='bfloat16', emb_dim=emb, num_heads=heads,
-            num_encoder_layers=0, num_decoder_layers=2, head_dim=64,
+            num_encoder_layers=0, num_decoder_layers=layers, head_dim=64,
             mlp_dim=mlp)
   ocfg = ot5.T5Config(**kw)
   cfg = network.T5Config(weight_dtype=weight_dtype, **kw)
   params = ot5.init_params(ocfg, seed=11, with_encoder=False)
+  if round_weights:
+    def rounded(node):
+      if isinstance(node, dict):
+        return {k: rounded(v) for k, v in node.items()}
+      return ot5.bf16_round(node)
+    params = rounded(params)
   oparams = quantized_tree(params) if weight_dtype == 'int8' else params
   rs = np.random.RandomState(3)
   R = B * K
   enc_tok = ragged_tokens(rs, B, E, 32128, Emin)
   encoded = ot5.bf16_round(rs.randn(B, E, emb).astype(np.float32))
-  ocache = ot5.init_cache(ocfg, R, L)
-  for lyr in ocache['decoder'].values():
-    sa = lyr['self_attention']
-    for n in ('cached_key', 'cached_value'):
-      sa[n][..., :t] = ot5.bf16_round(
-          rs.randn(R, heads, 64, t).astype(np.float32))
-    sa['cache_index'] = np.array(t, np.int32)
+  prefix = [[ot5.bf16_round(rs.randn(R, heads, 64, t).astype(np.float32))
+             for _ in range(2)] for _ in range(layers)]
+  tok = rs.randint(2, 32128, size=(R, 1)).astype(np.int32)
+
+  def oracle(cfg_):
+    cache = ot5.init_cache(cfg_, R, L)
+    for i in range(layers):
+      sa = cache['decoder'][f'layers_{i}']['self_attention']
+      sa['cached_key'][..., :t] = prefix[i][0]
+      sa['cached_value'][..., :t] = prefix[i][1]
+      sa['cache_index'] = np.array(t, np.int32)
+    cross_kv = ot5.project_cross_kv(oparams, cfg_, encoded)
+    cross_kv = [(np.repeat(k, K, 0), np.repeat(v, K, 0)) for k, v in cross_kv]
+    out, _ = ot5.decode(oparams, cfg_, None, np.repeat(enc_tok, K, axis=0),
+                        tok, tok, decode=True, cache=cache,
+                        max_decode_length=L, cross_kv=cross_kv)
+    return out[:, 0]
+
+  want = oracle(ocfg)
   module = network.Transformer(cfg)
   gcache = module.init_cache(R, L)
-  for lname, lyr in gcache['decoder'].items():
-    sa, osa = lyr['self_attention'], ocache['decoder'][lname]['self_attention']
-    for n in ('cached_key', 'cached_value'):
-      sa[n][..., :L].copy_(torch.as_tensor(osa[n]).to(torch.bfloat16))
+  for i in range(layers):
+    sa = gcache['decoder'][f'layers_{i}']['self_attention']
+    for n, src in zip(('cached_key', 'cached_value'), prefix[i]):
+      sa[n][..., :t].copy_(torch.as_tensor(src).to(torch.bfloat16))
     sa['cache_index'].fill_(t)
-  tok = rs.randint(2, 32128, size=(R, 1)).astype(np.int32)
-  cross_kv = ot5.project_cross_kv(oparams, ocfg, encoded)
-  cross_kv = [(np.repeat(k, K, 0), np.repeat(v, K, 0)) for k, v in cross_kv]
-  want, _ = ot5.decode(oparams, ocfg, None, np.repeat(enc_tok, K, axis=0), tok,
-                       tok, decode=True, cache=ocache, max_decode_length=L,
-                       cross_kv=cross_kv)
   got = module.apply(
       {'params': params, 'cache': gcache},
       network.BeamShared(torch.as_tensor(encoded, device='cuda').bfloat16(), K),
       network.BeamShared(enc_tok, K), torch.as_tensor(tok, device='cuda'),
       None, decode=True, max_decode_length=L, method=module.decode)
-  err = np.abs(host(got)[:, 0] - want[:, 0])
+  got = host(got)[:, 0]
+  if truth:
+    return got, want, oracle(ot5.T5Config(**dict(kw, dtype='float32')))
+  return got, want
+
+
+def _step_at_width(name, emb, heads, mlp, B, K, E, Emin, L, t,
+                   weight_dtype=None, layers=2):
+  got, want = step_at_width(emb, heads, mlp, B, K, E, Emin, L, t, weight_dtype,
+                            layers)
+  err = np.abs(got - want)
   print(f'{name}-size step: max |dlogit| = {err.max():.3g}, mean '
         f'{err.mean():.3g}, p99.9 {np.quantile(err, 0.999):.3g}')
-  check_logits(host(got)[:, 0], want[:, 0], 'bfloat16', name)
+  check_logits(got, want, 'bfloat16', name)
 
 
 def test_decoder_step_at_base_size_matches_oracle():
