@@ -19,11 +19,16 @@ class Transformer:
   """network.Transformer (t5x/examples/t5/network.py:295-461) behind a
   flax-like `apply`."""
 
-  scan_layers = False
-
-  def __init__(self, config: t5.T5Config, hoist_cross_kv: bool = True):
+  def __init__(self, config: t5.T5Config, hoist_cross_kv: bool = True,
+               scan_layers: bool = False):
     self.config = config
     self.dtype = config.dtype
+    # t5x/examples/scalable_t5/network.py:324-352: with the decoder stack under
+    # a scan (variable_axes={'cache': 0}) every cache leaf carries a leading
+    # layer axis, [layers, batch, ...], under one 'decoder' scope, and
+    # t5x/models.py:739-748 then decodes with cache_offset=1.  The layer
+    # arithmetic is unchanged; only the cache tree's layout differs.
+    self.scan_layers = scan_layers
     # Cross-attention K/V depend only on `encoded`; projecting them once per
     # batch is value-identical to the reference's per-step projection.
     self.hoist_cross_kv = hoist_cross_kv
@@ -62,11 +67,16 @@ class Transformer:
     del enable_dropout
     params = variables['params']
     if decode:
+      cache = variables['cache']
+      if self.scan_layers:
+        cache = _unstack_cache(cache, self.config.num_decoder_layers)
       logits, cache = t5.decode(
           params, self.config, encoded, encoder_input_tokens,
           decoder_input_tokens, decoder_target_tokens, decode=True,
-          cache=variables['cache'], max_decode_length=max_decode_length,
+          cache=cache, max_decode_length=max_decode_length,
           cross_kv=self._cross_kv(params, encoded))
+      if self.scan_layers:
+        cache = _stack_cache(cache, self.config.num_decoder_layers)
       return (logits, {'cache': cache}) if mutable else logits
     return t5.decode(params, self.config, encoded, encoder_input_tokens,
                      decoder_input_tokens, decoder_target_tokens)
@@ -77,12 +87,34 @@ class Transformer:
     if decode and 'cache' not in variables:
       # Cache-initialisation pass (t5x/models.py:542-552): only shapes matter.
       b, l = np.shape(decoder_input_tokens)
-      return None, {'cache': t5.init_cache(self.config, b, l)}
+      cache = t5.init_cache(self.config, b, l)
+      if self.scan_layers:
+        cache = _stack_cache(cache, self.config.num_decoder_layers)
+      return None, {'cache': cache}
     encoded = self._encode(variables, encoder_input_tokens)
     return self._decode(variables, encoded, encoder_input_tokens,
                         decoder_input_tokens, decoder_target_tokens,
                         enable_dropout=enable_dropout, decode=decode,
                         mutable=mutable)
+
+
+_CACHE_LEAVES = ('cached_key', 'cached_value', 'cache_index')
+
+
+def _stack_cache(cache, num_layers):
+  """Per-layer cache tree -> the scanned layout: one 'decoder' scope whose
+  leaves have a leading layer axis."""
+  per = [cache['decoder'][f'layers_{i}']['self_attention']
+         for i in range(num_layers)]
+  return {'decoder': {'decoder': {'self_attention': {
+      n: np.stack([np.asarray(p[n]) for p in per]) for n in _CACHE_LEAVES}}}}
+
+
+def _unstack_cache(cache, num_layers):
+  sa = cache['decoder']['decoder']['self_attention']
+  return {'decoder': {f'layers_{i}': {'self_attention': {
+      n: np.asarray(sa[n])[i] for n in _CACHE_LEAVES}}
+                      for i in range(num_layers)}}
 
 
 @dataclasses.dataclass

@@ -322,8 +322,8 @@ def temperature_sample(
   # cache must be the untouched zero cache, which is then not even expanded).
   use_fused = (getattr(tokens_to_logits, 'fused_sample_step', None) is not None
                and getattr(cache, 'fresh', False) and initial_index is None and
-               cache_offset == 0 and state_callback_fn is None and
-               logit_callback_fn is None)
+               cache_offset == getattr(tokens_to_logits, 'cache_offset', 0) and
+               state_callback_fn is None and logit_callback_fn is None)
   if not use_fused:
     _check_cache_room(cache, inputs.shape[1],
                       expect_empty=initial_index is None)

@@ -40,6 +40,8 @@ class StepFunction:
     self.encoded_inputs, self.raw_inputs = encoded_inputs, raw_inputs
     self.max_decode_length = max_decode_length
     module = model.module
+    # the beam / layer offset of the cache trees this step function works on
+    self.cache_offset = int(bool(getattr(module, 'scan_layers', False)))
     if hasattr(module, 'make_fused_beam_step'):
       self.fused_beam_step = lambda loop: module.make_fused_beam_step(
           loop, params, encoded_inputs, raw_inputs)

@@ -89,6 +89,20 @@ def relative_position_bucket(relative_position, bidirectional=True,
   return ret + np.where(is_small, n, val_if_large)
 
 
+def cache_tree(keys, values, index, scanned: bool):
+  """The cache tree of t5x/examples/t5/layers.py:231-244 over per-layer K/V
+  `keys[i]` / `values[i]` [rows, H, 64, L] and the int32 vector `index`
+  [layers]: one scope per layer, or (scanned) one 'decoder' scope with the
+  layer axis leading (t5x/examples/scalable_t5/network.py:324-352)."""
+  if scanned:
+    return {'decoder': {'decoder': {'self_attention': {
+        'cached_key': keys, 'cached_value': values, 'cache_index': index}}}}
+  return {'decoder': {
+      f'layers_{i}': {'self_attention': {
+          'cached_key': keys[i], 'cached_value': values[i],
+          'cache_index': index[i]}} for i in range(index.shape[0])}}
+
+
 class FreshCache(dict):
   """The zero cache as returned by cache initialisation.  While `fresh` is set
   a decode loop that owns its (beam-expanded) caches may skip expanding this
@@ -217,14 +231,20 @@ class Transformer:
   float32 leaves); it is cast/packed on first use and cached by identity.
   """
 
-  scan_layers = False
   # Batch slices a fused beam search steps on separate streams.  On MI355X
   # kernels of different streams do overlap, but the dispatch rate (about one
   # kernel per 1.5 us) is shared by all streams, and a decode step is bound by
   # its kernel count, so more lanes only add dispatches: 1 is fastest.
   decode_lanes = 1
 
-  def __init__(self, config: T5Config, device=None):
+  def __init__(self, config: T5Config, device=None, scan_layers: bool = False):
+    """scan_layers: hand out and accept the cache in the layout of a scanned
+    decoder stack (t5x/examples/scalable_t5/network.py:324-352): one 'decoder'
+    scope whose leaves carry a leading layer axis, [layers, rows, H, 64, L] and
+    cache_index [layers]; EncoderDecoderModel then decodes with
+    cache_offset=1 (t5x/models.py:739-748).  The parameter tree and the layer
+    arithmetic are the same."""
+    self.scan_layers = bool(scan_layers)
     if config.head_dim != 64:
       raise ValueError('the attention kernels are specialised for head_dim 64')
     if tuple(config.mlp_activations) != ('gelu', 'linear'):
@@ -287,15 +307,15 @@ class Transformer:
     # attended to (they lie beyond every cache_index).
     el = 16 // torch.empty((), dtype=act).element_size()
     length = (max_decode_length + el - 1) // el * el
-    kv = torch.zeros((cfg.num_decoder_layers, 2, batch, cfg.num_heads,
-                      cfg.head_dim, length), dtype=act, device=dev)
-    idx = torch.zeros((cfg.num_decoder_layers,), dtype=torch.int32, device=dev)
-    tree = FreshCache({'decoder': {
-        f'layers_{i}': {'self_attention': {
-            'cached_key': kv[i, 0], 'cached_value': kv[i, 1],
-            'cache_index': idx[i]}}
-        for i in range(cfg.num_decoder_layers)}})
-    return tree
+    nl = cfg.num_decoder_layers
+    idx = torch.zeros((nl,), dtype=torch.int32, device=dev)
+    if self.scan_layers:
+      kv = torch.zeros((2, nl, batch, cfg.num_heads, cfg.head_dim, length),
+                       dtype=act, device=dev)
+      return FreshCache(cache_tree(kv[0], kv[1], idx, True))
+    kv = torch.zeros((nl, 2, batch, cfg.num_heads, cfg.head_dim, length),
+                     dtype=act, device=dev)
+    return FreshCache(cache_tree(kv[:, 0], kv[:, 1], idx, False))
 
   def _call(self, variables, encoder_input_tokens, decoder_input_tokens,
             decoder_target_tokens, enable_dropout=False, decode=False,
@@ -463,8 +483,16 @@ class Transformer:
     b.ids.copy_(ids.reshape(R).to(torch.int32))
 
     layer_caches, index_leaves = [], []
+    scanned = 'decoder' in cache['decoder']
+    if scanned != self.scan_layers:
+      raise ValueError('cache tree layout (scanned layers or one scope per '
+                       'layer) does not match this module')
     for i in range(cfg.num_decoder_layers):
-      c = cache['decoder'][f'layers_{i}']['self_attention']
+      if scanned:
+        c = cache['decoder']['decoder']['self_attention']
+        c = {k: v[i] for k, v in c.items()}
+      else:
+        c = cache['decoder'][f'layers_{i}']['self_attention']
       ck, cv = c['cached_key'], c['cached_value']
       for t in (ck, cv):
         if (not t.is_contiguous() or t.dtype != w.act_dtype or
@@ -497,8 +525,11 @@ class Transformer:
     m = self._step_cache[1]
     _lib.call('t5d_decoder_step', _lib.stream_handle(), m, b.ids.data_ptr())
     if not consecutive:
-      for j, name in enumerate(cache['decoder']):
-        cache['decoder'][name]['self_attention']['cache_index'] = index_vec[j]
+      if scanned:
+        cache['decoder']['decoder']['self_attention']['cache_index'] = index_vec
+      else:
+        for j, name in enumerate(cache['decoder']):
+          cache['decoder'][name]['self_attention']['cache_index'] = index_vec[j]
     logits = b.logits.view(R, 1, cfg.vocab_size)
     return (logits, {'cache': cache}) if mutable else logits
 
@@ -509,7 +540,8 @@ class Transformer:
     object (caches, cross K/V buffers, state, captured graphs) is kept and
     re-bound to the next loop of the same shape and options, so a stream of
     batches pays for allocation and graph capture once."""
-    if not isinstance(encoded, BeamShared) or loop.cache_offset != 0:
+    if (not isinstance(encoded, BeamShared) or
+        loop.cache_offset != int(self.scan_layers)):
       return None
     if loop.beam_size > 8:
       return None
@@ -753,10 +785,9 @@ class FusedSampleStep:
     from t5x_amd import ops
     nl = self.kv.shape[0]
     value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return {'decoder': {
-        f'layers_{i}': {'self_attention': {
-            'cached_key': self.kv[i, 0], 'cached_value': value(self.kv[i, 1]),
-            'cache_index': self.cache_index[i]}} for i in range(nl)}}
+    return cache_tree(self.kv[:, 0],
+                      torch.stack([value(self.kv[i, 1]) for i in range(nl)]),
+                      self.cache_index, self.module.scan_layers)
 
   def __del__(self):
     try:
@@ -1079,10 +1110,9 @@ class FusedBeamStep:
     kv = torch.cat([lane.kv for lane in self.lanes], dim=2)
     idx = self.lanes[0].cache_index
     value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return {'decoder': {
-        f'layers_{i}': {'self_attention': {
-            'cached_key': kv[i, 0], 'cached_value': value(kv[i, 1]),
-            'cache_index': idx[i]}} for i in range(nl)}}
+    return cache_tree(kv[:, 0],
+                      torch.stack([value(kv[i, 1]) for i in range(nl)]), idx,
+                      self.module.scan_layers)
 
   def __del__(self):
     try:

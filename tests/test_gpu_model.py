@@ -350,7 +350,7 @@ def test_decoder_step_at_other_widths_matches_oracle(name, emb, heads, mlp, B,
   _step_at_width(name, emb, heads, mlp, B, K, E, Emin, L, t, wdt)
 
 
-def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
+def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0, scan_layers=False):
   """A step function over synthetic encoder output, as predict_batch builds
   it.  eos_bias > 0 scales up the logits column of EOS so decodes finish early."""
   from t5x_amd import decoding, models, network
@@ -359,7 +359,7 @@ def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0):
   params = network.init_params(gcfg, seed, dev, with_encoder=False)
   if eos_bias:
     params['decoder']['logits_dense']['kernel'][:, 1] *= eos_bias
-  module = network.Transformer(gcfg, dev)
+  module = network.Transformer(gcfg, dev, scan_layers=scan_layers)
   model = models.EncoderDecoderModel(module, decode_fn=decoding.beam_search)
   rs = np.random.RandomState(seed)
   tok = torch.as_tensor(ragged_tokens(rs, B, E, gcfg.vocab_size, 3), device=dev)
@@ -763,6 +763,10 @@ def test_predict_batch_with_decoder_prompts_float32_exact(decode_fn_name, kw):
                                         prompt_with_targets=True, **extra)
   np.testing.assert_array_equal(host(got), want)
   np.testing.assert_allclose(host(gaux['scores']), waux['scores'], atol=1e-4)
+  # forced prompts run on the graph-replay loops (their bookkeeping kernels
+  # read the prompt tokens), not on the kernel-per-call fallback: a decode
+  # context exists only when a fused loop was built
+  assert len(gm.module._beam_ctx) == 1
   # the forced prefix is reproduced in every returned decode
   flat = host(got).reshape(4, -1, 12)
   for i, n in enumerate((0, 3, 5, 1)):
@@ -807,3 +811,88 @@ def test_used_cache_is_not_taken_for_a_fresh_one():
     decoding.temperature_sample(inputs, cache, fn, 1, temperature=0.0)
   with pytest.raises(ValueError, match='already holds decode steps'):
     decoding.beam_search(inputs, cache, fn, 1, num_decodes=1)
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+@pytest.mark.parametrize('fn_name,kw', [
+    ('beam_search', dict(alpha=0.6)),
+    ('temperature_sample', dict(temperature=0.0)),
+    ('temperature_sample', dict(temperature=0.7, topk=20))])
+def test_predict_batch_with_a_scanned_layer_cache(dtype, fn_name, kw):
+  """The cache layout of a scanned decoder stack (leaves [layers, rows, ...]
+  under one scope, t5x/examples/scalable_t5/network.py:324-352) end to end:
+  predict_batch decodes with cache_offset=1 (t5x/models.py:739-748) on both
+  sides.  float32: tokens bit-exact."""
+  from t5x_amd import decoding, models, network
+  ocfg, cfg = tiny(dtype)
+  om = omodels.EncoderDecoderModel(
+      omodels.Transformer(ocfg, scan_layers=True),
+      decode_fn=functools.partial(getattr(odec, fn_name), **kw))
+  gm = models.EncoderDecoderModel(
+      network.Transformer(cfg, scan_layers=True),
+      decode_fn=functools.partial(getattr(decoding, fn_name), **kw))
+  assert gm.module.scan_layers and om.module.scan_layers
+  params = ot5.init_params(ocfg, seed=13)
+  rs = np.random.RandomState(6)
+  batch = {'encoder_input_tokens': ragged_tokens(rs, 3, 16, ocfg.vocab_size, 4),
+           'decoder_input_tokens': np.zeros((3, 10), np.int32)}
+  dp = lambda: ({'decode_rng': odec.GumbelNoise(seed=5)}
+                if fn_name == 'temperature_sample' else None)
+  want, waux = om.predict_batch_with_aux(params, batch, num_decodes=3,
+                                         return_all_decodes=True,
+                                         decoder_params=dp())
+  got, gaux = gm.predict_batch_with_aux(params, batch, num_decodes=3,
+                                        return_all_decodes=True,
+                                        decoder_params=dp())
+  got, gs = host(got), host(gaux['scores'])
+  if dtype == 'float32':
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_allclose(gs, waux['scores'], atol=1e-4)
+  else:
+    np.testing.assert_allclose(gs, waux['scores'], atol=10 * TOL[dtype])
+    assert (got == want).all(axis=-1).mean() >= 0.5
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_loops_on_a_scanned_layer_cache_generic_equals_fused(dtype):
+  """cache_offset=1 through both loop implementations: the kernel-per-call
+  loops expand, flatten and reorder [layers, batch, beams, ...] leaves; the
+  graph-replay loops own their caches and hand them out in that layout.  Same
+  sequences and scores, bit for bit, and the same caches."""
+  from t5x_amd import decoding
+  B, K, L = 3, 4, 12
+  module, fn = _decode_setup(dtype, B, K, 16, L, seed=17, scan_layers=True)
+  assert fn.cache_offset == 1
+  inputs = np.zeros((B, L), np.int32)
+  fresh = module.init_cache(B, L)
+  sa = fresh['decoder']['decoder']['self_attention']
+  assert sa['cached_key'].shape[:2] == (3, B) and sa['cache_index'].shape == (3,)
+
+  fused = decoding.BeamLoop(inputs, fresh, fn, 1, num_decodes=K, cache_offset=1)
+  plain = decoding.BeamLoop(inputs, dict(module.init_cache(B, L)), fn, 1,
+                            num_decodes=K, cache_offset=1)
+  assert fused.fused is not None and plain.fused is None
+  for step in range(L):
+    assert fused.cond() and plain.cond()
+    fused.body()
+    plain.body()
+  fc = fused.beam_cache['decoder']['decoder']['self_attention']
+  pc = plain.beam_cache['decoder']['decoder']['self_attention']
+  assert pc['cached_key'].shape[:3] == (3, B, K)
+  for which in ('cached_key', 'cached_value'):
+    a, b = fc[which], pc[which].reshape(3, B * K, *pc[which].shape[3:])
+    assert torch.equal(a[..., :L], b[..., :L]), which
+  assert torch.equal(fc['cache_index'].cpu(), pc['cache_index'].cpu())
+  got, gs = fused.finish()
+  want, ws = plain.finish()
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws))
+
+  noise = odec.GumbelNoise(seed=9)
+  a, la = decoding.temperature_sample(
+      inputs, module.init_cache(B, L), fn, 1, decode_rng=noise, num_decodes=K,
+      temperature=0.8, topk=10, cache_offset=1)
+  b, lb = decoding.temperature_sample(
+      inputs, dict(module.init_cache(B, L)), fn, 1, decode_rng=noise,
+      num_decodes=K, temperature=0.8, topk=10, cache_offset=1)
+  assert torch.equal(a, b) and torch.equal(la, lb)
