@@ -84,7 +84,7 @@ int t5d_embed(void* stream, int dtype, const void* table, const int32_t* ids,
 int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
                 void* out, int R, int d, float eps);
 
-/* Bias-free dense layer for M <= 128 rows (DenseGeneral,
+/* Bias-free dense layer for few rows (DenseGeneral,
  * t5x/examples/t5/layers.py:364-414; MlpBlock gate product :460-474; the
  * residual adds of t5x/examples/t5/network.py:146,163,177).
  *   A [M, K] act dtype; W packed (bf16 / int8, see t5d_pack_weight) or
@@ -93,6 +93,8 @@ int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
  *   out_dtype: dtype of C (T5D_F32 for the logits layer,
  *   t5x/examples/t5/network.py:286-291).
  *   T5D_EPI_GEGLU: W is a geglu-packed [K, 2F] kernel, N = 2F, C is [M, F].
+ *   The kernels are laid out for M <= 128 (the weights stream once); more rows
+ *   run as chunks of 128, each streaming the weights again.
  *   workspace/counters: reserved for kernel variants that need scratch
  *   memory; t5d_gemm_workspace_bytes currently returns 0 for every shape and
  *   both may be NULL. */

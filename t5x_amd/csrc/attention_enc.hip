@@ -113,7 +113,10 @@ enc_attn_kernel(EncAttnArgs a) {
     }
   };
 
-  float m = -INFINITY, l = 0.f;
+  // The running maximum starts at a finite floor: a lane whose 4 keys of the
+  // first tile all lie beyond E (E < 16) has only -inf scores, and
+  // exp(-inf - (-inf)) would poison its sum.
+  float m = -3.0e38f, l = 0.f;
   {
     FragE kcur[2], knext[2];
     load_k(0, kcur);

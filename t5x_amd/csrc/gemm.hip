@@ -892,6 +892,8 @@ static int tile_occupancy(int mp, int nt) {
   return acc == 8 && mp == 2 ? 3 : 2;
 }
 
+constexpr int kMaxRows = 128;  // rows one launch of the MFMA kernels covers
+
 static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
   const int mt_total = (M + 15) / 16;
   const int n_tiles = N / 16;
@@ -1038,29 +1040,37 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
                   (out_dtype == T5D_F32 && epilogue == T5D_EPI_NONE),
               T5D_EINVAL, "t5d_gemm: out_dtype %d with epilogue %d", out_dtype,
               epilogue);
-  T5D_REQUIRE(M <= 128, T5D_ELIMIT, "t5d_gemm: M=%d > 128 rows", M);
   T5D_REQUIRE(K % 32 == 0 && N % 16 == 0, T5D_EINVAL,
               "t5d_gemm: K=%d N=%d must tile 32x16", K, N);
   T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
               "t5d_gemm: A/W must be 16-byte aligned");
   (void)workspace; (void)counters;
-  GemmPlan p = plan_gemm(M, K, N, w_dtype == T5D_I8 ? 1 : 2);
-  GemmArgs g;
-  g.A = (const bf16_t*)A;
-  g.W = W;
-  g.scales = w_dtype == T5D_I8 ? scales : nullptr;
-  g.residual = residual;
-  g.C = C;
-  g.M = M; g.K = K; g.N = N;
-  g.m_parts = 1;
-  g.gate = tls_gate;
-  g.epilogue = epilogue;
-  g.out_f32 = out_dtype == T5D_F32;
-  g.norm_scale = nullptr;
-  g.eps = 0.f;
-  if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);
-  else launch_mfma<int8_t>(p, g, s);
-  T5D_CHECK_LAUNCH("t5d_gemm");
+  // The kernels cover up to kMaxRows rows; more rows go through in chunks
+  // (each streams the weights again: beyond a few hundred rows t5d_gemm_rows
+  // is the kernel to use).
+  const int n_out = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
+  const size_t out_elem = out_dtype == T5D_F32 ? 4 : 2;
+  for (int m0 = 0; m0 < M; m0 += kMaxRows) {
+    const int mc = min(kMaxRows, M - m0);
+    GemmPlan p = plan_gemm(mc, K, N, w_dtype == T5D_I8 ? 1 : 2);
+    GemmArgs g;
+    g.A = (const bf16_t*)A + (size_t)m0 * K;
+    g.W = W;
+    g.scales = w_dtype == T5D_I8 ? scales : nullptr;
+    g.residual = residual ? (const char*)residual + (size_t)m0 * n_out * 2
+                          : nullptr;
+    g.C = (char*)C + (size_t)m0 * n_out * out_elem;
+    g.M = mc; g.K = K; g.N = N;
+    g.m_parts = 1;
+    g.gate = tls_gate;
+    g.epilogue = epilogue;
+    g.out_f32 = out_dtype == T5D_F32;
+    g.norm_scale = nullptr;
+    g.eps = 0.f;
+    if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);
+    else launch_mfma<int8_t>(p, g, s);
+    T5D_CHECK_LAUNCH("t5d_gemm");
+  }
   return T5D_OK;
 }
 
@@ -1071,6 +1081,22 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
                              int epilogue) {
   T5D_REQUIRE(A && norm_scale && W && C, T5D_EINVAL,
               "t5d_norm_gemm: null pointer");
+  if (dtype == T5D_BF16 && M > kMaxRows) {
+    // in chunks of the rows the kernels cover (rows are independent)
+    T5D_REQUIRE(epilogue == T5D_EPI_NONE || epilogue == T5D_EPI_GEGLU,
+                T5D_EINVAL, "t5d_norm_gemm: epilogue %d (none or geglu)",
+                epilogue);
+    const int n_out = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
+    const size_t out_elem = out_dtype == T5D_F32 ? 4 : 2;
+    for (int m0 = 0; m0 < M; m0 += kMaxRows) {
+      const int rc = t5d_norm_gemm(
+          stream, dtype, w_dtype, out_dtype, (const char*)A + (size_t)m0 * K * 2,
+          norm_scale, eps, W, scales, (char*)C + (size_t)m0 * n_out * out_elem,
+          min(kMaxRows, M - m0), K, N, epilogue);
+      if (rc != T5D_OK) return rc;
+    }
+    return T5D_OK;
+  }
   if (dtype == T5D_F32) {
     T5D_REQUIRE(w_dtype == T5D_F32 && out_dtype == T5D_F32, T5D_EINVAL,
                 "t5d_norm_gemm: float32 activations need float32 weights / "
@@ -1101,7 +1127,7 @@ extern "C" int t5d_norm_gemm(void* stream, int dtype, int w_dtype,
               out_dtype, epilogue);
   T5D_REQUIRE(epilogue == T5D_EPI_NONE || epilogue == T5D_EPI_GEGLU, T5D_EINVAL,
               "t5d_norm_gemm: epilogue %d (none or geglu)", epilogue);
-  T5D_REQUIRE(M > 0 && M <= 128, T5D_ELIMIT, "t5d_norm_gemm: M=%d (1..128)", M);
+  T5D_REQUIRE(M > 0, T5D_EINVAL, "t5d_norm_gemm: M=%d", M);
   T5D_REQUIRE(K >= 64 && K % 64 == 0 && K <= 2048 && N > 0 && N % 16 == 0,
               T5D_ELIMIT,
               "t5d_norm_gemm: K=%d (multiple of 64, <= 2048), N=%d (multiple "

@@ -104,7 +104,9 @@ def _enc_attn_oracle(q, k, v, rel_emb, lens):
 
 
 @pytest.mark.parametrize('B,E,H', [(2, 16, 1), (3, 40, 2), (2, 100, 3),
-                                   (2, 512, 4), (1, 700, 2)])
+                                   (2, 512, 4), (1, 700, 2),
+                                   # shorter than one 16-key tile
+                                   (2, 4, 1), (3, 8, 2), (2, 12, 2)])
 def test_encoder_attention(ops, B, E, H):
   from t5x_amd import network
   rs = np.random.RandomState(B * 1000 + E + H)
@@ -145,7 +147,7 @@ def _tiny_cfgs(**kw):
   return ot5.T5Config(**base), network.T5Config(weight_dtype=wd, **base)
 
 
-@pytest.mark.parametrize('B,E', [(2, 16), (3, 40), (2, 132)])
+@pytest.mark.parametrize('B,E', [(2, 16), (3, 40), (2, 132), (3, 12), (2, 7)])
 def test_encoder_forward_matches_oracle(B, E):
   """Whole bf16 encoder on the HIP kernels.  Per-op agreement is to a bf16 ulp;
   over 3 layers the same chaotic amplification as in the decoder applies, so

@@ -896,3 +896,28 @@ def test_loops_on_a_scanned_layer_cache_generic_equals_fused(dtype):
       inputs, dict(module.init_cache(B, L)), fn, 1, decode_rng=noise,
       num_decodes=K, temperature=0.8, topk=10, cache_offset=1)
   assert torch.equal(a, b) and torch.equal(la, lb)
+
+
+def test_more_than_128_decoder_rows():
+  """batch x beams beyond the 128 rows one dense-kernel launch covers: the
+  decode runs (dense layers in chunks of rows) and every batch item gets what
+  it gets in a batch of its own size class."""
+  from t5x_amd import decoding, models, network
+  ocfg, cfg = tiny('bfloat16')
+  params = ot5.init_params(ocfg, seed=23)
+  rs = np.random.RandomState(8)
+  B, K = 44, 4   # 176 rows
+  enc = ragged_tokens(rs, B, 12, ocfg.vocab_size, 3)
+  gm = models.EncoderDecoderModel(
+      network.Transformer(cfg),
+      decode_fn=functools.partial(decoding.beam_search, alpha=0.6))
+  run = lambda e: gm.predict_batch_with_aux(
+      params, {'encoder_input_tokens': e,
+               'decoder_input_tokens': np.zeros((e.shape[0], 8), np.int32)},
+      num_decodes=K, return_all_decodes=True)
+  got, gaux = run(enc)
+  halves = [run(enc[:22]), run(enc[22:])]
+  want = np.concatenate([host(h[0]) for h in halves])
+  ws = np.concatenate([host(h[1]['scores']) for h in halves])
+  np.testing.assert_array_equal(host(got), want)
+  np.testing.assert_array_equal(host(gaux['scores']), ws)
