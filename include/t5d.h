@@ -411,7 +411,18 @@ typedef struct {
   /* non-zero: the layers' cached_value are in the blocked layout of
    * t5d_self_attention_step_gather (bfloat16, L a multiple of 32) */
   int value_blocked;
+  /* Measurement aid, normally 0: a mask of T5D_LEAVE_OUT_* bits; the step is
+   * enqueued WITHOUT the launches of those kernel families (their outputs keep
+   * whatever the buffers held, so the results are meaningless).  The time a
+   * loop of such steps saves against the full loop is what the family costs
+   * where it runs, between the step's other kernels. */
+  int leave_out;
 } t5d_model_step;
+
+enum {
+  T5D_LEAVE_OUT_CROSS_ATTENTION = 1,  /* t5d_cross_attention_step[_norm_q] */
+  T5D_LEAVE_OUT_SELF_ATTENTION = 2    /* t5d_self_attention_step[_gather] */
+};
 
 /* One decoder step for R rows (Decoder.__call__ with decode=True,
  * t5x/examples/t5/network.py:229-292, as driven by

@@ -13,6 +13,7 @@ from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int32,
 F32, BF16, I8 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_GEGLU = 0, 1, 2
 OUT_ROWS, OUT_HEADS_KEY, OUT_HEADS_VALUE = 0, 1, 2
+LEAVE_OUT_CROSS_ATTENTION, LEAVE_OUT_SELF_ATTENTION = 1, 2
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, 'csrc', 'libt5d.so')
@@ -44,7 +45,7 @@ class ModelStep(Structure):
                   'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
                   'ao', 'h', 'logits', 'gate', 'pending_src',
                   'pending_dst')] +
-              [('value_blocked', c_int)])
+              [('value_blocked', c_int), ('leave_out', c_int)])
 
 
 class BeamStep(Structure):

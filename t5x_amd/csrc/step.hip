@@ -87,7 +87,9 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
       T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
                        m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
     }
-    if (m->pending_src || m->value_blocked)
+    if (m->leave_out & T5D_LEAVE_OUT_SELF_ATTENTION) {
+      // measurement aid: see t5d_model_step::leave_out
+    } else if (m->pending_src || m->value_blocked)
       T5D_TRY(t5d_self_attention_step_gather(
           stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
           m->cache_index + l, m->ao, m->B, m->beams, m->H, m->L,
@@ -99,7 +101,10 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
                                       m->L));
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.self_out, w.self_out_scales,
                      x, m->x1, R, HD, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
-    if (fuse_cross_q) {
+    const bool no_cross = m->leave_out & T5D_LEAVE_OUT_CROSS_ATTENTION;
+    if (no_cross && fuse_cross_q) {
+      // measurement aid: see t5d_model_step::leave_out
+    } else if (fuse_cross_q) {
       T5D_TRY(t5d_cross_attention_step_norm_q(
           stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
           w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d));
@@ -114,9 +119,10 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
                          w.cross_q_scales, nullptr, m->q, R, d, HD,
                          T5D_EPI_NONE, nullptr, nullptr));
       }
-      T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
-                                       w.cross_value, m->enc_len, m->ao, m->B,
-                                       m->beams, m->H, m->E));
+      if (!no_cross)
+        T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
+                                         w.cross_value, m->enc_len, m->ao,
+                                         m->B, m->beams, m->H, m->E));
     }
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
                      w.cross_out_scales, m->x1, m->x2, R, HD, d,

@@ -440,6 +440,7 @@ class Transformer:
     m.gate = P(gate)
     m.pending_src, m.pending_dst = P(pending_src), P(pending_dst)
     m.value_blocked = int(bool(value_blocked))
+    m.leave_out = 0
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
                     pending_src, pending_dst)
     return m
@@ -718,8 +719,17 @@ class FusedSampleStep:
     self._lib.call('t5d_temperature_sample_step', self.stream.cuda_stream,
                    self.model, self.sample)
 
-  def _capture(self):
+  def _record(self):
     lib = self._lib
+    lib.call('t5d_graph_begin', self.stream.cuda_stream)
+    try:
+      self._enqueue()
+    finally:
+      handle = ctypes_void_p()
+      lib.call('t5d_graph_end', self.stream.cuda_stream, handle_ref(handle))
+    return handle
+
+  def _capture(self):
     self.stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(self.stream):
       # First launches load the code objects; with the gate closed they
@@ -727,15 +737,26 @@ class FusedSampleStep:
       self.keep_going.zero_()
       self._enqueue()
       self.stream.synchronize()
-      lib.call('t5d_graph_begin', self.stream.cuda_stream)
-      try:
-        self._enqueue()
-      finally:
-        handle = ctypes_void_p()
-        lib.call('t5d_graph_end', self.stream.cuda_stream, handle_ref(handle))
-      self.graph = handle
+      self.graph = self._record()
       self.keep_going.fill_(1)
     self.stream.synchronize()
+
+  def iteration_graph(self, leave_out=0):
+    """A graph of one iteration enqueued without the kernel families in the
+    `leave_out` mask (t5d_model_step::leave_out; 0: the full iteration), for
+    timing a family by difference.  The caller replays it with launch_graph
+    and destroys it with t5d_graph_destroy."""
+    self.stream.synchronize()
+    self.model.leave_out = int(leave_out)
+    try:
+      with torch.cuda.stream(self.stream):
+        return self._record()
+    finally:
+      self.model.leave_out = 0
+
+  def launch_graph(self, graph, n):
+    for _ in range(n):
+      self._lib.call('t5d_graph_launch', graph, self.stream.cuda_stream)
 
   def advance(self, n):
     """Enqueues n more iterations (fewer when the longest row ends sooner),
@@ -1028,6 +1049,31 @@ class FusedBeamStep:
       handle = ctypes_void_p()
       lib.call('t5d_graph_end', lane.stream.cuda_stream, handle_ref(handle))
     return handle
+
+  def iteration_graph(self, leave_out=0):
+    """A graph of one iteration enqueued without the kernel families in the
+    `leave_out` mask (t5d_model_step::leave_out; 0: the full iteration), for
+    timing a family by difference.  Single-lane loops.  The caller replays it
+    with launch_graph and destroys it with t5d_graph_destroy."""
+    if self.n_lanes != 1:
+      raise ValueError('iteration graphs are for the single-lane loop')
+    lane = self.lanes[0]
+    lane.stream.synchronize()
+    lane.model.leave_out = int(leave_out)
+    try:
+      with torch.cuda.stream(lane.stream):
+        return self._record(lane, 1)
+    finally:
+      lane.model.leave_out = 0
+
+  def launch_graph(self, graph, n):
+    stream = self.lanes[0].stream.cuda_stream
+    for _ in range(n):
+      self._lib.call('t5d_graph_launch', graph, stream)
+
+  @property
+  def stream(self):
+    return self.lanes[0].stream
 
   def _capture(self):
     loop = self.loop
