@@ -332,10 +332,12 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
     if fused:
       ops.cross_attention_step_norm_q(x, layers[i]['ln_cross'],
                                       layers[i]['cross_q'], cross['k'][i],
-                                      cross['v'][i], cross['enc_len'], w.K, out)
+                                      cross['v'][i], cross['enc_len'], w.K, out,
+                                      units=cross.get('units'))
     else:
       ops.cross_attention_step(q, cross['k'][i], cross['v'][i],
-                               cross['enc_len'], w.K, out)
+                               cross['enc_len'], w.K, out,
+                               units=cross.get('units'))
 
   reps = max(1, min(reps_per_layer, 96 // nl))
   replay_sec = time_kernel(torch, launch, reps * nl)

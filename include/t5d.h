@@ -196,11 +196,25 @@ int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
  *   t5d_gemm_rows writes both (T5D_OUT_HEADS_KEY / T5D_OUT_HEADS_VALUE).
  *   K/V are shared by the item's `beams` rows (<= 8).
  *   enc_len [B]: number of leading valid (non-padding) encoder positions.
- *   q [B*beams, H*64] -> out [B*beams, H*64]. */
+ *   q [B*beams, H*64] -> out [B*beams, H*64].
+ *   units: NULL or the table of t5d_cross_attention_units (bfloat16). */
 int t5d_cross_attention_step(void* stream, int dtype, const void* q,
                              const void* cross_key, const void* cross_value,
                              const int32_t* enc_len, void* out, int B,
-                             int beams, int H, int E);
+                             int beams, int H, int E, const int32_t* units);
+
+/* Work order for the bfloat16 cross-attention launches of one batch (no
+ * counterpart in the reference; a scheduling aid).  A launch has one workgroup
+ * per (item, head), and its work grows with the item's valid length; `units`
+ * [B*H] tells workgroup p which (item, head) to take so that the CUs end up
+ * evenly loaded: with at most two workgroups per CU the heaviest sit alone and
+ * the others are paired heaviest with lightest, larger launches go by falling
+ * length.  The entries also carry the valid length, so the table must be
+ * rebuilt whenever enc_len changes.  Passing units = NULL to the attention
+ * calls gives the natural order; results are identical either way.
+ * B, H <= 256. */
+int t5d_cross_attention_units(void* stream, const int32_t* enc_len, int B,
+                              int H, int E, int32_t* units);
 
 /* t5d_rmsnorm + the query projection (t5d_gemm) + t5d_cross_attention_step
  * in one kernel (pre_cross_attention_layer_norm, the `query` DenseGeneral and
@@ -216,7 +230,8 @@ int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
                                     const void* cross_key,
                                     const void* cross_value,
                                     const int32_t* enc_len, void* out, int B,
-                                    int beams, int H, int E, int d);
+                                    int beams, int H, int E, int d,
+                                    const int32_t* units);
 
 /* Encoder self-attention over whole sequences, bfloat16
  * (MultiHeadDotProductAttention without cache, t5x/examples/t5/layers.py:
@@ -395,6 +410,8 @@ typedef struct {
   const t5d_layer* layers;    /* HOST array of NL entries */
   int32_t* cache_index;       /* [NL] device, consecutive */
   const int32_t* enc_len;     /* [B] */
+  /* optional [B*H]: t5d_cross_attention_units of enc_len (bfloat16 only) */
+  const int32_t* cross_units;
   void *x, *x1, *x2, *xn;     /* [R, d] activations */
   void *qkv;                  /* [R, 3*H*64] */
   void *q, *ao;               /* [R, H*64] */

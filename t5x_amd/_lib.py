@@ -42,7 +42,8 @@ class ModelStep(Structure):
       'beams')] + [(n, c_void_p) for n in (
           'embedding', 'rel_bias', 'ln_final', 'logits_w', 'logits_scales')] +
               [('layers', POINTER(Layer))] + [(n, c_void_p) for n in (
-                  'cache_index', 'enc_len', 'x', 'x1', 'x2', 'xn', 'qkv', 'q',
+                  'cache_index', 'enc_len', 'cross_units', 'x', 'x1', 'x2',
+                  'xn', 'qkv', 'q',
                   'ao', 'h', 'logits', 'gate', 'pending_src',
                   'pending_dst')] +
               [('value_blocked', c_int), ('leave_out', c_int)])
@@ -109,11 +110,12 @@ _SIGNATURES = {
                                                _P, c_int, c_int, c_int, c_int,
                                                _P, _P, c_int]),
     't5d_cross_attention_step': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int,
-                                         c_int, c_int, c_int]),
+                                         c_int, c_int, c_int, _P]),
+    't5d_cross_attention_units': (c_int, [_P, _P, c_int, c_int, c_int, _P]),
     't5d_cross_attention_step_norm_q': (c_int, [_P, c_int, c_int, _P, _P,
                                                 c_float, _P, _P, _P, _P, _P,
                                                 c_int, c_int, c_int, c_int,
-                                                c_int]),
+                                                c_int, _P]),
     't5d_add_i32': (c_int, [_P, _P, c_int, c_int]),
     't5d_cache_gather_beams': (c_int, [_P, _P, c_int64, c_int, c_int, c_int,
                                        c_int, c_int, c_int, _P, _P, c_int]),

@@ -426,7 +426,7 @@ int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 const void* v, const int32_t* enc_len,
                                 void* out, int B, int beams, int H, int E,
                                 const void* x, const void* ln, const void* wq,
-                                int d, float eps);
+                                int d, float eps, const int32_t* units);
 int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                void* cv, const void* rel_bias,
                                const int32_t* cache_index, void* out, int R,
@@ -519,9 +519,12 @@ extern "C" int t5d_cross_attention_step(void* stream, int dtype, const void* q,
                                         const void* cross_key,
                                         const void* cross_value,
                                         const int32_t* enc_len, void* out,
-                                        int B, int beams, int H, int E) {
+                                        int B, int beams, int H, int E,
+                                        const int32_t* units) {
   int rc = check_common("t5d_cross_attention_step", dtype, H, E);
   if (rc) return rc;
+  T5D_REQUIRE(units == nullptr || dtype == T5D_BF16, T5D_EINVAL,
+              "t5d_cross_attention_step: a work order is for bfloat16 only");
   T5D_REQUIRE(q && cross_key && cross_value && enc_len && out && B > 0,
               T5D_EINVAL, "t5d_cross_attention_step: null pointer or B=%d", B);
   T5D_REQUIRE(beams >= 1 && beams <= 8, T5D_ELIMIT,
@@ -546,9 +549,76 @@ extern "C" int t5d_cross_attention_step(void* stream, int dtype, const void* q,
                 "32 positions, E=%d", E);
     launch_cross_attention_bf16(as_stream(stream), q, cross_key, cross_value,
                                 enc_len, out, B, beams, H, E, nullptr, nullptr,
-                                nullptr, 0, 0.f);
+                                nullptr, 0, 0.f, units);
   }
   T5D_CHECK_LAUNCH("t5d_cross_attention_step");
+  return T5D_OK;
+}
+
+// ---- work order of the cross-attention workgroups ---------------------------------
+// A cross-attention launch has one workgroup per (item, head) whose work grows
+// with the item's valid encoder length.  The dispatcher deals workgroups out
+// round-robin (position p goes to XCD p % 8 and, there, to CU (p / 8) % 32), two
+// to a CU at most, so with more workgroups than CUs position p shares its CU
+// with position p + n_cu, and the launch lasts as long as its most loaded CU.
+// This kernel writes the order that evens the CUs out: the heaviest units sit
+// alone on a CU, the rest are paired heaviest with lightest; launches of more
+// than two rounds get the units by falling length.  One workgroup; B <= 256.
+__global__ void __launch_bounds__(256)
+cross_units_kernel(const int32_t* __restrict__ enc_len, int B, int H, int E,
+                   int n_cu, int32_t* __restrict__ units) {
+  __shared__ int s_len[256];
+  __shared__ int s_item[256];  // items by falling length (ties: lower index)
+  const int tid = threadIdx.x;
+  if (tid < B) {
+    const int n = enc_len[tid];
+    s_len[tid] = n < 0 ? 0 : (n > E ? E : n);
+  }
+  __syncthreads();
+  if (tid < B) {
+    const int mine = s_len[tid];
+    int rank = 0;
+    for (int o = 0; o < B; ++o) {
+      const int other = s_len[o];
+      rank += (other > mine || (other == mine && o < tid)) ? 1 : 0;
+    }
+    s_item[rank] = tid;
+  }
+  __syncthreads();
+  const int n = B * H;
+  const int pairs = n - n_cu, alone = 2 * n_cu - n;
+  for (int r = tid; r < n; r += 256) {
+    const int b = s_item[r / H], h = r % H;
+    int p = r;
+    if (n > n_cu && n <= 2 * n_cu) {
+      const int rr = r - alone;
+      p = r < alone ? pairs + r : (rr < pairs ? rr : n_cu + (2 * pairs - 1 - rr));
+    }
+    // an item without a valid key keeps 0: the kernel then attends uniformly
+    units[p] = h | (b << 8) | (int)((uint32_t)s_len[b] << 16);
+  }
+}
+
+extern "C" int t5d_cross_attention_units(void* stream, const int32_t* enc_len,
+                                         int B, int H, int E, int32_t* units) {
+  T5D_REQUIRE(enc_len && units, T5D_EINVAL,
+              "t5d_cross_attention_units: null pointer");
+  T5D_REQUIRE(B > 0 && B <= 256 && H > 0 && H <= 256 && E > 0 && E < 32768,
+              T5D_ELIMIT,
+              "t5d_cross_attention_units: B=%d H=%d (1..256 each), E=%d "
+              "(below 32768)", B, H, E);
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) !=
+            hipSuccess || v <= 0)
+      v = 256;
+    n_cu = v;
+  }
+  hipLaunchKernelGGL(cross_units_kernel, dim3(1), dim3(256), 0,
+                     as_stream(stream), enc_len, B, H, E, n_cu, units);
+  T5D_CHECK_LAUNCH("t5d_cross_attention_units");
   return T5D_OK;
 }
 
@@ -556,7 +626,7 @@ extern "C" int t5d_cross_attention_step_norm_q(
     void* stream, int dtype, int w_dtype, const void* x, const void* ln_scale,
     float eps, const void* query_kernel, const void* cross_key,
     const void* cross_value, const int32_t* enc_len, void* out, int B,
-    int beams, int H, int E, int d) {
+    int beams, int H, int E, int d, const int32_t* units) {
   int rc = check_common("t5d_cross_attention_step_norm_q", dtype, H, E);
   if (rc) return rc;
   T5D_REQUIRE(dtype == T5D_BF16 && w_dtype == T5D_BF16, T5D_EINVAL,
@@ -581,7 +651,7 @@ extern "C" int t5d_cross_attention_step_norm_q(
               "t5d_cross_attention_step_norm_q: operands not 16-byte aligned");
   launch_cross_attention_bf16(as_stream(stream), nullptr, cross_key, cross_value,
                               enc_len, out, B, beams, H, E, x, ln_scale,
-                              query_kernel, d, eps);
+                              query_kernel, d, eps, units);
   T5D_CHECK_LAUNCH("t5d_cross_attention_step_norm_q");
   return T5D_OK;
 }

@@ -56,6 +56,10 @@ struct AttnMfmaArgs {
   int d;
   float eps;
   int v_blocked;  // self-attention: value cache stored as [S/32][64][32] per head
+  // cross-attention: optional work order, [B * H] entries
+  // head | item << 8 | valid length << 16; workgroup (x, y) takes entry
+  // y * H + x instead of (head x, item y, index[y])
+  const int32_t* units;
 };
 
 constexpr int kHeadDim = 64;
@@ -94,7 +98,7 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   __shared__ __attribute__((aligned(16))) float s_out[WM][NQP][kHeadDim];
   T5D_GATE_READ(a.gate);
 
-  const int h = blockIdx.x, b = blockIdx.y;
+  int h = blockIdx.x, b = blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nwaves = blockDim.x >> 6;
@@ -102,8 +106,17 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   const int q = n16 % NQP, rep = n16 / NQP;
   const int HD = a.H * kHeadDim;
 
-  int n = a.index[b];
-  T5D_GATE_TEST();  // after both scalar loads are in flight
+  int n;
+  if (a.units != nullptr) {
+    const int u = a.units[b * a.H + h];
+    T5D_GATE_TEST();  // after both scalar loads are in flight
+    h = u & 0xff;
+    b = (u >> 8) & 0xff;
+    n = (int)((uint32_t)u >> 16);
+  } else {
+    n = a.index[b];
+    T5D_GATE_TEST();
+  }
   n = n < 0 ? 0 : (n > a.S ? a.S : n);
   bool uniform = false;  // no valid key: the masked softmax is uniform
   if (n == 0) { uniform = true; n = a.S; }
@@ -736,9 +749,10 @@ int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 const void* v, const int32_t* enc_len,
                                 void* out, int B, int beams, int H, int E,
                                 const void* x, const void* ln, const void* wq,
-                                int d, float eps) {
+                                int d, float eps, const int32_t* units) {
   AttnMfmaArgs a;
   a.v_blocked = 0;
+  a.units = units;
   a.x = (const bf16_t*)x; a.ln = (const bf16_t*)ln; a.wq = wq;
   a.d = d; a.eps = eps;
   a.q = (const bf16_t*)q; a.k = (bf16_t*)k; a.v = (bf16_t*)v;
@@ -764,6 +778,7 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
   a.H = H; a.S = L; a.nq = 1; a.q_stride = 3 * H * kHeadDim;
   a.gate = tls_gate;
   a.x = nullptr; a.ln = nullptr; a.wq = nullptr; a.d = 0; a.eps = 0.f;
+  a.units = nullptr;
   a.nblk = (L + kBlockJ - 1) / kBlockJ;
   a.pending = pending;
   a.pending_dst = pending ? pending_dst : nullptr;

@@ -107,7 +107,8 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
     } else if (fuse_cross_q) {
       T5D_TRY(t5d_cross_attention_step_norm_q(
           stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
-          w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d));
+          w.cross_value, m->enc_len, m->ao, m->B, m->beams, m->H, m->E, d,
+          m->cross_units));
     } else {
       if (norm_rides(HD)) {
         T5D_TRY(t5d_norm_gemm(stream, dt, wd, dt, m->x1, w.ln_cross, 1e-6f,
@@ -122,7 +123,9 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
       if (!no_cross)
         T5D_TRY(t5d_cross_attention_step(stream, dt, m->q, w.cross_key,
                                          w.cross_value, m->enc_len, m->ao,
-                                         m->B, m->beams, m->H, m->E));
+                                         m->B, m->beams, m->H, m->E,
+                                         dt == T5D_BF16 ? m->cross_units
+                                                        : nullptr));
     }
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.cross_out,
                      w.cross_out_scales, m->x1, m->x2, R, HD, d,

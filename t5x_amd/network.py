@@ -343,6 +343,8 @@ class Transformer:
       for dst, src in zip(out['k'] + out['v'], res['k'] + res['v']):
         dst.copy_(src)
       out['enc_len'].copy_(res['enc_len'])
+      if out.get('units') is not None:
+        out['units'].copy_(res['units'])
       self._cross = (key, out, encoded)
       return out
     cfg = self.config
@@ -400,7 +402,12 @@ class Transformer:
       res = out
     else:
       res = dict(k=ks, v=vs, enc_len=lens.contiguous(), B=B, beams=beams,
-                 E=Ep)
+                 E=Ep, units=None)
+    # The order in which the cross-attention workgroups take the (item, head)
+    # pairs, chosen from the valid lengths so that the CUs are evenly loaded.
+    if bf16 and B <= 256 and H <= 256:
+      res['units'] = ops.cross_attention_units(res['enc_len'], H, Ep,
+                                               out=res.get('units'))
     self._cross = (key, res, encoded)
     return res
 
@@ -435,6 +442,7 @@ class Transformer:
     m.logits_scales = P(w.logits.scales)
     m.layers = layers
     m.cache_index, m.enc_len = P(cache_index), P(cross['enc_len'])
+    m.cross_units = P(cross.get('units'))
     for name in ('x', 'x1', 'x2', 'xn', 'qkv', 'q', 'ao', 'h', 'logits'):
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
@@ -852,7 +860,8 @@ class _BeamLane:
     lane_cross = dict(k=[t[b0:b1] for t in cross['k']],
                       v=[t[b0:b1] for t in cross['v']],
                       enc_len=cross['enc_len'][b0:b1], B=B, beams=K,
-                      E=cross['E'])
+                      E=cross['E'],
+                      units=cross.get('units') if owner.n_lanes == 1 else None)
     layer_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(nl)]
     self.model = module._model_step(
         w, lane_cross, self.bufs, layer_caches, self.cache_index, R, K, L,

@@ -323,7 +323,32 @@ def _cross_kv_dims(cross_key, cross_value):
   return B, H, E
 
 
-def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
+def cross_attention_units(enc_len, H, E, out=None):
+  """The work order of the bfloat16 cross-attention launches for a batch with
+  these valid lengths: int32 [B * H] (t5d_cross_attention_units)."""
+  _chk(enc_len, 'enc_len', torch.int32, 1)
+  B = enc_len.shape[0]
+  if out is None:
+    out = torch.empty((B * H,), dtype=torch.int32, device=enc_len.device)
+  _chk(out, 'units', torch.int32, 1)
+  if out.shape[0] != B * H:
+    raise ValueError(f'units must have {B * H} entries')
+  _lib.call('t5d_cross_attention_units', _s(), enc_len.data_ptr(), B, H, E,
+            out.data_ptr())
+  return out
+
+
+def _units_ptr(units, B, H):
+  if units is None:
+    return None
+  _chk(units, 'units', torch.int32, 1)
+  if units.shape[0] != B * H:
+    raise ValueError(f'units must have {B * H} entries')
+  return units.data_ptr()
+
+
+def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None,
+                         units=None):
   _chk(q, 'q', ndim=2)
   _chk(cross_key, 'cross_key', q.dtype)
   _chk(enc_len, 'enc_len', torch.int32, 1)
@@ -338,13 +363,14 @@ def cross_attention_step(q, cross_key, cross_value, enc_len, beams, out=None):
   _chk(out, 'out', q.dtype, 2)
   _lib.call('t5d_cross_attention_step', _s(), _lib.dtype_code(q.dtype),
             q.data_ptr(), cross_key.data_ptr(), cross_value.data_ptr(),
-            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E)
+            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E,
+            _units_ptr(units, B, H))
   return out
 
 
 def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
                                 cross_value, enc_len, beams, out=None,
-                                eps=1e-6):
+                                eps=1e-6, units=None):
   """rmsnorm(x, ln_scale) @ wq followed by cross_attention_step, one kernel."""
   _chk(x, 'x', torch.bfloat16, 2)
   _chk(ln_scale, 'ln_scale', torch.bfloat16, 1)
@@ -363,7 +389,8 @@ def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
   _lib.call('t5d_cross_attention_step_norm_q', _s(), _lib.dtype_code(x.dtype),
             wq.w_dtype, x.data_ptr(), ln_scale.data_ptr(), float(eps),
             wq.data.data_ptr(), cross_key.data_ptr(), cross_value.data_ptr(),
-            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E, d)
+            enc_len.data_ptr(), out.data_ptr(), B, beams, H, E, d,
+            _units_ptr(units, B, H))
   return out
 
 

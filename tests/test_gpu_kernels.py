@@ -625,6 +625,55 @@ def test_cross_attention_step(ops, dt, B, beams, H, E):
                              rtol=TOL[dt])
 
 
+@pytest.mark.parametrize('B,beams,H,E', [(3, 4, 2, 512), (32, 4, 12, 512),
+                                         (40, 1, 12, 256), (64, 1, 16, 512),
+                                         (20, 2, 12, 96)])
+def test_cross_attention_work_order(ops, B, beams, H, E):
+  """t5d_cross_attention_units: a permutation of the (item, head) pairs that
+  carries every item's valid length; with it the two cross-attention kernels
+  give bit for bit what they give in the natural order.  For a launch of one
+  to two workgroups per CU the heaviest units sit alone, i.e. every position
+  that shares its CU with another one (p and p + n_cu) holds a unit no longer
+  than any unit that sits alone."""
+  rs = np.random.RandomState(B * 7 + H)
+  D, d = 64, 256
+  lens = rs.randint(0, E + 1, size=(B,)).astype(np.int32)
+  lens[0] = E
+  lens_d = dev(lens)
+  units = ops.cross_attention_units(lens_d, H, E)
+  u = host(units).astype(np.int64) & 0xFFFFFFFF
+  h, b, n = u & 0xFF, (u >> 8) & 0xFF, u >> 16
+  assert sorted(zip(b.tolist(), h.tolist())) == [(i, j) for i in range(B)
+                                                 for j in range(H)]
+  np.testing.assert_array_equal(n, lens[b])
+  n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+  total = B * H
+  if n_cu < total <= 2 * n_cu:
+    pairs = total - n_cu
+    alone = n[pairs:n_cu]
+    assert alone.size == 0 or max(n[:pairs].max(), n[n_cu:].max()) <= alone.min()
+    # the paired: heaviest with lightest
+    assert (np.diff(n[:pairs]) <= 0).all() and (np.diff(n[n_cu:]) >= 0).all()
+  elif total > 2 * n_cu:
+    assert (np.diff(n) <= 0).all()
+  k = (0.5 * rs.randn(B, H, E, D)).astype(np.float32)
+  v = rs.randn(B, H, D, E).astype(np.float32)
+  kd = ops.tile_cross_key(dev(k, torch.bfloat16))
+  vd = ops.tile_cross_value(dev(v, torch.bfloat16))
+  q = dev(0.125 * rs.randn(B * beams, H * D).astype(np.float32), torch.bfloat16)
+  want = ops.cross_attention_step(q, kd, vd, lens_d, beams)
+  got = ops.cross_attention_step(q, kd, vd, lens_d, beams, units=units)
+  assert torch.equal(got, want)
+  x = dev(rs.randn(B * beams, d).astype(np.float32), torch.bfloat16)
+  scale = dev(1 + 0.1 * rs.randn(d).astype(np.float32), torch.bfloat16)
+  wq = ops.pack_weight(dev((rs.randn(d, H * D) / 16).astype(np.float32)),
+                       torch.bfloat16)
+  want = ops.cross_attention_step_norm_q(x, scale, wq, kd, vd, lens_d, beams)
+  got = ops.cross_attention_step_norm_q(x, scale, wq, kd, vd, lens_d, beams,
+                                        units=units)
+  assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize('rows,n,k', [(1, 10, 3), (4, 1000, 8), (3, 128512, 8),
                                       (2, 24, 24), (5, 77, 64)])
 def test_top_k_exact_with_ties(ops, rows, n, k):

@@ -36,12 +36,16 @@ def _both(B, beams, V, k, seed):
             want[3].data_ptr(), scratch.data_ptr(), B, beams, V, k)
   got = outputs()
   torch.cuda.synchronize()
-  before = torch.cuda.memory_allocated()
+  # the running count of allocation requests: unlike the bytes in use it cannot
+  # move when the garbage collector frees tensors of earlier tests meanwhile
+  def requests():
+    return torch.cuda.memory_stats()['allocation.all.allocated']
+  before = requests()
   _lib.call('t5d_beam_topk_static', s, logits.data_ptr(), live.data_ptr(),
             got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(),
             got[3].data_ptr(), B, beams, V, k)
   torch.cuda.synchronize()
-  assert torch.cuda.memory_allocated() == before
+  assert requests() == before
   for g, w in zip(got, want):
     np.testing.assert_array_equal(g.cpu().numpy(), w.cpu().numpy())
   assert int(got[1].min()) >= 0
