@@ -95,14 +95,31 @@ int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
  *   T5D_EPI_GEGLU: W is a geglu-packed [K, 2F] kernel, N = 2F, C is [M, F].
  *   The kernels are laid out for M <= 128 (the weights stream once); more rows
  *   run as chunks of 128, each streaming the weights again.
- *   workspace/counters: reserved for kernel variants that need scratch
- *   memory; t5d_gemm_workspace_bytes currently returns 0 for every shape and
- *   both may be NULL. */
+ *   Layers of 8 MB of weights and more run on large workgroup tiles (up to
+ *   128 x 128) chosen so that the most loaded CU reads the fewest bytes.
+ *   workspace/counters: reserved for plans that need scratch memory; no plan
+ *   does (t5d_gemm_workspace_bytes returns 0 for every shape) and both may
+ *   be NULL. */
 int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M, int K, int N);
 int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
              const void* A, const void* W, const float* scales,
              const void* residual, void* C, int M, int K, int N, int epilogue,
              void* workspace, int32_t* counters);
+
+/* t5d_gemm on a large-tile kernel of the caller's choice (bfloat16
+ * activations, M <= 128): a workgroup tile of mp*16 rows x nt*16 columns, K
+ * split over k_parts workgroups.  (mp, nt) one of (2,3) (2,4) (2,5) (4,4)
+ * (4,6) (4,8) (8,4) (8,5) (8,8).  k_parts > 1 needs the residual epilogue, a
+ * workspace of k_parts*M*N*4 bytes, N a multiple of 8 and <= 16384: the
+ * parts' float32 sums go there and a second kernel adds them in ascending
+ * order and applies the epilogue.  The result does not depend on (mp, nt)
+ * and equals t5d_gemm's bit for bit when k_parts == 1; it depends on k_parts
+ * (summation order).  For tuning and for testing every kernel variant;
+ * t5d_gemm picks the tile itself and never splits K. */
+int t5d_gemm_tiled(void* stream, int dtype, int w_dtype, int out_dtype,
+                   const void* A, const void* W, const float* scales,
+                   const void* residual, void* C, int M, int K, int N,
+                   int epilogue, void* workspace, int mp, int nt, int k_parts);
 
 /* t5d_rmsnorm followed by t5d_gemm in one kernel (a pre-attention / pre-MLP
  * LayerNorm feeding its dense layer, t5x/examples/t5/network.py:134-139,

@@ -21,95 +21,9 @@
 #include <cstring>
 
 #include "common.h"
+#include "gemm_tiles.h"
 
 namespace t5d {
-
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_v;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_v;
-
-union Frag {
-  uint4 u;
-  bf16x8_v v;
-};
-
-__device__ __forceinline__ uint32_t pack_i8x2_to_bf16x2(int a, int b) {
-  // int8 values are exactly representable in bfloat16.
-  return pack_bf16x2((float)a, (float)b);
-}
-
-// A packed weight tile as it travels from memory (`Raw`, kept in registers
-// while the load is in flight) and as the matrix cores take it (`Frag`).
-// int8 tiles are half the bytes, so twice as many can be in flight (kDepth);
-// they are widened only when consumed — converting at load time would put a
-// wait for the load right behind it.
-template <typename WT> struct WeightTile;
-template <> struct WeightTile<bf16_t> {
-  static constexpr int kTileBytes = 1024;
-  static constexpr int kDepth = 1;
-  typedef uint4 Raw;
-  __device__ static __forceinline__ Raw load(const void* tile, int lane) {
-    return reinterpret_cast<const uint4*>(tile)[lane];
-  }
-  __device__ static __forceinline__ Raw zero() { return make_uint4(0, 0, 0, 0); }
-  __device__ static __forceinline__ Frag frag(const Raw& r) {
-    Frag f;
-    f.u = r;
-    return f;
-  }
-};
-template <> struct WeightTile<int8_t> {
-  static constexpr int kTileBytes = 512;
-  static constexpr int kDepth = 2;
-  typedef uint2 Raw;
-  __device__ static __forceinline__ Raw load(const void* tile, int lane) {
-    return reinterpret_cast<const uint2*>(tile)[lane];
-  }
-  __device__ static __forceinline__ Raw zero() { return make_uint2(0, 0); }
-  __device__ static __forceinline__ Frag frag(const Raw& q) {
-    Frag f;
-    f.u.x = pack_i8x2_to_bf16x2((int8_t)(q.x), (int8_t)(q.x >> 8));
-    f.u.y = pack_i8x2_to_bf16x2((int8_t)(q.x >> 16), (int8_t)(q.x >> 24));
-    f.u.z = pack_i8x2_to_bf16x2((int8_t)(q.y), (int8_t)(q.y >> 8));
-    f.u.w = pack_i8x2_to_bf16x2((int8_t)(q.y >> 16), (int8_t)(q.y >> 24));
-    return f;
-  }
-};
-
-struct GemmArgs {
-  const bf16_t* A;      // [M, K]
-  const void* W;        // packed tiles
-  const float* scales;  // [N] or null
-  const void* residual; // [M, Nout] act dtype or null
-  void* C;              // [M, Nout]
-  int M, K, N;          // N = number of weight columns
-  int m_parts;          // workgroups along M
-  const int32_t* gate;  // optional device-side enable flag
-  int epilogue;
-  int out_f32;
-  const bf16_t* norm_scale;  // norm_gemm_kernel: [K] layer-norm scale
-  float eps;
-};
-
-// Apply scale + epilogue to one finished column (pair) of row m; `res` is the
-// residual element (fetched early by the caller).
-__device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
-                                             float v, float v_gate, float res) {
-  if (g.epilogue == T5D_EPI_GEGLU) {
-    const int f = (n >> 4) * 8 + (n & 7);
-    const int F = g.N >> 1;
-    float a0 = round_bf16(v), a1 = round_bf16(v_gate);
-    float h = round_bf16(round_bf16(gelu_tanh(a0)) * a1);
-    reinterpret_cast<bf16_t*>(g.C)[(size_t)m * F + f] = f32_to_bf16(h);
-    return;
-  }
-  const size_t o = (size_t)m * g.N + n;
-  if (g.out_f32) {
-    reinterpret_cast<float*>(g.C)[o] = v;
-    return;
-  }
-  if (g.epilogue == T5D_EPI_RESIDUAL) v = round_bf16(v) + res;
-  reinterpret_cast<bf16_t*>(g.C)[o] = f32_to_bf16(v);
-}
 
 template <int MP, int NT, typename WT>
 __global__ void __launch_bounds__(256)
@@ -874,10 +788,6 @@ __global__ void pack_weight_kernel(const WT* __restrict__ src,
   dst[idx] = v;
 }
 
-struct GemmPlan {
-  int mp, nt, m_parts, n_groups;
-};
-
 // Pick the workgroup tile.  Model: the workgroups run in rounds of as many
 // as are resident at once (256 CUs x the tile's occupancy, which its register
 // count sets); a round costs a fixed latency plus the time one workgroup needs
@@ -897,7 +807,7 @@ constexpr int kMaxRows = 128;  // rows one launch of the MFMA kernels covers
 static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
   const int mt_total = (M + 15) / 16;
   const int n_tiles = N / 16;
-  GemmPlan best = {1, 1, 1, 1};
+  GemmPlan best = {1, 1, 1, 1, 1, false};
   double best_cost = 1e30;
   const int mps[4] = {1, 2, 4, 8};
   const int nts[3] = {1, 2, 4};
@@ -915,10 +825,93 @@ static GemmPlan plan_gemm(int M, int K, int N, int w_bytes) {
       const double cost = rounds * (3.0 + bytes / 40e3) + wgs * bytes / 40e6;
       if (cost < best_cost) {
         best_cost = cost;
-        best = {mp, nt, m_parts, n_groups};
+        best = {mp, nt, m_parts, n_groups, 1, false};
       }
     }
   return best;
+}
+
+// CUs of the current device (256 on MI355X).
+static int cu_count() {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) !=
+            hipSuccess || v <= 0)
+      v = 256;
+    n_cu = v;
+  }
+  return n_cu;
+}
+
+// Layers whose weights are at least this many bytes are planned for
+// gemm_big_kernel; smaller ones are bound by launch latency and keep the
+// small tiles (measured: the large-tile kernel is slower on every layer of
+// T5.1.1-large and on the 4-21 MB layers of T5.1.1-XL with int8 weights).
+constexpr double kBigWeightBytes = 24e6;
+constexpr double kCuBytesPerUs = 45e3;   // what one CU takes in from L2
+
+// Microseconds of a large-tile launch: rounds of one workgroup per CU, each
+// lasting the bytes that workgroup reads over a CU's intake rate; the larger
+// the accumulator tile, the fewer registers are left for loads in flight and
+// the further the kernel stays below that rate (fitted to measurements).  A
+// split over K additionally costs the kernel that adds the parts.
+static double big_cost(int M, int K, int N, int w_bytes, int mp, int nt,
+                       int k_parts) {
+  const int mt_total = (M + 15) / 16, n_tiles = N / 16;
+  const int m_parts = (mt_total + mp - 1) / mp;
+  const int n_groups = (n_tiles + nt - 1) / nt;
+  const double wgs = (double)m_parts * n_groups * k_parts;
+  const double rounds = (double)(long)((wgs + cu_count() - 1) / cu_count());
+  const double bytes = (double)K / k_parts *
+                       (2.0 * min(mp * 16, M) + (double)w_bytes * nt * 16);
+  double t = 4.0 + rounds * bytes * (1.0 + 0.012 * mp * nt) / kCuBytesPerUs;
+  if (k_parts > 1) t += 4.5 + 2.0 * k_parts * (double)M * N * 4.0 / 4e6;
+  return t;
+}
+
+// Tiles measured best for the layer shapes of the benchmark models (rows up
+// to M, K, N, bytes per weight); the cost model covers everything else.
+struct TunedTile { int M, K, N, wb, mp, nt; };
+static const TunedTile kTunedTiles[] = {
+    {128, 4096, 4096, 2, 2, 4},    // XXL attention projections: 19 us
+    {128, 4096, 12288, 2, 4, 6},   // XXL q, k, v: 40 us
+    {128, 4096, 20480, 2, 8, 5},   // XXL MLP in: 67 us
+    {128, 10240, 4096, 2, 2, 4},   // XXL MLP out: 40 us
+    {128, 4096, 32128, 2, 8, 8},   // XXL vocabulary projection: 93 us
+    {64, 2048, 32128, 1, 4, 4},    // XL int8 vocabulary projection: 30 us
+};
+
+// The plan never splits K by itself: at these shapes the split was measured
+// equal at best once the kernel that adds the parts is counted
+// (K = 10240, N = 4096: 39.3 + finish against 40.1 us); t5d_gemm_tiled runs
+// it on request.
+static bool plan_big(int M, int K, int N, int w_bytes, GemmPlan* out) {
+  if ((double)K * N * w_bytes < kBigWeightBytes || M < 32 || K < 2048)
+    return false;
+  const int mt_total = (M + 15) / 16, n_tiles = N / 16;
+  for (const TunedTile& t : kTunedTiles)
+    if (M <= t.M && 2 * M > t.M && K == t.K && N == t.N && w_bytes == t.wb) {
+      *out = {t.mp, t.nt, (mt_total + t.mp - 1) / t.mp,
+              (n_tiles + t.nt - 1) / t.nt, 1, true};
+      return true;
+    }
+  double best_cost = 1e30;
+  bool found = false;
+  for (int mp = 2; mp <= 8; mp *= 2)
+    for (int nt = 3; nt <= 8; ++nt) {
+      if (!gemm_big_has_tile(mp, nt)) continue;
+      if (mp > mt_total && (mp >> 1) >= mt_total) continue;
+      const double c = big_cost(M, K, N, w_bytes, mp, nt, 1);
+      if (c < best_cost) {
+        best_cost = c;
+        *out = {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt, 1,
+                true};
+        found = true;
+      }
+    }
+  return found;
 }
 
 template <typename WT>
@@ -1006,7 +999,7 @@ extern "C" int t5d_pack_weight(void* stream, int w_dtype, const void* src,
 extern "C" int64_t t5d_gemm_workspace_bytes(int dtype, int w_dtype, int M,
                                             int K, int N) {
   (void)dtype; (void)w_dtype; (void)M; (void)K; (void)N;
-  return 0;  // no kernel variant needs scratch memory
+  return 0;  // no plan needs scratch memory (see plan_big)
 }
 
 extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
@@ -1044,15 +1037,18 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
               "t5d_gemm: K=%d N=%d must tile 32x16", K, N);
   T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
               "t5d_gemm: A/W must be 16-byte aligned");
-  (void)workspace; (void)counters;
+  (void)counters;
   // The kernels cover up to kMaxRows rows; more rows go through in chunks
   // (each streams the weights again: beyond a few hundred rows t5d_gemm_rows
   // is the kernel to use).
   const int n_out = epilogue == T5D_EPI_GEGLU ? N / 2 : N;
   const size_t out_elem = out_dtype == T5D_F32 ? 4 : 2;
+  const int wb = w_dtype == T5D_I8 ? 1 : 2;
+  (void)workspace;
   for (int m0 = 0; m0 < M; m0 += kMaxRows) {
     const int mc = min(kMaxRows, M - m0);
-    GemmPlan p = plan_gemm(mc, K, N, w_dtype == T5D_I8 ? 1 : 2);
+    GemmPlan p;
+    if (!plan_big(mc, K, N, wb, &p)) p = plan_gemm(mc, K, N, wb);
     GemmArgs g;
     g.A = (const bf16_t*)A + (size_t)m0 * K;
     g.W = W;
@@ -1067,9 +1063,84 @@ extern "C" int t5d_gemm(void* stream, int dtype, int w_dtype, int out_dtype,
     g.out_f32 = out_dtype == T5D_F32;
     g.norm_scale = nullptr;
     g.eps = 0.f;
-    if (w_dtype == T5D_BF16) launch_mfma<bf16_t>(p, g, s);
-    else launch_mfma<int8_t>(p, g, s);
+    if (p.big) {
+      launch_gemm_big(w_dtype, p, g, nullptr, s);
+    } else if (w_dtype == T5D_BF16) {
+      launch_mfma<bf16_t>(p, g, s);
+    } else {
+      launch_mfma<int8_t>(p, g, s);
+    }
     T5D_CHECK_LAUNCH("t5d_gemm");
+  }
+  return T5D_OK;
+}
+
+// Shared argument checks of the bfloat16 MFMA entry points.
+static int check_mfma_args(const char* name, int dtype, int w_dtype,
+                           const void* A, const void* W, const float* scales,
+                           int M, int K, int N) {
+  T5D_REQUIRE(dtype == T5D_BF16 && (w_dtype == T5D_BF16 || w_dtype == T5D_I8),
+              T5D_EINVAL,
+              "%s: bfloat16 activations with packed bfloat16 or int8 weights",
+              name);
+  T5D_REQUIRE(A && W, T5D_EINVAL, "%s: null pointer", name);
+  T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
+              "%s: int8 weights need scales", name);
+  T5D_REQUIRE(M > 0 && M <= kMaxRows && K > 0 && N > 0 && K % 32 == 0 &&
+                  N % 16 == 0,
+              T5D_EINVAL, "%s: M=%d (1..%d), K=%d N=%d must tile 32x16", name,
+              M, kMaxRows, K, N);
+  T5D_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, T5D_EINVAL,
+              "%s: A/W must be 16-byte aligned", name);
+  return T5D_OK;
+}
+
+extern "C" int t5d_gemm_tiled(void* stream, int dtype, int w_dtype,
+                              int out_dtype, const void* A, const void* W,
+                              const float* scales, const void* residual,
+                              void* C, int M, int K, int N, int epilogue,
+                              void* workspace, int mp, int nt, int k_parts) {
+  int rc = check_mfma_args("t5d_gemm_tiled", dtype, w_dtype, A, W, scales, M, K,
+                           N);
+  if (rc != T5D_OK) return rc;
+  T5D_REQUIRE(C && epilogue >= T5D_EPI_NONE && epilogue <= T5D_EPI_GEGLU &&
+                  (epilogue != T5D_EPI_RESIDUAL || residual) &&
+                  (out_dtype == T5D_BF16 ||
+                   (out_dtype == T5D_F32 && epilogue == T5D_EPI_NONE)),
+              T5D_EINVAL, "t5d_gemm_tiled: epilogue %d, out_dtype %d", epilogue,
+              out_dtype);
+  T5D_REQUIRE(gemm_big_has_tile(mp, nt), T5D_EINVAL,
+              "t5d_gemm_tiled: no kernel for a tile of %d x %d", mp * 16,
+              nt * 16);
+  T5D_REQUIRE(k_parts >= 1 && k_parts <= 16, T5D_EINVAL,
+              "t5d_gemm_tiled: k_parts=%d", k_parts);
+  T5D_REQUIRE(k_parts == 1 ||
+                  (workspace && epilogue == T5D_EPI_RESIDUAL && N % 8 == 0 &&
+                   N <= 16384 &&
+                   ((uintptr_t)workspace | (uintptr_t)residual | (uintptr_t)C) %
+                           16 == 0),
+              T5D_EINVAL,
+              "t5d_gemm_tiled: a split over K needs a workspace, the residual "
+              "epilogue, 16-byte aligned rows and N <= 16384");
+  const int mt_total = (M + 15) / 16, n_tiles = N / 16;
+  GemmPlan p = {mp, nt, (mt_total + mp - 1) / mp, (n_tiles + nt - 1) / nt,
+                k_parts, true};
+  GemmArgs g;
+  g.A = (const bf16_t*)A; g.W = W;
+  g.scales = w_dtype == T5D_I8 ? scales : nullptr;
+  g.residual = residual; g.C = C;
+  g.M = M; g.K = K; g.N = N; g.m_parts = p.m_parts;
+  g.gate = tls_gate; g.epilogue = epilogue;
+  g.out_f32 = out_dtype == T5D_F32;
+  g.norm_scale = nullptr; g.eps = 0.f;
+  hipStream_t s = as_stream(stream);
+  launch_gemm_big(w_dtype, p, g, k_parts > 1 ? (float*)workspace : nullptr, s);
+  T5D_CHECK_LAUNCH("t5d_gemm_tiled");
+  if (k_parts > 1) {
+    rc = launch_splitk_finish(s, (const float*)workspace, k_parts, g.scales,
+                              residual, C, nullptr, nullptr, M, N, 0.f);
+    if (rc != T5D_OK) return rc;
+    T5D_CHECK_LAUNCH("t5d_gemm_tiled(finish)");
   }
   return T5D_OK;
 }

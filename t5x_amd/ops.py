@@ -145,34 +145,8 @@ def rmsnorm(x, scale, out=None, eps=1e-6):
   return out
 
 
-class GemmScratch:
-  """Split-K workspace + counters, grown on demand and reused."""
-
-  def __init__(self, device):
-    self.device = device
-    self.workspace = None
-    self.counters = torch.zeros(4096, dtype=torch.int32, device=device)
-
-  def get(self, nbytes):
-    if nbytes and (self.workspace is None or
-                   self.workspace.numel() < nbytes):
-      self.workspace = torch.empty(nbytes, dtype=torch.uint8,
-                                   device=self.device)
-    return self.workspace
-
-
-_scratch = {}
-
-
-def _default_scratch(device):
-  key = (device.type, device.index)
-  if key not in _scratch:
-    _scratch[key] = GemmScratch(device)
-  return _scratch[key]
-
-
 def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
-         scratch=None, norm_scale=None, eps=1e-6):
+         norm_scale=None, eps=1e-6):
   """C = epilogue(a @ W).  a [M, K]; geglu weights give [M, F].  With
   norm_scale [K] the rows of a are RMS-normalised first, in the same kernel."""
   _chk(a, 'a', ndim=2)
@@ -202,18 +176,37 @@ def gemm(a, w: PackedWeight, out=None, residual=None, out_dtype=None,
               float(eps), w.data.data_ptr(), _lib.ptr(w.scales),
               out.data_ptr(), M, K, w.N, epi)
     return out
-  ws_bytes = _lib.load().t5d_gemm_workspace_bytes(dt, w.w_dtype, M, K, w.N)
-  ws = cnt = None
-  if ws_bytes:
-    scratch = scratch or _default_scratch(a.device)
-    ws = scratch.get(ws_bytes)
-    cnt = scratch.counters
-    if w.N // 16 > cnt.numel():
-      raise ValueError('too many column tiles for the counter buffer')
   _lib.call('t5d_gemm', _s(), dt, w.w_dtype, _lib.dtype_code(out_dtype),
             a.data_ptr(), w.data.data_ptr(), _lib.ptr(w.scales),
-            _lib.ptr(residual), out.data_ptr(), M, K, w.N, epi, _lib.ptr(ws),
-            _lib.ptr(cnt))
+            _lib.ptr(residual), out.data_ptr(), M, K, w.N, epi, None, None)
+  return out
+
+
+def gemm_tiled(a, w: PackedWeight, mp, nt, k_parts=1, out=None, residual=None,
+               out_dtype=None):
+  """gemm on the large-tile kernel (mp*16 rows x nt*16 columns per workgroup,
+  K split over k_parts workgroups)."""
+  _chk(a, 'a', torch.bfloat16, 2)
+  M, K = a.shape
+  if K != w.K:
+    raise ValueError(f'a is [{M}, {K}] but the kernel has K={w.K}')
+  epi = EPI_GEGLU if w.geglu else (EPI_RESIDUAL if residual is not None
+                                   else EPI_NONE)
+  out_dtype = out_dtype or a.dtype
+  if out is None:
+    out = torch.empty((M, w.out_features), dtype=out_dtype, device=a.device)
+  _chk(out, 'out', out_dtype, 2)
+  if residual is not None:
+    _chk(residual, 'residual', a.dtype, 2)
+    if tuple(residual.shape) != (M, w.out_features):
+      raise ValueError('residual shape mismatch')
+  ws = None
+  if k_parts > 1:
+    ws = torch.empty((k_parts, M, w.N), dtype=torch.float32, device=a.device)
+  _lib.call('t5d_gemm_tiled', _s(), _lib.dtype_code(a.dtype), w.w_dtype,
+            _lib.dtype_code(out_dtype), a.data_ptr(), w.data.data_ptr(),
+            _lib.ptr(w.scales), _lib.ptr(residual), out.data_ptr(), M, K, w.N,
+            epi, _lib.ptr(ws), int(mp), int(nt), int(k_parts))
   return out
 
 

@@ -94,6 +94,61 @@ def test_gemm_bf16(ops, M, K, N, epi):
   np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
 
 
+BIG_TILES = [(2, 3), (2, 4), (2, 5), (4, 4), (4, 6), (4, 8), (8, 4), (8, 5),
+             (8, 8)]
+
+
+@pytest.mark.parametrize('mp,nt', BIG_TILES)
+@pytest.mark.parametrize('wdt', [torch.bfloat16, torch.int8])
+def test_gemm_large_tiles(ops, mp, nt, wdt):
+  """Every large-tile kernel (t5d_gemm_tiled) against the oracle's dense layer
+  and, bit for bit, against t5d_gemm on its small tiles (same split of K over
+  the wavefronts, same summation order), for the three epilogues, with rows
+  and columns that do not fill the last tile; then K split over 2 and 3
+  workgroups (float32 parts added by a second kernel) against the oracle."""
+  rs = np.random.RandomState(mp * 10 + nt + (wdt == torch.int8))
+  M, K, N = 100, 1088, 16 * (2 * nt + 1)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+  if wdt == torch.int8:
+    k0, k1 = ot5.quantize_int8(w0), ot5.quantize_int8(w1)
+  else:
+    k0, k1 = w0, w1
+  pw = ops.pack_weight(dev(w0), torch.bfloat16, wdt)
+  pg = ops.pack_weight(dev(w0), torch.bfloat16, wdt, gate_kernel=dev(w1))
+  plain = ot5.dense_general(host(a), k0, 'bfloat16')
+  want = {
+      'none': plain,
+      'residual': ot5.bf16_round(plain + host(res)),
+      'geglu': ot5.mlp_block(
+          {'wi_0': {'kernel': k0}, 'wi_1': {'kernel': k1},
+           'wo': {'kernel': np.eye(N, dtype=np.float32)}}, host(a),
+          ('gelu', 'linear'), 'bfloat16')}
+  for epi in ('none', 'residual', 'geglu'):
+    w = pg if epi == 'geglu' else pw
+    r = res if epi == 'residual' else None
+    got = ops.gemm_tiled(a, w, mp, nt, residual=r)
+    np.testing.assert_allclose(host(got), want[epi], atol=2e-2, rtol=2**-7)
+    assert torch.equal(got, ops.gemm(a, w, residual=r)), epi
+  f32 = ops.gemm_tiled(a, pw, mp, nt, out_dtype=torch.float32)
+  assert torch.equal(f32, ops.gemm(a, pw, out_dtype=torch.float32))
+  for k_parts in (2, 3):
+    got = ops.gemm_tiled(a, pw, mp, nt, k_parts, residual=res)
+    np.testing.assert_allclose(host(got), want['residual'], atol=2e-2,
+                               rtol=2**-7)
+
+
+def test_gemm_tiled_rejects_what_it_cannot_run(ops):
+  a = dev(np.zeros((16, 64), np.float32), torch.bfloat16)
+  pw = ops.pack_weight(dev(np.zeros((64, 64), np.float32)), torch.bfloat16)
+  with pytest.raises(ValueError, match='no kernel for a tile'):
+    ops.gemm_tiled(a, pw, 3, 3)
+  with pytest.raises(ValueError, match='a split over K needs'):
+    ops.gemm_tiled(a, pw, 2, 4, 2)  # no residual epilogue
+
+
 @pytest.mark.parametrize('M,K,N', [(1, 768, 768), (5, 256, 512), (32, 768, 2304),
                                    (128, 768, 768), (128, 768, 4096),
                                    (100, 1024, 1024), (128, 64, 48),
