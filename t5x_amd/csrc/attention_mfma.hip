@@ -110,8 +110,10 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
   if (a.units != nullptr) {
     const int u = a.units[b * a.H + h];
     T5D_GATE_TEST();  // after both scalar loads are in flight
-    h = u & 0xff;
-    b = (u >> 8) & 0xff;
+    // (clamped: a table that does not belong to this launch must not become
+    // an address)
+    h = min(u & 0xff, a.H - 1);
+    b = min((u >> 8) & 0xff, (int)gridDim.y - 1);
     n = (int)((uint32_t)u >> 16);
   } else {
     n = a.index[b];
