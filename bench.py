@@ -61,6 +61,10 @@ def parse_args():
                   help="'encoder': the once-per-batch stage before the decode "
                        'loop (encoder forward + cross K/V projection); a step '
                        'is one batch')
+  ap.add_argument('--replay-roofline', action='store_true',
+                  help='time the roofline kernel by back-to-back replay only '
+                       '(no decodes enqueued without it); for runs under '
+                       'hardware counters, which serialise every dispatch')
   ap.add_argument('--roofline-only', action='store_true',
                   help='only the dominant-kernel replay plus a plain copy of '
                        'known size (for counter runs under rocprofv3 --pmc)')
@@ -629,7 +633,8 @@ def main():
                  't_first': windows[-1][0], 't_last': windows[-1][1],
                  'timed_windows': [list(x) for x in windows],
                  'rows_x_steps_per_s': round(B * K * args.steps / elapsed, 1)},
-      'roofline': roofline_cross_attention(w),
+      'roofline': roofline_cross_attention(
+          w, in_loop=not args.replay_roofline),
   }
   # (the oracle's float32 copy of the XXL weights alone is 45 GB and minutes
   # of initialisation: no CPU figure for that shape)
