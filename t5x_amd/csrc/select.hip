@@ -1236,14 +1236,22 @@ sample_tokens_fast_kernel(SampleArgs a) {
   double sum = 0.0;
   float wtok = 0.f;
   bool mine = false;
+  // After a top-k / top-p mask all but a few elements are -1e7, and with a
+  // maximum this far above them exp(x - max) is exactly 0 in float32: chunks
+  // that are masked throughout add nothing and skip the four exponentials.
+  const bool far = mx > kNegInf + 1000.f;
 #pragma unroll
   for (int u = 0; u < 8; ++u) {
     const float4 w =
         a.rescale ? y[u] : (u * 1024 + tid < nvec ? x4[u * 1024 + tid] : kPad);
-    sum += (double)expf(w.x - mx);
-    sum += (double)expf(w.y - mx);
-    sum += (double)expf(w.z - mx);
-    sum += (double)expf(w.w - mx);
+    const bool masked = far && w.x <= kNegInf && w.y <= kNegInf &&
+                        w.z <= kNegInf && w.w <= kNegInf;
+    if (!masked) {
+      sum += (double)expf(w.x - mx);
+      sum += (double)expf(w.y - mx);
+      sum += (double)expf(w.z - mx);
+      sum += (double)expf(w.w - mx);
+    }
     const int j = 4 * (u * 1024 + tid);
     if (best.i == j) { wtok = w.x; mine = true; }
     if (best.i == j + 1) { wtok = w.y; mine = true; }
