@@ -61,6 +61,10 @@ def parse_args():
                   help="'encoder': the once-per-batch stage before the decode "
                        'loop (encoder forward + cross K/V projection); a step '
                        'is one batch')
+  ap.add_argument('--in-flight', type=int, default=None,
+                  help='also measure this many whole decodes of different '
+                       'batches running on the device at once (default: 3 '
+                       'for the default config, 0 = skip for the others)')
   ap.add_argument('--replay-roofline', action='store_true',
                   help='time the roofline kernel by back-to-back replay only '
                        '(no decodes enqueued without it); for runs under '
@@ -380,6 +384,70 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
   return out
 
 
+def in_flight_throughput(w, n, groups=3):
+  """Whole decodes of n different batches (same shape, same weights) running
+  on the device at once, each on its own streams, driven by one host thread
+  through the loops' start / poll protocol (chunks of 8 iterations enqueued
+  ahead, the loop flag read back without waiting): the throughput of
+  EncoderDecoderModel.predict_batches.  Like the single-decode figure, decode
+  starts are outside the clock; everything the loops do until the last one has
+  ended, read-backs and the iterations enqueued past the end included, is
+  inside."""
+  import torch
+  from t5x_amd import decoding, models, network
+  dev = w.encoded.device
+  fns = []
+  for i in range(n):
+    rs = np.random.Generator(np.random.PCG64(w.seed + 101 + i))
+    tok = rs.integers(2, 32128, size=(w.B, w.E)).astype(np.int32)
+    lens = rs.integers(w.enc_lens.min(), w.E + 1, size=(w.B,))
+    tok[np.arange(w.E)[None, :] >= lens[:, None]] = 0
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(w.seed + 201 + i)
+    encoded = torch.randn(tuple(w.encoded.shape), generator=gen,
+                          device=dev).to(w.encoded.dtype)
+    fns.append(models.StepFunction(
+        w.model, w.params, network.BeamShared(encoded, w.K),
+        network.BeamShared(torch.as_tensor(tok, device=dev), w.K), w.L))
+
+  def group():
+    loops = []
+    for i, fn in enumerate(fns):
+      cache = w.module.init_cache(w.B, w.L)
+      if w.loop_kind == 'beam':
+        loops.append(decoding.BeamLoop(w.inputs, cache, fn, eos_id=1,
+                                       num_decodes=w.K, alpha=0.6))
+      else:
+        _, temperature, topk = w.loop_kind
+        w.decodes += 1
+        loops.append(decoding.SampleLoop(
+            w.inputs, cache, fn, 1, w.seed + w.decodes, w.K, temperature,
+            topk, use_fused=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    decoding.run_in_flight(loops)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for loop in loops:
+      loop.finish()
+      count = int((loop.cur.cur_index if w.loop_kind == 'beam' else
+                   loop.fused.step_count).item())
+      if count != w.L:
+        raise RuntimeError(f'decode in flight stopped at step {count}')
+    return dt
+
+  w.loop = None
+  for _ in range(2):   # builds the n contexts; first pass of re-binding them
+    group()
+  seconds = sum(group() for _ in range(groups))
+  steps = groups * n * w.L
+  return {'decodes': n, 'value': round(w.B * steps / seconds, 1),
+          'unit': 'tokens/s', 'steps': steps,
+          'ms_per_step': round(seconds / steps * 1e3, 4),
+          'what': (f'{n} batches of the same shape decoding at once '
+                   '(separate streams, one host thread), whole decodes')}
+
+
 def copy_calibration(torch, nbytes=256 << 20, reps=5):
   """A plain device copy of known size, so FETCH_SIZE / WRITE_SIZE readings can
   be scaled: it reads nbytes and writes nbytes."""
@@ -638,6 +706,11 @@ def main():
   }
   # (the oracle's float32 copy of the XXL weights alone is 45 GB and minutes
   # of initialisation: no CPU figure for that shape)
+  n_in_flight = args.in_flight
+  if n_in_flight is None:
+    n_in_flight = 3 if args.config == DEFAULT_CONFIG else 0
+  if n_in_flight > 1:
+    out['in_flight'] = in_flight_throughput(w, n_in_flight)
   if not args.no_cpu_baseline and size != 'xxl':
     out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
   print(json.dumps(out))

@@ -18,6 +18,7 @@ caller that follows the protocol:
     (jax.random.categorical(key, x) == argmax(x + gumbel)).
 """
 
+import collections
 import dataclasses
 import functools
 from typing import Any, Callable, Mapping, Optional, Tuple, Union
@@ -300,18 +301,12 @@ def _noise_source(decode_rng):
 # ------------------------------------------------------------------------------
 
 
-def temperature_sample(
-    inputs, cache, tokens_to_logits, eos_id: int, decode_rng=None,
-    num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
-    topk: int = 1, topp: float = 0.0, cache_offset: int = 0,
-    initial_index=None, max_decode_steps=None,
-    max_decode_steps_hard_limit: Optional[int] = None,
-    rescale_log_probs: bool = True,
-    state_callback_fn: Optional[Callable] = None,
-    logit_callback_fn: Optional[Callable] = None,
-):
-  """:115-409 -> (decodes [B, num_decodes, L] i32, log_prob [B, num_decodes])
-  sorted ascending by log-prob."""
+def _sample_setup(inputs, cache, tokens_to_logits, num_decodes, cache_offset,
+                  initial_index, max_decode_steps,
+                  max_decode_steps_hard_limit, state_callback_fn,
+                  logit_callback_fn):
+  """:340-385, what temperature_sample does before its trial: the arguments of
+  the single trial (inputs, cache, initial_index, max_decode_steps, use_fused)."""
   if (max_decode_steps_hard_limit is not None and
       max_decode_steps_hard_limit > 0 and max_decode_steps is not None):
     max_decode_steps = np.minimum(max_decode_steps,
@@ -342,19 +337,16 @@ def temperature_sample(
           _dev(initial_index, torch.int32), num_decodes)
   else:
     expanded_inputs, expanded_cache = inputs, cache
+  return (expanded_inputs, expanded_cache, initial_index, max_decode_steps,
+          use_fused)
 
-  expanded_decodes, expanded_log_prob = _temperature_sample_single_trial(
-      expanded_inputs, expanded_cache, tokens_to_logits, eos_id, decode_rng,
-      num_decodes, temperature, topk, topp, initial_index=initial_index,
-      max_decode_steps=max_decode_steps, rescale_log_probs=rescale_log_probs,
-      state_callback_fn=state_callback_fn, logit_callback_fn=logit_callback_fn,
-      use_fused=use_fused)
 
-  batch_size = inputs.shape[0]
+def _sort_trials(expanded_decodes, expanded_log_prob, batch_size, num_decodes):
+  """:387-409, the trials of each batch item sorted ascending by log-prob."""
   decodes = unflatten_beam_dim(expanded_decodes, batch_size, num_decodes)
   log_prob = unflatten_beam_dim(expanded_log_prob, batch_size, num_decodes)
-  # :401-409 ascending, stable.  top_k of the negated scores is a stable
-  # descending order of -log_prob, i.e. a stable ascending order of log_prob.
+  # Ascending, stable.  top_k of the negated scores is a stable descending
+  # order of -log_prob, i.e. a stable ascending order of log_prob.
   if num_decodes > 1:
     _, idxs = ops.top_k((-log_prob).contiguous(), num_decodes)
     decodes = ops.gather_beams(decodes.contiguous(), idxs)
@@ -362,7 +354,173 @@ def temperature_sample(
   return decodes, log_prob
 
 
-class SampleLoop:
+def temperature_sample(
+    inputs, cache, tokens_to_logits, eos_id: int, decode_rng=None,
+    num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
+    topk: int = 1, topp: float = 0.0, cache_offset: int = 0,
+    initial_index=None, max_decode_steps=None,
+    max_decode_steps_hard_limit: Optional[int] = None,
+    rescale_log_probs: bool = True,
+    state_callback_fn: Optional[Callable] = None,
+    logit_callback_fn: Optional[Callable] = None,
+):
+  """:115-409 -> (decodes [B, num_decodes, L] i32, log_prob [B, num_decodes])
+  sorted ascending by log-prob."""
+  (expanded_inputs, expanded_cache, initial_index, max_decode_steps,
+   use_fused) = _sample_setup(
+       inputs, cache, tokens_to_logits, num_decodes, cache_offset,
+       initial_index, max_decode_steps, max_decode_steps_hard_limit,
+       state_callback_fn, logit_callback_fn)
+  expanded_decodes, expanded_log_prob = _temperature_sample_single_trial(
+      expanded_inputs, expanded_cache, tokens_to_logits, eos_id, decode_rng,
+      num_decodes, temperature, topk, topp, initial_index=initial_index,
+      max_decode_steps=max_decode_steps, rescale_log_probs=rescale_log_probs,
+      state_callback_fn=state_callback_fn, logit_callback_fn=logit_callback_fn,
+      use_fused=use_fused)
+  return _sort_trials(expanded_decodes, expanded_log_prob,
+                      np.shape(inputs)[0], num_decodes)
+
+
+def begin_temperature_sample(
+    inputs, cache, tokens_to_logits, eos_id: int, decode_rng=None,
+    num_decodes: int = 1, temperature: Union[float, np.ndarray] = 1.0,
+    topk: int = 1, topp: float = 0.0, cache_offset: int = 0,
+    initial_index=None, max_decode_steps=None,
+    max_decode_steps_hard_limit: Optional[int] = None,
+    rescale_log_probs: bool = True,
+    state_callback_fn: Optional[Callable] = None,
+    logit_callback_fn: Optional[Callable] = None,
+):
+  """temperature_sample set up but not run -> Decode."""
+  (expanded_inputs, expanded_cache, initial_index, max_decode_steps,
+   use_fused) = _sample_setup(
+       inputs, cache, tokens_to_logits, num_decodes, cache_offset,
+       initial_index, max_decode_steps, max_decode_steps_hard_limit,
+       state_callback_fn, logit_callback_fn)
+  loop = SampleLoop(expanded_inputs, expanded_cache, tokens_to_logits, eos_id,
+                    decode_rng, num_decodes, temperature, topk, topp,
+                    initial_index, max_decode_steps, rescale_log_probs,
+                    state_callback_fn, logit_callback_fn, use_fused)
+  return Decode(loop, functools.partial(_sort_trials,
+                                        batch_size=np.shape(inputs)[0],
+                                        num_decodes=num_decodes))
+
+
+temperature_sample.begin = begin_temperature_sample
+
+
+class Decode:
+  """A decode that has been set up but not necessarily run: the loop object
+  plus what turns the loop's final state into the function's return value.
+  `run()` runs it to its end; `start()` / `poll()` run it without waiting, so
+  that several can be in flight; `result()` is the decode function's return
+  value (it runs whatever is left of the loop)."""
+
+  def __init__(self, loop, epilogue=None):
+    self.loop, self._epilogue = loop, epilogue
+    self._result = None
+    self._ran = False
+
+  def run(self):
+    self.loop.run()
+    self._ran = True
+
+  def start(self, check_every: int = 8):
+    self.loop.start(check_every)
+
+  def poll(self, block: bool = False) -> bool:
+    if self._ran:
+      return True
+    self._ran = self.loop.poll(block)
+    return self._ran
+
+  def result(self):
+    if self._result is None:
+      if not self._ran:
+        if self.loop._tickets is None:
+          self.loop.run()
+        else:
+          while not self.loop.poll(block=True):
+            pass
+        self._ran = True
+      out = self.loop.finish()
+      self._result = out if self._epilogue is None else self._epilogue(*out)
+    return self._result
+
+
+class _InFlight:
+  """start() / poll() for a loop object: the loop runs on the device in chunks
+  of iterations, a few of them enqueued ahead, and the host only asks whether
+  the oldest chunk has ended and what the loop condition was then.  Nothing
+  here waits unless asked to, so one host thread can keep several decodes (each
+  on its own streams) in flight.  Iterations enqueued after the condition
+  turned false change nothing on the device, so the final state is the one the
+  plain loop reaches."""
+
+  finished = False   # set by finish(): the decode context may serve another loop
+  _ended = False
+  _tickets = None
+
+  def start(self, check_every: int = 8, ahead: int = 2):
+    """Begins running the loop; returns at once (without a fused step: after
+    running it to its end)."""
+    self._tickets = collections.deque()
+    if self.fused is None:
+      self.run()
+      self._ended = True
+      return
+    if ahead > self.fused.CHUNK_SLOTS:
+      raise ValueError(f'at most {self.fused.CHUNK_SLOTS} chunks ahead')
+    self._check_every = int(check_every)
+    if not self.cond():
+      self._ended = True
+      return
+    for _ in range(ahead):
+      self._push_chunk()
+
+  def _push_chunk(self):
+    ticket = self.fused.launch_chunk(self._check_every)
+    if ticket is not None:
+      self._tickets.append(ticket)
+      self.step += self._check_every
+
+  def poll(self, block: bool = False) -> bool:
+    """True once the loop has ended (finish() then returns its results).
+    Enqueues further chunks as earlier ones end; with `block`, first waits
+    for the oldest chunk in flight."""
+    if self._tickets is None:
+      raise ValueError('poll() before start()')
+    while not self._ended:
+      if not self._tickets:  # nothing left to enqueue
+        self._ended = True
+        break
+      running = self.fused.chunk_running(self._tickets[0], block)
+      block = False
+      if running is None:
+        break
+      self._tickets.popleft()
+      if running:
+        self._push_chunk()
+      else:
+        self._ended = True
+        self._tickets.clear()
+    return self._ended
+
+
+def run_in_flight(loops, check_every: int = 8):
+  """Runs loop objects (BeamLoop, SampleLoop, or anything with start / poll)
+  to their ends together: all are started, then the host waits on one of them
+  at a time while keeping the others fed."""
+  loops = list(loops)
+  for loop in loops:
+    loop.start(check_every)
+  pending = [l for l in loops if not l.poll()]
+  while pending:
+    pending[0].poll(block=True)
+    pending = [l for l in pending if not l.poll()]
+
+
+class SampleLoop(_InFlight):
   """The loop of _temperature_sample_single_trial (:412-715) as an object:
   `cond()` / `body()` are the while-loop's condition and body, `finish()` the
   epilogue; `advance(n)` runs n iterations without reading the condition back
@@ -435,7 +593,8 @@ class SampleLoop:
           max_decode_len=self.mdl, initial_eos_count=self.eos0,
           temperature=self.temps_dev, all_ended=self.all_ended, eos_id=eos_id,
           topk=topk, topp=topp, rescale=rescale_log_probs,
-          noise_source=self.source if self.any_sampling else None)
+          noise_source=self.source if self.any_sampling else None,
+          owner=self)
 
   def _loop_state(self):
     return SamplingLoopState(
@@ -502,9 +661,13 @@ class SampleLoop:
   def finish(self):
     if self.fused is not None:
       self.fused.finish()
+      if self._tickets is not None:  # ran in chunks: iterations executed
+        self.step = int(self.fused.step_count.item())
       # the context's buffers serve the next call too: hand out copies
-      return (self.fused.sequences[:, 1:-1].clone(),
-              self.fused.log_prob.clone())
+      out = (self.fused.sequences[:, 1:-1].clone(),
+             self.fused.log_prob.clone())
+      self.finished = True
+      return out
     if self.state_callback_fn is not None:
       st = self.state_callback_fn(self._loop_state())
       self.sequences = _dev(st.sequences, torch.int32)
@@ -589,7 +752,7 @@ def beam_init(batch_size, beam_size, max_decode_len, cache, offset=0,
   return st, beam_cache
 
 
-class BeamLoop:
+class BeamLoop(_InFlight):
   """The beam_search loop (:1131-1569) as an object: `cond()` / `body()` are
   the while-loop's condition and body, `finish()` the epilogue.  beam_search()
   below is `while loop.cond(): loop.body()`; exposing the pieces lets a caller
@@ -769,7 +932,21 @@ class BeamLoop:
       finished_seqs = torch.as_tensor(np.ascontiguousarray(seqs), device=dev)
     else:
       finished_seqs = finished_seqs[:, :, 1:]  # :1567
+    self.finished = True
     return finished_seqs, finished_scores
+
+
+def begin_beam_search(
+    inputs, cache, tokens_to_logits, eos_id: int, num_decodes: int = 4,
+    alpha: float = 0.6, max_decode_len: Optional[int] = None,
+    max_decode_step: int = -1, min_log_prob: float = NEG_INF_VALUE,
+    decode_rng=None, cache_offset: int = 0, initial_index=None,
+):
+  """beam_search (:1131-1569) set up but not run -> Decode."""
+  del decode_rng
+  return Decode(BeamLoop(inputs, cache, tokens_to_logits, eos_id, num_decodes,
+                         alpha, max_decode_len, max_decode_step, min_log_prob,
+                         cache_offset, initial_index))
 
 
 def beam_search(
@@ -780,9 +957,12 @@ def beam_search(
 ):
   """:1131-1569 -> (sequences [B, K, L] i32, scores [B, K] f32), the beam axis
   sorted ascending by score."""
-  del decode_rng
-  loop = BeamLoop(inputs, cache, tokens_to_logits, eos_id, num_decodes, alpha,
-                  max_decode_len, max_decode_step, min_log_prob, cache_offset,
-                  initial_index)
-  loop.run()  # :1509
-  return loop.finish()
+  decode = begin_beam_search(inputs, cache, tokens_to_logits, eos_id,
+                             num_decodes, alpha, max_decode_len,
+                             max_decode_step, min_log_prob, decode_rng,
+                             cache_offset, initial_index)
+  decode.run()  # :1509
+  return decode.result()
+
+
+beam_search.begin = begin_beam_search

@@ -15,6 +15,8 @@ One process drives one GPU here, so "partitioning" reduces to the data layout
 object with `as_numpy_iterator()` such as a tf.data.Dataset).
 """
 
+import collections
+import functools
 import inspect
 from typing import Any, Callable, Mapping, Optional, Sequence
 
@@ -72,10 +74,33 @@ def _stack(examples):
                   examples[0], *examples[1:])
 
 
+def _begin_of(infer_step):
+  """`begin_<name>` of the object whose bound method `infer_step` is (through
+  functools.partial wrappers), with the wrappers' arguments bound again: the
+  variant of the step that returns, without waiting, an object with poll() and
+  result().  None when there is no such variant."""
+  fn, args, kwargs = infer_step, (), {}
+  while isinstance(fn, functools.partial):
+    args, kwargs = fn.args + args, {**fn.keywords, **kwargs}
+    fn = fn.func
+  begin = getattr(getattr(fn, '__self__', None),
+                  'begin_' + getattr(fn, '__name__', ''), None)
+  if begin is None:
+    return None
+  return functools.partial(begin, *args, **kwargs)
+
+
 def get_infer_fn(infer_step: Callable, batch_size: int,
                  train_state_axes: Any = None, partitioner: Any = None,
-                 keep_aux_as_numpy: bool = False):
-  """t5x/utils.py:1543-1817 -> infer_fn(ds, train_state, rng=None)."""
+                 keep_aux_as_numpy: bool = False,
+                 decodes_in_flight: int = 1):
+  """t5x/utils.py:1543-1817 -> infer_fn(ds, train_state, rng=None).
+
+  `decodes_in_flight` (no counterpart in the reference): when `infer_step` is
+  `predict_batch` / `predict_batch_with_aux` of a model that can start a
+  prediction without waiting for it, up to that many batches decode on the
+  device at once (each holds its own caches and cross K/V); each batch's
+  result is unchanged.  1: one batch after the other, as the reference."""
   del train_state_axes  # one device: parameters are not partitioned
   params_of_step = inspect.signature(infer_step).parameters
   takes_rng = 'rng' in params_of_step
@@ -119,6 +144,19 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
     batched_results, all_indices = [], []
     params = getattr(train_state, 'params', train_state)
     mutables = getattr(train_state, 'flax_mutables', None)
+    begin = _begin_of(infer_step) if decodes_in_flight > 1 else None
+    if takes_mutables or 'rng' not in params_of_step:
+      begin = None
+    in_flight = collections.deque()
+
+    def collect_oldest():
+      oldest = in_flight[0]
+      while not oldest.poll():
+        for other in list(in_flight)[1:]:
+          other.poll()
+        oldest.poll(block=True)
+      batched_results.append(in_flight.popleft().result())
+
     for i in range(n_batches):
       chunk = shard[i * per_shard_batch_size:(i + 1) * per_shard_batch_size]
       index = np.asarray([c[0] for c in chunk], dtype=np.int64)
@@ -127,12 +165,20 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
         step_rng = None
       else:
         step_rng, rng = split_rng(rng)
+      if begin is not None:
+        in_flight.append(begin(params, infer_batch, step_rng))
+        all_indices.append(index)
+        while len(in_flight) >= decodes_in_flight:
+          collect_oldest()
+        continue
       batch_indices, batch_result = infer_step_with_indices(
           params, infer_batch, step_rng, index, mutables)
       # Results stay on the device until everything is enqueued; the copies
       # below are what the reference's copy_to_host_async overlaps.
       batched_results.append(batch_result)
       all_indices.append(batch_indices)
+    while in_flight:
+      collect_oldest()
 
     batched_results = [tree_map(_to_numpy, r) for r in batched_results]
     all_inferences = tree_map(lambda *xs: np.concatenate(xs),

@@ -4,6 +4,7 @@
 Arrays are torch tensors on the GPU; NumPy inputs are uploaded.
 """
 
+import collections
 import dataclasses
 import functools
 import inspect
@@ -126,6 +127,43 @@ class EncoderDecoderModel:
       return_all_decodes: bool = None, num_decodes: int = None,
       prompt_with_targets: bool = False):
     """t5x/models.py:584-758."""
+    return self.begin_predict_batch_with_aux(
+        params, batch, rng, decoder_params, return_all_decodes, num_decodes,
+        prompt_with_targets).result()
+
+  def begin_predict_batch(self, params, batch, rng=None):
+    """predict_batch set up and started but not waited for -> Prediction."""
+    return self.begin_predict_batch_with_aux(params, batch, rng).first()
+
+  def predict_batches(self, params, batches, rngs=None, in_flight: int = 3,
+                      **kwargs):
+    """predict_batch_with_aux over an iterable of batches, yielding each
+    batch's result in order, with up to `in_flight` decodes running on the
+    device at once (each on its own streams): the device spends most of a
+    decode step of one batch waiting on dependent launches, which the other
+    batches' steps fill.  Every batch's result is what predict_batch_with_aux
+    returns for it alone.  `rngs`: one per batch, or None.  With decode
+    functions other than beam_search / temperature_sample the batches run one
+    after the other."""
+    rngs = iter(rngs) if rngs is not None else None
+    active = collections.deque()
+    for batch in batches:
+      rng = next(rngs) if rngs is not None else None
+      active.append(self.begin_predict_batch_with_aux(params, batch, rng,
+                                                      **kwargs))
+      while len(active) >= max(1, in_flight):
+        yield _wait_for_oldest(active)
+    while active:
+      yield _wait_for_oldest(active)
+
+  def begin_predict_batch_with_aux(
+      self, params, batch, rng=None,
+      decoder_params: Optional[MutableMapping[str, Any]] = None,
+      return_all_decodes: bool = None, num_decodes: int = None,
+      prompt_with_targets: bool = False):
+    """predict_batch_with_aux (t5x/models.py:584-758) up to and including the
+    start of its decode loop -> Prediction; `.result()` is the method's return
+    value."""
     if return_all_decodes is None:
       return_all_decodes = self._default_decoder_params.return_all_decodes
     if num_decodes is None:
@@ -181,11 +219,86 @@ class EncoderDecoderModel:
     scanned = hasattr(self.module, 'scan_layers') and self.module.scan_layers
     if 'eos_id' not in decoder_params:
       decoder_params['eos_id'] = self.output_vocabulary.eos_id or 1
-    decodes, scores = self._decode_fn(
+    decode_kwargs = dict(
         inputs=decoder_prompt_inputs, cache=cache,
         tokens_to_logits=tokens_ids_to_logits, num_decodes=num_decodes,
         cache_offset=1 if scanned else 0, **decoder_params)
+    begin, bound = _begin_of(self._decode_fn)
+    if begin is None:  # some other decode function: it runs here and now
+      decode = decoding.Decode(_Ran(self._decode_fn(**decode_kwargs)))
+    else:
+      decode = begin(**bound, **decode_kwargs)
+      decode.start()
+    return Prediction(decode, return_all_decodes)
 
-    if return_all_decodes:
-      return decodes, {'scores': scores}
-    return decodes[:, -1, :], {'scores': scores[:, -1]}
+
+def _begin_of(decode_fn):
+  """The `begin` variant of a decode function (what decoding.beam_search and
+  temperature_sample carry) behind any functools.partial wrappers, and the
+  keyword arguments those wrappers bind; (None, {}) if there is none."""
+  fn, bound = decode_fn, {}
+  while isinstance(fn, functools.partial):
+    if fn.args:
+      return None, {}
+    bound = {**fn.keywords, **bound}
+    fn = fn.func
+  begin = getattr(fn, 'begin', None)
+  return (begin, bound) if begin is not None else (None, {})
+
+
+class _Ran:
+  """A decode loop that has already run: the loop interface over its result."""
+  _tickets = None
+
+  def __init__(self, result):
+    self._result = result
+
+  def run(self):
+    pass
+
+  def start(self, check_every=8):
+    del check_every
+
+  def poll(self, block=False):
+    del block
+    return True
+
+  def finish(self):
+    return self._result
+
+
+class Prediction:
+  """A predict_batch_with_aux call whose decode loop may still be running on
+  the device.  poll(): has it ended (never waits unless `block`); result():
+  the call's return value (waits)."""
+
+  def __init__(self, decode, return_all_decodes, first_only=False):
+    self._decode = decode
+    self._all, self._first_only = return_all_decodes, first_only
+
+  def first(self):
+    """The same prediction, with predict_batch's return value."""
+    return Prediction(self._decode, self._all, first_only=True)
+
+  def poll(self, block: bool = False) -> bool:
+    return self._decode.poll(block)
+
+  def result(self):
+    decodes, scores = self._decode.result()
+    if self._all:
+      out = decodes, {'scores': scores}
+    else:
+      out = decodes[:, -1, :], {'scores': scores[:, -1]}
+    return out[0] if self._first_only else out
+
+
+def _wait_for_oldest(active):
+  """Waits for the oldest of the predictions in flight, polling the others so
+  that their loops stay fed; removes it and returns its result."""
+  oldest = active[0]
+  while not oldest.poll():
+    for other in list(active)[1:]:
+      other.poll()
+    oldest.poll(block=True)
+  active.popleft()
+  return oldest.result()

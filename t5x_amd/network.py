@@ -13,6 +13,7 @@ the layers it uses (t5x/examples/t5/layers.py).  What runs where:
 """
 
 import dataclasses
+import weakref
 from typing import Any, Mapping, Optional, Sequence
 
 import numpy as np
@@ -260,6 +261,7 @@ class Transformer:
     self._cross = None
     self._step_cache = None
     self._beam_ctx = {}
+    self._streams = None
 
   # -- plumbing ---------------------------------------------------------------
   def _dev(self):
@@ -561,25 +563,68 @@ class Transformer:
            int(loop.eos_id), float(loop.min_brevity), float(loop.min_log_prob),
            int(loop.max_decode_step), int(loop.min_initial),
            int(self.decode_lanes))
-    ctx = self._beam_ctx.get(key)
-    if ctx is not None and ctx.w is not w:  # an id reused by other weights
+    return self._decode_context(
+        key, w, loop,
+        make=lambda slot: FusedBeamStep(self, loop, params, encoded,
+                                        enc_tokens, slot=slot),
+        rebind=lambda ctx: ctx.rebind(loop, encoded, enc_tokens))
+
+  # Decode contexts of one (weights, shapes, options) key that are kept for
+  # re-binding: more than one only when several decodes are in flight at once.
+  MAX_CONTEXTS_PER_KEY = 4
+
+  def _decode_context(self, key, w, owner, make, rebind):
+    """A decode context for `owner` (the loop object that will drive it): a
+    kept one of this key that no live, unfinished loop owns any more, re-bound,
+    or a new one.  Contexts are kept in small pools per key, so that a caller
+    who keeps several decodes in flight (each on its own stream) pays for
+    their allocation and graph capture once.  make(slot) builds a context for
+    pool slot `slot`, whose stream is decode_stream(slot)."""
+    pool = self._beam_ctx.get(key)
+    if pool and pool[0].w is not w:  # an id reused by other weights
       del self._beam_ctx[key]
-      ctx = None
-    if ctx is not None:
-      ctx.rebind(loop, encoded, enc_tokens)
-      return ctx
-    ctx = FusedBeamStep(self, loop, params, encoded, enc_tokens)
-    if len(self._beam_ctx) >= 2:  # a context holds the caches: keep few
-      self._beam_ctx.pop(next(iter(self._beam_ctx)))
-    self._beam_ctx[key] = ctx
+      pool = None
+    if pool is None:
+      if len(self._beam_ctx) >= 2:  # a context holds the caches: keep few
+        self._beam_ctx.pop(next(iter(self._beam_ctx)))
+      pool = self._beam_ctx[key] = []
+    for ctx in pool:
+      if ctx.is_free():
+        rebind(ctx)
+        ctx.claim(owner)
+        return ctx
+    ctx = make(len(pool))
+    ctx.claim(owner)
+    if len(pool) < self.MAX_CONTEXTS_PER_KEY:
+      pool.append(ctx)
     return ctx
 
+  def decode_stream(self, slot):
+    """The stream of the decode contexts in pool slot `slot`.  The device
+    runs streams side by side only when they sit on different hardware
+    queues, of which a process has few (4 by default) and which streams are
+    given in turn as they are first used; so the module makes its streams
+    once, together, and uses each once right away: consecutive slots then sit
+    on different queues whatever streams the caller makes in between."""
+    if self._streams is None:
+      dev = self._dev()
+      self._streams = [torch.cuda.Stream(device=dev)
+                       for _ in range(self.MAX_CONTEXTS_PER_KEY)]
+      touch = torch.zeros((16,), dtype=torch.int32, device=dev)
+      torch.cuda.current_stream().synchronize()
+      for stream in self._streams:
+        with torch.cuda.stream(stream):
+          touch.zero_()
+        stream.synchronize()
+    return self._streams[slot % len(self._streams)]
 
   # -- fused sampling: one graph replay per loop iteration --------------------------
-  def make_fused_sample_step(self, params, encoded, enc_tokens, **kw):
+  def make_fused_sample_step(self, params, encoded, enc_tokens, owner=None,
+                             **kw):
     """Returns a FusedSampleStep (see there for the arguments).  Like the beam
     contexts, the step object is kept per (weights, shapes, options) and
-    re-bound to the next call's state."""
+    re-bound to the next call's state; `owner` is the loop object that drives
+    it (a context without owner is free for the next call at once)."""
     beams = encoded.beams if isinstance(encoded, BeamShared) else 1
     enc = encoded.x if isinstance(encoded, BeamShared) else encoded
     rows = kw['sequences'].shape[0]
@@ -591,21 +636,63 @@ class Transformer:
            tuple(kw['sequences'].shape), int(kw['eos_id']), int(kw['topk']),
            float(kw['topp']), bool(kw['rescale']),
            kw.get('noise_source') is not None)
-    ctx = self._beam_ctx.get(key)
-    if ctx is not None and ctx.w is not w:
-      del self._beam_ctx[key]
-      ctx = None
-    if ctx is not None:
-      ctx.rebind(encoded, enc_tokens, **kw)
-      return ctx
-    ctx = FusedSampleStep(self, params, encoded, enc_tokens, **kw)
-    if len(self._beam_ctx) >= 2:
-      self._beam_ctx.pop(next(iter(self._beam_ctx)))
-    self._beam_ctx[key] = ctx
-    return ctx
+    return self._decode_context(
+        key, w, owner,
+        make=lambda slot: FusedSampleStep(self, params, encoded, enc_tokens,
+                                          slot=slot, **kw),
+        rebind=lambda ctx: ctx.rebind(encoded, enc_tokens, **kw))
 
 
-class FusedSampleStep:
+class _OwnedContext:
+  """What the kept decode contexts share: who drives them, and chunks of
+  iterations whose end the host can ask about without waiting.
+
+  A context is free for the next decode when nothing owns it, its owner is
+  gone, or its owner has finished (`owner.finished`); contexts never keep
+  their loop alive."""
+
+  CHUNK_SLOTS = 4  # chunks a caller may have outstanding per context
+  _owner = None
+  _flag_host = None
+  _n_chunks = 0
+
+  def claim(self, owner):
+    self._owner = None if owner is None else weakref.ref(owner)
+
+  def is_free(self) -> bool:
+    if self._owner is None:
+      return True
+    owner = self._owner()
+    return owner is None or bool(getattr(owner, 'finished', False))
+
+  def _end_chunk(self, flag, stream):
+    """After a chunk of iterations was enqueued on `stream`: copies the
+    device flag to pinned host memory and records an event behind it.
+    Returns the ticket for _chunk_flag()."""
+    if self._flag_host is None:
+      self._flag_host = torch.zeros((self.CHUNK_SLOTS,), dtype=torch.int32,
+                                    pin_memory=True)
+      self._chunk_events = [torch.cuda.Event()
+                            for _ in range(self.CHUNK_SLOTS)]
+    slot = self._n_chunks % self.CHUNK_SLOTS
+    self._n_chunks += 1
+    with torch.cuda.stream(stream):
+      self._flag_host[slot:slot + 1].copy_(flag.reshape(1), non_blocking=True)
+    self._chunk_events[slot].record(stream)
+    return slot
+
+  def _chunk_flag(self, ticket, block=False):
+    """The flag as the chunk left it, or None while the chunk is running
+    (block: wait for it)."""
+    event = self._chunk_events[ticket]
+    if block:
+      event.synchronize()
+    elif not event.query():
+      return None
+    return int(self._flag_host[ticket])
+
+
+class FusedSampleStep(_OwnedContext):
   """Whole temperature_sample iterations as replays of one captured HIP graph
   (decoder step on the current tokens, token choice, bookkeeping, loop flag).
   Owns the self-attention caches of its rows as one block
@@ -616,7 +703,7 @@ class FusedSampleStep:
   def __init__(self, module, params, encoded, enc_tokens, *, sequences,
                cur_index, cur_token, ended, log_prob, max_decode_len,
                initial_eos_count, temperature, all_ended, eos_id, topk, topp,
-               rescale, noise_source=None, ring=8):
+               rescale, noise_source=None, ring=8, slot=0):
     from t5x_amd import _lib
     self._lib = _lib
     cfg, dev = module.config, module._dev()
@@ -687,7 +774,7 @@ class FusedSampleStep:
     self.sample = st
     self._keepalive = (sequences, cur_index, cur_token, ended, log_prob,
                        max_decode_len, initial_eos_count, temperature)
-    self.stream = torch.cuda.Stream(device=dev)
+    self.stream = module.decode_stream(slot)
     self.graph = None
     self.step = 0
     self._capture()
@@ -766,19 +853,19 @@ class FusedSampleStep:
     for _ in range(n):
       self._lib.call('t5d_graph_launch', graph, self.stream.cuda_stream)
 
-  def advance(self, n):
+  def advance(self, n, wait=True):
     """Enqueues n more iterations (fewer when the longest row ends sooner),
-    refilling the noise ring for each group of `ring` steps; the host waits
-    for a group only when it has to overwrite its noise."""
+    refilling the noise ring for each group of `ring` steps.  The refills are
+    enqueued on the loop's stream, behind the iterations that read the slots
+    they overwrite; with `wait` the host also stays at most one ring ahead of
+    the device."""
     lib = self._lib
     with torch.cuda.stream(self.stream):
       todo = min(int(n), self.max_steps - self.step)
       while todo > 0:
-        # up to the next multiple of `ring`: a refill never overwrites noise
-        # of a step that is enqueued but not yet executed
         m = min(todo, self.ring - self.step % self.ring)
         if self.noise is not None:
-          if self.step % self.ring == 0:
+          if wait and self.step % self.ring == 0:
             self.stream.synchronize()
           for step in range(self.step, self.step + m):
             g = self.noise_source.noise(step, tuple(self.noise.shape[1:]))
@@ -793,6 +880,20 @@ class FusedSampleStep:
     """The loop condition (not every row ended), read back from the device."""
     self.stream.synchronize()
     return not bool(self.all_ended.item())
+
+  def launch_chunk(self, n):
+    """Enqueues up to n iterations without waiting for anything and returns a
+    ticket for chunk_running(); None when the loop has no iterations left."""
+    if self.step >= self.max_steps:
+      return None
+    self.advance(n, wait=False)
+    return self._end_chunk(self.all_ended, self.stream)
+
+  def chunk_running(self, ticket, block=False):
+    """Whether the loop condition still held after that chunk; None while the
+    chunk is running (block: wait for it)."""
+    flag = self._chunk_flag(ticket, block)
+    return None if flag is None else flag == 0
 
   def finish(self):
     self.stream.synchronize()
@@ -900,13 +1001,16 @@ class _BeamLane:
       bs.cache_slot, bs.cache_src, bs.cache_dst = (
           P(self.cache_slot), P(self.cache_src), P(self.cache_dst))
     self.beam = bs
-    self.stream = torch.cuda.Stream(device=dev)
+    # the first lane runs on the pool slot's stream; further lanes (an option
+    # for one decode at a time) on streams of their own
+    self.stream = (module.decode_stream(owner.slot) if index == 0 else
+                   torch.cuda.Stream(device=dev))
     self.event = torch.cuda.Event()
     self.graph = None
     self.graph_long = None
 
 
-class FusedBeamStep:
+class FusedBeamStep(_OwnedContext):
   """Whole beam-search iterations as replays of captured HIP graphs.
 
   The batch is cut into lanes (batch items never interact in beam search).
@@ -921,11 +1025,13 @@ class FusedBeamStep:
   without the host.  Iterations enqueued after the flag turned 0 change
   nothing, so the host may look at it only every few iterations."""
 
-  def __init__(self, module, loop, params, encoded, enc_tokens, lanes=None):
+  def __init__(self, module, loop, params, encoded, enc_tokens, lanes=None,
+               slot=0):
     from t5x_amd import _lib
     self._lib = _lib
     cfg, dev = module.config, module._dev()
-    self.module, self.loop, self.device = module, loop, dev
+    self.module, self.device = module, dev
+    self.loop = loop
     w = module.decoder_weights(params)
     enc_tok = enc_tokens.x
     enc_tok = torch.as_tensor(np.asarray(enc_tok), device=dev) if not isinstance(
@@ -966,6 +1072,7 @@ class FusedBeamStep:
       lanes = module.decode_lanes
     n = max(1, min(int(lanes), B))
     self.n_lanes = n
+    self.slot = slot
     bounds = [B * i // n for i in range(n + 1)]
     self.lane_cur_index = loop.cur.cur_index.to(torch.int32).reshape(1).repeat(n)
     self.cond_event = torch.cuda.Event()
@@ -979,6 +1086,15 @@ class FusedBeamStep:
     self.lanes = [_BeamLane(self, i, bounds[i], bounds[i + 1], w, cross)
                   for i in range(n)]
     self._capture()
+
+  @property
+  def loop(self):
+    """The loop bound to this context (None once it is gone)."""
+    return self._loop()
+
+  @loop.setter
+  def loop(self, loop):
+    self._loop = weakref.ref(loop)
 
   _STATE_FIELDS = ('cur_index', 'live_logprobs', 'finished_scores', 'live_seqs',
                    'finished_seqs', 'finished_flags')
@@ -1124,6 +1240,20 @@ class FusedBeamStep:
       self.cond_event.record(first)
       for lane in lanes[1:]:
         lane.stream.wait_event(self.cond_event)
+
+  def launch_chunk(self, n):
+    """launch(n), and a ticket for chunk_running().  (The loop condition
+    bounds the loop: there is always a next iteration to enqueue.)"""
+    self.launch(n)
+    # the last condition of a chunk is evaluated on the first lane's stream
+    # after all lanes joined; a single lane's kernels are on that stream too
+    return self._end_chunk(self.flag, self.lanes[0].stream)
+
+  def chunk_running(self, ticket, block=False):
+    """Whether the loop condition still held after that chunk; None while the
+    chunk is running (block: wait for it)."""
+    flag = self._chunk_flag(ticket, block)
+    return None if flag is None else flag != 0
 
   def synchronize(self):
     for lane in self.lanes:

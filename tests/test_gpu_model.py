@@ -23,6 +23,7 @@ logit tolerance.
 """
 
 import functools
+import time
 import types
 
 import numpy as np
@@ -494,6 +495,112 @@ def test_fused_loop_context_is_reused_across_batches(dtype):
     assert int(fused.cur.cur_index.item()) == int(plain.cur.cur_index.item())
     assert torch.equal(torch.as_tensor(got), torch.as_tensor(want)), batch
     assert torch.equal(torch.as_tensor(gs), torch.as_tensor(ws)), batch
+
+
+@pytest.mark.parametrize('dtype,decode_fn_name,kw,lanes', [
+    ('bfloat16', 'beam_search', dict(alpha=0.6), 1),
+    ('bfloat16', 'beam_search', dict(alpha=0.6), 2),
+    ('float32', 'beam_search', dict(alpha=0.6), 1),
+    ('bfloat16', 'temperature_sample', dict(temperature=0.0), 1),
+    ('bfloat16', 'temperature_sample', dict(temperature=0.8, topk=20), 1),
+])
+def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
+                                                    lanes):
+  """Seven batches through predict_batches with three decodes in flight on the
+  device: every batch's tokens and scores are bit-identical to
+  predict_batch_with_aux on that batch alone, in order, although the loops
+  (of different lengths: an EOS-heavy vocabulary column ends some early)
+  interleave, and three kept contexts serve all seven."""
+  from t5x_amd import network
+  ocfg, _, gm = _models(dtype, decode_fn_name, **kw)
+  gm.module.decode_lanes = lanes
+  dev = torch.device('cuda')
+  params = network.init_params(gm.module.config, 11, dev)
+  params['decoder']['logits_dense']['kernel'][:, 1] *= 3.0
+  rs = np.random.RandomState(8)
+  B, E, L = 4, 24, 19
+  batches = [{'encoder_input_tokens': ragged_tokens(rs, B, E, ocfg.vocab_size,
+                                                    3),
+              'decoder_input_tokens': np.zeros((B, L), np.int32)}
+             for _ in range(7)]
+  sampling = decode_fn_name == 'temperature_sample'
+  n = 1 if sampling else 4
+  rngs = list(range(40, 47)) if sampling else None
+  common = dict(num_decodes=n, return_all_decodes=True)
+  want = [gm.predict_batch_with_aux(
+      params, b, rng=None if rngs is None else rngs[i], **common)
+          for i, b in enumerate(batches)]
+  if not kw.get('temperature'):
+    lengths = {int((host(w[0]) != 0).sum(-1).max()) for w in want}
+    assert len(lengths) > 1, lengths   # the loops do differ in length
+  gm.module._beam_ctx.clear()
+  got = list(gm.predict_batches(params, batches, rngs, in_flight=3, **common))
+  assert len(got) == len(want)
+  for i, ((gd, ga), (wd, wa)) in enumerate(zip(got, want)):
+    assert torch.equal(gd, wd), i
+    assert torch.equal(ga['scores'], wa['scores']), i
+  pools = list(gm.module._beam_ctx.values())
+  assert len(pools) == 1 and len(pools[0]) == 3
+  # afterwards every context is free again: one more batch re-binds the first
+  again = gm.predict_batch_with_aux(
+      params, batches[2], rng=None if rngs is None else rngs[2], **common)
+  assert torch.equal(again[0], want[2][0])
+  assert len(pools[0]) == 3
+
+
+def test_loops_in_flight_with_poll_equal_run():
+  """BeamLoop.start / poll (chunks enqueued ahead, the flag read without
+  waiting) against BeamLoop.run, two loops interleaved by hand, and
+  decoding.run_in_flight over three."""
+  from t5x_amd import decoding, models, network
+  B, K, E, L = 3, 4, 16, 27
+  _, gcfg = tiny('bfloat16')
+  dev = torch.device('cuda')
+  params = network.init_params(gcfg, 3, dev, with_encoder=False)
+  params['decoder']['logits_dense']['kernel'][:, 1] *= 3.0
+  module = network.Transformer(gcfg, dev)
+  model = models.EncoderDecoderModel(module, decode_fn=decoding.beam_search)
+  inputs = np.zeros((B, L), np.int32)
+
+  def step_fn(seed):
+    rs = np.random.RandomState(seed)
+    tok = torch.as_tensor(ragged_tokens(rs, B, E, gcfg.vocab_size, 3),
+                          device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    encoded = torch.randn((B, E, gcfg.emb_dim), generator=gen,
+                          device=dev).to(torch.bfloat16)
+    return models.StepFunction(model, params, network.BeamShared(encoded, K),
+                               network.BeamShared(tok, K), L)
+
+  def new_loop(seed):
+    return decoding.BeamLoop(inputs, module.init_cache(B, L), step_fn(seed),
+                             eos_id=1, num_decodes=K)
+
+  want = []
+  for seed in (1, 2, 3):
+    loop = new_loop(seed)
+    loop.run()
+    want.append(loop.finish())
+  a, b = new_loop(1), new_loop(2)
+  assert a.fused is not b.fused
+  a.start(check_every=3)
+  b.start(check_every=5)
+  with pytest.raises(ValueError):
+    new_loop(3).poll()
+  done = [False, False]
+  deadline = time.monotonic() + 60
+  while not all(done) and time.monotonic() < deadline:
+    done = [a.poll(), b.poll()]
+  assert all(done)
+  for loop, (ws, wsc) in zip((a, b), want):
+    gs, gsc = loop.finish()
+    assert torch.equal(gs, ws) and torch.equal(gsc, wsc)
+  loops = [new_loop(seed) for seed in (1, 2, 3)]
+  decoding.run_in_flight(loops)
+  for loop, (ws, wsc) in zip(loops, want):
+    gs, gsc = loop.finish()
+    assert torch.equal(gs, ws) and torch.equal(gsc, wsc)
 
 
 class _SuppliedNoise:

@@ -141,3 +141,133 @@ def test_cache_room_check_on_host_tensors():
     decoding._check_cache_room(mk(16, 0), 17, expect_empty=True)
   with pytest.raises(ValueError, match='already holds decode steps'):
     decoding._check_cache_room(mk(16, 5), 16, expect_empty=True)
+
+
+# ---- several decodes in flight: host protocol (no GPU) ---------------------------
+
+
+class _FakePrediction:
+  """What begin_predict_batch returns, with a scripted number of polls."""
+  log = []
+
+  def __init__(self, name, polls_needed, value):
+    self.name, self.left, self.value = name, polls_needed, value
+
+  def poll(self, block=False):
+    self.log.append((self.name, 'block' if block else 'poll'))
+    if block:
+      self.left = 0
+    else:
+      self.left = max(0, self.left - 1)
+    return self.left == 0
+
+  def result(self):
+    assert self.left == 0
+    self.log.append((self.name, 'result'))
+    return self.value
+
+
+class _FakeModel:
+  def __init__(self):
+    self.begun = []
+
+  def predict_batch(self, params, batch, rng=None):
+    return batch['a'][:, 0] * params['w']
+
+  def begin_predict_batch(self, params, batch, rng=None):
+    self.begun.append(int(batch['a'][0, 0]))
+    # later batches finish sooner: results must still come back in order
+    return _FakePrediction(len(self.begun), 9 - 2 * len(self.begun),
+                           self.predict_batch(params, batch, rng))
+
+
+def test_decodes_in_flight_keep_order_and_bound_the_number_in_flight():
+  import functools
+  _FakePrediction.log = []
+  model = _FakeModel()
+  fn = infer.get_infer_fn(functools.partial(model.predict_batch), 2,
+                          decodes_in_flight=3)
+  out = fn(_dataset(8), {'w': 3})
+  assert out == [(i, 3 * i) for i in range(8)]
+  assert model.begun == [0, 2, 4, 6]
+  log = _FakePrediction.log
+  order = [name for name, what in log if what == 'result']
+  assert order == [1, 2, 3, 4]
+  # never more than 3 begun and not yet collected; the 4th batch begins only
+  # after the first result was taken
+  first_result = log.index((1, 'result'))
+  assert all(name != 4 for name, _ in log[:first_result])
+  # while waiting for the oldest, the others are polled (kept fed)
+  assert (2, 'poll') in log[:first_result] and (3, 'poll') in log[:first_result]
+
+
+def test_decodes_in_flight_falls_back_to_the_plain_step():
+  model = _FakeModel()
+  # 1 in flight, or a step that is no bound method with a begin_ variant
+  for fn in (infer.get_infer_fn(model.predict_batch, 2, decodes_in_flight=1),
+             infer.get_infer_fn(lambda params, batch, rng=None:
+                                model.predict_batch(params, batch), 2,
+                                decodes_in_flight=3)):
+    assert fn(_dataset(4), {'w': 2}) == [(i, 2 * i) for i in range(4)]
+  assert model.begun == []
+
+
+class _FakeFused:
+  """A fused step context: the loop condition turns false after `end`
+  iterations; chunks complete one poll after they are asked about."""
+  CHUNK_SLOTS = 4
+
+  def __init__(self, end):
+    self.end, self.enqueued, self.chunks, self.asked = end, 0, [], set()
+
+  def keep_going(self):
+    return self.end > 0
+
+  def launch_chunk(self, n):
+    self.enqueued += n
+    self.chunks.append(self.enqueued)
+    return len(self.chunks) - 1
+
+  def chunk_running(self, ticket, block=False):
+    if not block and ticket not in self.asked:
+      self.asked.add(ticket)
+      return None
+    return self.chunks[ticket] < self.end
+
+  def finish(self):
+    pass
+
+
+def test_loop_start_poll_protocol():
+  import sys
+  from t5x_amd import decoding
+
+  class Loop(decoding._InFlight):
+    def __init__(self, end):
+      self.fused, self.step = _FakeFused(end), 0
+
+    def cond(self):
+      return self.fused.keep_going()
+
+  loop = Loop(end=20)
+  with pytest.raises(ValueError):
+    loop.poll()
+  loop.start(check_every=8)
+  assert loop.fused.enqueued == 16          # two chunks ahead
+  polls = 0
+  while not loop.poll():
+    polls += 1
+    assert polls < 50
+  # the condition turned false inside the third chunk: exactly one chunk was
+  # enqueued past it, and none after the end was seen
+  assert loop.fused.enqueued == 32 and loop.step == 32
+  assert loop.poll()                         # stays ended
+  done = Loop(end=0)
+  done.start()
+  assert done.poll() and done.fused.enqueued == 0
+  # run_in_flight: blocks on one loop at a time, ends them all
+  loops = [Loop(end=e) for e in (5, 40, 17)]
+  decoding.run_in_flight(loops, check_every=8)
+  assert all(l.poll() for l in loops)
+  assert [l.fused.enqueued >= l.fused.end for l in loops] == [True] * 3
+  assert all(l.fused.enqueued <= l.fused.end + 16 for l in loops)
