@@ -307,7 +307,12 @@ def in_loop_kernel_times(w, families, repeats=3):
     return start.elapsed_time(end) * 1e-3
 
   masks = [0] + list(families)
-  best = {m: min(one_decode(m) for _ in range(repeats)) for m in masks}
+  lanes, w.module.decode_lanes = w.module.decode_lanes, 1  # one chain of kernels
+  try:
+    best = {m: min(one_decode(m) for _ in range(repeats)) for m in masks}
+  finally:
+    w.module.decode_lanes = lanes
+    w.loop = None
   launches = nl * (w.L - 1)
   return {m: ((best[0] - best[m]) / launches, launches) for m in families}
 
@@ -366,8 +371,9 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
     times = in_loop_kernel_times(w, (_lib.LEAVE_OUT_CROSS_ATTENTION,
                                      _lib.LEAVE_OUT_SELF_ATTENTION))
     sec, n = times[_lib.LEAVE_OUT_CROSS_ATTENTION]
-    where = (f'inside the decode loop, by difference: {n} launches of one '
-             'whole decode left out')
+    where = (f'inside the decode loop (the whole batch as one chain of '
+             f'kernels), by difference: {n} launches of one whole decode '
+             'left out')
     out['replay_launch_us'] = round(replay_sec * 1e6, 2)
     ssec, sn = times[_lib.LEAVE_OUT_SELF_ATTENTION]
     sbytes = float(np.mean([w.self_attention_bytes(t)
@@ -408,7 +414,8 @@ def in_flight_throughput(w, n, groups=3):
                           device=dev).to(w.encoded.dtype)
     fns.append(models.StepFunction(
         w.model, w.params, network.BeamShared(encoded, w.K),
-        network.BeamShared(torch.as_tensor(tok, device=dev), w.K), w.L))
+        network.BeamShared(torch.as_tensor(tok, device=dev), w.K), w.L,
+        in_flight=True))
 
   def group():
     loops = []
@@ -696,6 +703,9 @@ def main():
       'config': {'workload': f'T5.1.1-{size} {what}, encoder {E} ({Emin}..{E} '
                              f'valid), max decode length {L}',
                  'name': args.config, 'beam_rows': B * K,
+                 # batch slices stepped side by side on separate streams
+                 'batch_lanes': getattr(getattr(w.loop, 'fused', None),
+                                        'n_lanes', 1),
                  # positions t of the decode the timed iterations covered:
                  # whole decodes, then a window centred on (L-1)/2
                  't_first': windows[-1][0], 't_last': windows[-1][1],

@@ -166,7 +166,7 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
       else:
         step_rng, rng = split_rng(rng)
       if begin is not None:
-        in_flight.append(begin(params, infer_batch, step_rng))
+        in_flight.append(begin(params, infer_batch, step_rng, in_flight=True))
         all_indices.append(index)
         while len(in_flight) >= decodes_in_flight:
           collect_oldest()

@@ -36,7 +36,9 @@ class StepFunction:
   for a fused on-device step (`fused_beam_step`, `fused_sample_step`)."""
 
   def __init__(self, model, params, encoded_inputs, raw_inputs,
-               max_decode_length):
+               max_decode_length, in_flight=False):
+    """in_flight: the caller keeps several decodes running at once (a fused
+    beam step then does not cut its batch into lanes)."""
     self.model, self.params = model, params
     self.encoded_inputs, self.raw_inputs = encoded_inputs, raw_inputs
     self.max_decode_length = max_decode_length
@@ -45,7 +47,7 @@ class StepFunction:
     self.cache_offset = int(bool(getattr(module, 'scan_layers', False)))
     if hasattr(module, 'make_fused_beam_step'):
       self.fused_beam_step = lambda loop: module.make_fused_beam_step(
-          loop, params, encoded_inputs, raw_inputs)
+          loop, params, encoded_inputs, raw_inputs, in_flight=in_flight)
     if hasattr(module, 'make_fused_sample_step'):
       self.fused_sample_step = lambda **kw: module.make_fused_sample_step(
           params, encoded_inputs, raw_inputs, **kw)
@@ -131,9 +133,10 @@ class EncoderDecoderModel:
         params, batch, rng, decoder_params, return_all_decodes, num_decodes,
         prompt_with_targets).result()
 
-  def begin_predict_batch(self, params, batch, rng=None):
+  def begin_predict_batch(self, params, batch, rng=None, in_flight=False):
     """predict_batch set up and started but not waited for -> Prediction."""
-    return self.begin_predict_batch_with_aux(params, batch, rng).first()
+    return self.begin_predict_batch_with_aux(params, batch, rng,
+                                             in_flight=in_flight).first()
 
   def predict_batches(self, params, batches, rngs=None, in_flight: int = 3,
                       **kwargs):
@@ -149,8 +152,8 @@ class EncoderDecoderModel:
     active = collections.deque()
     for batch in batches:
       rng = next(rngs) if rngs is not None else None
-      active.append(self.begin_predict_batch_with_aux(params, batch, rng,
-                                                      **kwargs))
+      active.append(self.begin_predict_batch_with_aux(
+          params, batch, rng, in_flight=in_flight > 1, **kwargs))
       while len(active) >= max(1, in_flight):
         yield _wait_for_oldest(active)
     while active:
@@ -160,10 +163,11 @@ class EncoderDecoderModel:
       self, params, batch, rng=None,
       decoder_params: Optional[MutableMapping[str, Any]] = None,
       return_all_decodes: bool = None, num_decodes: int = None,
-      prompt_with_targets: bool = False):
+      prompt_with_targets: bool = False, in_flight: bool = False):
     """predict_batch_with_aux (t5x/models.py:584-758) up to and including the
     start of its decode loop -> Prediction; `.result()` is the method's return
-    value."""
+    value.  in_flight: the caller will have other predictions running beside
+    this one."""
     if return_all_decodes is None:
       return_all_decodes = self._default_decoder_params.return_all_decodes
     if num_decodes is None:
@@ -201,7 +205,7 @@ class EncoderDecoderModel:
       expand = lambda x: decoding.flat_batch_beam_expand(x, num_decodes)
     tokens_ids_to_logits = StepFunction(
         self, params, expand(encoded_inputs), expand(encoder_input_tokens),
-        decoder_input_tokens.shape[1])
+        decoder_input_tokens.shape[1], in_flight=in_flight)
 
     if decoder_params is None:
       decoder_params = {}

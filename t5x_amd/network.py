@@ -232,11 +232,15 @@ class Transformer:
   float32 leaves); it is cast/packed on first use and cached by identity.
   """
 
-  # Batch slices a fused beam search steps on separate streams.  On MI355X
-  # kernels of different streams do overlap, but the dispatch rate (about one
-  # kernel per 1.5 us) is shared by all streams, and a decode step is bound by
-  # its kernel count, so more lanes only add dispatches: 1 is fastest.
-  decode_lanes = 1
+  # Batch slices ("lanes") that a fused beam search steps on separate streams.
+  # A decode step is a chain of dependent kernels that leaves most of the
+  # device waiting, so two half-batches side by side finish an iteration
+  # sooner than the whole batch in one chain (measured: base beam 4
+  # 0.789 -> 0.738 ms, XL int8 2.61 -> 2.46 ms; three lanes are slower
+  # again, and a fourth stream shares a hardware queue).  None: 2 lanes for a
+  # decode on its own, 1 when several batches are in flight (those fill the
+  # device better than lanes do, and streams that run side by side are few).
+  decode_lanes = None
 
   def __init__(self, config: T5Config, device=None, scan_layers: bool = False):
     """scan_layers: hand out and accept the cache in the layout of a scanned
@@ -545,28 +549,31 @@ class Transformer:
     return (logits, {'cache': cache}) if mutable else logits
 
   # -- fused beam search: one graph replay per loop iteration ------------------------
-  def make_fused_beam_step(self, loop, params, encoded, enc_tokens):
+  def make_fused_beam_step(self, loop, params, encoded, enc_tokens,
+                           in_flight=False):
     """Returns a FusedBeamStep driving `loop` (a decoding.BeamLoop), or None
     when this configuration has to use the generic per-call path.  The step
     object (caches, cross K/V buffers, state, captured graphs) is kept and
     re-bound to the next loop of the same shape and options, so a stream of
-    batches pays for allocation and graph capture once."""
+    batches pays for allocation and graph capture once.  in_flight: the
+    caller keeps several decodes running at once (see decode_lanes)."""
     if (not isinstance(encoded, BeamShared) or
         loop.cache_offset != int(self.scan_layers)):
       return None
     if loop.beam_size > 8:
       return None
     w = self.decoder_weights(params)
+    lanes = self.decode_lanes or (1 if in_flight else 2)
+    lanes = max(1, min(int(lanes), loop.batch_size))
     key = (id(w), tuple(encoded.x.shape), encoded.x.dtype, encoded.beams,
            loop.batch_size, loop.beam_size, loop.max_decode_len,
            tuple(loop.inputs_dev.shape), tuple(loop.brevity.shape),
            int(loop.eos_id), float(loop.min_brevity), float(loop.min_log_prob),
-           int(loop.max_decode_step), int(loop.min_initial),
-           int(self.decode_lanes))
+           int(loop.max_decode_step), int(loop.min_initial), lanes)
     return self._decode_context(
         key, w, loop,
         make=lambda slot: FusedBeamStep(self, loop, params, encoded,
-                                        enc_tokens, slot=slot),
+                                        enc_tokens, lanes=lanes, slot=slot),
         rebind=lambda ctx: ctx.rebind(loop, encoded, enc_tokens))
 
   # Decode contexts of one (weights, shapes, options) key that are kept for
@@ -600,7 +607,8 @@ class Transformer:
     return ctx
 
   def decode_stream(self, slot):
-    """The stream of the decode contexts in pool slot `slot`.  The device
+    """The stream of the decode contexts in pool slot `slot` (with batch
+    lanes: of lane l of the context in slot s, at s * lanes + l).  The device
     runs streams side by side only when they sit on different hardware
     queues, of which a process has few (4 by default) and which streams are
     given in turn as they are first used; so the module makes its streams
@@ -1001,10 +1009,7 @@ class _BeamLane:
       bs.cache_slot, bs.cache_src, bs.cache_dst = (
           P(self.cache_slot), P(self.cache_src), P(self.cache_dst))
     self.beam = bs
-    # the first lane runs on the pool slot's stream; further lanes (an option
-    # for one decode at a time) on streams of their own
-    self.stream = (module.decode_stream(owner.slot) if index == 0 else
-                   torch.cuda.Stream(device=dev))
+    self.stream = module.decode_stream(owner.slot * owner.n_lanes + index)
     self.event = torch.cuda.Event()
     self.graph = None
     self.graph_long = None
@@ -1068,9 +1073,7 @@ class FusedBeamStep(_OwnedContext):
     # [0]: slot of beam e; [1], [2]: source / destination slots in flight
     self.cache_slots = torch.arange(K, dtype=torch.int32, device=dev).expand(
         3, B, K).contiguous()
-    if lanes is None:
-      lanes = module.decode_lanes
-    n = max(1, min(int(lanes), B))
+    n = max(1, min(int(lanes or 1), B))
     self.n_lanes = n
     self.slot = slot
     bounds = [B * i // n for i in range(n + 1)]

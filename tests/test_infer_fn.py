@@ -174,7 +174,8 @@ class _FakeModel:
   def predict_batch(self, params, batch, rng=None):
     return batch['a'][:, 0] * params['w']
 
-  def begin_predict_batch(self, params, batch, rng=None):
+  def begin_predict_batch(self, params, batch, rng=None, in_flight=False):
+    assert in_flight
     self.begun.append(int(batch['a'][0, 0]))
     # later batches finish sooner: results must still come back in order
     return _FakePrediction(len(self.begun), 9 - 2 * len(self.begun),
