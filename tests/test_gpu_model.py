@@ -738,6 +738,54 @@ def test_full_size_base_beam4_fused_loop_equals_generic_loop():
   assert np.isfinite(scores).all()
 
 
+def test_full_size_base_beam4_three_batches_in_flight_equal_one_by_one():
+  """The benchmark workload with three different batches decoding at once
+  (one chain of kernels each, started and polled without waiting) against the
+  same three decoded one after the other (two batch lanes each): tokens,
+  scores and step counts bit for bit."""
+  from t5x_amd import decoding, models, network
+  B, K, E, L = 32, 4, 512, 128
+  module, fn0 = _full_size_setup('base', B, K, E, 128, L, decoding.beam_search)
+  dev = torch.device('cuda')
+  cfg = module.config
+  inputs = np.zeros((B, L), np.int32)
+
+  def step_fn(seed, in_flight):
+    rs = np.random.Generator(np.random.PCG64(seed))
+    tok = rs.integers(2, 32128, size=(B, E)).astype(np.int32)
+    lens = rs.integers(128, E + 1, size=(B,))
+    tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    encoded = torch.randn((B, E, cfg.emb_dim), generator=gen,
+                          device=dev).to(torch.bfloat16)
+    return models.StepFunction(
+        fn0.model, fn0.params, network.BeamShared(encoded, K),
+        network.BeamShared(torch.as_tensor(tok, device=dev), K), L,
+        in_flight=in_flight)
+
+  def new_loop(seed, in_flight):
+    return decoding.BeamLoop(inputs, module.init_cache(B, L),
+                             step_fn(seed, in_flight), eos_id=1,
+                             num_decodes=K, alpha=0.6)
+
+  want = []
+  for seed in (11, 12, 13):
+    loop = new_loop(seed, False)
+    assert loop.fused.n_lanes == 2
+    loop.run()
+    want.append(loop.finish() + (int(loop.cur.cur_index.item()),))
+  loops = [new_loop(seed, True) for seed in (11, 12, 13)]
+  assert [l.fused.n_lanes for l in loops] == [1, 1, 1]
+  assert len({id(l.fused) for l in loops}) == 3
+  assert len({l.fused.stream.cuda_stream for l in loops}) == 3
+  decoding.run_in_flight(loops)
+  for loop, (ws, wsc, steps) in zip(loops, want):
+    gs, gsc = loop.finish()
+    assert int(loop.cur.cur_index.item()) == steps
+    assert torch.equal(gs, ws) and torch.equal(gsc, wsc)
+
+
 @pytest.mark.parametrize('K', [2, 3, 4, 8])
 def test_fused_beam_loop_slot_maps_follow_the_inheritance_rule(K):
   """Where the graph-replay loop keeps the beams' cache rows: after every
