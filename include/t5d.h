@@ -186,11 +186,13 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
  * unless that is where it read it, and the new column goes there.  Per item
  * pending_dst must be a permutation of 0..beams-1 and no slot that some row
  * writes without reading it may be read by another row.
- * value_blocked != 0: cached_value is stored per (row, head) as
+ * value_blocked 1: cached_value is stored per (row, head) as
  * [L/32][64][32] (blocks of 32 positions, L a multiple of 32) instead of the
- * reference's [64][L]; a caller that owns its caches (a decode loop) gets
- * loads of consecutive memory for them and converts when it hands the cache
- * tree out. */
+ * reference's [64][L]; 2: cached_key as well.  A caller that owns its caches
+ * (a decode loop) gets loads of consecutive memory for them — a head's cache
+ * is then read as whole 4 KB blocks up to the current length instead of the
+ * first part of each of 64 rows — and converts when it hands the cache tree
+ * out.  0: both in the reference layout. */
 int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
                                    void* cached_key, void* cached_value,
                                    const void* rel_bias,
@@ -442,8 +444,9 @@ typedef struct {
    * optional destination slots (NULL: row e keeps slot e) */
   const int32_t* pending_src;
   const int32_t* pending_dst;
-  /* non-zero: the layers' cached_value are in the blocked layout of
-   * t5d_self_attention_step_gather (bfloat16, L a multiple of 32) */
+  /* 1: the layers' cached_value are in the blocked layout of
+   * t5d_self_attention_step_gather (bfloat16, L a multiple of 32); 2: the
+   * cached_key too */
   int value_blocked;
   /* Measurement aid, normally 0: a mask of T5D_LEAVE_OUT_* bits; the step is
    * enqueued WITHOUT the launches of those kernel families (their outputs keep

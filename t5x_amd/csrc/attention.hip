@@ -500,8 +500,10 @@ extern "C" int t5d_self_attention_step_gather(
               "%d wavefronts per workgroup", beams, L, kMaxWaves);
   T5D_REQUIRE(pending_dst == nullptr || pending_src != nullptr, T5D_EINVAL,
               "t5d_self_attention_step_gather: pending_dst without pending_src");
+  T5D_REQUIRE(value_blocked >= 0 && value_blocked <= 2, T5D_EINVAL,
+              "t5d_self_attention_step_gather: value_blocked=%d", value_blocked);
   T5D_REQUIRE(!value_blocked || L % 32 == 0, T5D_EINVAL,
-              "t5d_self_attention_step_gather: blocked values need L %% 32 == 0 "
+              "t5d_self_attention_step_gather: blocked caches need L %% 32 == 0 "
               "(L=%d)", L);
   T5D_REQUIRE(((uintptr_t)cached_key % 16) == 0 &&
                   ((uintptr_t)cached_value % 16) == 0,
@@ -509,8 +511,7 @@ extern "C" int t5d_self_attention_step_gather(
               "t5d_self_attention_step_gather: cache not 16-byte aligned");
   launch_self_attention_bf16(as_stream(stream), qkv, cached_key, cached_value,
                              rel_bias, cache_index, out, B * beams, H, L,
-                             pending_src, pending_dst, beams,
-                             value_blocked ? 1 : 0);
+                             pending_src, pending_dst, beams, value_blocked);
   T5D_CHECK_LAUNCH("t5d_self_attention_step_gather");
   return T5D_OK;
 }

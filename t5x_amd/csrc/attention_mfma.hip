@@ -56,6 +56,7 @@ struct AttnMfmaArgs {
   int d;
   float eps;
   int v_blocked;  // self-attention: value cache stored as [S/32][64][32] per head
+  int k_blocked;  // self-attention: key cache stored the same way
   // cross-attention: optional work order, [B * H] entries
   // head | item << 8 | valid length << 16; workgroup (x, y) takes entry
   // y * H + x instead of (head x, item y, index[y])
@@ -525,15 +526,25 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   // groups are skipped by wave-uniform branches, together with their matrix
   // products.  Offsets are clamped to the row end when S is not a multiple of
   // the tile (those positions are masked).
+  // K: head dim 16 dg + i, positions j0 .. j0 + 7.  Reference layout [64][S]:
+  // a head dim's positions are contiguous, a lane's 16 chunks are S apart.
+  // Blocked layout [S/32][64][32]: the chunk sits in block j0 / 32, the 16
+  // chunks are 64 bytes apart and the cache of a head is read as whole 4 KB
+  // blocks up to the current length instead of the first part of 64 rows.
   const int j0 = jw + 8 * jc;
   const bool live = j0 < n;
-  const uint32_t koff = (uint32_t)(16 * dg * S + min(j0, S - 8)) * 2u;
+  const int j0c = min(j0, S - 8);
+  const uint32_t koff =
+      a.k_blocked
+          ? (uint32_t)(((j0c >> 5) * kHeadDim + 16 * dg) * 32 + (j0c & 31)) * 2u
+          : (uint32_t)(16 * dg * S + j0c) * 2u;
+  const uint32_t kdim = (a.k_blocked ? 32u : (uint32_t)S) * 2u;  // next head dim
   uint4 kc[16];
   if (live) {
 #pragma unroll
     for (int i = 0; i < 16; ++i)
       kc[i] = *reinterpret_cast<const uint4*>(
-          reinterpret_cast<const char*>(ksrc + (size_t)i * S) + koff);
+          reinterpret_cast<const char*>(ksrc) + i * kdim + koff);
   }
   // Byte offset of this lane's chunk of V tile (jb, dt) inside the head's
   // slot.  Reference layout [64][S]: row 16 dt + n16, positions 32 jb + 8 g ..;
@@ -595,8 +606,8 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
       if (live) {
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          *reinterpret_cast<uint4*>(
-              reinterpret_cast<char*>(kdst + (size_t)i * S) + koff) = kc[i];
+          *reinterpret_cast<uint4*>(reinterpret_cast<char*>(kdst) + i * kdim +
+                                    koff) = kc[i];
       }
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
@@ -617,9 +628,10 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   auto store_column = [&]() {
     if (wave_has_t) {
       if (rw != rs) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      kdst[(size_t)lane * S + t] = knew_d;
-      vdst[a.v_blocked ? ((size_t)(t >> 5) * kHeadDim + lane) * 32 + (t & 31)
-                       : (size_t)lane * S + t] = vnew_d;
+      const size_t plain = (size_t)lane * S + t;
+      const size_t blocked = ((size_t)(t >> 5) * kHeadDim + lane) * 32 + (t & 31);
+      kdst[a.k_blocked ? blocked : plain] = knew_d;
+      vdst[a.v_blocked ? blocked : plain] = vnew_d;
     }
   };
 
@@ -758,6 +770,7 @@ int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,
                                 int d, float eps, const int32_t* units) {
   AttnMfmaArgs a;
   a.v_blocked = 0;
+  a.k_blocked = 0;
   a.units = units;
   a.x = (const bf16_t*)x; a.ln = (const bf16_t*)ln; a.wq = wq;
   a.d = d; a.eps = eps;
@@ -777,7 +790,8 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
                                const int32_t* pending_dst, int beams,
                                int value_blocked) {
   AttnMfmaArgs a;
-  a.v_blocked = value_blocked;
+  a.v_blocked = value_blocked != 0;
+  a.k_blocked = value_blocked == 2;
   a.q = (const bf16_t*)qkv; a.k = (bf16_t*)ck; a.v = (bf16_t*)cv;
   a.rel_bias = (const bf16_t*)rel_bias; a.index = cache_index;
   a.out = (bf16_t*)out;

@@ -453,7 +453,8 @@ class Transformer:
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
     m.pending_src, m.pending_dst = P(pending_src), P(pending_dst)
-    m.value_blocked = int(bool(value_blocked))
+    # the loops that block their value caches block their key caches too
+    m.value_blocked = 2 if value_blocked else 0
     m.leave_out = 0
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
                     pending_src, pending_dst)
@@ -735,8 +736,8 @@ class FusedSampleStep(_OwnedContext):
     self.temperature = temperature
     R, S = sequences.shape
     act = w.act_dtype
-    # bfloat16: the value caches are kept in blocks of 32 positions (loads of
-    # consecutive memory); cache_tree() converts back.
+    # bfloat16: the key and value caches are kept in blocks of 32 positions
+    # (loads of consecutive memory); cache_tree() converts back.
     self.value_blocked = act == torch.bfloat16
     el = 32 if self.value_blocked else 16 // torch.empty(
         (), dtype=act).element_size()
@@ -922,9 +923,9 @@ class FusedSampleStep(_OwnedContext):
     self.stream.synchronize()
     from t5x_amd import ops
     nl = self.kv.shape[0]
-    value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return cache_tree(self.kv[:, 0],
-                      torch.stack([value(self.kv[i, 1]) for i in range(nl)]),
+    plain = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
+    return cache_tree(torch.stack([plain(self.kv[i, 0]) for i in range(nl)]),
+                      torch.stack([plain(self.kv[i, 1]) for i in range(nl)]),
                       self.cache_index, self.module.scan_layers)
 
   def __del__(self):
@@ -1056,8 +1057,8 @@ class FusedBeamStep(_OwnedContext):
     # copied), so the reorder in flight is a pair of slot maps, cache_slots.
     self.deferred_gather = (K > 1 and act == torch.bfloat16 and
                             K * ((L + 127) // 128) <= 16)
-    # The value caches are then kept in blocks of 32 positions (loads of
-    # consecutive memory); cache_tree() converts back.  (The stand-alone
+    # The key and value caches are then kept in blocks of 32 positions (loads
+    # of consecutive memory); cache_tree() converts back.  (The stand-alone
     # reorder kernel of the other path copies row prefixes, which only the
     # reference layout has.)
     self.value_blocked = self.deferred_gather or (K == 1 and
@@ -1297,9 +1298,9 @@ class FusedBeamStep(_OwnedContext):
     nl = self.lanes[0].kv.shape[0]
     kv = torch.cat([lane.kv for lane in self.lanes], dim=2)
     idx = self.lanes[0].cache_index
-    value = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return cache_tree(kv[:, 0],
-                      torch.stack([value(kv[i, 1]) for i in range(nl)]), idx,
+    plain = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
+    return cache_tree(torch.stack([plain(kv[i, 0]) for i in range(nl)]),
+                      torch.stack([plain(kv[i, 1]) for i in range(nl)]), idx,
                       self.module.scan_layers)
 
   def __del__(self):

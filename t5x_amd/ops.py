@@ -211,8 +211,8 @@ def gemm_tiled(a, w: PackedWeight, mp, nt, k_parts=1, out=None, residual=None,
 
 
 def block_cached_value(v):
-  """[R, H, 64, L] value cache -> the blocked [R, H, L/32, 64, 32] layout
-  (same bytes count; L a multiple of 32)."""
+  """[R, H, 64, L] value (or key) cache -> the blocked [R, H, L/32, 64, 32]
+  layout (same bytes count; L a multiple of 32)."""
   R, H, D, L = v.shape
   return v.reshape(R, H, D, L // 32, 32).permute(0, 1, 3, 2, 4).contiguous()
 
@@ -228,12 +228,15 @@ def unblock_cached_value(v):
 
 def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
                         out=None, pending_src=None, value_blocked=False,
-                        pending_dst=None):
+                        pending_dst=None, key_blocked=False):
   """One cached self-attention step; with pending_src [B, beams] the rows'
   caches are first gathered from their source beams inside the kernel, into
   slot e of row (b, e) or, with pending_dst [B, beams], into slot
   pending_dst[b, e].  value_blocked: cached_value holds the blocked layout
-  (see block_cached_value) in a tensor of the usual [R, H, 64, L] shape."""
+  (see block_cached_value) in a tensor of the usual [R, H, 64, L] shape;
+  key_blocked (with value_blocked): cached_key as well."""
+  if key_blocked and not value_blocked:
+    raise ValueError('key_blocked goes with value_blocked')
   _chk(qkv, 'qkv', ndim=2)
   _chk(cached_key, 'cached_key', qkv.dtype, 4)
   _chk(cached_value, 'cached_value', qkv.dtype, 4)
@@ -269,7 +272,7 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
               cached_key.data_ptr(), cached_value.data_ptr(),
               rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), B,
               beams, H, L, _lib.ptr(pending_src), _lib.ptr(pending_dst),
-              int(bool(value_blocked)))
+              2 if key_blocked else int(bool(value_blocked)))
     return out
   _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
             qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),

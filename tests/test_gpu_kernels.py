@@ -548,6 +548,29 @@ def test_self_attention_step_with_pending_gather(ops, B, beams, H, L, t):
   assert torch.equal(ops.unblock_cached_value(cv_d)[..., :t + 1],
                      cv_a[..., :t + 1])
 
+  # ... and with the key cache in the same blocks
+  ck_f = ops.block_cached_value(ck).view(R, H, D, L)
+  cv_f = ops.block_cached_value(cv).view(R, H, D, L)
+  got_f = ops.self_attention_step(qkv, ck_f, cv_f, rel_bias, idx,
+                                  pending_src=src, value_blocked=True,
+                                  key_blocked=True)
+  assert torch.equal(got_f, want)
+  assert torch.equal(ops.unblock_cached_value(ck_f)[..., :t + 1],
+                     ck_a[..., :t + 1])
+  assert torch.equal(ops.unblock_cached_value(cv_f)[..., :t + 1],
+                     cv_a[..., :t + 1])
+  ck_plain = ck.clone()
+  ops.cache_gather_beams(ck_plain.view(B, beams, H, D, L), src, valid_len=valid)
+  ck_g = ops.block_cached_value(ck_plain).view(R, H, D, L)
+  cv_g = ops.block_cached_value(cv_plain).view(R, H, D, L)
+  got_g = ops.self_attention_step(qkv, ck_g, cv_g, rel_bias, idx,
+                                  value_blocked=True, key_blocked=True)
+  assert torch.equal(got_g, want)
+  assert torch.equal(ops.unblock_cached_value(ck_g)[..., :t + 1],
+                     ck_a[..., :t + 1])
+  with pytest.raises(ValueError):
+    ops.self_attention_step(qkv, ck_g, cv_g, rel_bias, idx, key_blocked=True)
+
 
 def _lib_call_norm_gemm_mixed(ops, x, pw):
   """float32 activations with packed bfloat16 weights, straight at the C entry
@@ -582,7 +605,7 @@ def inherit_slots(slot_of, parents):
 @pytest.mark.parametrize('B,beams,H,L,t', [(3, 4, 2, 128, 0), (3, 4, 3, 128, 77),
                                            (2, 2, 2, 32, 9), (2, 8, 2, 256, 200),
                                            (32, 4, 12, 128, 64)])
-@pytest.mark.parametrize('blocked', [False, True])
+@pytest.mark.parametrize('blocked', [0, 1, 2])
 def test_self_attention_step_with_destination_slots(ops, B, beams, H, L, t,
                                                      blocked):
   """Beams that inherit their parents' slots: with the caches of the old beams
@@ -625,21 +648,25 @@ def test_self_attention_step_with_destination_slots(ops, B, beams, H, L, t,
   cv_a = logical_v[(rows + pa).reshape(-1)].clone()
   want = ops.self_attention_step(qkv, ck_a, cv_a, rel_bias, idx)
 
-  ck_b = ck.clone()
+  # blocked 1: the value cache in blocks of 32 positions, 2: the key cache too
+  ck_b = (ops.block_cached_value(ck).view(R, H, D, L) if blocked == 2
+          else ck.clone())
   cv_b = (ops.block_cached_value(cv).view(R, H, D, L) if blocked
           else cv.clone())
   got = ops.self_attention_step(qkv, ck_b, cv_b, rel_bias, idx,
                                 pending_src=src, pending_dst=dst,
-                                value_blocked=blocked)
+                                value_blocked=blocked > 0,
+                                key_blocked=blocked == 2)
   assert torch.equal(got, want)
+  ck_out = ops.unblock_cached_value(ck_b) if blocked == 2 else ck_b
   cv_out = ops.unblock_cached_value(cv_b) if blocked else cv_b
   at = (rows + dst.long()).reshape(-1)      # where new beam e's cache is now
-  assert torch.equal(ck_b[at][..., :t + 1], ck_a[..., :t + 1])
+  assert torch.equal(ck_out[at][..., :t + 1], ck_a[..., :t + 1])
   assert torch.equal(cv_out[at][..., :t + 1], cv_a[..., :t + 1])
   # inherited slots were not rewritten beyond the new column
   keep = (src == dst).reshape(-1)
   if t + 1 < L and bool(keep.any()):
-    assert torch.equal(ck_b[at][keep][..., t + 1:],
+    assert torch.equal(ck_out[at][keep][..., t + 1:],
                        ck[(rows + src.long()).reshape(-1)][keep][..., t + 1:])
 
 
