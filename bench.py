@@ -63,8 +63,10 @@ def parse_args():
                        'is one batch')
   ap.add_argument('--in-flight', type=int, default=None,
                   help='also measure this many whole decodes of different '
-                       'batches running on the device at once (default: 3 '
-                       'for the default config, 0 = skip for the others)')
+                       'batches running on the device at once (default for '
+                       'the default config: as many as the device runs side '
+                       'by side, 3 with 4 hardware queues; 0 = skip, the '
+                       'default for the other configs)')
   ap.add_argument('--replay-roofline', action='store_true',
                   help='time the roofline kernel by back-to-back replay only '
                        '(no decodes enqueued without it); for runs under '
@@ -718,7 +720,8 @@ def main():
   # of initialisation: no CPU figure for that shape)
   n_in_flight = args.in_flight
   if n_in_flight is None:
-    n_in_flight = 3 if args.config == DEFAULT_CONFIG else 0
+    n_in_flight = (w.module.streams_side_by_side()
+                   if args.config == DEFAULT_CONFIG else 0)
   if n_in_flight > 1:
     out['in_flight'] = in_flight_throughput(w, n_in_flight)
   if not args.no_cpu_baseline and size != 'xxl':

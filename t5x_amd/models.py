@@ -138,16 +138,20 @@ class EncoderDecoderModel:
     return self.begin_predict_batch_with_aux(params, batch, rng,
                                              in_flight=in_flight).first()
 
-  def predict_batches(self, params, batches, rngs=None, in_flight: int = 3,
-                      **kwargs):
+  def predict_batches(self, params, batches, rngs=None,
+                      in_flight: Optional[int] = None, **kwargs):
     """predict_batch_with_aux over an iterable of batches, yielding each
     batch's result in order, with up to `in_flight` decodes running on the
     device at once (each on its own streams): the device spends most of a
     decode step of one batch waiting on dependent launches, which the other
     batches' steps fill.  Every batch's result is what predict_batch_with_aux
-    returns for it alone.  `rngs`: one per batch, or None.  With decode
-    functions other than beam_search / temperature_sample the batches run one
-    after the other."""
+    returns for it alone.  `rngs`: one per batch, or None.  in_flight None: as
+    many as the device runs side by side (3 with the runtime's default number
+    of hardware queues).  With decode functions other than beam_search /
+    temperature_sample the batches run one after the other."""
+    if in_flight is None:
+      side_by_side = getattr(self.module, 'streams_side_by_side', None)
+      in_flight = side_by_side() if side_by_side is not None else 1
     rngs = iter(rngs) if rngs is not None else None
     active = collections.deque()
     for batch in batches:
