@@ -93,14 +93,15 @@ def _begin_of(infer_step):
 def get_infer_fn(infer_step: Callable, batch_size: int,
                  train_state_axes: Any = None, partitioner: Any = None,
                  keep_aux_as_numpy: bool = False,
-                 decodes_in_flight: int = 1):
+                 decodes_in_flight: Optional[int] = None):
   """t5x/utils.py:1543-1817 -> infer_fn(ds, train_state, rng=None).
 
   `decodes_in_flight` (no counterpart in the reference): when `infer_step` is
   `predict_batch` / `predict_batch_with_aux` of a model that can start a
   prediction without waiting for it, up to that many batches decode on the
   device at once (each holds its own caches and cross K/V); each batch's
-  result is unchanged.  1: one batch after the other, as the reference."""
+  result is unchanged.  None: what the model's batches_in_flight() says for
+  the first batch; 1: one batch after the other, as the reference."""
   del train_state_axes  # one device: parameters are not partitioned
   params_of_step = inspect.signature(infer_step).parameters
   takes_rng = 'rng' in params_of_step
@@ -144,9 +145,10 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
     batched_results, all_indices = [], []
     params = getattr(train_state, 'params', train_state)
     mutables = getattr(train_state, 'flax_mutables', None)
-    begin = _begin_of(infer_step) if decodes_in_flight > 1 else None
+    begin = _begin_of(infer_step) if decodes_in_flight != 1 else None
     if takes_mutables or 'rng' not in params_of_step:
       begin = None
+    n_in_flight = decodes_in_flight
     in_flight = collections.deque()
 
     def collect_oldest():
@@ -165,10 +167,16 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
         step_rng = None
       else:
         step_rng, rng = split_rng(rng)
+      if begin is not None and n_in_flight is None:
+        ask = getattr(begin.func.__self__, 'batches_in_flight', None)
+        n_in_flight = (ask(infer_batch, begin.keywords.get('num_decodes'))
+                       if ask is not None else 1)
+        if n_in_flight <= 1:
+          begin = None
       if begin is not None:
         in_flight.append(begin(params, infer_batch, step_rng, in_flight=True))
         all_indices.append(index)
-        while len(in_flight) >= decodes_in_flight:
+        while len(in_flight) >= n_in_flight:
           collect_oldest()
         continue
       batch_indices, batch_result = infer_step_with_indices(

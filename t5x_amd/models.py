@@ -145,16 +145,14 @@ class EncoderDecoderModel:
     device at once (each on its own streams): the device spends most of a
     decode step of one batch waiting on dependent launches, which the other
     batches' steps fill.  Every batch's result is what predict_batch_with_aux
-    returns for it alone.  `rngs`: one per batch, or None.  in_flight None: as
-    many as the device runs side by side (3 with the runtime's default number
-    of hardware queues).  With decode functions other than beam_search /
-    temperature_sample the batches run one after the other."""
-    if in_flight is None:
-      side_by_side = getattr(self.module, 'streams_side_by_side', None)
-      in_flight = side_by_side() if side_by_side is not None else 1
+    returns for it alone.  `rngs`: one per batch, or None.  in_flight None:
+    batches_in_flight() of the first batch.  With decode functions other than
+    beam_search / temperature_sample the batches run one after the other."""
     rngs = iter(rngs) if rngs is not None else None
     active = collections.deque()
     for batch in batches:
+      if in_flight is None:
+        in_flight = self.batches_in_flight(batch, kwargs.get('num_decodes'))
       rng = next(rngs) if rngs is not None else None
       active.append(self.begin_predict_batch_with_aux(
           params, batch, rng, in_flight=in_flight > 1, **kwargs))
@@ -162,6 +160,20 @@ class EncoderDecoderModel:
         yield _wait_for_oldest(active)
     while active:
       yield _wait_for_oldest(active)
+
+  def batches_in_flight(self, batch, num_decodes=None) -> int:
+    """How many batches shaped like `batch` to keep decoding at once: as many
+    as the device runs side by side (3 with the runtime's default number of
+    hardware queues) unless their caches would not fit comfortably; 1 for
+    modules and decode functions that cannot run that way."""
+    ask = getattr(self.module, 'batches_in_flight', None)
+    if ask is None or _begin_of(self._decode_fn)[0] is None:
+      return 1
+    if num_decodes is None:
+      num_decodes = self._default_decoder_params.num_decodes
+    B, E = np.shape(batch['encoder_input_tokens'])[:2]
+    L = np.shape(batch['decoder_input_tokens'])[1]
+    return ask(B, num_decodes, E, L)
 
   def begin_predict_batch_with_aux(
       self, params, batch, rng=None,

@@ -621,6 +621,28 @@ class Transformer:
       queues = 4
     return 4 if queues >= 8 else 3
 
+  def decode_context_bytes(self, batch_size, num_decodes, enc_len,
+                           decode_len) -> int:
+    """What one decode in flight keeps on the device besides the shared
+    weights: its beam-expanded self-attention caches and the cross K/V of its
+    batch (activations and beam state are small beside them)."""
+    cfg = self.config
+    el = 2 if self.dtype == 'bfloat16' else 4
+    per_position = cfg.num_decoder_layers * 2 * cfg.num_heads * cfg.head_dim * el
+    return per_position * (batch_size * num_decodes * decode_len +
+                           batch_size * enc_len)
+
+  def batches_in_flight(self, batch_size, num_decodes, enc_len,
+                        decode_len) -> int:
+    """How many batches of this shape to keep decoding at once: as many as the
+    device runs side by side, fewer when their caches and cross K/V would
+    take more than half of the free device memory."""
+    n = self.streams_side_by_side()
+    need = self.decode_context_bytes(batch_size, num_decodes, enc_len,
+                                     decode_len)
+    free, _ = torch.cuda.mem_get_info(self._dev())
+    return max(1, min(n, int(free // 2 // max(1, need))))
+
   def decode_stream(self, slot):
     """The stream of the decode contexts in pool slot `slot` (with batch
     lanes: of lane l of the context in slot s, at s * lanes + l).  The device

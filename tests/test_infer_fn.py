@@ -272,3 +272,33 @@ def test_loop_start_poll_protocol():
   assert all(l.poll() for l in loops)
   assert [l.fused.enqueued >= l.fused.end for l in loops] == [True] * 3
   assert all(l.fused.enqueued <= l.fused.end + 16 for l in loops)
+
+
+def test_decode_context_bytes_and_in_flight_count_of_a_model():
+  from t5x_amd import decoding, models, network
+  base = network.Transformer.__new__(network.Transformer)
+  base.config, base.dtype = network.t5_1_1_config('base', dtype='bfloat16'), 'bfloat16'
+  # caches [12, 2, 128 rows, 12, 64, 128] + cross K/V [12, 2, 32, 12, 64, 512], bf16
+  assert base.decode_context_bytes(32, 4, 512, 128) == 2 * 12 * 2 * 12 * 64 * (
+      128 * 128 + 32 * 512)
+  xxl = network.Transformer.__new__(network.Transformer)
+  xxl.config, xxl.dtype = network.t5_1_1_config('xxl', dtype='bfloat16'), 'bfloat16'
+  assert 60e9 < xxl.decode_context_bytes(128, 1, 1024, 256) < 70e9
+
+  class Module:
+    asked = None
+
+    def batches_in_flight(self, *shape):
+      Module.asked = shape
+      return 2
+
+  batch = {'encoder_input_tokens': np.zeros((5, 40), np.int32),
+           'decoder_input_tokens': np.zeros((5, 16), np.int32)}
+  model = models.EncoderDecoderModel(Module(), decode_fn=decoding.beam_search)
+  assert model.batches_in_flight(batch, 4) == 2
+  assert Module.asked == (5, 4, 40, 16)
+  # a decode function that cannot be started without waiting: one at a time
+  other = models.EncoderDecoderModel(Module(), decode_fn=lambda **kw: None)
+  assert other.batches_in_flight(batch) == 1
+  # a module that cannot say: one at a time
+  assert models.EncoderDecoderModel(object()).batches_in_flight(batch) == 1
