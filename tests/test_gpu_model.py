@@ -503,6 +503,7 @@ def test_fused_loop_context_is_reused_across_batches(dtype):
     ('float32', 'beam_search', dict(alpha=0.6), 1),
     ('bfloat16', 'temperature_sample', dict(temperature=0.0), 1),
     ('bfloat16', 'temperature_sample', dict(temperature=0.8, topk=20), 1),
+    ('bfloat16', 'temperature_sample', dict(temperature=0.9, topk=5), 3),
 ])
 def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
                                                     lanes):
@@ -513,7 +514,8 @@ def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
   interleave, and three kept contexts serve all seven."""
   from t5x_amd import network
   ocfg, _, gm = _models(dtype, decode_fn_name, **kw)
-  gm.module.decode_lanes = lanes
+  if decode_fn_name == 'beam_search':
+    gm.module.decode_lanes = lanes
   dev = torch.device('cuda')
   params = network.init_params(gm.module.config, 11, dev)
   params['decoder']['logits_dense']['kernel'][:, 1] *= 3.0
@@ -524,7 +526,8 @@ def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
               'decoder_input_tokens': np.zeros((B, L), np.int32)}
              for _ in range(7)]
   sampling = decode_fn_name == 'temperature_sample'
-  n = 1 if sampling else 4
+  # (for the sampling loops the last parameter is num_decodes: they have no lanes)
+  n = lanes if sampling else 4
   rngs = list(range(40, 47)) if sampling else None
   common = dict(num_decodes=n, return_all_decodes=True)
   want = [gm.predict_batch_with_aux(
