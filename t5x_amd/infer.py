@@ -18,6 +18,7 @@ object with `as_numpy_iterator()` such as a tf.data.Dataset).
 import collections
 import functools
 import inspect
+import itertools
 from typing import Any, Callable, Mapping, Optional, Sequence
 
 import numpy as np
@@ -74,6 +75,49 @@ def _stack(examples):
                   examples[0], *examples[1:])
 
 
+def map_in_flight(begin, items, in_flight: int, max_unclaimed: int = 16):
+  """begin(item) for every item of an iterable, with up to `in_flight` of the
+  returned objects running at once, yielding their result() in the order of
+  the items.  An object has poll(block=False) -> bool (has it ended; waits
+  only when asked to) and result().  What has ended is collected at once —
+  which frees whatever it holds for the next item — also when an older one is
+  still running, so one slow item does not idle the others' places; at most
+  `max_unclaimed` results wait for an older item that way."""
+  in_flight = max(1, int(in_flight))
+  todo = iter(items)
+  pending = collections.deque()   # [object or None once collected, result]
+
+  def collect():
+    for entry in pending:
+      if entry[0] is not None and entry[0].poll():
+        entry[1] = entry[0].result()
+        entry[0] = None
+
+  def running():
+    return [e[0] for e in pending if e[0] is not None]
+
+  exhausted = False
+  while True:
+    collect()
+    while pending and pending[0][0] is None:
+      yield pending.popleft()[1]
+    if exhausted and not pending:
+      return
+    active = running()
+    if (not exhausted and len(active) < in_flight and
+        len(pending) < in_flight + max_unclaimed):
+      try:
+        item = next(todo)
+      except StopIteration:
+        exhausted = True
+        continue
+      pending.append([begin(item), None])
+      continue
+    # nothing to start: wait for the oldest one running (the others keep
+    # their chunks enqueued ahead and are looked at right after)
+    active[0].poll(block=True)
+
+
 def _begin_of(infer_step):
   """`begin_<name>` of the object whose bound method `infer_step` is (through
   functools.partial wrappers), with the wrappers' arguments bound again: the
@@ -106,14 +150,6 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
   params_of_step = inspect.signature(infer_step).parameters
   takes_rng = 'rng' in params_of_step
   takes_mutables = 'flax_mutables' in params_of_step
-
-  def infer_step_with_indices(params, batch, rng, indices, flax_mutables):
-    kwargs = {'flax_mutables': flax_mutables} if takes_mutables else {}
-    if takes_rng:
-      res = infer_step(params, batch, rng, **kwargs)
-    else:
-      res = infer_step(params, batch, **kwargs)
-    return indices, res
 
   if partitioner is not None:
     layout = partitioner.get_data_layout(batch_size)
@@ -149,44 +185,41 @@ def get_infer_fn(infer_step: Callable, batch_size: int,
     if takes_mutables or 'rng' not in params_of_step:
       begin = None
     n_in_flight = decodes_in_flight
-    in_flight = collections.deque()
 
-    def collect_oldest():
-      oldest = in_flight[0]
-      while not oldest.poll():
-        for other in list(in_flight)[1:]:
-          other.poll()
-        oldest.poll(block=True)
-      batched_results.append(in_flight.popleft().result())
-
-    for i in range(n_batches):
-      chunk = shard[i * per_shard_batch_size:(i + 1) * per_shard_batch_size]
-      index = np.asarray([c[0] for c in chunk], dtype=np.int64)
-      infer_batch = _stack([c[1] for c in chunk])
-      if rng is None:
-        step_rng = None
-      else:
-        step_rng, rng = split_rng(rng)
-      if begin is not None and n_in_flight is None:
-        ask = getattr(begin.func.__self__, 'batches_in_flight', None)
-        n_in_flight = (ask(infer_batch, begin.keywords.get('num_decodes'))
-                       if ask is not None else 1)
-        if n_in_flight <= 1:
-          begin = None
-      if begin is not None:
-        in_flight.append(begin(params, infer_batch, step_rng, in_flight=True))
+    def batches():
+      nonlocal rng
+      for i in range(n_batches):
+        chunk = shard[i * per_shard_batch_size:(i + 1) * per_shard_batch_size]
+        index = np.asarray([c[0] for c in chunk], dtype=np.int64)
+        infer_batch = _stack([c[1] for c in chunk])
+        if rng is None:
+          step_rng = None
+        else:
+          step_rng, rng = split_rng(rng)
         all_indices.append(index)
-        while len(in_flight) >= n_in_flight:
-          collect_oldest()
-        continue
-      batch_indices, batch_result = infer_step_with_indices(
-          params, infer_batch, step_rng, index, mutables)
+        yield infer_batch, step_rng
+
+    todo = batches()
+    if begin is not None and n_in_flight is None and n_batches:
+      first = next(todo)
+      ask = getattr(begin.func.__self__, 'batches_in_flight', None)
+      n_in_flight = (ask(first[0], begin.keywords.get('num_decodes'))
+                     if ask is not None else 1)
+      todo = itertools.chain([first], todo)
+    if begin is not None and (n_in_flight or 1) > 1:
+      batched_results.extend(map_in_flight(
+          lambda b: begin(params, b[0], b[1], in_flight=True), todo,
+          n_in_flight))
+    else:
       # Results stay on the device until everything is enqueued; the copies
       # below are what the reference's copy_to_host_async overlaps.
-      batched_results.append(batch_result)
-      all_indices.append(batch_indices)
-    while in_flight:
-      collect_oldest()
+      for infer_batch, step_rng in todo:
+        kwargs = {'flax_mutables': mutables} if takes_mutables else {}
+        if takes_rng:
+          batched_results.append(infer_step(params, infer_batch, step_rng,
+                                            **kwargs))
+        else:
+          batched_results.append(infer_step(params, infer_batch, **kwargs))
 
     batched_results = [tree_map(_to_numpy, r) for r in batched_results]
     all_inferences = tree_map(lambda *xs: np.concatenate(xs),

@@ -4,16 +4,17 @@
 Arrays are torch tensors on the GPU; NumPy inputs are uploaded.
 """
 
-import collections
 import dataclasses
 import functools
 import inspect
+import itertools
 from typing import Any, Callable, Mapping, MutableMapping, Optional, Tuple
 
 import numpy as np
 import torch
 
 from t5x_amd import decoding
+from t5x_amd import infer
 from t5x_amd import network
 
 
@@ -149,17 +150,21 @@ class EncoderDecoderModel:
     batches_in_flight() of the first batch.  With decode functions other than
     beam_search / temperature_sample the batches run one after the other."""
     rngs = iter(rngs) if rngs is not None else None
-    active = collections.deque()
-    for batch in batches:
-      if in_flight is None:
-        in_flight = self.batches_in_flight(batch, kwargs.get('num_decodes'))
+    batches = iter(batches)
+    try:
+      first = next(batches)
+    except StopIteration:
+      return
+    if in_flight is None:
+      in_flight = self.batches_in_flight(first, kwargs.get('num_decodes'))
+
+    def begin(batch):
       rng = next(rngs) if rngs is not None else None
-      active.append(self.begin_predict_batch_with_aux(
-          params, batch, rng, in_flight=in_flight > 1, **kwargs))
-      while len(active) >= max(1, in_flight):
-        yield _wait_for_oldest(active)
-    while active:
-      yield _wait_for_oldest(active)
+      return self.begin_predict_batch_with_aux(
+          params, batch, rng, in_flight=in_flight > 1, **kwargs)
+
+    yield from infer.map_in_flight(
+        begin, itertools.chain([first], batches), in_flight)
 
   def batches_in_flight(self, batch, num_decodes=None) -> int:
     """How many batches shaped like `batch` to keep decoding at once: as many
@@ -310,15 +315,3 @@ class Prediction:
     else:
       out = decodes[:, -1, :], {'scores': scores[:, -1]}
     return out[0] if self._first_only else out
-
-
-def _wait_for_oldest(active):
-  """Waits for the oldest of the predictions in flight, polling the others so
-  that their loops stay fed; removes it and returns its result."""
-  oldest = active[0]
-  while not oldest.poll():
-    for other in list(active)[1:]:
-      other.poll()
-    oldest.poll(block=True)
-  active.popleft()
-  return oldest.result()

@@ -511,7 +511,7 @@ def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
   device: every batch's tokens and scores are bit-identical to
   predict_batch_with_aux on that batch alone, in order, although the loops
   (of different lengths: an EOS-heavy vocabulary column ends some early)
-  interleave, and three kept contexts serve all seven."""
+  interleave, and at most three kept contexts serve all seven."""
   from t5x_amd import network
   ocfg, _, gm = _models(dtype, decode_fn_name, **kw)
   if decode_fn_name == 'beam_search':
@@ -542,13 +542,16 @@ def test_batches_in_flight_equal_batches_one_by_one(dtype, decode_fn_name, kw,
   for i, ((gd, ga), (wd, wa)) in enumerate(zip(got, want)):
     assert torch.equal(gd, wd), i
     assert torch.equal(ga['scores'], wa['scores']), i
+  # (at most three contexts; fewer when the short loops of this small model
+  # end before a third batch is begun)
   pools = list(gm.module._beam_ctx.values())
-  assert len(pools) == 1 and len(pools[0]) == 3
+  assert len(pools) == 1 and 1 <= len(pools[0]) <= 3
+  n_contexts = len(pools[0])
   # afterwards every context is free again: one more batch re-binds the first
   again = gm.predict_batch_with_aux(
       params, batches[2], rng=None if rngs is None else rngs[2], **common)
   assert torch.equal(again[0], want[2][0])
-  assert len(pools[0]) == 3
+  assert len(pools[0]) == n_contexts
 
 
 def test_loops_in_flight_with_poll_equal_run():

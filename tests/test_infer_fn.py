@@ -168,8 +168,8 @@ class _FakePrediction:
 
 
 class _FakeModel:
-  def __init__(self):
-    self.begun = []
+  def __init__(self, polls_needed=lambda k: 9 - 2 * k):
+    self.begun, self.polls_needed = [], polls_needed
 
   def predict_batch(self, params, batch, rng=None):
     return batch['a'][:, 0] * params['w']
@@ -177,9 +177,20 @@ class _FakeModel:
   def begin_predict_batch(self, params, batch, rng=None, in_flight=False):
     assert in_flight
     self.begun.append(int(batch['a'][0, 0]))
-    # later batches finish sooner: results must still come back in order
-    return _FakePrediction(len(self.begun), 9 - 2 * len(self.begun),
+    k = len(self.begun)
+    _FakePrediction.log.append((k, 'begin'))
+    # by default later batches finish sooner: results must still come back in
+    # order
+    return _FakePrediction(k, self.polls_needed(k),
                            self.predict_batch(params, batch, rng))
+
+
+def _max_running(log):
+  running = most = 0
+  for _, what in log:
+    running += {'begin': 1, 'result': -1}.get(what, 0)
+    most = max(most, running)
+  return most
 
 
 def test_decodes_in_flight_keep_order_and_bound_the_number_in_flight():
@@ -192,14 +203,29 @@ def test_decodes_in_flight_keep_order_and_bound_the_number_in_flight():
   assert out == [(i, 3 * i) for i in range(8)]
   assert model.begun == [0, 2, 4, 6]
   log = _FakePrediction.log
-  order = [name for name, what in log if what == 'result']
-  assert order == [1, 2, 3, 4]
+  assert sorted(name for name, what in log if what == 'result') == [1, 2, 3, 4]
   # never more than 3 begun and not yet collected; the 4th batch begins only
-  # after the first result was taken
-  first_result = log.index((1, 'result'))
+  # after a result was taken
+  assert _max_running(log) == 3
+  first_result = min(i for i, (_, what) in enumerate(log) if what == 'result')
   assert all(name != 4 for name, _ in log[:first_result])
-  # while waiting for the oldest, the others are polled (kept fed)
-  assert (2, 'poll') in log[:first_result] and (3, 'poll') in log[:first_result]
+  # while one is waited for, the others are looked at (kept fed)
+  assert {name for name, what in log[:first_result] if what == 'poll'} == {
+      1, 2, 3}
+
+
+def test_a_slow_batch_does_not_idle_the_places_of_the_others():
+  _FakePrediction.log = []
+  # the first batch needs far longer than the others
+  model = _FakeModel(polls_needed=lambda k: 60 if k == 1 else 2)
+  fn = infer.get_infer_fn(model.predict_batch, 1, decodes_in_flight=3)
+  out = fn(_dataset(7), {'w': 2})
+  assert out == [(i, 2 * i) for i in range(7)]      # still in order
+  log = _FakePrediction.log
+  assert _max_running(log) == 3
+  done = [name for name, what in log if what == 'result']
+  # every later batch was begun and collected while the first still ran
+  assert done[-1] == 1 and sorted(done[:-1]) == [2, 3, 4, 5, 6, 7]
 
 
 def test_decodes_in_flight_falls_back_to_the_plain_step():
