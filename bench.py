@@ -723,7 +723,12 @@ def main():
     n_in_flight = (w.module.streams_side_by_side()
                    if args.config == DEFAULT_CONFIG else 0)
   if n_in_flight > 1:
-    out['in_flight'] = in_flight_throughput(w, n_in_flight)
+    # an extra figure: whatever goes wrong in it must not cost the line
+    try:
+      out['in_flight'] = in_flight_throughput(w, n_in_flight)
+    except Exception as e:  # pylint: disable=broad-except
+      out['in_flight'] = {'decodes': n_in_flight, 'value': None,
+                          'error': f'{type(e).__name__}: {e}'}
   if not args.no_cpu_baseline and size != 'xxl':
     out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
   print(json.dumps(out))
