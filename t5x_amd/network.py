@@ -225,6 +225,10 @@ class _StepBuffers:
                               device=device)
 
 
+# device index -> the decode streams of that device (Transformer.decode_stream)
+_DECODE_STREAMS = {}
+
+
 class Transformer:
   """network.Transformer with `apply(variables, *args, method=..., **kwargs)`.
 
@@ -265,7 +269,6 @@ class Transformer:
     self._cross = None
     self._step_cache = None
     self._beam_ctx = {}
-    self._streams = None
 
   # -- plumbing ---------------------------------------------------------------
   def _dev(self):
@@ -648,20 +651,26 @@ class Transformer:
     lanes: of lane l of the context in slot s, at s * lanes + l).  The device
     runs streams side by side only when they sit on different hardware
     queues, of which a process has few (4 by default) and which streams are
-    given in turn as they are first used; so the module makes its streams
-    once, together, and uses each once right away: consecutive slots then sit
-    on different queues whatever streams the caller makes in between."""
-    if self._streams is None:
-      dev = self._dev()
-      self._streams = [torch.cuda.Stream(device=dev)
-                       for _ in range(self.MAX_CONTEXTS_PER_KEY)]
+    given in turn as they are first used; so the decode streams of a device
+    are made once per process, together, and each is used once right away:
+    consecutive slots then sit on different queues whatever streams the
+    caller, or another model on the same device, makes later."""
+    dev = self._dev()
+    key = torch.device(dev).index
+    if key is None:
+      key = torch.cuda.current_device()
+    streams = _DECODE_STREAMS.get(key)
+    if streams is None:
+      streams = [torch.cuda.Stream(device=dev)
+                 for _ in range(self.MAX_CONTEXTS_PER_KEY)]
       touch = torch.zeros((16,), dtype=torch.int32, device=dev)
       torch.cuda.current_stream().synchronize()
-      for stream in self._streams:
+      for stream in streams:
         with torch.cuda.stream(stream):
           touch.zero_()
         stream.synchronize()
-    return self._streams[slot % len(self._streams)]
+      _DECODE_STREAMS[key] = streams
+    return streams[slot % len(streams)]
 
   # -- fused sampling: one graph replay per loop iteration --------------------------
   def make_fused_sample_step(self, params, encoded, enc_tokens, owner=None,
