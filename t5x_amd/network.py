@@ -227,6 +227,47 @@ class _StepBuffers:
 
 # device index -> the decode streams of that device (Transformer.decode_stream)
 _DECODE_STREAMS = {}
+# device index -> how many of them (the first n) were measured to run side by
+# side, or None where that could not be measured
+_DECODE_STREAMS_SIDE_BY_SIDE = {}
+
+
+def _measure_side_by_side(streams):
+  """The largest n for which busy kernels on the first n streams overlap: n
+  kernels of about half a millisecond, one per stream, must finish in less
+  than 1.5 times what one takes.  None without a busy kernel to use."""
+  import time
+  sleep = getattr(torch.cuda, '_sleep', None)
+  if sleep is None:
+    return None
+
+  def timed(group, cycles):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for stream in group:
+      with torch.cuda.stream(stream):
+        sleep(cycles)
+    for stream in group:
+      stream.synchronize()
+    return time.perf_counter() - t0
+
+  cycles = 100_000
+  one = timed(streams[:1], cycles)
+  for _ in range(8):  # the unit of `cycles` is the device's business
+    if one >= 4e-4:
+      break
+    cycles *= 4
+    one = timed(streams[:1], cycles)
+  if one < 4e-4:
+    return None
+  one = min(one, timed(streams[:1], cycles))
+  n = 1
+  while n < len(streams):
+    together = min(timed(streams[:n + 1], cycles) for _ in range(2))
+    if together > 1.5 * one:
+      break
+    n += 1
+  return n
 
 
 class Transformer:
@@ -567,7 +608,8 @@ class Transformer:
     if loop.beam_size > 8:
       return None
     w = self.decoder_weights(params)
-    lanes = self.decode_lanes or (1 if in_flight else 2)
+    lanes = self.decode_lanes or (
+        1 if in_flight or self.streams_side_by_side() < 2 else 2)
     lanes = max(1, min(int(lanes), loop.batch_size))
     key = (id(w), tuple(encoded.x.shape), encoded.x.dtype, encoded.beams,
            loop.batch_size, loop.beam_size, loop.max_decode_len,
@@ -610,19 +652,30 @@ class Transformer:
       pool.append(ctx)
     return ctx
 
-  @staticmethod
-  def streams_side_by_side() -> int:
-    """How many decode streams the device runs side by side: one hardware
+  def streams_side_by_side(self) -> int:
+    """How many decode streams the device runs side by side.  One hardware
     queue of the process serves the default stream, the others are dealt to
     the streams in turn, and queues beyond the fourth share command
-    processors (measured: 3 decodes in flight pay with the runtime's default
-    of 4 queues, 4 with GPU_MAX_HW_QUEUES=8 or more, a fifth never)."""
+    processors (3 decodes in flight pay with the runtime's default of 4
+    queues, 4 with GPU_MAX_HW_QUEUES=8 or more, a fifth never).  Which queue a
+    stream got cannot be asked, so it is measured once per device when the
+    decode streams are made: the first n streams count when n short busy
+    kernels, one per stream, take about as long as one."""
+    self.decode_stream(0)
+    key = self._stream_key()
+    measured = _DECODE_STREAMS_SIDE_BY_SIDE.get(key)
+    if measured is not None:
+      return measured
     import os
     try:
       queues = int(os.environ.get('GPU_MAX_HW_QUEUES', '4'))
     except ValueError:
       queues = 4
     return 4 if queues >= 8 else 3
+
+  def _stream_key(self):
+    key = torch.device(self._dev()).index
+    return torch.cuda.current_device() if key is None else key
 
   def decode_context_bytes(self, batch_size, num_decodes, enc_len,
                            decode_len) -> int:
@@ -655,10 +708,7 @@ class Transformer:
     are made once per process, together, and each is used once right away:
     consecutive slots then sit on different queues whatever streams the
     caller, or another model on the same device, makes later."""
-    dev = self._dev()
-    key = torch.device(dev).index
-    if key is None:
-      key = torch.cuda.current_device()
+    dev, key = self._dev(), self._stream_key()
     streams = _DECODE_STREAMS.get(key)
     if streams is None:
       streams = [torch.cuda.Stream(device=dev)
@@ -670,6 +720,7 @@ class Transformer:
           touch.zero_()
         stream.synchronize()
       _DECODE_STREAMS[key] = streams
+      _DECODE_STREAMS_SIDE_BY_SIDE[key] = _measure_side_by_side(streams)
     return streams[slot % len(streams)]
 
   # -- fused sampling: one graph replay per loop iteration --------------------------
