@@ -184,35 +184,71 @@ class Workload:
         sync()
         seconds += time.perf_counter() - t0
         windows.append((first, first + take - 1))
+        # A loop flag that had closed would turn every kernel of the window
+        # into an early return and the window would read fast: the device's
+        # own step count must have advanced by what was timed.
+        if self.steps_on_device() != first + take:
+          raise RuntimeError(
+              f'timed window {first}..{first + take - 1}: the device is at '
+              f'step {self.steps_on_device()}, not {first + take}')
       done += take
     if timed and self.loop.step >= self.L:
       self.check_full_decode()
     return seconds, windows
 
+  def steps_on_device(self):
+    """Loop iterations the device has completed in the current decode."""
+    if self.loop_kind == 'beam':
+      return int(self.loop.cur.cur_index.item())
+    return int(self.loop.fused.step_count.item())
+
   def check_full_decode(self):
     if self.loop.cond():
       raise RuntimeError('decode did not stop at max_decode_len')
-    if self.loop_kind == 'beam':
-      count = int(self.loop.cur.cur_index.item())
-    else:
-      count = int(self.loop.fused.step_count.item())
+    count = self.steps_on_device()
     if count != self.L:
       raise RuntimeError(f'decode stopped early at step {count}; the step '
                          'count of this run would be wrong')
 
   # -- algorithmic traffic (bytes) of one launch, by kernel ---------------------
-  def cross_attention_bytes(self, fused=True):
-    """Valid K and V rows once per batch item and the attention output out;
-    in: the residual-stream rows, the layer-norm scale and the query kernel
-    (fused projection), or the projected queries."""
+  def cross_attention_bytes(self):
+    """Algorithmic bytes of one cross-attention launch: the valid K and V
+    rows once per batch item (shared by its beams, padded keys skipped), the
+    queries in and the attention output out."""
+    s = self.encoded.element_size()
+    hd = self.cfg.num_heads * self.cfg.head_dim
+    R = self.B * self.K
+    return int(self.enc_lens.sum()) * hd * 2 * s + 2 * R * hd * s
+
+  def fused_query_bytes(self):
+    """What the launch moves on top of that when the pre-attention layer norm
+    and the query projection ride inside it: residual-stream rows and the
+    norm scale in and the query kernel once, instead of the queries in.  It
+    belongs to the dense layers' account, not to the attention's."""
     s = self.encoded.element_size()
     hd = self.cfg.num_heads * self.cfg.head_dim
     d = self.cfg.emb_dim
     R = self.B * self.K
-    kv = int(self.enc_lens.sum()) * hd * 2 * s
-    if fused:
-      return kv + R * d * s + d * s + d * hd * s + R * hd * s
-    return kv + 2 * R * hd * s
+    return R * d * s + d * s + d * hd * s - R * hd * s
+
+  def step_bytes(self):
+    """Algorithmic bytes of one loop iteration, averaged over the positions
+    of a decode: every decoder weight once, the valid self-attention prefix
+    and the valid cross K/V once per batch item per layer, the cache rows
+    the beam reorder has to move (none here: beams inherit their parents'
+    slots; the reference's gather is not counted), activations."""
+    c = self.cfg
+    s = self.encoded.element_size()
+    wbytes = 1 if c.weight_dtype == 'int8' else s
+    d, F, V = c.emb_dim, c.mlp_dim, c.vocab_size
+    hd = c.num_heads * c.head_dim
+    R, nl = self.B * self.K, c.num_decoder_layers
+    weights = nl * (d * 3 * hd + hd * d + d * hd + hd * d + d * 2 * F +
+                    F * d) * wbytes + d * V * wbytes
+    self_kv = nl * float(np.mean([self.self_attention_bytes(t)
+                                  for t in range(self.L)]))
+    cross = nl * self.cross_attention_bytes()
+    return int(weights + self_kv + cross)
 
   def self_attention_bytes(self, t):
     s = 2
@@ -258,17 +294,57 @@ PROFILE_NOTE = os.path.join(os.path.dirname(os.path.abspath(__file__)),
                             'cross_attn_mfma_kernel_base-beam4_pmc.txt')
 
 
+STEP_TRAFFIC_NOTE = os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                 'profiles',
+                                 'decode_step_base-beam4_hbm_traffic_pmc.txt')
+
+
+def _noted(path, key):
+  if not os.path.exists(path):
+    return None
+  with open(path) as f:
+    for line in f:
+      if line.startswith(key + ':'):
+        return int(float(line.split(':', 1)[1]))
+  return None
+
+
 def measured_traffic(name):
   """HBM bytes per launch of the dominant kernel from the committed counter
   summary (FETCH_SIZE + WRITE_SIZE, calibrated against a plain copy), or None
   when no summary exists for this workload."""
-  if name != 'base-beam4' or not os.path.exists(PROFILE_NOTE):
+  if name != 'base-beam4':
     return None
-  with open(PROFILE_NOTE) as f:
-    for line in f:
-      if line.startswith('traffic_bytes_per_launch:'):
-        return int(float(line.split(':', 1)[1]))
-  return None
+  return _noted(PROFILE_NOTE, 'traffic_bytes_per_launch')
+
+
+def device_level(w, ms_per_step, in_flight):
+  """Bytes per loop iteration over the wall-clock time of an iteration, for
+  the modes the product runs in (batch lanes side by side; several batches in
+  flight): the device-level counterpart of the per-launch roofline figure,
+  which is measured on a single chain of kernels.  `algorithmic`: the bytes an
+  iteration has to move (Workload.step_bytes); `traffic`: what the memory
+  counters read for all kernels of an iteration (FETCH_SIZE + WRITE_SIZE summed
+  over a kernel trace of the loop, from the committed summary; the counters
+  serialise dispatches, which changes when bytes move, not how many)."""
+  alg = w.step_bytes()
+  traffic = (_noted(STEP_TRAFFIC_NOTE, 'step_traffic_bytes')
+             if w.name == 'base-beam4' else None)
+
+  def rates(ms):
+    out = {'ms_per_step': ms,
+           'algorithmic_gbps': round(alg / ms / 1e6, 1),
+           'algorithmic_frac': round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    if traffic:
+      out['traffic_gbps'] = round(traffic / ms / 1e6, 1)
+      out['traffic_frac'] = round(traffic / ms / 1e6 / HBM_PEAK_GBPS, 4)
+    return out
+
+  out = {'algorithmic_bytes_per_step': alg, 'traffic_bytes_per_step': traffic,
+         'one_batch': rates(ms_per_step)}
+  if in_flight and in_flight.get('value'):
+    out['batches_in_flight'] = rates(in_flight['ms_per_step'])
+  return out
 
 
 def in_loop_kernel_times(w, families, repeats=3):
@@ -356,13 +432,16 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
 
   reps = max(1, min(reps_per_layer, 96 // nl))
   replay_sec = time_kernel(torch, launch, reps * nl)
-  nbytes = w.cross_attention_bytes(fused)
+  nbytes = w.cross_attention_bytes()
   if fused:
     name = 'cross_attn_mfma_kernel<4,4,%d>' % ((cfg.emb_dim // 64 + 3) // 4)
   else:
     name = 'cross_attn_mfma_kernel (query projected separately)'
   out = {'kernel': name, 'bound': 'hbm', 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-         'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes}
+         'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes,
+         # moved by the same launch for the dense layers' account (layer norm
+         # + query projection fused in); not part of `achieved`
+         'fused_query_bytes': w.fused_query_bytes() if fused else 0}
   sec, where = replay_sec, 'back-to-back replay over the layers'
   if in_loop and w.bf16:
     # The figure that counts is the kernel's duration inside the decode loop
@@ -708,6 +787,9 @@ def main():
                  # batch slices stepped side by side on separate streams
                  'batch_lanes': getattr(getattr(w.loop, 'fused', None),
                                         'n_lanes', 1),
+                 # decode streams the device was found (or told) to run side
+                 # by side: decides the lanes above and the batches in flight
+                 'streams_side_by_side': w.module.streams_side_by_side(),
                  # positions t of the decode the timed iterations covered:
                  # whole decodes, then a window centred on (L-1)/2
                  't_first': windows[-1][0], 't_last': windows[-1][1],
@@ -729,6 +811,8 @@ def main():
     except Exception as e:  # pylint: disable=broad-except
       out['in_flight'] = {'decodes': n_in_flight, 'value': None,
                           'error': f'{type(e).__name__}: {e}'}
+  out['roofline']['device_level'] = device_level(
+      w, out['ms_per_step'], out.get('in_flight'))
   if not args.no_cpu_baseline and size != 'xxl':
     out['cpu_baseline'] = cpu_baseline(args.config, args.cpu_steps, args.seed)
   print(json.dumps(out))

@@ -95,8 +95,11 @@ int t5d_rmsnorm(void* stream, int dtype, const void* x, const void* scale,
  *   T5D_EPI_GEGLU: W is a geglu-packed [K, 2F] kernel, N = 2F, C is [M, F].
  *   The kernels are laid out for M <= 128 (the weights stream once); more rows
  *   run as chunks of 128, each streaming the weights again.
- *   Layers of 8 MB of weights and more run on large workgroup tiles (up to
- *   128 x 128) chosen so that the most loaded CU reads the fewest bytes.
+ *   Which workgroup tile a shape runs on is internal (layers of 24 MB of
+ *   weights and more with M >= 32 and K >= 2048 take large tiles of up to
+ *   128 x 128, chosen so that the most loaded CU reads the fewest bytes);
+ *   every tile splits and sums K the same way, so the result's bits do not
+ *   depend on it.
  *   workspace/counters: reserved for plans that need scratch memory; no plan
  *   does (t5d_gemm_workspace_bytes returns 0 for every shape) and both may
  *   be NULL. */
@@ -448,18 +451,7 @@ typedef struct {
    * t5d_self_attention_step_gather (bfloat16, L a multiple of 32); 2: the
    * cached_key too */
   int value_blocked;
-  /* Measurement aid, normally 0: a mask of T5D_LEAVE_OUT_* bits; the step is
-   * enqueued WITHOUT the launches of those kernel families (their outputs keep
-   * whatever the buffers held, so the results are meaningless).  The time a
-   * loop of such steps saves against the full loop is what the family costs
-   * where it runs, between the step's other kernels. */
-  int leave_out;
 } t5d_model_step;
-
-enum {
-  T5D_LEAVE_OUT_CROSS_ATTENTION = 1,  /* t5d_cross_attention_step[_norm_q] */
-  T5D_LEAVE_OUT_SELF_ATTENTION = 2    /* t5d_self_attention_step[_gather] */
-};
 
 /* One decoder step for R rows (Decoder.__call__ with decode=True,
  * t5x/examples/t5/network.py:229-292, as driven by

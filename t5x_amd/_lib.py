@@ -46,7 +46,7 @@ class ModelStep(Structure):
                   'xn', 'qkv', 'q',
                   'ao', 'h', 'logits', 'gate', 'pending_src',
                   'pending_dst')] +
-              [('value_blocked', c_int), ('leave_out', c_int)])
+              [('value_blocked', c_int)])
 
 
 class BeamStep(Structure):
@@ -88,6 +88,7 @@ _SIGNATURES = {
     't5d_graph_launch': (c_int, [_P, _P]),
     't5d_graph_destroy': (c_int, [_P]),
     't5d_version': (c_int, []),
+    't5d_measure_leave_out': (c_int, [c_int]),
     't5d_last_error': (c_char_p, []),
     't5d_packed_weight_bytes': (c_int64, [c_int, c_int, c_int]),
     't5d_pack_weight': (c_int, [_P, c_int, _P, _P, _P, c_int, c_int, c_int]),
@@ -168,6 +169,13 @@ def load():
 
 def exported_names():
   return sorted(_SIGNATURES)
+
+
+def measure_leave_out(mask: int) -> int:
+  """t5d_measure_leave_out (include/t5d_measure.h, a measurement aid that is
+  not part of the boundary): sets the calling thread's mask of kernel
+  families that fused steps are enqueued without; returns the previous one."""
+  return int(load().t5d_measure_leave_out(int(mask)))
 
 
 def last_error() -> str:

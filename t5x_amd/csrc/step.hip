@@ -5,10 +5,15 @@
 #include <vector>
 
 #include "common.h"
+#include "../../include/t5d_measure.h"
 
 using namespace t5d;
 
 namespace {
+
+// t5d_measure_leave_out: kernel families the calling thread's fused steps are
+// enqueued without (a measurement aid, 0 in every product call).
+thread_local int tls_leave_out = 0;
 
 struct GateScope {
   explicit GateScope(const int32_t* g) { tls_gate = g; }
@@ -87,8 +92,8 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
       T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->xn, w.qkv, w.qkv_scales, nullptr,
                        m->qkv, R, d, 3 * HD, T5D_EPI_NONE, nullptr, nullptr));
     }
-    if (m->leave_out & T5D_LEAVE_OUT_SELF_ATTENTION) {
-      // measurement aid: see t5d_model_step::leave_out
+    if (tls_leave_out & T5D_LEAVE_OUT_SELF_ATTENTION) {
+      // measurement aid: see t5d_measure_leave_out
     } else if (m->pending_src || m->value_blocked)
       T5D_TRY(t5d_self_attention_step_gather(
           stream, dt, m->qkv, w.cached_key, w.cached_value, m->rel_bias,
@@ -101,9 +106,9 @@ int decoder_step_impl(void* stream, const t5d_model_step* m, const int32_t* ids,
                                       m->L));
     T5D_TRY(t5d_gemm(stream, dt, wd, dt, m->ao, w.self_out, w.self_out_scales,
                      x, m->x1, R, HD, d, T5D_EPI_RESIDUAL, nullptr, nullptr));
-    const bool no_cross = m->leave_out & T5D_LEAVE_OUT_CROSS_ATTENTION;
+    const bool no_cross = tls_leave_out & T5D_LEAVE_OUT_CROSS_ATTENTION;
     if (no_cross && fuse_cross_q) {
-      // measurement aid: see t5d_model_step::leave_out
+      // measurement aid: see t5d_measure_leave_out
     } else if (fuse_cross_q) {
       T5D_TRY(t5d_cross_attention_step_norm_q(
           stream, dt, wd, m->x1, w.ln_cross, 1e-6f, w.cross_q, w.cross_key,
@@ -245,6 +250,12 @@ extern "C" int t5d_temperature_sample_step(void* stream,
   GateScope gate(s->keep_going);
   return launch_sample_step(as_stream(stream), m->logits, s, m->R, m->V,
                             m->cache_index, m->NL);
+}
+
+extern "C" int t5d_measure_leave_out(int mask) {
+  const int before = tls_leave_out;
+  tls_leave_out = mask;
+  return before;
 }
 
 // ---- HIP graph capture --------------------------------------------------------

@@ -118,19 +118,39 @@ def map_in_flight(begin, items, in_flight: int, max_unclaimed: int = 16):
     active[0].poll(block=True)
 
 
+def _defined_at(obj, name):
+  """Position in type(obj)'s method resolution order of the class that defines
+  `name` (0: the most derived class); None if no class does."""
+  for depth, cls in enumerate(type(obj).__mro__):
+    if name in vars(cls):
+      return depth
+  return None
+
+
 def _begin_of(infer_step):
   """`begin_<name>` of the object whose bound method `infer_step` is (through
   functools.partial wrappers), with the wrappers' arguments bound again: the
   variant of the step that returns, without waiting, an object with poll() and
-  result().  None when there is no such variant."""
+  result().  None when there is no such variant, and also when a subclass has
+  overridden the step (or a method the variant stands for, listed in its
+  `stands_for`) without overriding the variant: the override is then what the
+  reference's `infer_step(params, batch, rng)` contract calls, and the
+  inherited variant would bypass it."""
   fn, args, kwargs = infer_step, (), {}
   while isinstance(fn, functools.partial):
     args, kwargs = fn.args + args, {**fn.keywords, **kwargs}
     fn = fn.func
-  begin = getattr(getattr(fn, '__self__', None),
-                  'begin_' + getattr(fn, '__name__', ''), None)
-  if begin is None:
+  owner, name = getattr(fn, '__self__', None), getattr(fn, '__name__', '')
+  begin = getattr(owner, 'begin_' + name, None)
+  if begin is None or not inspect.ismethod(fn) or not inspect.ismethod(begin):
     return None
+  begin_depth = _defined_at(owner, 'begin_' + name)
+  if begin_depth is None:
+    return None
+  for covered in getattr(begin, 'stands_for', (name,)):
+    depth = _defined_at(owner, covered)
+    if depth is None or depth < begin_depth:
+      return None
   return functools.partial(begin, *args, **kwargs)
 
 

@@ -139,6 +139,11 @@ class EncoderDecoderModel:
     return self.begin_predict_batch_with_aux(params, batch, rng,
                                              in_flight=in_flight).first()
 
+  # the methods a caller may hold instead of which begin_predict_batch can be
+  # called: a subclass that overrides one of them without overriding the
+  # begin variant must be called through its override (infer._begin_of)
+  begin_predict_batch.stands_for = ('predict_batch', 'predict_batch_with_aux')
+
   def predict_batches(self, params, batches, rngs=None,
                       in_flight: Optional[int] = None, **kwargs):
     """predict_batch_with_aux over an iterable of batches, yielding each
@@ -255,6 +260,10 @@ class EncoderDecoderModel:
       decode = begin(**bound, **decode_kwargs)
       decode.start()
     return Prediction(decode, return_all_decodes)
+
+
+EncoderDecoderModel.begin_predict_batch_with_aux.stands_for = (
+    'predict_batch_with_aux',)
 
 
 def _begin_of(decode_fn):

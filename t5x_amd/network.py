@@ -235,7 +235,10 @@ _DECODE_STREAMS_SIDE_BY_SIDE = {}
 def _measure_side_by_side(streams):
   """The largest n for which busy kernels on the first n streams overlap: n
   kernels of about half a millisecond, one per stream, must finish in less
-  than 1.5 times what one takes.  None without a busy kernel to use."""
+  than 1.5 times what one takes (the shortest of three runs each; on a busy
+  device a single run can read long).  The whole measurement is taken twice;
+  None when the two disagree or when there is no busy kernel to use: the
+  caller then goes by the number of hardware queues instead."""
   import time
   sleep = getattr(torch.cuda, '_sleep', None)
   if sleep is None:
@@ -260,14 +263,19 @@ def _measure_side_by_side(streams):
     one = timed(streams[:1], cycles)
   if one < 4e-4:
     return None
-  one = min(one, timed(streams[:1], cycles))
-  n = 1
-  while n < len(streams):
-    together = min(timed(streams[:n + 1], cycles) for _ in range(2))
-    if together > 1.5 * one:
-      break
-    n += 1
-  return n
+
+  def count():
+    alone = min(timed(streams[:1], cycles) for _ in range(3))
+    n = 1
+    while n < len(streams):
+      together = min(timed(streams[:n + 1], cycles) for _ in range(3))
+      if together > 1.5 * alone:
+        break
+      n += 1
+    return n
+
+  first, second = count(), count()
+  return first if first == second else None
 
 
 class Transformer:
@@ -286,6 +294,13 @@ class Transformer:
   # decode on its own, 1 when several batches are in flight (those fill the
   # device better than lanes do, and streams that run side by side are few).
   decode_lanes = None
+
+  # How many decode streams the device runs side by side.  None: the
+  # environment variable T5X_AMD_STREAMS_SIDE_BY_SIDE if set, else measured
+  # once per device and process (streams_side_by_side).  A fixed value makes
+  # the number of batch lanes and of batches in flight, hence what is
+  # captured and held, the same in every run; results never depend on it.
+  side_by_side = None
 
   def __init__(self, config: T5Config, device=None, scan_layers: bool = False):
     """scan_layers: hand out and accept the cache in the layout of a scanned
@@ -499,7 +514,6 @@ class Transformer:
     m.pending_src, m.pending_dst = P(pending_src), P(pending_dst)
     # the loops that block their value caches block their key caches too
     m.value_blocked = 2 if value_blocked else 0
-    m.leave_out = 0
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
                     pending_src, pending_dst)
     return m
@@ -661,12 +675,17 @@ class Transformer:
     stream got cannot be asked, so it is measured once per device when the
     decode streams are made: the first n streams count when n short busy
     kernels, one per stream, take about as long as one."""
-    self.decode_stream(0)
+    import os
+    fixed = self.side_by_side
+    if fixed is None and os.environ.get('T5X_AMD_STREAMS_SIDE_BY_SIDE'):
+      fixed = int(os.environ['T5X_AMD_STREAMS_SIDE_BY_SIDE'])
+    if fixed is not None:
+      return max(1, min(int(fixed), self.MAX_CONTEXTS_PER_KEY))
+    self.decode_stream(0, measure=True)
     key = self._stream_key()
     measured = _DECODE_STREAMS_SIDE_BY_SIDE.get(key)
     if measured is not None:
       return measured
-    import os
     try:
       queues = int(os.environ.get('GPU_MAX_HW_QUEUES', '4'))
     except ValueError:
@@ -699,7 +718,7 @@ class Transformer:
     free, _ = torch.cuda.mem_get_info(self._dev())
     return max(1, min(n, int(free // 2 // max(1, need))))
 
-  def decode_stream(self, slot):
+  def decode_stream(self, slot, measure=False):
     """The stream of the decode contexts in pool slot `slot` (with batch
     lanes: of lane l of the context in slot s, at s * lanes + l).  The device
     runs streams side by side only when they sit on different hardware
@@ -720,6 +739,7 @@ class Transformer:
           touch.zero_()
         stream.synchronize()
       _DECODE_STREAMS[key] = streams
+    if measure and key not in _DECODE_STREAMS_SIDE_BY_SIDE:
       _DECODE_STREAMS_SIDE_BY_SIDE[key] = _measure_side_by_side(streams)
     return streams[slot % len(streams)]
 
@@ -943,16 +963,16 @@ class FusedSampleStep(_OwnedContext):
 
   def iteration_graph(self, leave_out=0):
     """A graph of one iteration enqueued without the kernel families in the
-    `leave_out` mask (t5d_model_step::leave_out; 0: the full iteration), for
+    `leave_out` mask (t5d_measure_leave_out; 0: the full iteration), for
     timing a family by difference.  The caller replays it with launch_graph
     and destroys it with t5d_graph_destroy."""
     self.stream.synchronize()
-    self.model.leave_out = int(leave_out)
+    before = self._lib.measure_leave_out(int(leave_out))
     try:
       with torch.cuda.stream(self.stream):
         return self._record()
     finally:
-      self.model.leave_out = 0
+      self._lib.measure_leave_out(before)
 
   def launch_graph(self, graph, n):
     for _ in range(n):
@@ -1277,19 +1297,19 @@ class FusedBeamStep(_OwnedContext):
 
   def iteration_graph(self, leave_out=0):
     """A graph of one iteration enqueued without the kernel families in the
-    `leave_out` mask (t5d_model_step::leave_out; 0: the full iteration), for
+    `leave_out` mask (t5d_measure_leave_out; 0: the full iteration), for
     timing a family by difference.  Single-lane loops.  The caller replays it
     with launch_graph and destroys it with t5d_graph_destroy."""
     if self.n_lanes != 1:
       raise ValueError('iteration graphs are for the single-lane loop')
     lane = self.lanes[0]
     lane.stream.synchronize()
-    lane.model.leave_out = int(leave_out)
+    before = self._lib.measure_leave_out(int(leave_out))
     try:
       with torch.cuda.stream(lane.stream):
         return self._record(lane, 1)
     finally:
-      lane.model.leave_out = 0
+      self._lib.measure_leave_out(before)
 
   def launch_graph(self, graph, n):
     stream = self.lanes[0].stream.cuda_stream

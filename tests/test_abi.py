@@ -1,5 +1,5 @@
-"""The C-ABI library loads and exports every entry point include/t5d.h
-declares (no compute calls: this runs without a GPU)."""
+"""The C-ABI library loads and exports every entry point include/*.h
+declare (no compute calls: this runs without a GPU)."""
 
 import ctypes
 import os
@@ -13,7 +13,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_names():
-  text = open(os.path.join(ROOT, 'include', 't5d.h')).read()
+  inc = os.path.join(ROOT, 'include')
+  text = ''.join(open(os.path.join(inc, f)).read()
+                 for f in sorted(os.listdir(inc)) if f.endswith('.h'))
   text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
   return sorted(set(re.findall(r'\b(t5d_[a-z0-9_]+)\s*\(', text)))
 
@@ -34,6 +36,37 @@ def test_library_exports_every_declared_symbol():
 
 def test_binding_covers_every_declared_symbol():
   assert set(declared_names()) == set(_lib.exported_names())
+
+
+def test_measurement_aids_stay_out_of_the_boundary():
+  """The work-skipping switch bench.py uses lives in its own header and entry
+  point; the boundary's structs and declarations carry none."""
+  boundary = open(os.path.join(ROOT, 'include', 't5d.h')).read()
+  assert 'leave_out' not in boundary and 'LEAVE_OUT' not in boundary
+  aids = open(os.path.join(ROOT, 'include', 't5d_measure.h')).read()
+  assert 't5d_measure_leave_out' in aids
+  if not os.path.exists(_lib.LIB_PATH):
+    pytest.fail(f'{_lib.LIB_PATH} not built: run __graft_entry__.build()')
+  assert hasattr(ctypes.CDLL(_lib.LIB_PATH), 't5d_measure_leave_out')
+  assert _lib.measure_leave_out(0) == 0
+  # no product module calls it
+  pkg = os.path.join(ROOT, 't5x_amd')
+  users = [f for f in os.listdir(pkg) if f.endswith('.py') and
+           'measure_leave_out(' in open(os.path.join(pkg, f)).read()]
+  assert sorted(users) == ['_lib.py', 'network.py']  # iteration_graph only
+
+
+def test_static_entry_point_calls_no_allocator():
+  """Source check: neither the entry point nor its address look-up names an
+  allocating or freeing HIP call."""
+  src = open(os.path.join(ROOT, 't5x_amd', 'csrc', 'select.hip')).read()
+  start = src.index('static int static_topk_scratch(')
+  entry = src.index('extern "C" int t5d_beam_topk_static(')
+  end = src.index('\n}\n', entry)
+  body = src[start:end]
+  assert 'hipGetSymbolAddress' in body
+  assert not re.search(r'hipMalloc|hipFree|hipMallocAsync|hipHostMalloc|'
+                       r'hipExtMalloc|hipMemPool', body)
 
 
 def test_version_and_error_string_without_gpu():

@@ -239,6 +239,56 @@ def test_decodes_in_flight_falls_back_to_the_plain_step():
   assert model.begun == []
 
 
+def test_an_overridden_step_is_called_not_the_inherited_begin_variant():
+  """t5x/utils.py:1684-1700 calls `infer_step(params, batch, rng)`: a subclass
+  that overrides the step keeps being called through its override, also when
+  several decodes in flight are asked for; one that overrides the begin
+  variant as well gets the overlap back."""
+
+  class Doubling(_FakeModel):
+    def predict_batch(self, params, batch, rng=None):
+      return 2 * super().predict_batch(params, batch, rng)
+
+  model = Doubling()
+  fn = infer.get_infer_fn(model.predict_batch, 2, decodes_in_flight=3)
+  assert fn(_dataset(4), {'w': 3}) == [(i, 6 * i) for i in range(4)]
+  assert model.begun == []
+
+  class DoublingBoth(Doubling):
+    def begin_predict_batch(self, params, batch, rng=None, in_flight=False):
+      return super().begin_predict_batch(params, batch, rng, in_flight)
+
+  _FakePrediction.log = []
+  model = DoublingBoth()
+  fn = infer.get_infer_fn(model.predict_batch, 2, decodes_in_flight=3)
+  assert fn(_dataset(4), {'w': 3}) == [(i, 6 * i) for i in range(4)]
+  assert model.begun == [0, 2]
+
+
+def test_model_subclass_overriding_predict_batch_with_aux_is_honoured():
+  """The product's EncoderDecoderModel: `predict_batch` of a subclass that
+  overrides only predict_batch_with_aux must reach the override, so the
+  inherited begin_predict_batch (which would bypass it) is not used."""
+  from t5x_amd import models
+
+  class Post(models.EncoderDecoderModel):
+    def predict_batch_with_aux(self, params, batch, rng=None, **kw):
+      return batch['a'][:, 0] + params['w'], {'scores': batch['a'][:, 0]}
+
+  model = Post(module=None)
+  assert infer._begin_of(model.predict_batch) is None
+  assert infer._begin_of(model.predict_batch_with_aux) is None
+  base = models.EncoderDecoderModel(module=None)
+  assert infer._begin_of(base.predict_batch) is not None
+  assert infer._begin_of(base.predict_batch_with_aux) is not None
+  fn = infer.get_infer_fn(model.predict_batch, 2)
+  assert fn(_dataset(4), {'w': 5}) == [(i, i + 5) for i in range(4)]
+  fn = infer.get_infer_fn(model.predict_batch_with_aux, 2)
+  out, aux = fn(_dataset(4), {'w': 5})
+  assert out == [(i, i + 5) for i in range(4)]
+  assert aux == {'scores': [0, 1, 2, 3]}
+
+
 class _FakeFused:
   """A fused step context: the loop condition turns false after `end`
   iterations; chunks complete one poll after they are asked about."""

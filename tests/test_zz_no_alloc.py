@@ -35,17 +35,22 @@ def _both(B, beams, V, k, seed):
             want[0].data_ptr(), want[1].data_ptr(), want[2].data_ptr(),
             want[3].data_ptr(), scratch.data_ptr(), B, beams, V, k)
   got = outputs()
+
+  def static_call():
+    _lib.call('t5d_beam_topk_static', s, logits.data_ptr(), live.data_ptr(),
+              got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(),
+              got[3].data_ptr(), B, beams, V, k)
+    torch.cuda.synchronize()
+
   torch.cuda.synchronize()
-  # the running count of allocation requests: unlike the bytes in use it cannot
-  # move when the garbage collector frees tensors of earlier tests meanwhile
-  def requests():
-    return torch.cuda.memory_stats()['allocation.all.allocated']
-  before = requests()
-  _lib.call('t5d_beam_topk_static', s, logits.data_ptr(), live.data_ptr(),
-            got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(),
-            got[3].data_ptr(), B, beams, V, k)
-  torch.cuda.synchronize()
-  assert requests() == before
+  static_call()   # the first call on a device looks the array's address up
+  # What the driver reports as free device memory (the library calls HIP
+  # directly, so torch's allocator statistics would not see a hipMalloc of
+  # its own); nothing else runs between the two readings.
+  free_before, _ = torch.cuda.mem_get_info()
+  static_call()
+  free_after, _ = torch.cuda.mem_get_info()
+  assert free_after == free_before
   for g, w in zip(got, want):
     np.testing.assert_array_equal(g.cpu().numpy(), w.cpu().numpy())
   assert int(got[1].min()) >= 0
