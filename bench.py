@@ -198,9 +198,12 @@ class Workload:
 
   def steps_on_device(self):
     """Loop iterations the device has completed in the current decode."""
+    fused = getattr(self.loop, 'fused', None)
     if self.loop_kind == 'beam':
+      if fused is not None:
+        fused.synchronize()   # brings the lanes' counter into loop.cur
       return int(self.loop.cur.cur_index.item())
-    return int(self.loop.fused.step_count.item())
+    return int(fused.step_count.item())
 
   def check_full_decode(self):
     if self.loop.cond():
@@ -460,7 +463,7 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
     sbytes = float(np.mean([w.self_attention_bytes(t)
                             for t in range(1, w.L)]))
     out['self_attention'] = {
-        'kernel': 'self_attn_mfma_kernel', 'avg_launch_us': round(ssec * 1e6, 2),
+        'kernel': 'self_attn_tail_kernel', 'avg_launch_us': round(ssec * 1e6, 2),
         'launches': sn, 'mean_bytes_per_launch': int(sbytes),
         'achieved': round(sbytes / ssec / 1e9, 1),
         'frac': round(sbytes / ssec / 1e9 / HBM_PEAK_GBPS, 4)}

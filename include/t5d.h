@@ -195,7 +195,21 @@ int t5d_self_attention_step(void* stream, int dtype, const void* qkv,
  * (a decode loop) gets loads of consecutive memory for them — a head's cache
  * is then read as whole 4 KB blocks up to the current length instead of the
  * first part of each of 64 rows — and converts when it hands the cache tree
- * out.  0: both in the reference layout. */
+ * out.  0: both in the reference layout.
+ * value_blocked 3, the layout for a decode loop that owns its caches: a
+ * (row, head) slot has (L + 32) * 64 elements in both caches;
+ *   cached_key   [L + 32][64]: position-major (rows 0 .. L-1 in use), so the
+ *                key a step appends is one full 128-byte line;
+ *   cached_value [L/32 + 1][64][32]: finished blocks of 32 positions as with
+ *                value_blocked 1, and in the last block (the tail) the
+ *                positions of the block being filled, as [32][64]
+ *                position-major; the step whose position completes a block
+ *                writes the block and the tail starts over.
+ * A reference-layout step appends a position as 64 separate 2-byte stores per
+ * cache, each a partial cache line (measured: 2 of 14 us per launch at 128
+ * rows x 12 heads, 21 of 73 us at 128 x 64); here it is two full lines.
+ * Results have the same bits in every layout.  L a multiple of 32 and at
+ * most 256 (128 for a pending_src without pending_dst); T5D_ELIMIT beyond. */
 int t5d_self_attention_step_gather(void* stream, int dtype, const void* qkv,
                                    void* cached_key, void* cached_value,
                                    const void* rel_bias,
@@ -447,9 +461,8 @@ typedef struct {
    * optional destination slots (NULL: row e keeps slot e) */
   const int32_t* pending_src;
   const int32_t* pending_dst;
-  /* 1: the layers' cached_value are in the blocked layout of
-   * t5d_self_attention_step_gather (bfloat16, L a multiple of 32); 2: the
-   * cached_key too */
+  /* the layers' cache layout, as value_blocked of
+   * t5d_self_attention_step_gather (bfloat16; 0: the reference layout) */
   int value_blocked;
 } t5d_model_step;
 

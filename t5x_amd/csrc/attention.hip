@@ -500,8 +500,16 @@ extern "C" int t5d_self_attention_step_gather(
               "%d wavefronts per workgroup", beams, L, kMaxWaves);
   T5D_REQUIRE(pending_dst == nullptr || pending_src != nullptr, T5D_EINVAL,
               "t5d_self_attention_step_gather: pending_dst without pending_src");
-  T5D_REQUIRE(value_blocked >= 0 && value_blocked <= 2, T5D_EINVAL,
+  T5D_REQUIRE(value_blocked >= 0 && value_blocked <= 3, T5D_EINVAL,
               "t5d_self_attention_step_gather: value_blocked=%d", value_blocked);
+  const bool in_place = pending_src != nullptr && pending_dst == nullptr;
+  T5D_REQUIRE(value_blocked != 3 || L <= (in_place ? 128 : 256), T5D_ELIMIT,
+              "t5d_self_attention_step_gather: the tail layout covers L <= %d "
+              "%s (L=%d)", in_place ? 128 : 256,
+              in_place ? "for a gather without destination slots" : "", L);
+  T5D_REQUIRE(value_blocked != 3 || beams <= 8, T5D_ELIMIT,
+              "t5d_self_attention_step_gather: beams=%d (tail layout: 1..8)",
+              beams);
   T5D_REQUIRE(!value_blocked || L % 32 == 0, T5D_EINVAL,
               "t5d_self_attention_step_gather: blocked caches need L %% 32 == 0 "
               "(L=%d)", L);

@@ -49,6 +49,7 @@ struct AttnMfmaArgs {
   const int32_t* pending;  // [B, beams] source slot per row, or null
   const int32_t* pending_dst;  // [B, beams] slot per row (null: row e, slot e)
   int beams, nblk;         // rows per workgroup, wavefronts per row
+  int n_units;             // self_attn_rows_kernel: rows * heads
   // cross-attention with the query projection fused in (q == nullptr)
   const bf16_t* x;         // [R, d] residual stream
   const bf16_t* ln;        // [d] pre-attention layer-norm scale
@@ -739,6 +740,379 @@ self_attn_mfma_kernel(AttnMfmaArgs a) {
   store_column();
 }
 
+
+// ---- self-attention on caches laid out for the decode loop -----------------------
+// The column a step appends is 64 head dims of ONE position.  In the reference
+// layout (and in the blocked ones above) those are 64 separate 2-byte stores
+// into 64 different cache lines per (row, head) and cache: partial-line
+// writes, which the memory system turns into read-modify-write cycles —
+// measured at 2.1 us of a 13.8 us launch over 128 rows x 12 heads and 21 us
+// of 73 us over 128 x 64, against nothing measurable for one 128-byte line.
+// A loop that owns its caches therefore keeps them like this ("tail" layout,
+// value_blocked == 3), per (row, head) slot of (L + 32) * 64 elements:
+//   keys    [L + 32][64]: position-major, a new key is one full line.  The
+//           score arithmetic does not care: lane (dg, jc) still multiplies
+//           head dims 16 dg .. +16 with positions 8 jc .. +8 in the same
+//           order, it just finds a position's 16 dims in two 16-byte loads
+//           instead of a dim's 8 positions in one.
+//   values  [L / 32 + 1][64][32]: blocks of 32 positions as before (the layout
+//           the matrix cores take operands from), but a block is written
+//           once, whole, when its 32nd position arrives.  Until then its
+//           positions live in the slot's last block, the tail, as [32][64]
+//           position-major (a new value is one full line); a step reads the
+//           tail lane-linearly, turns it into the operand layout through LDS
+//           and, on the block's last position, stores the operand registers
+//           as the finished block (4 KB of consecutive memory).
+// One wavefront does all of a (row, head) pair and walks its NC chunks of 128
+// positions itself, so nothing is exchanged between wavefronts, and a
+// workgroup is just WM consecutive pairs without any barrier.  That holds for
+// rows that are never reordered (the sampling loops) and equally for a beam
+// search's rows when every row has a slot of its own to keep its cache in
+// (pending_dst): the slot rule — a new beam keeps the slot it read unless an
+// earlier one does, and then takes one that no new beam reads — means no
+// wavefront writes what another reads.  Pairs being independent, the launch
+// is cut into workgroups of 4, 2 or 1 so that the CUs get equal shares (128
+// rows x 12 heads as 768 workgroups of 2: 3 per CU, where workgroups of one
+// batch item's 4 beams put 2 on half of the CUs and 1 on the others).
+//   BARRIER: a gather WITHOUT destination slots permutes an item's rows in
+//     place; a workgroup is then the item's `beams` rows, with the one
+//     barrier of self_attn_mfma_kernel when the item's beams moved; NC == 1.
+// Operation for operation the arithmetic is that of self_attn_mfma_kernel
+// (per-chunk partial sums added by rising chunk), so the results have the
+// same bits whatever the layout.
+constexpr int kTailRow = 144;  // bytes per position of the tail tile in LDS
+constexpr int kCUs = 256;       // compute units of the device (MI355X)
+
+template <int NC, int WM, bool BARRIER>
+__global__ void __launch_bounds__(64 * WM, BARRIER ? 1 : 2)
+self_attn_tail_kernel(AttnMfmaArgs a) {
+  static_assert(!BARRIER || NC == 1, "a row permuted in place is one chunk");
+  __shared__ __attribute__((aligned(16))) bf16_t s_p[WM][NC * kBlockJ];
+  __shared__ __attribute__((aligned(16))) unsigned char s_tail[WM][32 * kTailRow];
+  __shared__ float s_pt[WM];
+  T5D_GATE_READ(a.gate);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int jc = lane & 15, dg = lane >> 4;  // score layout
+  const int n16 = lane & 15, g = lane >> 4;  // MFMA layout
+  const int HD = a.H * kHeadDim;
+  const int S = a.S;
+
+  int r, h;              // row of the step, head
+  if (BARRIER) {
+    h = blockIdx.x;
+    r = blockIdx.y * a.beams + wave;
+  } else {
+    const int unit = blockIdx.x * WM + wave;
+    r = unit / a.H;
+    h = unit - r * a.H;
+    if (r >= a.n_units / a.H) return;  // no barrier on this path
+  }
+  int rs = r, rw = r;    // slot the row reads; slot it keeps
+  bool permuted = false; // BARRIER: does this batch item need rows moved?
+  if (a.pending != nullptr) {
+    const int b0 = r / a.beams * a.beams;
+    auto in_range = [&](int v) { return v < 0 ? 0 : (v >= a.beams ? a.beams - 1 : v); };
+    rs = b0 + in_range(a.pending[r]);
+    if (a.pending_dst) rw = b0 + in_range(a.pending_dst[r]);
+    if (BARRIER)
+      for (int q = 0; q < a.beams; ++q)
+        permuted = permuted || a.pending[b0 + q] != q;
+  }
+  const int t_in = *a.index;
+  T5D_GATE_TEST();  // after the scalar loads above are in flight
+  const bool copy = rw != rs;  // what the row reads goes into its own slot
+
+  // (self_attn_mfma_kernel explains the index outside [0, S).)  By then every
+  // block is finished: nothing is in the tail.
+  const bool past_end = t_in < 0 || t_in >= S;
+  const int t = past_end ? S - 1 : t_in;
+  const int n = t + 1;
+  const int pb = past_end ? (S >> 5) : (t >> 5);  // the block still in the tail
+  const int tl = past_end ? 0 : (t & 31);         // positions the tail holds
+  const size_t slot = (size_t)kHeadDim * (S + 32) * 2;  // bytes
+  const size_t tail_at = (size_t)(S >> 5) * 4096;
+  const char* ksrc = reinterpret_cast<const char*>(a.k) + ((size_t)rs * a.H + h) * slot;
+  const char* vsrc = reinterpret_cast<const char*>(a.v) + ((size_t)rs * a.H + h) * slot;
+  char* kdst = reinterpret_cast<char*>(a.k) + ((size_t)rw * a.H + h) * slot;
+  char* vdst = reinterpret_cast<char*>(a.v) + ((size_t)rw * a.H + h) * slot;
+  const bf16_t* qrow = a.q + (size_t)r * a.q_stride + h * kHeadDim;
+
+  // Keys of every chunk in use: lane (dg, jc) takes head dims 16 dg .. +16 of
+  // positions 128 c + 8 jc .. +8, 32 bytes of each position's line.
+  uint4 kr[NC][8][2];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int j0 = c * kBlockJ + 8 * jc;
+    if (j0 < n) {
+      const char* p = ksrc + ((size_t)j0 * kHeadDim + 16 * dg) * 2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        kr[c][e][0] = *reinterpret_cast<const uint4*>(p + e * 128);
+        kr[c][e][1] = *reinterpret_cast<const uint4*>(p + e * 128 + 16);
+      }
+    }
+  }
+  // The step's own row: query (this lane's 16 head dims for the scores, its
+  // own element for the new column's score), new key / value elements.
+  float qv[16];
+  {
+    const uint4* qp = reinterpret_cast<const uint4*>(qrow + 16 * dg);
+    float f[8];
+    unpack16(qp[0], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[e] = f[e];
+    unpack16(qp[1], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[8 + e] = f[e];
+  }
+  const bf16_t q_d = qrow[lane];
+  const bf16_t knew_d = qrow[HD + lane];
+  const bf16_t vnew_d = qrow[2 * HD + lane];
+  // (the new value again, as this lane's 4 outputs per tile need it: with two
+  // chunks of keys in flight the registers are short, and it is asked for
+  // after the scores instead, behind the softmax)
+  uint2 vn[4];
+  auto load_vn = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+      vn[dt] = *reinterpret_cast<const uint2*>(qrow + 2 * HD + 16 * dt + 4 * g);
+  };
+  if (NC == 1) load_vn();
+  // Relative-position bias of this lane's 2 positions per chunk, by distance.
+  float bias[NC][2];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int jp = c * kBlockJ + 8 * jc + 4 * (dg >> 1) + 2 * (dg & 1);
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      bias[c][e] = jp + e < n
+                       ? bf16_to_f32(a.rel_bias[(size_t)h * S + (t - jp - e)])
+                       : 0.f;
+  }
+  // The tail: positions 32 pb .. t - 1, 128 bytes each, read lane-linearly
+  // (lane l of load k has 8 head dims of position 8 k + l / 8).
+  uint4 tr[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    tr[k] = make_uint4(0, 0, 0, 0);
+    if (8 * k + (lane >> 3) < tl)
+      tr[k] = *reinterpret_cast<const uint4*>(vsrc + tail_at + k * 1024 + lane * 16);
+  }
+  // Finished value blocks: whole 32-position groups (1 KB per tile).
+  Frag16 vb[NC][4][4];
+  auto load_values = [&](int c) {
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      if (c * 4 + jb < pb) {
+        const char* p = vsrc + ((size_t)((c * 4 + jb) * kHeadDim + n16) * 32 + 8 * g) * 2;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+          vb[c][jb][dt].u = *reinterpret_cast<const uint4*>(p + dt * 1024);
+      }
+    }
+  };
+  // One chunk: keys and values in flight together.  Two: the registers hold
+  // both chunks' keys or one chunk's keys and values, so a chunk's values are
+  // requested when its scores have freed the registers of its keys.
+  if (NC == 1) load_values(0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  const float snew = wave_sum(bf16_to_f32(q_d) * bf16_to_f32(knew_d));
+  float sc[NC][2];
+  float m = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    if (c * kBlockJ < n) {
+      float s8[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // position e of this lane: its 16 head dims in rising order
+        float kf[8], acc = 0.f;
+        unpack16(kr[c][e][0], kf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = fmaf(qv[i], kf[i], acc);
+        unpack16(kr[c][e][1], kf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = fmaf(qv[8 + i], kf[i], acc);
+        s8[e] = acc;
+      }
+      if (BARRIER && permuted) {
+        // Every wavefront of the item has its source data in registers
+        // before any slot is written.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+      }
+      if (copy && c * kBlockJ + 8 * jc < n) {
+        char* p = kdst + ((size_t)(c * kBlockJ + 8 * jc) * kHeadDim + 16 * dg) * 2;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          *reinterpret_cast<uint4*>(p + e * 128) = kr[c][e][0];
+          *reinterpret_cast<uint4*>(p + e * 128 + 16) = kr[c][e][1];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (NC > 1) load_values(c);  // into the registers the keys have left
+      __builtin_amdgcn_sched_barrier(0);
+      reduce_scatter_8(s8, sc[c]);
+      const int jp = c * kBlockJ + 8 * jc + 4 * (dg >> 1) + 2 * (dg & 1);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int j = jp + e;
+        float x = (j == t && !past_end) ? snew : sc[c][e];
+        x = round_bf16(x);
+        if (j < n) x = round_bf16(x + bias[c][e]);
+        else x = -INFINITY;
+        sc[c][e] = x;
+        m = fmaxf(m, x);
+      }
+    } else {
+      sc[c][0] = sc[c][1] = -INFINITY;
+    }
+  }
+  if (NC > 1) load_vn();
+  // The tail into LDS, one position per row, the new value as position tl (it
+  // takes part in the matrix product with probability 0, see below, and
+  // completes the block when tl == 31); positions beyond are zero.
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    *reinterpret_cast<uint4*>(&s_tail[wave][(8 * k + (lane >> 3)) * kTailRow +
+                                            (lane & 7) * 16]) = tr[k];
+  if (copy) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (8 * k + (lane >> 3) < tl)
+        *reinterpret_cast<uint4*>(vdst + tail_at + k * 1024 + lane * 16) = tr[k];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (!past_end)
+    *reinterpret_cast<bf16_t*>(&s_tail[wave][tl * kTailRow + lane * 2]) = vnew_d;
+
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    float part = 0.f;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      sc[c][e] = __expf(sc[c][e] - m);  // exp(-inf) == 0
+      part += sc[c][e];
+    }
+    part = wave_sum(part);
+    sum = c == 0 ? part : sum + part;
+  }
+  {
+    // Normalised probabilities, rounded to bf16 where the reference rounds.
+    // Position t is kept out of the matrix product: its probability goes to
+    // s_pt and its output share is added from the new value below.
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int jp = c * kBlockJ + 8 * jc + 4 * (dg >> 1) + 2 * (dg & 1);
+      float p0 = round_bf16(sc[c][0] * inv), p1 = round_bf16(sc[c][1] * inv);
+      if (jp == t && !past_end) { s_pt[wave] = p0; p0 = 0.f; }
+      if (jp + 1 == t && !past_end) { s_pt[wave] = p1; p1 = 0.f; }
+      *reinterpret_cast<uint32_t*>(&s_p[wave][jp]) = pack_bf16x2(p0, p1);
+    }
+  }
+  // The wavefront's own LDS writes above are read back below in another lane
+  // order; no other wavefront is involved, so ordering within the wavefront
+  // is all that is needed.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // The tail block as matrix operand: lane (n16, g) of tile dt holds head dim
+  // 16 dt + n16 of positions 8 g .. +8.
+  Frag16 vt[4];
+  const bool tail_used = !past_end && tl > 0;
+  if (tail_used) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        vt[dt].h[e] = *reinterpret_cast<const bf16_t*>(
+            &s_tail[wave][(8 * g + e) * kTailRow + (16 * dt + n16) * 2]);
+  }
+
+  f32x4_v acc[4];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    f32x4_v oc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      const int gb = c * 4 + jb;
+      if (gb < pb || (gb == pb && tail_used)) {
+        Frag16 pb16;
+        pb16.u = *reinterpret_cast<const uint4*>(
+            &s_p[wave][c * kBlockJ + 32 * jb + 8 * g]);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          Frag16 v;
+          v.u = gb < pb ? vb[c][jb][dt].u : vt[dt].u;
+          oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.v, pb16.v, oc[dt],
+                                                           0, 0, 0);
+        }
+      }
+    }
+    if (copy) {
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        if (c * 4 + jb < pb) {
+          char* p = vdst + ((size_t)((c * 4 + jb) * kHeadDim + n16) * 32 + 8 * g) * 2;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+            *reinterpret_cast<uint4*>(p + dt * 1024) = vb[c][jb][dt].u;
+        }
+      }
+    }
+    if (!past_end && t >= c * kBlockJ && t < (c + 1) * kBlockJ) {
+      const float p_t = s_pt[wave];
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        oc[dt][0] = fmaf(p_t, bf16lo_to_f32(vn[dt].x), oc[dt][0]);
+        oc[dt][1] = fmaf(p_t, bf16hi_to_f32(vn[dt].x), oc[dt][1]);
+        oc[dt][2] = fmaf(p_t, bf16lo_to_f32(vn[dt].y), oc[dt][2]);
+        oc[dt][3] = fmaf(p_t, bf16hi_to_f32(vn[dt].y), oc[dt][3]);
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      if (c == 0) acc[dt] = oc[dt];
+      else acc[dt] += oc[dt];
+    }
+  }
+  if (n16 == 0) {
+    bf16_t* o = a.out + (size_t)r * HD + h * kHeadDim + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      uint2 pk;
+      pk.x = pack_bf16x2(acc[dt][0], acc[dt][1]);
+      pk.y = pack_bf16x2(acc[dt][2], acc[dt][3]);
+      *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
+    }
+  }
+  // The step's column: the key as one line of its cache; the value as one
+  // line of the tail, or, when it is its block's last, the finished block.
+  // The key line must land after the copy of the old line above.
+  if (!past_end) {
+    if (copy) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    *reinterpret_cast<bf16_t*>(kdst + ((size_t)t * kHeadDim + lane) * 2) = knew_d;
+    if (tl == 31) {
+      char* p = vdst + ((size_t)(pb * kHeadDim + n16) * 32 + 8 * g) * 2;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+        *reinterpret_cast<uint4*>(p + dt * 1024) = vt[dt].u;
+    } else {
+      *reinterpret_cast<bf16_t*>(vdst + tail_at + tl * 128 + lane * 2) = vnew_d;
+    }
+  }
+}
+
 // ---- dispatch -------------------------------------------------------------------
 template <int NQP>
 static void launch_cross(const AttnMfmaArgs& a, int B, hipStream_t s) {
@@ -800,6 +1174,46 @@ int launch_self_attention_bf16(hipStream_t s, const void* qkv, void* ck,
   a.x = nullptr; a.ln = nullptr; a.wq = nullptr; a.d = 0; a.eps = 0.f;
   a.units = nullptr;
   a.nblk = (L + kBlockJ - 1) / kBlockJ;
+  a.n_units = R * H;
+  if (value_blocked == 3) {
+    // caches in the decode loop's own layout (checked by the caller: one
+    // chunk for a gather in place, two at most otherwise)
+    a.v_blocked = a.k_blocked = 1;
+    a.pending = pending;
+    a.pending_dst = pending ? pending_dst : nullptr;
+    a.beams = pending ? beams : 1;
+    if (pending != nullptr && pending_dst == nullptr) {
+      dim3 grid(H, R / beams), block(64 * beams);
+      if (beams <= 4)
+        hipLaunchKernelGGL((self_attn_tail_kernel<1, 4, true>), grid, block, 0, s, a);
+      else
+        hipLaunchKernelGGL((self_attn_tail_kernel<1, 8, true>), grid, block, 0, s, a);
+      return 0;
+    }
+    // independent (row, head) pairs: workgroups of 4, 2 or 1 of them,
+    // whichever leaves the most loaded CU the fewest wavefronts
+    int wm = 4, worst = 1 << 30;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+      const int groups = (a.n_units + cand - 1) / cand;
+      const int load = (groups + kCUs - 1) / kCUs * cand;
+      if (load < worst) { worst = load; wm = cand; }
+    }
+    dim3 grid((a.n_units + wm - 1) / wm), block(64 * wm);
+#define T5D_LAUNCH_TAIL(NC_, WM_)                                              \
+  hipLaunchKernelGGL((self_attn_tail_kernel<NC_, WM_, false>), grid, block, 0, \
+                     s, a)
+    if (a.nblk == 1) {
+      if (wm == 4) T5D_LAUNCH_TAIL(1, 4);
+      else if (wm == 2) T5D_LAUNCH_TAIL(1, 2);
+      else T5D_LAUNCH_TAIL(1, 1);
+    } else {
+      if (wm == 4) T5D_LAUNCH_TAIL(2, 4);
+      else if (wm == 2) T5D_LAUNCH_TAIL(2, 2);
+      else T5D_LAUNCH_TAIL(2, 1);
+    }
+#undef T5D_LAUNCH_TAIL
+    return 0;
+  }
   a.pending = pending;
   a.pending_dst = pending ? pending_dst : nullptr;
   a.beams = pending ? beams : 1;

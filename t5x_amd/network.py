@@ -278,6 +278,36 @@ def _measure_side_by_side(streams):
   return first if first == second else None
 
 
+def decode_cache_layout(act_dtype, beams, length):
+  """The layout a decode loop keeps the self-attention caches it owns in, as
+  t5d_self_attention_step_gather names them, and the cache length to use.
+  bfloat16 caches are kept for the loop's access pattern — 3: keys by
+  position, values in finished blocks of 32 positions plus a position-major
+  tail, so that the column a step appends is two full cache lines instead of
+  128 two-byte stores into 128 lines (the kernels cover 256 positions);
+  2: keys and values in blocks of 32 positions, for longer caches — and
+  converted back by cache_tree().
+  float32 caches stay in the reference layout (0)."""
+  if act_dtype != torch.bfloat16:
+    return 0, (length + 3) // 4 * 4
+  L = (length + 31) // 32 * 32
+  if beams <= 8 and L <= 256:
+    return 3, L
+  return 2, L
+
+
+def _plain_caches(kv, layout, n):
+  """[2, R, H, 64, L(+32)] keys and values of one layer in `layout`, holding n
+  positions -> the pair in the reference layout [R, H, 64, L]."""
+  from t5x_amd import ops
+  if layout == 3:
+    return (ops.untail_cached_key(kv[0].reshape(*kv.shape[1:3], -1, 64)),
+            ops.untail_cached_value(kv[1], n))
+  if layout == 2:
+    return ops.unblock_cached_value(kv[0]), ops.unblock_cached_value(kv[1])
+  return kv[0], kv[1]
+
+
 class Transformer:
   """network.Transformer with `apply(variables, *args, method=..., **kwargs)`.
 
@@ -478,7 +508,7 @@ class Transformer:
 
   # -- the decode step -------------------------------------------------------------
   def _model_step(self, w, cross, bufs, layer_caches, cache_index, R, beams,
-                  L, gate=None, pending_src=None, value_blocked=False,
+                  L, gate=None, pending_src=None, cache_layout=0,
                   pending_dst=None):
     """Fills a t5d_model_step for one call of t5d_decoder_step."""
     from t5x_amd import _lib
@@ -512,8 +542,9 @@ class Transformer:
       setattr(m, name, P(getattr(bufs, name)))
     m.gate = P(gate)
     m.pending_src, m.pending_dst = P(pending_src), P(pending_dst)
-    # the loops that block their value caches block their key caches too
-    m.value_blocked = 2 if value_blocked else 0
+    # 0: the reference layout; 2: keys and values in blocks of 32 positions;
+    # 3: the decode loops' own layout (decode_cache_layout)
+    m.value_blocked = int(cache_layout)
     m._keepalive = (layers, w, cross, bufs, layer_caches, cache_index, gate,
                     pending_src, pending_dst)
     return m
@@ -852,14 +883,13 @@ class FusedSampleStep(_OwnedContext):
     self.temperature = temperature
     R, S = sequences.shape
     act = w.act_dtype
-    # bfloat16: the key and value caches are kept in blocks of 32 positions
-    # (loads of consecutive memory); cache_tree() converts back.
-    self.value_blocked = act == torch.bfloat16
-    el = 32 if self.value_blocked else 16 // torch.empty(
-        (), dtype=act).element_size()
-    self.L = L = (S - 2 + el - 1) // el * el
+    # bfloat16: the caches are kept in a layout of the loop's own
+    # (decode_cache_layout); cache_tree() converts back.
+    self.cache_layout, self.L = decode_cache_layout(act, 1, S - 2)
+    L = self.L
     nl = cfg.num_decoder_layers
-    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
+    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim,
+                           L + (32 if self.cache_layout == 3 else 0)),
                           dtype=act, device=dev)
     self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
     self.bufs = _StepBuffers(cfg, R, dev, act)
@@ -881,7 +911,7 @@ class FusedSampleStep(_OwnedContext):
     self.model = module._model_step(w, cross, self.bufs, layer_caches,
                                     self.cache_index, R, beams, L,
                                     gate=self.keep_going,
-                                    value_blocked=self.value_blocked)
+                                    cache_layout=self.cache_layout)
     P = _lib.ptr
     st = _lib.SampleStep()
     st.sequences, st.cur_index, st.cur_token = (P(sequences), P(cur_index),
@@ -1039,9 +1069,11 @@ class FusedSampleStep(_OwnedContext):
     self.stream.synchronize()
     from t5x_amd import ops
     nl = self.kv.shape[0]
-    plain = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return cache_tree(torch.stack([plain(self.kv[i, 0]) for i in range(nl)]),
-                      torch.stack([plain(self.kv[i, 1]) for i in range(nl)]),
+    held = self.cache_index.tolist()
+    plain = [_plain_caches(self.kv[i], self.cache_layout, held[i])
+             for i in range(nl)]
+    return cache_tree(torch.stack([k for k, _ in plain]),
+                      torch.stack([v for _, v in plain]),
                       self.cache_index, self.module.scan_layers)
 
   def __del__(self):
@@ -1065,7 +1097,8 @@ class _BeamLane:
     R, S, L = B * K, loop.max_decode_len, owner.L
     act = w.act_dtype
     nl = cfg.num_decoder_layers
-    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim, L),
+    self.kv = torch.zeros((nl, 2, R, cfg.num_heads, cfg.head_dim,
+                           L + (32 if owner.cache_layout == 3 else 0)),
                           dtype=act, device=dev)
     self.cache_index = torch.zeros((nl,), dtype=torch.int32, device=dev)
     self.bufs = _StepBuffers(cfg, R, dev, act)
@@ -1094,7 +1127,7 @@ class _BeamLane:
         gate=self.keep_going,
         pending_src=self.cache_src if owner.deferred_gather else None,
         pending_dst=self.cache_dst if owner.deferred_gather else None,
-        value_blocked=owner.value_blocked)
+        cache_layout=owner.cache_layout)
     st = loop.cur
     P = _lib.ptr
     ptrs = _lib.BeamStatePtrs()
@@ -1173,17 +1206,17 @@ class FusedBeamStep(_OwnedContext):
     # copied), so the reorder in flight is a pair of slot maps, cache_slots.
     self.deferred_gather = (K > 1 and act == torch.bfloat16 and
                             K * ((L + 127) // 128) <= 16)
-    # The key and value caches are then kept in blocks of 32 positions (loads
-    # of consecutive memory); cache_tree() converts back.  (The stand-alone
+    # The caches are then kept in a layout of the loop's own
+    # (decode_cache_layout); cache_tree() converts back.  (The stand-alone
     # reorder kernel of the other path copies row prefixes, which only the
     # reference layout has.)
-    self.value_blocked = self.deferred_gather or (K == 1 and
-                                                  act == torch.bfloat16)
-    if self.value_blocked:
-      L = (L + 31) // 32 * 32
-      if K * ((L + 127) // 128) > 16:
-        self.value_blocked = self.deferred_gather = False
-        L = (S - 1 + el - 1) // el * el
+    self.cache_layout = 0
+    if self.deferred_gather or (K == 1 and act == torch.bfloat16):
+      layout, L32 = decode_cache_layout(act, K, S - 1)
+      if K * ((L32 + 127) // 128) <= 16:
+        self.cache_layout, L = layout, L32
+      else:
+        self.deferred_gather = False
     self.L = L
     loop.top_alive.copy_(torch.arange(K, dtype=torch.int32,
                                       device=dev).expand(B, K))
@@ -1414,9 +1447,11 @@ class FusedBeamStep(_OwnedContext):
     nl = self.lanes[0].kv.shape[0]
     kv = torch.cat([lane.kv for lane in self.lanes], dim=2)
     idx = self.lanes[0].cache_index
-    plain = (ops.unblock_cached_value if self.value_blocked else (lambda v: v))
-    return cache_tree(torch.stack([plain(kv[i, 0]) for i in range(nl)]),
-                      torch.stack([plain(kv[i, 1]) for i in range(nl)]), idx,
+    held = idx.tolist()
+    plain = [_plain_caches(kv[i], self.cache_layout, held[i])
+             for i in range(nl)]
+    return cache_tree(torch.stack([k for k, _ in plain]),
+                      torch.stack([v for _, v in plain]), idx,
                       self.module.scan_layers)
 
   def __del__(self):

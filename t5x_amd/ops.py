@@ -226,26 +226,90 @@ def unblock_cached_value(v):
       R, H, 64, L)
 
 
+def tail_cached_key(k):
+  """[R, H, 64, L] key cache -> the decode loops' [R, H, L + 32, 64]
+  (position-major; the last 32 rows are unused)."""
+  R, H, D, L = k.shape
+  out = k.new_zeros((R, H, L + 32, D))
+  out[:, :, :L] = k.transpose(2, 3)
+  return out
+
+
+def untail_cached_key(k):
+  """Inverse of tail_cached_key -> [R, H, 64, L]."""
+  return k[:, :, :-32].transpose(2, 3).contiguous()
+
+
+def tail_cached_value(v, n):
+  """[R, H, 64, L] value cache holding n positions -> the decode loops'
+  [R, H, L/32 + 1, 64, 32]: the finished blocks of 32 positions, and in the
+  last block the n % 32 positions of the block being filled as [32, 64]
+  position-major."""
+  R, H, D, L = v.shape
+  n = int(n)
+  out = v.new_zeros((R, H, L // 32 + 1, D, 32))
+  full = n // 32
+  out[:, :, :full] = block_cached_value(v)[:, :, :full]
+  rest = n - 32 * full
+  if rest:
+    tail = out[:, :, -1].reshape(R, H, 32, D)  # a view: same memory
+    tail[:, :, :rest] = v[:, :, :, 32 * full:n].transpose(2, 3)
+  return out
+
+
+def untail_cached_value(v, n):
+  """Inverse of tail_cached_value for a cache holding n positions ->
+  [R, H, 64, L]; positions n and beyond read zero."""
+  R, H = v.shape[:2]
+  v = v.reshape(R, H, -1, 64, 32)
+  L = (v.shape[2] - 1) * 32
+  n = int(n)
+  full = min(n // 32, L // 32)
+  out = v.new_zeros((R, H, 64, L))
+  if full:
+    out[:, :, :, :32 * full] = unblock_cached_value(
+        v[:, :, :full].contiguous())
+  rest = n - 32 * full
+  if rest > 0 and full < L // 32:
+    tail = v[:, :, -1].reshape(R, H, 32, 64)
+    out[:, :, :, 32 * full:n] = tail[:, :, :rest].transpose(2, 3)
+  return out
+
+
 def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
                         out=None, pending_src=None, value_blocked=False,
-                        pending_dst=None, key_blocked=False):
+                        pending_dst=None, key_blocked=False, tail=False):
   """One cached self-attention step; with pending_src [B, beams] the rows'
   caches are first gathered from their source beams inside the kernel, into
   slot e of row (b, e) or, with pending_dst [B, beams], into slot
   pending_dst[b, e].  value_blocked: cached_value holds the blocked layout
   (see block_cached_value) in a tensor of the usual [R, H, 64, L] shape;
-  key_blocked (with value_blocked): cached_key as well."""
+  key_blocked (with value_blocked): cached_key as well.  tail: both caches in
+  the decode loops' layout (tail_cached_key / tail_cached_value), as tensors
+  of [R, H, 64, L + 32] elements."""
   if key_blocked and not value_blocked:
     raise ValueError('key_blocked goes with value_blocked')
+  if tail and (value_blocked or key_blocked):
+    raise ValueError('tail is a layout of its own')
   _chk(qkv, 'qkv', ndim=2)
-  _chk(cached_key, 'cached_key', qkv.dtype, 4)
-  _chk(cached_value, 'cached_value', qkv.dtype, 4)
   _chk(rel_bias, 'rel_bias', qkv.dtype, 2)
   _chk(cache_index, 'cache_index', torch.int32)
-  R, H, D, L = cached_key.shape
+  if tail:
+    _chk(cached_key, 'cached_key', qkv.dtype)
+    _chk(cached_value, 'cached_value', qkv.dtype)
+    R, H = cached_key.shape[:2]
+    D = 64
+    L = cached_key.numel() // (R * H * D) - 32
+    if cached_value.numel() != cached_key.numel() or L <= 0 or L % 32:
+      raise ValueError('tail layout: both caches hold [R, H, (L + 32) * 64] '
+                       'elements, L a multiple of 32')
+  else:
+    _chk(cached_key, 'cached_key', qkv.dtype, 4)
+    _chk(cached_value, 'cached_value', qkv.dtype, 4)
+    R, H, D, L = cached_key.shape
   if D != 64:
     raise ValueError('head_dim must be 64')
-  if cached_value.shape != cached_key.shape:
+  if not tail and cached_value.shape != cached_key.shape:
     raise ValueError('cached_key / cached_value shapes differ')
   if tuple(qkv.shape) != (R, 3 * H * D):
     raise ValueError(f'qkv shape {tuple(qkv.shape)} != {(R, 3 * H * D)}')
@@ -256,7 +320,7 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
   if out is None:
     out = torch.empty((R, H * D), dtype=qkv.dtype, device=qkv.device)
   _chk(out, 'out', qkv.dtype, 2)
-  if pending_src is not None or value_blocked:
+  if pending_src is not None or value_blocked or tail:
     B, beams = R, 1
     if pending_src is not None:
       _chk(pending_src, 'pending_src', torch.int32, 2)
@@ -272,7 +336,7 @@ def self_attention_step(qkv, cached_key, cached_value, rel_bias, cache_index,
               cached_key.data_ptr(), cached_value.data_ptr(),
               rel_bias.data_ptr(), cache_index.data_ptr(), out.data_ptr(), B,
               beams, H, L, _lib.ptr(pending_src), _lib.ptr(pending_dst),
-              2 if key_blocked else int(bool(value_blocked)))
+              3 if tail else 2 if key_blocked else int(bool(value_blocked)))
     return out
   _lib.call('t5d_self_attention_step', _s(), _lib.dtype_code(qkv.dtype),
             qkv.data_ptr(), cached_key.data_ptr(), cached_value.data_ptr(),

@@ -670,6 +670,115 @@ def test_self_attention_step_with_destination_slots(ops, B, beams, H, L, t,
                        ck[(rows + src.long()).reshape(-1)][keep][..., t + 1:])
 
 
+_TAIL_CASES = [
+    (3, 4, 2, 128, 0, 40),      # from an empty cache across the first block
+    (2, 4, 3, 128, 58, 70),     # two block ends, up to the cache end
+    (2, 8, 2, 64, 20, 44),      # 8 beams (the wider workgroup)
+    (5, 1, 3, 256, 118, 20),    # rows never reordered: into the second chunk
+    (3, 1, 2, 256, 250, 6),     # ... up to the cache end
+    (9, 1, 2, 96, 0, 96),       # ... one chunk, every position
+    (32, 4, 12, 128, 60, 6),    # the benchmark shape
+    (2, 4, 2, 256, 120, 12),    # beams over two chunks
+    (3, 4, 2, 128, 27, 8, True),   # gathered in place (no destination slots)
+    (2, 8, 1, 96, 60, 6, True),
+]
+
+
+@pytest.mark.parametrize('B,beams,H,L,t0,steps,in_place', [
+    c if len(c) == 7 else c + (False,) for c in _TAIL_CASES])
+def test_self_attention_steps_in_the_decode_loop_layout(ops, B, beams, H, L, t0,
+                                                         steps, in_place):
+  """Consecutive steps on caches in the decode loops' own layout (keys by
+  position, values in finished blocks plus a position-major tail, a block
+  written when its last position arrives) with the beams re-ranked, dropped
+  and duplicated at every step: outputs equal gather-then-step on
+  reference-layout caches bit for bit at every step, and so do the caches
+  converted back.  beams == 1: rows that are never reordered.  in_place: the
+  gather without destination slots (beam e keeps slot e)."""
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(B * 7 + beams * 131 + L + t0)
+  rs = np.random.RandomState(B + beams + L + t0)
+  R, D, dt = B * beams, 64, torch.bfloat16
+  # reference-layout caches holding t0 positions (zeros beyond, as a decode
+  # leaves them)
+  ck = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  cv = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  ck[..., t0:] = 0
+  cv[..., t0:] = 0
+  rel_bias = torch.randn((H, L), generator=gen, device='cuda').to(dt)
+  rows = torch.arange(B, device='cuda')[:, None] * beams
+  # tail-layout caches with the beams scattered over the slots
+  slot_of = np.stack([np.arange(beams) if in_place else rs.permutation(beams)
+                      for _ in range(B)])
+  so = torch.as_tensor(slot_of, device='cuda').long()
+  phys_k, phys_v = torch.empty_like(ck), torch.empty_like(cv)
+  phys_k[(rows + so).reshape(-1)] = ck
+  phys_v[(rows + so).reshape(-1)] = cv
+  tk = ops.tail_cached_key(phys_k)
+  tv = ops.tail_cached_value(phys_v, t0)
+  assert torch.equal(ops.untail_cached_key(tk), phys_k)
+  assert torch.equal(ops.untail_cached_value(tv, t0), phys_v)
+  for t in range(t0, t0 + steps):
+    qkv = torch.randn((R, 3 * H * D), generator=gen, device='cuda').to(dt)
+    idx = torch.tensor(t, dtype=torch.int32, device='cuda')
+    if beams > 1:
+      parents = rs.randint(0, beams, size=(B, beams))
+      parents[0] = np.arange(beams)         # nothing moves
+      if B > 1:
+        parents[1] = rs.permutation(beams)  # a re-ranking: nothing is copied
+      if in_place:
+        maps = [(list(parents[b]), list(range(beams))) for b in range(B)]
+      else:
+        maps = [inherit_slots(slot_of[b], parents[b]) for b in range(B)]
+      src = torch.tensor([m[0] for m in maps], dtype=torch.int32, device='cuda')
+      dst = (None if in_place else
+             torch.tensor([m[1] for m in maps], dtype=torch.int32,
+                          device='cuda'))
+      pa = torch.as_tensor(parents, device='cuda').long()
+      ck = ck[(rows + pa).reshape(-1)].clone()
+      cv = cv[(rows + pa).reshape(-1)].clone()
+      slot_of = np.array([m[1] for m in maps])
+    else:
+      src = dst = None
+    want = ops.self_attention_step(qkv, ck, cv, rel_bias, idx)
+    got = ops.self_attention_step(qkv, tk, tv, rel_bias, idx, pending_src=src,
+                                  pending_dst=dst, tail=True)
+    assert torch.equal(got, want), t
+    n = min(t + 1, L)
+    at = (rows + torch.as_tensor(slot_of, device='cuda').long()).reshape(-1)
+    if t % 7 == 0 or t == t0 + steps - 1 or t % 32 in (30, 31, 0):
+      assert torch.equal(ops.untail_cached_key(tk)[at][..., :n], ck[..., :n]), t
+      assert torch.equal(ops.untail_cached_value(tv, n)[at][..., :n],
+                         cv[..., :n]), t
+
+
+def test_self_attention_step_past_the_cache_end_in_the_decode_loop_layout(ops):
+  """A cache index at or beyond L: nothing is inserted and all L columns are
+  attended, as the reference-layout kernel does."""
+  gen = torch.Generator(device='cuda')
+  gen.manual_seed(5)
+  R, H, D, L, dt = 6, 2, 64, 64, torch.bfloat16
+  ck = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  cv = torch.randn((R, H, D, L), generator=gen, device='cuda').to(dt)
+  rel_bias = torch.randn((H, L), generator=gen, device='cuda').to(dt)
+  qkv = torch.randn((R, 3 * H * D), generator=gen, device='cuda').to(dt)
+  tk, tv = ops.tail_cached_key(ck), ops.tail_cached_value(cv, L)
+  for t in (L, L + 3, -1):
+    idx = torch.tensor(t, dtype=torch.int32, device='cuda')
+    ck_a, cv_a = ck.clone(), cv.clone()
+    want = ops.self_attention_step(qkv, ck_a, cv_a, rel_bias, idx)
+    got = ops.self_attention_step(qkv, tk, tv, rel_bias, idx, tail=True)
+    assert torch.equal(got, want), t
+    assert torch.equal(ops.untail_cached_key(tk), ck_a)
+    assert torch.equal(ops.untail_cached_value(tv, L), cv_a)
+  with pytest.raises(Exception, match='tail layout covers'):
+    big = torch.zeros((1, 1, 64, 512 + 32), dtype=dt, device='cuda')
+    ops.self_attention_step(
+        torch.zeros((1, 192), dtype=dt, device='cuda'), big, big.clone(),
+        torch.zeros((1, 512), dtype=dt, device='cuda'),
+        torch.tensor(0, dtype=torch.int32, device='cuda'), tail=True)
+
+
 @pytest.mark.parametrize('dt', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('B,beams,H,E', [(2, 1, 3, 64), (3, 4, 2, 512),
                                          (2, 2, 2, 128), (1, 8, 2, 264),
