@@ -171,6 +171,49 @@ def test_encoder_forward_matches_oracle(B, E):
   assert err.max() < 0.25, err.max()
 
 
+def test_encoder_forward_at_base_width_matches_oracle():
+  """The whole T5.1.1-base encoder (12 layers, d = 768, 12 heads, gated MLP of
+  2048) over B = 4 rows of E = 512 tokens with ragged lengths, as
+  bench.py --stage encoder runs it (t5x/examples/t5/network.py:47-96,315-343).
+  Twelve bfloat16 layers amplify single-ulp differences, so the yardstick is
+  the oracle with float32 activations on the same bfloat16-valued parameters:
+  the HIP encoder may be no further from it than the bfloat16 oracle is
+  (factor 1.25 on mean, 99.9th percentile and maximum over the valid rows)."""
+  from t5x_amd import network
+  B, E = 4, 512
+  kw = dict(network.T5_1_1['base'], num_decoder_layers=1)
+  ocfg = ot5.T5Config(dtype='bfloat16', **kw)
+  tcfg = ot5.T5Config(dtype='float32', **kw)
+  gcfg = network.T5Config(dtype='bfloat16', **kw)
+
+  def rounded(node):
+    if isinstance(node, dict):
+      return {k: rounded(v) for k, v in node.items()}
+    return ot5.bf16_round(node)
+
+  params = rounded(ot5.init_params(ocfg, seed=2))
+  rs = np.random.RandomState(12)
+  tok = rs.randint(2, ocfg.vocab_size, size=(B, E)).astype(np.int32)
+  lens = np.array([E, 128, 301, 437])
+  tok[np.arange(E)[None, :] >= lens[:, None]] = 0
+  want = ot5.encode(params, ocfg, tok)
+  truth = ot5.encode(params, tcfg, tok)
+  module = network.Transformer(gcfg, torch.device('cuda'))
+  got = host(module.apply({'params': params}, tok, enable_dropout=False,
+                          method=module.encode))
+  assert got.shape == want.shape == (B, E, 768)
+  valid = np.arange(E)[None, :] < lens[:, None]
+  stats = lambda e: (e.mean(), np.quantile(e, 0.999), e.max())
+  h = stats(np.abs(got - truth)[valid])
+  o = stats(np.abs(want - truth)[valid])
+  print(f'base encoder: |hip - truth| mean {h[0]:.3g} p99.9 {h[1]:.3g} max '
+        f'{h[2]:.3g}; |oracle - truth| mean {o[0]:.3g} p99.9 {o[1]:.3g} max '
+        f'{o[2]:.3g}', flush=True)
+  for name, x, y in zip(('mean', 'p99.9', 'max'), h, o):
+    assert x <= 1.25 * y, (name, x, y)
+  assert np.abs(got - want)[valid].mean() < 2e-2
+
+
 @pytest.mark.parametrize('B,E', [(2, 18), (3, 41)])
 def test_encoder_forward_at_lengths_off_the_tile_matches_oracle(B, E):
   """bf16 encoder at lengths that are not a multiple of 4 (the rows are padded

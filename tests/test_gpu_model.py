@@ -855,10 +855,10 @@ def test_full_size_xl_int8_beam4_fused_loop_equals_generic_loop():
 
 def test_full_size_large_sampling_fused_loop_equals_generic_loop():
   """T5.1.1-large, batch 64, temperature 0.7, top-k 40, encoder 512, with the
-  Gumbel noise supplied to both loops; 64 of the 256 positions (the full decode
-  only repeats the same step)."""
+  Gumbel noise supplied to both loops; 160 of the 256 positions (past the
+  128th, where a row's cache takes a second chunk of positions)."""
   from t5x_amd import decoding
-  B, E, L, steps = 64, 512, 256, 64
+  B, E, L, steps = 64, 512, 256, 160
   module, fn = _full_size_setup('large', B, 1, E, 512, L,
                                 decoding.temperature_sample)
   gen = torch.Generator(device='cuda')
@@ -876,6 +876,32 @@ def test_full_size_large_sampling_fused_loop_equals_generic_loop():
   assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp))
   seqs = host(got)[:, 0]
   assert (seqs[:, steps:] == 0).all() and (seqs[:, :steps] != 0).mean() > 0.9
+
+
+def test_full_size_xxl_greedy_fused_loop_equals_generic_loop():
+  """T5.1.1-XXL as a whole (24 decoder layers, d = 4096, 64 heads, batch 128,
+  encoder 1024, 256 positions, greedy): the graph-replay loop (caches in the
+  loop's own layout, large-tile dense kernels on every layer's buffers) against
+  the kernel-per-call loop on reference-layout caches, bit for bit, over the
+  first 20 positions; greedy rows never end early with these weights, so every
+  row must hold 20 tokens."""
+  from t5x_amd import decoding
+  B, E, L, steps = 128, 1024, 256, 20
+  print('XXL greedy: fused loop vs kernel-per-call loop, 24 layers', flush=True)
+  module, fn = _full_size_setup('xxl', B, 1, E, 1024, L,
+                                decoding.temperature_sample)
+  inputs = np.zeros((B, L), np.int32)
+  kw = dict(temperature=0.0, max_decode_steps=steps)
+  want, wlp = decoding.temperature_sample(
+      inputs, dict(module.init_cache(B, L)), fn, 1, **kw)
+  got, glp = decoding.temperature_sample(
+      inputs, module.init_cache(B, L), fn, 1, **kw)
+  assert torch.equal(torch.as_tensor(got), torch.as_tensor(want))
+  assert torch.equal(torch.as_tensor(glp), torch.as_tensor(wlp))
+  seqs = host(got)[:, 0]
+  assert (seqs[:, steps:] == 0).all() and (seqs[:, :steps] != 0).mean() > 0.9
+  del module, fn
+  torch.cuda.empty_cache()
 
 
 def test_infer_fn_over_predict_batch_with_aux_matches_oracle():
