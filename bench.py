@@ -74,6 +74,11 @@ def parse_args():
   ap.add_argument('--roofline-only', action='store_true',
                   help='only the dominant-kernel replay plus a plain copy of '
                        'known size (for counter runs under rocprofv3 --pmc)')
+  ap.add_argument('--counter-copy', action='store_true',
+                  help='end the run with a plain device copy of 256 MiB, 5 '
+                       'times (for runs under rocprofv3 --pmc: what FETCH_SIZE '
+                       '/ WRITE_SIZE read for a copy of known size scales the '
+                       "kernels' readings)")
   ap.add_argument('--cpu-steps', type=int, default=6,
                   help='size of the CPU oracle sample: decode steps (batch '
                        'rows with --stage encoder)')
@@ -814,6 +819,8 @@ def main():
     except Exception as e:  # pylint: disable=broad-except
       out['in_flight'] = {'decodes': n_in_flight, 'value': None,
                           'error': f'{type(e).__name__}: {e}'}
+  if args.counter_copy:
+    out['counter_copy_bytes'] = copy_calibration(torch)
   out['roofline']['device_level'] = device_level(
       w, out['ms_per_step'], out.get('in_flight'))
   if not args.no_cpu_baseline and size != 'xxl':

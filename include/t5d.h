@@ -279,18 +279,27 @@ int t5d_cross_attention_step_norm_q(void* stream, int dtype, int w_dtype,
  *   T5D_OUT_HEADS_VALUE), Ep a multiple of 32;
  *   rel_bias [H, 2E-1] bfloat16 indexed by (key - query + E - 1);
  *   enc_len [B]: keys and queries at positions >= enc_len[b] are padding
- *   (masked with -1e10 as in the reference); out [B*E, H*64]. */
+ *   (masked with -1e10 as in the reference);
+ *   valid_bits: NULL, or [B, (E + 31) / 32] words whose bit e says that
+ *   position e of the item is valid (encoder_input_tokens > 0 element-wise,
+ *   network.py:325-328: a padding token inside the text); positions at and
+ *   beyond enc_len[b] (then: the last valid position + 1) are padding
+ *   whatever their bits;
+ *   out [B*E, H*64]. */
 int t5d_encoder_attention(void* stream, const void* q, const void* k,
                           const void* v_t, const void* rel_bias,
-                          const int32_t* enc_len, void* out, int B, int H,
-                          int E, int Ep, int q_stride, int k_stride);
+                          const int32_t* enc_len, const uint32_t* valid_bits,
+                          void* out, int B, int H, int E, int Ep, int q_stride,
+                          int k_stride);
 
 /* The same attention in float32 (the dtype of the exactness tests), straight
  * from the fused projection: qkv [B*E, 3*H*64] holds q | k | v per row;
- * rel_bias [H, 2E-1] float32; out [B*E, H*64].  E <= 2048. */
+ * rel_bias [H, 2E-1] float32; enc_len / valid_bits as above; out
+ * [B*E, H*64].  E <= 2048. */
 int t5d_encoder_attention_f32(void* stream, const float* qkv,
                               const float* rel_bias, const int32_t* enc_len,
-                              float* out, int B, int H, int E);
+                              const uint32_t* valid_bits, float* out, int B,
+                              int H, int E);
 
 /* Add `delta` to n int32 values (cache_index += 1, layers.py:275). */
 int t5d_add_i32(void* stream, int32_t* x, int n, int delta);

@@ -34,7 +34,8 @@ struct EncAttnArgs {
   const bf16_t* k;    // same layout as q
   const bf16_t* vt;   // [B, H, Ep / 32, 64, 32]: 32-key blocks
   const bf16_t* bias; // [H, 2E-1]: by (key - query + E - 1)
-  const int32_t* len; // [B] valid prefix length
+  const int32_t* len; // [B] valid prefix length (with `valid`: last valid + 1)
+  const uint32_t* valid;  // optional [B, (E + 31) / 32]: bit e = position e valid
   bf16_t* out;        // [B*E, H*64]
   int H, E, Ep, q_stride, k_stride;
 };
@@ -45,6 +46,7 @@ __global__ void __launch_bounds__(256)
 enc_attn_kernel(EncAttnArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t s_p[4][16][32];
   __shared__ float s_bias[2 * kMaxEncLen];  // this head's bias by distance
+  __shared__ uint32_t s_valid[kMaxEncLen / 32];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, gq = lane >> 4;
@@ -53,10 +55,22 @@ enc_attn_kernel(EncAttnArgs a) {
   const int E = a.E;
   for (int i = threadIdx.x; i < 2 * E - 1; i += 256)
     s_bias[i] = bf16_to_f32(a.bias[(size_t)h * (2 * E - 1) + i]);
-  __syncthreads();
-  if (q0 >= E) return;
   int n = a.len[b];
   n = n < 0 ? 0 : (n > E ? E : n);
+  // Which positions are valid: the prefix [0, n), or the caller's bits (a
+  // padding token inside the text: encoder_input_tokens > 0 element-wise).
+  const int words = (E + 31) >> 5;
+  for (int i = threadIdx.x; i < words; i += 256) {
+    const int left = n - 32 * i;
+    const uint32_t prefix =
+        left >= 32 ? 0xffffffffu : (left <= 0 ? 0u : ((1u << left) - 1u));
+    s_valid[i] = a.valid ? (a.valid[(size_t)b * words + i] & prefix) : prefix;
+  }
+  __syncthreads();
+  if (q0 >= E) return;
+  auto is_valid = [&](int pos) {
+    return pos < E && ((s_valid[pos >> 5] >> (pos & 31)) & 1u) != 0;
+  };
   const float kMasked = -9.9857e9f;  // bf16(-1e10), layers.py:309-311
   const size_t row0 = (size_t)b * E;
 
@@ -67,15 +81,17 @@ enc_attn_kernel(EncAttnArgs a) {
   for (int c = 0; c < 2; ++c)
     qb[c].u = *reinterpret_cast<const uint4*>(
         a.q + (row0 + qi) * a.q_stride + h * 64 + 32 * c + 8 * gq);
-  const bool q_valid = (q0 + l16) < n;
+  const bool q_valid = is_valid(q0 + l16);
   const float* bias_row = s_bias + (E - 1) - qi;
 
   // Keys past the valid length get -1e10, whose exp underflows to exactly 0
   // next to any valid key: when all 16 queries of this wavefront are valid,
   // the key tiles that hold only padding are skipped.  (A padded query attends
   // uniformly over ALL keys, so a wavefront with one walks them all.)
-  const int n_tiles =
-      (q0 + 15 < n) ? (n + 15) >> 4 : (E + 15) >> 4;
+  const bool all_valid =
+      q0 + 15 < E &&
+      ((s_valid[q0 >> 5] >> (q0 & 31)) & 0xffffu) == 0xffffu;  // q0 % 16 == 0
+  const int n_tiles = all_valid ? (n + 15) >> 4 : (E + 15) >> 4;
 
   // K tile kt as the A operand: lane (row = key l16, g) holds K[key][32c + 8g .. +8].
   // It is fetched with four neighbouring lanes on 64 contiguous bytes of one key
@@ -104,7 +120,7 @@ enc_attn_kernel(EncAttnArgs a) {
       const int key = 16 * kt + 4 * gq + i;
       float x = round_bf16(acc[i]);
       if (key < E) {
-        const bool ok = q_valid && key < n;
+        const bool ok = q_valid && is_valid(key);
         x = ok ? round_bf16(x + bias_row[key]) : kMasked;
       } else {
         x = -INFINITY;
@@ -219,6 +235,7 @@ struct EncAttnF32Args {
   const float* qkv;   // [B*E, 3*H*64]
   const float* bias;  // [H, 2E-1], by (key - query + E - 1)
   const int32_t* len; // [B]
+  const uint32_t* valid;  // optional [B, (E + 31) / 32], as EncAttnArgs
   float* out;         // [B*E, H*64]
   int H, E;
 };
@@ -240,7 +257,13 @@ enc_attn_f32_kernel(EncAttnF32Args a) {
   const float* base = a.qkv + (size_t)b * a.E * row_stride + h * kHeadDim;
   s_q[wave][lane] = base[(size_t)e * row_stride + lane];
   const float* bias = a.bias + (size_t)h * (2 * a.E - 1) + (a.E - 1) - e;
-  const bool q_valid = e < n;
+  const int words = (a.E + 31) >> 5;
+  auto is_valid = [&](int pos) {
+    return pos < n &&
+           (a.valid == nullptr ||
+            ((a.valid[(size_t)b * words + (pos >> 5)] >> (pos & 31)) & 1u) != 0);
+  };
+  const bool q_valid = is_valid(e);
 
   float m = -INFINITY;
   for (int j = lane; j < a.E; j += 64) {
@@ -256,7 +279,7 @@ enc_attn_f32_kernel(EncAttnF32Args a) {
       s = fmaf(qv.z, kv.z, s);
       s = fmaf(qv.w, kv.w, s);
     }
-    const float mask = (q_valid && j < n) ? 0.f : -1e10f;
+    const float mask = (q_valid && is_valid(j)) ? 0.f : -1e10f;
     const float x = s + (mask + bias[j]);
     s_w[wave][j] = x;
     m = fmaxf(m, x);
@@ -283,8 +306,9 @@ using namespace t5d;
 
 extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
                                      const void* v_t, const void* rel_bias,
-                                     const int32_t* enc_len, void* out, int B,
-                                     int H, int E, int Ep, int q_stride,
+                                     const int32_t* enc_len,
+                                     const uint32_t* valid_bits, void* out,
+                                     int B, int H, int E, int Ep, int q_stride,
                                      int k_stride) {
   T5D_REQUIRE(q && k && v_t && rel_bias && enc_len && out, T5D_EINVAL,
               "t5d_encoder_attention: null pointer");
@@ -305,6 +329,7 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
   EncAttnArgs a;
   a.q = (const bf16_t*)q; a.k = (const bf16_t*)k; a.vt = (const bf16_t*)v_t;
   a.bias = (const bf16_t*)rel_bias; a.len = enc_len; a.out = (bf16_t*)out;
+  a.valid = valid_bits;
   a.H = H; a.E = E; a.Ep = Ep; a.q_stride = q_stride; a.k_stride = k_stride;
   dim3 grid((E + 63) / 64, H, B), block(256);
   hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
@@ -314,8 +339,9 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
 
 extern "C" int t5d_encoder_attention_f32(void* stream, const float* qkv,
                                          const float* rel_bias,
-                                         const int32_t* enc_len, float* out,
-                                         int B, int H, int E) {
+                                         const int32_t* enc_len,
+                                         const uint32_t* valid_bits,
+                                         float* out, int B, int H, int E) {
   T5D_REQUIRE(qkv && rel_bias && enc_len && out, T5D_EINVAL,
               "t5d_encoder_attention_f32: null pointer");
   T5D_REQUIRE(B > 0 && H > 0 && E > 0, T5D_EINVAL,
@@ -329,6 +355,7 @@ extern "C" int t5d_encoder_attention_f32(void* stream, const float* qkv,
               "t5d_encoder_attention_f32: qkv must be 16-byte aligned");
   EncAttnF32Args a;
   a.qkv = qkv; a.bias = rel_bias; a.len = enc_len; a.out = out;
+  a.valid = valid_bits;
   a.H = H; a.E = E;
   dim3 grid((E + kEncF32Rows - 1) / kEncF32Rows, H, B);
   hipLaunchKernelGGL(enc_attn_f32_kernel, grid, dim3(64 * kEncF32Rows), 0,

@@ -67,7 +67,7 @@ def _encode_hip(module, params, tokens):
   B, E = tokens.shape
   H = cfg.num_heads
   HD = H * 64
-  lens = _suffix_lengths(tokens, dev)
+  lens, bits = _key_mask(tokens, dev)
   Ep = (E + 31) // 32 * 32  # values are stored in blocks of 32 positions
   bias = w.rel_bias(E)
   ids = tokens.reshape(-1).to(torch.int32).contiguous()
@@ -78,7 +78,8 @@ def _encode_hip(module, params, tokens):
     xn = ops.rmsnorm(x, l['ln_attn'])
     qk = ops.gemm_rows(xn, l['qk'])                       # [M, q | k]
     ops.gemm_rows(xn, l['v'], out=v_t, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep)
-    attn = ops.encoder_attention(qk[:, :HD], qk[:, HD:], v_t, bias, lens)
+    attn = ops.encoder_attention(qk[:, :HD], qk[:, HD:], v_t, bias, lens,
+                                 valid_bits=bits)
     x = ops.gemm_rows(attn, l['o'], residual=x)
     y = ops.rmsnorm(x, l['ln_mlp'])
     h = ops.gemm_rows(y, l['wi'])
@@ -125,15 +126,21 @@ class EncoderKernelWeightsF32:
     return self._bias[E]
 
 
-def _suffix_lengths(tokens, dev):
-  """Valid length per row; padding must be a suffix of zeros."""
+def _key_mask(tokens, dev):
+  """The padding mask of t5x/examples/t5/network.py:325-328 (token > 0,
+  element-wise) as the kernels take it: (lengths, bits).  Padding that is a
+  suffix of zeros, the usual case, is a length per row and bits None; a
+  padding token inside the text gives the last valid position + 1 and one bit
+  per position (ops.pack_valid_bits)."""
+  from t5x_amd import ops
   B, E = tokens.shape
   valid = tokens > 0
   lens = valid.sum(dim=1).to(torch.int32)
   prefix = torch.arange(E, device=dev)[None, :] < lens[:, None]
-  if not bool((prefix == valid).all()):
-    raise ValueError('encoder padding must be a suffix of zeros')
-  return lens.contiguous()
+  if bool((prefix == valid).all()):
+    return lens.contiguous(), None
+  last = (valid * torch.arange(1, E + 1, device=dev)[None, :]).max(dim=1).values
+  return last.to(torch.int32).contiguous(), ops.pack_valid_bits(valid)
 
 
 def _encode_hip_f32(module, params, tokens):
@@ -147,12 +154,12 @@ def _encode_hip_f32(module, params, tokens):
   w = module._enc_weights[key][1]
   B, E = tokens.shape
   H = cfg.num_heads
-  lens = _suffix_lengths(tokens, dev)
+  lens, bits = _key_mask(tokens, dev)
   bias = w.rel_bias(E)
   x = ops.embed(w.embedding, tokens.reshape(-1).to(torch.int32).contiguous())
   for l in w.layers:
     qkv = ops.gemm(x, l['qkv'], norm_scale=l['ln_attn'])
-    attn = ops.encoder_attention_f32(qkv, bias, lens, H)
+    attn = ops.encoder_attention_f32(qkv, bias, lens, H, valid_bits=bits)
     x = ops.gemm(attn, l['o'], residual=x)
     h = ops.gemm(x, l['wi'], norm_scale=l['ln_mlp'])
     x = ops.gemm(h, l['wo'], residual=x)

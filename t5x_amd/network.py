@@ -453,7 +453,22 @@ class Transformer:
     Ep = (E + pad - 1) // pad * pad
     if out is not None and (out['B'], out['E']) != (B, Ep):
       raise ValueError('cross K/V buffers of another shape')
-    x = encoded.reshape(B * E, d).contiguous()
+    # The mask keeps exactly the keys whose token is > 0 (network.py:366-370).
+    # Keys and values of a position depend on that position alone and
+    # cross-attention has no position term, so masking a key equals leaving
+    # it out: the kernels take a count of valid keys per item, and where the
+    # padding is not a suffix of zeros (a padding token inside the text) the
+    # valid positions' encoder outputs are moved to the front first, in order.
+    tok = enc_tokens.reshape(B, E)
+    valid = tok > 0
+    lens = valid.sum(dim=1).to(torch.int32)
+    prefix = torch.arange(E, device=tok.device)[None, :] < lens[:, None]
+    if not bool((prefix == valid).all()):
+      order = torch.sort((~valid).to(torch.int8), dim=1, stable=True).indices
+      x = torch.gather(encoded, 1, order[:, :, None].expand(B, E, d))
+    else:
+      x = encoded
+    x = x.reshape(B * E, d).contiguous()
     ks, vs = [], []
     hip = bf16 and E % 4 == 0
     for i, l in enumerate(w.layers):
@@ -483,15 +498,6 @@ class Transformer:
         if out is not None:
           buf = (out['k'] if dst is ks else out['v'])[i].copy_(buf)
         dst.append(buf)
-    tok = enc_tokens.reshape(B, E)
-    valid = tok > 0
-    # The mask keeps exactly the positions with token > 0 (network.py:366-370).
-    # The kernel takes a prefix length; inputs are right-padded.
-    lens = valid.sum(dim=1).to(torch.int32)
-    prefix = (torch.arange(E, device=tok.device)[None, :] <
-              lens[:, None])
-    if not bool((prefix == valid).all()):
-      raise ValueError('encoder padding must be a suffix of zeros')
     if out is not None:
       out['enc_len'].copy_(lens)
       res = out

@@ -489,10 +489,34 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
   return out
 
 
-def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
+def _valid_bits(valid_bits, B, E):
+  if valid_bits is None:
+    return None
+  _chk(valid_bits, 'valid_bits', torch.int32, 2)
+  if tuple(valid_bits.shape) != (B, (E + 31) // 32):
+    raise ValueError(f'valid_bits {tuple(valid_bits.shape)}, expected '
+                     f'{(B, (E + 31) // 32)}')
+  return valid_bits.data_ptr()
+
+
+def pack_valid_bits(valid):
+  """[B, E] bool -> [B, (E + 31) / 32] int32 words, bit e % 32 of word e / 32
+  = valid[b, e] (what the encoder attention kernels take as valid_bits)."""
+  B, E = valid.shape
+  words = (E + 31) // 32
+  padded = torch.zeros((B, words * 32), dtype=torch.int64, device=valid.device)
+  padded[:, :E] = valid.to(torch.int64)
+  weights = (1 << torch.arange(32, device=valid.device, dtype=torch.int64))
+  packed = (padded.view(B, words, 32) * weights).sum(-1)
+  packed = torch.where(packed >= 2**31, packed - 2**32, packed)
+  return packed.to(torch.int32).contiguous()
+
+
+def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None, valid_bits=None):
   """q, k: [B*E, >= H*64] row-major views (row stride = stride(0)); v_t
   [B, H, Ep/32, 64, 32] (tile_cross_value of [B, H, 64, Ep]); rel_bias
-  [H, 2E-1]; enc_len [B] -> out [B*E, H*64]."""
+  [H, 2E-1]; enc_len [B]; valid_bits: None or pack_valid_bits of the
+  per-position mask -> out [B*E, H*64]."""
   _chk(v_t, 'v_t', torch.bfloat16, 5)
   _chk(rel_bias, 'rel_bias', torch.bfloat16, 2)
   _chk(enc_len, 'enc_len', torch.int32, 1)
@@ -514,13 +538,16 @@ def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None):
   _chk(out, 'out', torch.bfloat16, 2)
   _lib.call('t5d_encoder_attention', _s(), q.data_ptr(), k.data_ptr(),
             v_t.data_ptr(), rel_bias.data_ptr(), enc_len.data_ptr(),
-            out.data_ptr(), B, H, E, Ep, q.stride(0), k.stride(0))
+            _valid_bits(valid_bits, B, E), out.data_ptr(), B, H, E, Ep,
+            q.stride(0), k.stride(0))
   return out
 
 
-def encoder_attention_f32(qkv, rel_bias, enc_len, H, out=None):
+def encoder_attention_f32(qkv, rel_bias, enc_len, H, out=None,
+                          valid_bits=None):
   """float32 encoder self-attention from the fused projection: qkv
-  [B*E, 3*H*64] (q | k | v), rel_bias [H, 2E-1], enc_len [B] -> [B*E, H*64]."""
+  [B*E, 3*H*64] (q | k | v), rel_bias [H, 2E-1], enc_len [B], valid_bits as
+  encoder_attention -> [B*E, H*64]."""
   _chk(qkv, 'qkv', torch.float32, 2)
   _chk(rel_bias, 'rel_bias', torch.float32, 2)
   _chk(enc_len, 'enc_len', torch.int32, 1)
@@ -534,7 +561,8 @@ def encoder_attention_f32(qkv, rel_bias, enc_len, H, out=None):
     out = torch.empty((B * E, H * 64), dtype=torch.float32, device=qkv.device)
   _chk(out, 'out', torch.float32, 2)
   _lib.call('t5d_encoder_attention_f32', _s(), qkv.data_ptr(),
-            rel_bias.data_ptr(), enc_len.data_ptr(), out.data_ptr(), B, H, E)
+            rel_bias.data_ptr(), enc_len.data_ptr(),
+            _valid_bits(valid_bits, B, E), out.data_ptr(), B, H, E)
   return out
 
 
