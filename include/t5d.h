@@ -401,11 +401,21 @@ int t5d_beam_cond(void* stream, const t5d_beam_state* state, int B, int K,
  *   log-prob = log_softmax(rescale ? scaled : logits)[token]
  *   (0 for the greedy branch when rescale).
  *   logits, gumbel [R, V] f32 (gumbel may be NULL when every T <= 1e-4);
- *   temperature [R] f32; tokens [R] i32, logprobs [R] f32 (out). */
+ *   temperature [R] f32; tokens [R] i32, logprobs [R] f32 (out).
+ *   workspace: NULL, or t5d_sample_tokens_workspace_bytes(R) bytes of device
+ *   memory of the caller's (4-byte aligned, contents irrelevant): with it a
+ *   top-k choice (topk <= 64, rescale, R <= 128 rows of >= 4096 logits) runs
+ *   as two launches — every row cut into 4 parts that list their own k
+ *   largest, then one workgroup per row on those lists alone, which reads
+ *   Gumbel noise only for the kept candidates — instead of one workgroup per
+ *   row over everything (46 -> 13 us at 64 rows of 32128, k = 40).  The chosen
+ *   tokens are the same; log-probs are summed in another order (both exact to
+ *   float32 rounding). */
+int64_t t5d_sample_tokens_workspace_bytes(int R);
 int t5d_sample_tokens(void* stream, const float* logits, const float* gumbel,
                       const float* temperature, int32_t* tokens,
                       float* logprobs, int R, int V, int topk, float topp,
-                      int rescale);
+                      int rescale, void* workspace);
 
 /* Bookkeeping of one temperature_sample step (t5x/decoding.py:631-700):
  * prompt teacher forcing, log-prob accumulation, sequence write at i+1, EOS
@@ -545,6 +555,7 @@ typedef struct {
   int32_t* step_count;             /* device counter of executed steps */
   int32_t* tokens;                 /* [R] scratch */
   float* token_logprobs;           /* [R] scratch */
+  void* workspace;                 /* NULL or as t5d_sample_tokens takes it */
   int32_t* all_ended;              /* out: every row ended */
   int32_t* keep_going;             /* loop flag = !all_ended; == model->gate */
   int S, eos_id, topk, rescale;

@@ -69,8 +69,8 @@ class SampleStep(Structure):
       'sequences', 'cur_index', 'cur_token', 'ended', 'log_prob',
       'max_decode_len', 'initial_eos_count', 'temperature', 'gumbel')] +
               [('noise_ring', c_int)] + [(n, c_void_p) for n in (
-                  'step_count', 'tokens', 'token_logprobs', 'all_ended',
-                  'keep_going')] +
+                  'step_count', 'tokens', 'token_logprobs', 'workspace',
+                  'all_ended', 'keep_going')] +
               [('S', c_int), ('eos_id', c_int), ('topk', c_int),
                ('rescale', c_int), ('topp', c_float)])
 
@@ -135,8 +135,9 @@ _SIGNATURES = {
                                 c_int, c_int, c_int, c_int, c_int, c_int]),
     't5d_beam_cond': (c_int, [_P, POINTER(BeamStatePtrs), c_int, c_int, c_int,
                               c_float, c_float, c_int, c_int, _P]),
+    't5d_sample_tokens_workspace_bytes': (c_int64, [c_int]),
     't5d_sample_tokens': (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int,
-                                  c_float, c_int]),
+                                  c_float, c_int, _P]),
     't5d_sample_update': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
                                   c_int, c_int, c_int]),
 }

@@ -804,6 +804,9 @@ struct SampleArgs {
   const int32_t* noise_step; // null: slot 0
   int noise_ring, R;
   const int32_t* gate;
+  // optional: the rows' top-k candidates found by sample_topk_parts_kernel
+  // (sample_parts_* below), or null
+  int32_t* parts;
 };
 
 // One workgroup per row.
@@ -1013,6 +1016,135 @@ __device__ __forceinline__ float kth_largest_by_radix(const float4 (&y)[8],
   return key_to_float(prefix);
 }
 
+// ---- top-k sampling in two launches ------------------------------------------------
+// A row per workgroup leaves three quarters of the device idle at 64 rows, and
+// the workgroup spends its time in a dozen block-wide exchanges.  With a
+// top-k mask only the k largest scaled logits (and their ties) can be chosen
+// or enter the log-softmax — everything else is -1e7, whose exponential is
+// exactly 0 next to them — so the row is first cut into kSampleParts parts,
+// one small workgroup each (every CU gets some), which emit their own k
+// largest, ties at the k-th included; the row's k largest are among those
+// 4 k.  The row's workgroup then works on that list alone: the k-th largest
+// overall, Gumbel noise gathered for the kept candidates only (the noise
+// tensor is not read otherwise), argmax, log-softmax.  A part whose list
+// overflows (long runs of equal values), a greedy row, logits so low that
+// -1e7 is not far below them: the row is marked and its workgroup runs
+// the one-launch algorithm on the whole row.
+// Workspace (int32 words): counts [R][kSampleParts] (-1: marked), then values
+// [R][kSampleParts][kSamplePartCap] (float bits), then indices of the same
+// shape.
+constexpr int kSampleParts = 4;
+constexpr int kSamplePartCap = 64;   // candidates a part may emit
+constexpr int kSamplePartList = 256; // elements at or above a part's bound
+__host__ __device__ inline size_t sample_parts_words(int R) {
+  return (size_t)R * kSampleParts * (1 + 2 * kSamplePartCap);
+}
+__device__ __forceinline__ int32_t* sample_parts_count(int32_t* ws, int r, int p) {
+  return ws + (size_t)r * kSampleParts + p;
+}
+__device__ __forceinline__ int32_t* sample_parts_vals(int32_t* ws, int R, int r, int p) {
+  return ws + (size_t)R * kSampleParts +
+         ((size_t)r * kSampleParts + p) * kSamplePartCap;
+}
+__device__ __forceinline__ int32_t* sample_parts_idx(int32_t* ws, int R, int r, int p) {
+  return ws + (size_t)R * kSampleParts * (1 + kSamplePartCap) +
+         ((size_t)r * kSampleParts + p) * kSamplePartCap;
+}
+
+__global__ void __launch_bounds__(256)
+sample_topk_parts_kernel(SampleArgs a) {
+  __shared__ float s_wm[4];
+  __shared__ float s_lv[kSamplePartList];
+  __shared__ int s_li[kSamplePartList];
+  __shared__ int s_count, s_out;
+  __shared__ float s_cut;
+  T5D_GATED(a.gate);
+  const int p = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int V = a.V, nvec = V >> 2;
+  const int chunk = (nvec + kSampleParts - 1) / kSampleParts;  // <= 2048
+  const int v0 = p * chunk, v1 = min(nvec, v0 + chunk);
+  const float4 kPad = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  const float4* x4 = reinterpret_cast<const float4*>(a.logits + (size_t)r * V);
+  float4 y[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int vi = v0 + u * 256 + tid;
+    y[u] = vi < v1 ? x4[vi] : kPad;
+  }
+  const float T = a.temperature[r];
+  const float kMinT = 1e-4f;
+  if (tid == 0) { s_count = 0; s_out = 0; }
+  int32_t* count = sample_parts_count(a.parts, r, p);
+  if (!(T > kMinT)) {  // greedy rows take the one-launch path
+    if (tid == 0) *count = -1;
+    return;
+  }
+  const float Tm = fmaxf(T, kMinT);
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    y[u].x /= Tm; y[u].y /= Tm; y[u].z /= Tm; y[u].w /= Tm;
+  }
+  // bound: the smallest over the 4 wavefronts of a wavefront's m-th largest
+  // per-thread maximum, m = ceil(k / 4): at least k elements reach it
+  const int m = (a.topk + 3) >> 2;
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    tmax = fmaxf(fmaxf(tmax, fmaxf(y[u].x, y[u].y)), fmaxf(y[u].z, y[u].w));
+  float rest = tmax, wm = -INFINITY;
+  for (int it = 0; it < m; ++it) {
+    wm = wave_max(rest);
+    const unsigned long long hit = __builtin_amdgcn_ballot_w64(rest == wm);
+    if (lane == (int)__builtin_ctzll(hit | (1ull << 63))) rest = -INFINITY;
+  }
+  if (lane == 0) s_wm[wave] = wm;
+  __syncthreads();
+  const float bound = fminf(fminf(s_wm[0], s_wm[1]), fminf(s_wm[2], s_wm[3]));
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const float top = fmaxf(fmaxf(y[u].x, y[u].y), fmaxf(y[u].z, y[u].w));
+    if (top >= bound) {  // (-inf pads never reach a finite bound)
+      const float e[4] = {y[u].x, y[u].y, y[u].z, y[u].w};
+      const int j = 4 * (v0 + u * 256 + tid);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (e[c] >= bound) {
+          const int q = atomicAdd(&s_count, 1);
+          if (q < kSamplePartList) { s_lv[q] = e[c]; s_li[q] = j + c; }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int ncand = s_count;
+  // fewer than k (a -inf bound: rows of -inf) or more than the list holds
+  bool ok = ncand >= a.topk && ncand <= kSamplePartList && bound > -INFINITY;
+  if (ok) {
+    if (tid < ncand) {
+      const float v = s_lv[tid];
+      int gt = 0, ge = 0;
+      for (int c = 0; c < ncand; ++c) {
+        const float o = s_lv[c];
+        gt += o > v ? 1 : 0;
+        ge += o >= v ? 1 : 0;
+      }
+      if (gt < a.topk && a.topk <= ge) s_cut = v;  // equal candidates: same bits
+    }
+    __syncthreads();
+    const float cut = s_cut;
+    float* vals = reinterpret_cast<float*>(sample_parts_vals(a.parts, a.R, r, p));
+    int32_t* idx = sample_parts_idx(a.parts, a.R, r, p);
+    if (tid < ncand && s_lv[tid] >= cut) {
+      const int q = atomicAdd(&s_out, 1);
+      if (q < kSamplePartCap) { vals[q] = s_lv[tid]; idx[q] = s_li[tid]; }
+    }
+    __syncthreads();
+    ok = s_out <= kSamplePartCap;
+  }
+  if (tid == 0) *count = ok ? s_out : -1;
+}
+
 __global__ void __launch_bounds__(1024)
 sample_tokens_fast_kernel(SampleArgs a) {
   __shared__ Cand cscratch[16];
@@ -1027,6 +1159,68 @@ sample_tokens_fast_kernel(SampleArgs a) {
   const int r = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int V = a.V, nvec = V >> 2;
+  if (a.parts != nullptr) {
+    // The row's candidates from sample_topk_parts_kernel: at most
+    // kSampleParts * kSamplePartCap = 256 of them, one per thread.
+    int n[kSampleParts], total = 0;
+    bool usable = true;
+#pragma unroll
+    for (int p = 0; p < kSampleParts; ++p) {
+      n[p] = *sample_parts_count(a.parts, r, p);
+      usable = usable && n[p] >= 0;
+      total += n[p];
+    }
+    if (usable) {
+      float v = -INFINITY;
+      int j = 0x7FFFFFFF;
+      int base = 0;
+#pragma unroll
+      for (int p = 0; p < kSampleParts; ++p) {
+        if (tid >= base && tid < base + n[p]) {
+          v = reinterpret_cast<const float*>(
+              sample_parts_vals(a.parts, a.R, r, p))[tid - base];
+          j = sample_parts_idx(a.parts, a.R, r, p)[tid - base];
+        }
+        base += n[p];
+      }
+      if (tid < total) s_lv[tid] = v;
+      __syncthreads();
+      // the k-th largest of the row (ties kept): by counting
+      int gt = 0, ge = 0;
+      if (tid < total) {
+        for (int c = 0; c < total; ++c) {
+          const float o = s_lv[c];
+          gt += o > v ? 1 : 0;
+          ge += o >= v ? 1 : 0;
+        }
+        if (gt < a.topk && a.topk <= ge) s_cut = v;
+      }
+      const float mx = block_max_f32(v, fscratch);  // (a barrier: s_cut is set)
+      const float cutoff = s_cut;
+      // -1e7 must be so far below the kept values that its exponential is 0
+      if (mx > kNegInf + 1000.f) {
+        const bool kept = tid < total && v >= cutoff;
+        const int slot = a.noise_step ? *a.noise_step % a.noise_ring : 0;
+        Cand best = {-INFINITY, 0x7FFFFFFF};
+        if (kept) {
+          best.v = v + a.gumbel[((size_t)slot * a.R + r) * V + j];
+          best.i = j;
+        }
+        best = block_best(best, cscratch);
+        double sum = kept ? (double)expf(v - mx) : 0.0;
+        sum = block_sum_f64(sum, dscratch);
+        __syncthreads();
+        if (kept && j == best.i) fscratch[0] = v;  // one thread holds the token
+        __syncthreads();
+        if (tid == 0) {
+          a.tokens[r] = best.i;
+          a.logprobs[r] = (fscratch[0] - mx) - (float)log(sum);
+        }
+        return;
+      }
+      __syncthreads();  // (everyone has read what the path below reuses)
+    }
+  }
   const float4 kPad = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
   const float4* x4 = reinterpret_cast<const float4*>(a.logits + (size_t)r * V);
   float4 y[8];
@@ -1291,39 +1485,59 @@ struct SampleUpdateArgs {
   const int32_t* gate;
 };
 
-// One workgroup; 16 lanes per row (rows are dealt round-robin to the 64 groups
-// of 16 lanes), which count the row's EOS tokens in parallel.
+// One workgroup; 8 lanes per row (128 rows per pass), which read the row's
+// sequence once — counting its EOS tokens and picking up the forced token at
+// position i + 1 on the way — so that every load of a row is asked for
+// before the first one is waited for: the kernel costs one trip to memory on
+// top of its launch (with 16 lanes per row, 64 rows per pass and the loads
+// chained index -> forced token -> row it took 13 us for 64 rows and 23 us
+// for 128).
 constexpr int kSampleUpdateThreads = 1024;
+constexpr int kSampleUpdateLanes = 8;
+__device__ __forceinline__ int lanes8_sum(int v) {
+  v += dpp_move<kDppXor1>(v);
+  v += dpp_move<kDppXor2>(v);
+  return v + dpp_move<kDppHalfMirror>(v);
+}
+
 __global__ void __launch_bounds__(kSampleUpdateThreads)
 sample_update_kernel(SampleUpdateArgs a) {
   __shared__ int iscratch[kSampleUpdateThreads / 64];
   T5D_GATED(a.gate);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int group = threadIdx.x >> 4, gl = threadIdx.x & 15;
-  int not_ended = 0;  // rows of this group still running (its 16 lanes agree)
-  for (int r0 = 0; r0 < a.R; r0 += kSampleUpdateThreads / 16) {
-    // whole wavefronts stay in the loop (the reduction below is wave-wide);
+  const int group = threadIdx.x / kSampleUpdateLanes;
+  const int gl = threadIdx.x % kSampleUpdateLanes;
+  int not_ended = 0;  // rows of this group still running (its lanes agree)
+  for (int r0 = 0; r0 < a.R; r0 += kSampleUpdateThreads / kSampleUpdateLanes) {
+    // whole wavefronts stay in the loop (the reductions below cross lanes);
     // groups past the last row work on row 0 and discard the result
     const bool real = r0 + group < a.R;
     const int r = real ? r0 + group : 0;
     int32_t* seq = a.sequences + (size_t)r * a.S;
     const int mdl = a.max_decode_len[r];
-    const int i = min(a.cur_index[r], mdl);
-    const int next_input = seq[i + 1];
-    const bool oop = next_input == 0;
+    const int ci = a.cur_index[r];
     const bool was_ended = a.ended[r] != 0;
-    const int tok = oop ? a.tokens[r] : next_input;
+    const int sampled = a.tokens[r];
+    const float sampled_lp = a.token_logprobs[r];
+    const float lp = a.log_prob[r];
+    const int initial_eos = a.initial_eos_count[r];
+    const int i = min(ci, mdl);
+    // EOS count of the row without position i + 1, and that position's token
+    int eos = 0, next_input = 0;
+    for (int j = gl; j < a.S; j += kSampleUpdateLanes) {
+      const int v = seq[j];
+      if (j == i + 1) next_input = v;
+      else eos += (v == a.eos_id) ? 1 : 0;
+    }
+    eos = lanes8_sum(eos);
+    next_input = lanes8_sum(next_input);  // one lane held it
+    const bool oop = next_input == 0;
+    const int tok = oop ? sampled : next_input;
     const int out_tok = was_ended ? 0 : tok;
-    // EOS count of the row with position i + 1 already holding out_tok
-    int eos = 0;
-    for (int j = gl; j < a.S; j += 16)
-      eos += ((j == i + 1 ? out_tok : seq[j]) == a.eos_id) ? 1 : 0;
-    eos = lanes16_sum(eos);
-    const bool ended = was_ended || (eos > a.initial_eos_count[r]) ||
-                       (i >= mdl - 1);
+    eos += (out_tok == a.eos_id) ? 1 : 0;
+    const bool ended = was_ended || (eos > initial_eos) || (i >= mdl - 1);
     if (real && gl == 0) {
-      if (oop && !was_ended)
-        a.log_prob[r] = a.log_prob[r] + a.token_logprobs[r];
+      if (oop && !was_ended) a.log_prob[r] = lp + sampled_lp;
       seq[i + 1] = out_tok;
       a.ended[r] = ended ? 1 : 0;
       a.cur_index[r] = i + 1;
@@ -1331,7 +1545,8 @@ sample_update_kernel(SampleUpdateArgs a) {
     }
     if (real && gl == 0 && !ended) ++not_ended;
   }
-  // lanes 0, 16, 32, 48 hold their groups' counts
+  // lanes 0, 8, .., 56 hold their groups' counts
+  not_ended += __shfl_xor(not_ended, 8, 64);
   not_ended += __shfl_xor(not_ended, 16, 64);
   not_ended += __shfl_xor(not_ended, 32, 64);
   if (lane == 0) iscratch[wave] = not_ended;
@@ -1604,19 +1819,36 @@ int t5d::launch_beam_tail(hipStream_t s, const t5d_beam_state* state, int B,
   return T5D_OK;
 }
 
-static void launch_sample_tokens(hipStream_t s, const SampleArgs& a, int R) {
+static void launch_sample_tokens(hipStream_t s, SampleArgs a, int R) {
   const bool aligned = ((uintptr_t)a.logits % 16) == 0 &&
                        (a.gumbel == nullptr || ((uintptr_t)a.gumbel % 16) == 0);
-  if (a.V % 4 == 0 && a.V <= 32768 && aligned)
+  const bool fast = a.V % 4 == 0 && a.V <= 32768 && aligned;
+  // Two launches when the rows' candidates can be found by parts: a top-k
+  // mask of at most kSamplePartCap, log-probs of the masked row, rows long
+  // enough that every part holds k elements, few enough rows to leave CUs
+  // idle otherwise.
+  const bool by_parts = fast && a.parts != nullptr && a.gumbel != nullptr &&
+                        a.topk > 0 && a.topk <= kSamplePartCap && a.rescale &&
+                        !(a.topp > 0.f) && a.V >= 4096 && R <= 128;
+  if (!by_parts) a.parts = nullptr;
+  if (by_parts)
+    hipLaunchKernelGGL(sample_topk_parts_kernel, dim3(kSampleParts, R),
+                       dim3(256), 0, s, a);
+  if (fast)
     hipLaunchKernelGGL(sample_tokens_fast_kernel, dim3(R), dim3(1024), 0, s, a);
   else
     hipLaunchKernelGGL(sample_tokens_kernel, dim3(R), dim3(256), 0, s, a);
 }
 
+extern "C" int64_t t5d_sample_tokens_workspace_bytes(int R) {
+  return R > 0 ? (int64_t)(sample_parts_words(R) * sizeof(int32_t)) : 0;
+}
+
 extern "C" int t5d_sample_tokens(void* stream, const float* logits,
                                  const float* gumbel, const float* temperature,
                                  int32_t* tokens, float* logprobs, int R,
-                                 int V, int topk, float topp, int rescale) {
+                                 int V, int topk, float topp, int rescale,
+                                 void* workspace) {
   T5D_REQUIRE(logits && temperature && tokens && logprobs, T5D_EINVAL,
               "t5d_sample_tokens: null pointer");
   T5D_REQUIRE(R > 0 && V > 0 && topk >= 0 && topp >= 0.f, T5D_EINVAL,
@@ -1629,6 +1861,9 @@ extern "C" int t5d_sample_tokens(void* stream, const float* logits,
   a.tokens = tokens; a.logprobs = logprobs;
   a.V = V; a.topk = topk; a.rescale = rescale; a.topp = topp;
   a.noise_step = nullptr; a.noise_ring = 1; a.R = R; a.gate = tls_gate;
+  T5D_REQUIRE(((uintptr_t)workspace % 4) == 0, T5D_EINVAL,
+              "t5d_sample_tokens: workspace alignment");
+  a.parts = static_cast<int32_t*>(workspace);
   launch_sample_tokens(as_stream(stream), a, R);
   T5D_CHECK_LAUNCH("t5d_sample_tokens");
   return T5D_OK;
@@ -1643,6 +1878,7 @@ int t5d::launch_sample_step(hipStream_t s, const float* logits,
   a.V = V; a.topk = st->topk; a.rescale = st->rescale; a.topp = st->topp;
   a.noise_step = st->step_count; a.noise_ring = st->noise_ring; a.R = R;
   a.gate = tls_gate;
+  a.parts = static_cast<int32_t*>(st->workspace);
   launch_sample_tokens(s, a, R);
   T5D_CHECK_LAUNCH("sample step (tokens)");
   SampleUpdateArgs u;

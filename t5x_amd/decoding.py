@@ -583,6 +583,9 @@ class SampleLoop(_InFlight):
     self.all_ended = torch.zeros((), dtype=torch.int32, device=dev)
     self.tokens = torch.empty((batch_size,), dtype=torch.int32, device=dev)
     self.tok_lp = torch.empty((batch_size,), dtype=torch.float32, device=dev)
+    # scratch memory for the token choice (both loops hand one over, so both
+    # take the same kernels)
+    self.sample_ws = ops.sample_tokens_workspace(batch_size, dev)
     self.source = _noise_source(prng_key)
     self.step = 0
     self.fused = None
@@ -635,7 +638,8 @@ class SampleLoop(_InFlight):
       gumbel = _dev(self.source.noise(self.step, tuple(logits.shape)),
                     torch.float32).contiguous()
     ops.sample_tokens(logits, gumbel, self.temps_dev, self.topk, self.topp,
-                      self.rescale_log_probs, self.tokens, self.tok_lp)
+                      self.rescale_log_probs, self.tokens, self.tok_lp,
+                      workspace=self.sample_ws)
     ops.sample_update(self.tokens, self.tok_lp, self.sequences, self.cur_index,
                       self.cur_token, self.ended, self.log_prob, self.mdl,
                       self.eos0, self.all_ended, self.eos_id)

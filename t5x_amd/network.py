@@ -929,6 +929,9 @@ class FusedSampleStep(_OwnedContext):
     st.noise_ring = self.ring
     st.step_count, st.tokens, st.token_logprobs = (
         P(self.step_count), P(self.tokens), P(self.tok_lp))
+    from t5x_amd import ops
+    self.sample_ws = ops.sample_tokens_workspace(R, dev)
+    st.workspace = P(self.sample_ws)
     st.all_ended, st.keep_going = P(all_ended), P(self.keep_going)
     st.S, st.eos_id, st.topk = S, int(eos_id), int(topk)
     st.rescale, st.topp = int(bool(rescale)), float(topp)

@@ -700,8 +700,15 @@ def beam_cond(state: BeamBuffers, min_brevity, min_log_prob, max_decode_step,
             int(min_initial_index), keep_going.data_ptr())
 
 
+def sample_tokens_workspace(R, device):
+  """Scratch memory that lets sample_tokens cut a top-k choice into two
+  launches (t5d_sample_tokens_workspace_bytes)."""
+  n = int(_lib.load().t5d_sample_tokens_workspace_bytes(int(R)))
+  return torch.empty(((n + 3) // 4,), dtype=torch.int32, device=device)
+
+
 def sample_tokens(logits, gumbel, temperature, topk, topp, rescale, tokens=None,
-                  logprobs=None):
+                  logprobs=None, workspace=None):
   _chk(logits, 'logits', torch.float32, 2)
   _chk(temperature, 'temperature', torch.float32, 1)
   R, V = logits.shape
@@ -715,9 +722,15 @@ def sample_tokens(logits, gumbel, temperature, topk, topp, rescale, tokens=None,
     tokens = torch.empty((R,), dtype=torch.int32, device=logits.device)
   if logprobs is None:
     logprobs = torch.empty((R,), dtype=torch.float32, device=logits.device)
+  if workspace is not None:
+    _chk(workspace, 'workspace', torch.int32, 1)
+    need = int(_lib.load().t5d_sample_tokens_workspace_bytes(R))
+    if workspace.numel() * 4 < need:
+      raise ValueError(f'workspace of {workspace.numel() * 4} bytes, need {need}')
   _lib.call('t5d_sample_tokens', _s(), logits.data_ptr(), _lib.ptr(gumbel),
             temperature.data_ptr(), tokens.data_ptr(), logprobs.data_ptr(), R,
-            V, int(topk), float(topp), int(bool(rescale)))
+            V, int(topk), float(topp), int(bool(rescale)),
+            _lib.ptr(workspace))
   return tokens, logprobs
 
 

@@ -1092,6 +1092,51 @@ def test_sample_tokens_topk_cutoff_with_ties(ops, k):
   np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize('R,V,k', [(6, 32128, 40), (64, 32128, 40),
+                                   (3, 32128, 1), (5, 32128, 64),
+                                   (128, 4096, 7), (4, 8000, 33)])
+def test_sample_tokens_topk_in_two_launches(ops, R, V, k):
+  """The top-k choice with a workspace (rows cut into parts that list their own
+  k largest, then one workgroup per row on the lists) against the oracle and
+  against the one-launch path: same tokens; log-probs to float32 rounding.
+  Rows are mixed: plain random rows, ties at the cutoff, a run of equal values
+  longer than a part's list (that row falls back to the whole-row path), a
+  greedy row (temperature 0), a row whose k largest sit in one part."""
+  rs = np.random.RandomState(R + V + k)
+  logits = (2 * rs.randn(R, V)).astype(np.float32)
+  logits[0, ::4] = logits[0, 1]                       # ties everywhere
+  logits[1 % R, rs.permutation(V)[:600]] = 60.0       # 600 equal maxima
+  logits[2 % R, :k + 5] += 30.0                       # all winners in part 0
+  temps = np.full((R,), 0.7, np.float32)
+  if R > 3:
+    temps[3] = 0.0                                    # a greedy row
+  if R > 4:
+    temps[4] = 1.3                                    # its own temperature
+  g = odec.GumbelNoise(seed=k).noise(0, (R, V))
+  ws = ops.sample_tokens_workspace(R, 'cuda')
+  ws.fill_(-7)                                        # contents are irrelevant
+  tok, lp = ops.sample_tokens(dev(logits), dev(g), dev(temps), k, 0.0, True,
+                              workspace=ws)
+  tok1, lp1 = ops.sample_tokens(dev(logits), dev(g), dev(temps), k, 0.0, True)
+  scaled = (logits / np.maximum(temps, np.float32(1e-4))[:, None]).astype(
+      np.float32)
+  masked = obs.topk_mask(scaled, k, np.float32(-1e7))
+  want_tok = np.argmax(masked + g, axis=-1)
+  want_lp = odec.log_softmax(masked)[np.arange(R), want_tok]
+  greedy = temps <= 1e-4
+  want_tok[greedy] = np.argmax(logits, axis=-1)[greedy]
+  want_lp[greedy] = 0.0
+  np.testing.assert_array_equal(host(tok), want_tok)
+  np.testing.assert_array_equal(host(tok1), want_tok)
+  np.testing.assert_allclose(host(lp), want_lp, atol=1e-5, rtol=1e-5)
+  np.testing.assert_allclose(host(lp), host(lp1), atol=2e-6, rtol=2e-6)
+  # which rows took the lists: all but the greedy row and the 600-tie row
+  counts = host(ws)[:R * 4].reshape(R, 4)
+  assert (counts[1 % R] < 0).any() and (counts[0] >= 0).all()
+  if R > 3:
+    assert (counts[3] < 0).all()
+
+
 def test_sample_tokens_topp_table(ops):
   # t5x/binary_search_test.py:143-209 through the kernel: with a huge Gumbel
   # bonus on one index the sampled token reveals whether it survived the mask.
