@@ -313,7 +313,7 @@ def _noted(path, key):
   with open(path) as f:
     for line in f:
       if line.startswith(key + ':'):
-        return int(float(line.split(':', 1)[1]))
+        return int(float(line.split(':', 1)[1].split()[0]))
   return None
 
 
