@@ -57,10 +57,14 @@ def parse_args():
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--lanes', type=int, default=None,
                   help='batch slices stepped concurrently (default: library)')
-  ap.add_argument('--stage', default='decode', choices=['decode', 'encoder'],
+  ap.add_argument('--stage', default='decode',
+                  choices=['decode', 'encoder', 'dense'],
                   help="'encoder': the once-per-batch stage before the decode "
                        'loop (encoder forward + cross K/V projection); a step '
-                       'is one batch')
+                       "is one batch.  'dense': the decoder's dense layers on "
+                       'their own, each kind replayed over the layers (a step '
+                       'is one pass over every dense layer of the decoder): '
+                       'weight streaming rate and matrix-core rate per kind')
   ap.add_argument('--in-flight', type=int, default=None,
                   help='also measure this many whole decodes of different '
                        'batches running on the device at once (default for '
@@ -701,6 +705,106 @@ class EncoderStage:
             'sample': f'{rows} of the {self.B} batch rows, one pass'}
 
 
+def main_dense(args):
+  """The dense layers of the configuration's decoder at its decode rows: every
+  kind (q/k/v with its layer norm, the two attention outputs, the gated MLP
+  input with its norm, the MLP output, the vocabulary projection with the
+  final norm) replayed back to back over the layers' weights, so no launch
+  finds its weights cached; time per launch from HIP events on the launch
+  stream.  `value`: passes over all dense layers of the decoder per second."""
+  import torch
+  from t5x_amd import network, ops
+  size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[args.config]
+  if dtype != 'bfloat16':
+    raise SystemExit('bench.py --stage dense measures the matrix-core kernels '
+                     f'(bfloat16 activations); {args.config} is {dtype}')
+  cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
+  dev = torch.device('cuda')
+  params = network.init_params(cfg, args.seed, dev, with_encoder=False)
+  module = network.Transformer(cfg, dev)
+  w = module.decoder_weights(params)
+  R, d, F, V = B * K, cfg.emb_dim, cfg.mlp_dim, cfg.vocab_size
+  hd = cfg.num_heads * cfg.head_dim
+  act = torch.bfloat16
+  wb = 1 if wdt == 'int8' else 2
+  rnd = lambda *s: torch.randn(s, device=dev).to(act)
+  x, ao, h = rnd(R, d), rnd(R, hd), rnd(R, F)
+  norm_rides = d <= 1024 or (wdt == 'int8' and d <= 2048)
+  nl = len(w.layers)
+  state = {'i': 0}
+
+  def layer():
+    state['i'] = (state['i'] + 1) % nl
+    return w.layers[state['i']]
+
+  def normed(name, ln):
+    def run():
+      l = layer()
+      if norm_rides and (d <= 1024 or l[name].N <= 2048):
+        ops.gemm(x, l[name], norm_scale=l[ln])
+      else:
+        ops.gemm(ops.rmsnorm(x, l[ln]), l[name])
+    return run
+
+  kinds = [
+      ('q, k, v (+ layer norm)', normed('qkv', 'ln_self'), d, 3 * hd, 1),
+      ('attention output + residual',
+       lambda: ops.gemm(ao, layer()['self_out'], residual=x), hd, d, 2),
+      ('cross-attention query (+ layer norm)', normed('cross_q', 'ln_cross'),
+       d, hd, 1),
+      ('gated MLP input (+ layer norm)', normed('wi', 'ln_mlp'), d, 2 * F, 1),
+      ('MLP output + residual',
+       lambda: ops.gemm(h, layer()['wo'], residual=x), F, d, 1),
+  ]
+  rows, total = [], 0.0
+  for name, fn, k, n, per_layer in kinds:
+    sec = time_kernel(torch, fn, 2 * nl)
+    nbytes = k * n * wb + R * (k + n) * 2
+    rows.append({'layer': name, 'K': k, 'N': n, 'launches_per_step':
+                 per_layer * nl, 'us': round(sec * 1e6, 2),
+                 'weight_gbps': round(k * n * wb / sec / 1e9, 1),
+                 'tflops': round(2.0 * R * k * n / sec / 1e12, 1),
+                 'bytes': nbytes})
+    total += sec * per_layer * nl
+  if norm_rides and d <= 1024:
+    vocab = lambda: ops.gemm(x, w.logits, norm_scale=w.ln_final,
+                             out_dtype=torch.float32)
+  else:
+    vocab = lambda: ops.gemm(ops.rmsnorm(x, w.ln_final), w.logits,
+                             out_dtype=torch.float32)
+  sec = time_kernel(torch, vocab, 8)
+  rows.append({'layer': 'vocabulary projection (+ final norm)', 'K': d, 'N': V,
+               'launches_per_step': 1, 'us': round(sec * 1e6, 2),
+               'weight_gbps': round(d * V * wb / sec / 1e9, 1),
+               'tflops': round(2.0 * R * d * V / sec / 1e12, 1),
+               'bytes': d * V * wb + R * d * 2 + R * V * 4})
+  total += sec
+  best = max(rows, key=lambda r: r['weight_gbps'])
+  weights = sum(r['K'] * r['N'] * wb * r['launches_per_step'] for r in rows)
+  out = {
+      'metric': f'passes over the decoder\'s dense layers per second, '
+                f'{args.config} at {R} rows on 1 GPU',
+      'value': round(1.0 / total, 1), 'unit': 'passes/s', 'n_gpus': 1,
+      'steps': 1, 'warmup': 0, 'ms_per_step': round(total * 1e3, 4),
+      'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+      'dtype': 'bf16' if wdt is None else f'bf16 act / {wdt} weights',
+      'data': 'synthetic',
+      'config': {'workload': f'T5.1.1-{size} decoder dense layers at {R} rows',
+                 'name': args.config, 'stage': 'dense', 'layers': rows,
+                 'weight_bytes_per_pass': weights,
+                 'weights_gbps_whole_pass': round(weights / total / 1e9, 1)},
+      'roofline': {'kernel': best['layer'], 'bound': 'hbm',
+                   'achieved': best['weight_gbps'], 'peak': HBM_PEAK_GBPS,
+                   'unit': 'GB/s',
+                   'frac': round(best['weight_gbps'] / HBM_PEAK_GBPS, 4),
+                   'traffic': None, 'bytes_per_launch': best['bytes'],
+                   'avg_launch_us': best['us']},
+  }
+  if args.counter_copy:
+    out['counter_copy_bytes'] = copy_calibration(torch)
+  print(json.dumps(out))
+
+
 def host_threads():
   try:
     from threadpoolctl import threadpool_info
@@ -757,6 +861,8 @@ def main():
     sys.exit(3)
   if args.stage == 'encoder':
     return main_encoder(args)
+  if args.stage == 'dense':
+    return main_dense(args)
   w = Workload(args.config, args.seed, args.lanes)
   if args.roofline_only:
     w.new_decode()  # builds the cross-attention K/V

@@ -1488,10 +1488,9 @@ struct SampleUpdateArgs {
 // One workgroup; 8 lanes per row (128 rows per pass), which read the row's
 // sequence once — counting its EOS tokens and picking up the forced token at
 // position i + 1 on the way — so that every load of a row is asked for
-// before the first one is waited for: the kernel costs one trip to memory on
-// top of its launch (with 16 lanes per row, 64 rows per pass and the loads
-// chained index -> forced token -> row it took 13 us for 64 rows and 23 us
-// for 128).
+// before the first one is waited for (with 16 lanes per row, 64 rows per pass,
+// one row element per trip to the L2 and the loads chained index -> forced
+// token -> row it took 13 us for 64 rows and 23 us for 128).
 constexpr int kSampleUpdateThreads = 1024;
 constexpr int kSampleUpdateLanes = 8;
 __device__ __forceinline__ int lanes8_sum(int v) {
@@ -1523,11 +1522,23 @@ sample_update_kernel(SampleUpdateArgs a) {
     const int initial_eos = a.initial_eos_count[r];
     const int i = min(ci, mdl);
     // EOS count of the row without position i + 1, and that position's token
+    // (12 loads in flight per lane and pass: a row of 258 takes three passes;
+    // one load per pass would be one trip to the L2 per element)
+    constexpr int kU = 12;
     int eos = 0, next_input = 0;
-    for (int j = gl; j < a.S; j += kSampleUpdateLanes) {
-      const int v = seq[j];
-      if (j == i + 1) next_input = v;
-      else eos += (v == a.eos_id) ? 1 : 0;
+    for (int j0 = gl; j0 < a.S; j0 += kSampleUpdateLanes * kU) {
+      int v[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int j = j0 + kSampleUpdateLanes * u;
+        v[u] = j < a.S ? seq[j] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int j = j0 + kSampleUpdateLanes * u;
+        if (j == i + 1) next_input = v[u];
+        else if (j < a.S) eos += (v[u] == a.eos_id) ? 1 : 0;
+      }
     }
     eos = lanes8_sum(eos);
     next_input = lanes8_sum(next_input);  // one lane held it
