@@ -737,22 +737,33 @@ def main_dense(args):
     state['i'] = (state['i'] + 1) % nl
     return w.layers[state['i']]
 
+  xn = ops.rmsnorm(x, w.layers[0]['ln_self'])
+  own_norm = []
+
   def normed(name, ln):
+    # The layer norm rides in the projection's kernel where the step does so;
+    # elsewhere it is a launch of its own, timed as its own row below.
+    rides = norm_rides and (d <= 1024 or w.layers[0][name].N <= 2048)
+    if not rides:
+      own_norm.append(name)
     def run():
       l = layer()
-      if norm_rides and (d <= 1024 or l[name].N <= 2048):
+      if rides:
         ops.gemm(x, l[name], norm_scale=l[ln])
       else:
-        ops.gemm(ops.rmsnorm(x, l[ln]), l[name])
+        ops.gemm(xn, l[name])
     return run
 
+  with_norm = lambda name, key: name + (
+      '' if key in own_norm else ' with its layer norm')
+  qkv_fn, cq_fn, wi_fn = (normed('qkv', 'ln_self'),
+                          normed('cross_q', 'ln_cross'), normed('wi', 'ln_mlp'))
   kinds = [
-      ('q, k, v (+ layer norm)', normed('qkv', 'ln_self'), d, 3 * hd, 1),
+      (with_norm('q, k, v', 'qkv'), qkv_fn, d, 3 * hd, 1),
       ('attention output + residual',
        lambda: ops.gemm(ao, layer()['self_out'], residual=x), hd, d, 2),
-      ('cross-attention query (+ layer norm)', normed('cross_q', 'ln_cross'),
-       d, hd, 1),
-      ('gated MLP input (+ layer norm)', normed('wi', 'ln_mlp'), d, 2 * F, 1),
+      (with_norm('cross-attention query', 'cross_q'), cq_fn, d, hd, 1),
+      (with_norm('gated MLP input', 'wi'), wi_fn, d, 2 * F, 1),
       ('MLP output + residual',
        lambda: ops.gemm(h, layer()['wo'], residual=x), F, d, 1),
   ]
@@ -770,17 +781,27 @@ def main_dense(args):
     vocab = lambda: ops.gemm(x, w.logits, norm_scale=w.ln_final,
                              out_dtype=torch.float32)
   else:
-    vocab = lambda: ops.gemm(ops.rmsnorm(x, w.ln_final), w.logits,
-                             out_dtype=torch.float32)
+    own_norm.append('logits')
+    vocab = lambda: ops.gemm(xn, w.logits, out_dtype=torch.float32)
+  if own_norm:
+    sec = time_kernel(torch, lambda: ops.rmsnorm(x, layer()['ln_mlp']), 2 * nl)
+    n_norms = nl * sum(k in own_norm for k in ('qkv', 'cross_q', 'wi')) + (
+        'logits' in own_norm)
+    rows.append({'layer': 'layer norm as a launch of its own', 'K': d, 'N': d,
+                 'launches_per_step': n_norms, 'us': round(sec * 1e6, 2),
+                 'weight_gbps': 0.0, 'tflops': 0.0, 'bytes': 2 * R * d * 2})
+    total += sec * n_norms
   sec = time_kernel(torch, vocab, 8)
-  rows.append({'layer': 'vocabulary projection (+ final norm)', 'K': d, 'N': V,
+  rows.append({'layer': with_norm('vocabulary projection', 'logits'),
+               'K': d, 'N': V,
                'launches_per_step': 1, 'us': round(sec * 1e6, 2),
                'weight_gbps': round(d * V * wb / sec / 1e9, 1),
                'tflops': round(2.0 * R * d * V / sec / 1e12, 1),
                'bytes': d * V * wb + R * d * 2 + R * V * 4})
   total += sec
   best = max(rows, key=lambda r: r['weight_gbps'])
-  weights = sum(r['K'] * r['N'] * wb * r['launches_per_step'] for r in rows)
+  weights = sum(r['K'] * r['N'] * wb * r['launches_per_step'] for r in rows
+                if r['weight_gbps'])
   out = {
       'metric': f'passes over the decoder\'s dense layers per second, '
                 f'{args.config} at {R} rows on 1 GPU',

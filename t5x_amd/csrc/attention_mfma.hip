@@ -84,7 +84,7 @@ constexpr int kBlockJ = 128;  // positions per wavefront
 // accumulation and summation order as gemm_mfma_kernel, so q has the same
 // bits as the stand-alone dense layer given the same row statistics.  NJ is
 // the number of k-tile pairs per wavefront (d / 256, rounded up).
-template <int NQP, int WM, int NJ>
+template <int NQP, int WM, int NJ, bool ONCE = false>
 // fused, d <= 768: 2 workgroups per CU (256 registers hold both streams);
 // not fused: V is requested once the scores have consumed K, so a wavefront
 // needs under 128 registers and every workgroup of a launch of 64 x 16 or
@@ -189,9 +189,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
     if (16 * jt < nw) {
 #pragma unroll
       for (int c = 0; c < 2; ++c)
-        kb[jt][c].u = *reinterpret_cast<const uint4*>(
+        kb[jt][c].u = load_kv<ONCE>(reinterpret_cast<const uint4*>(
             kbase + ((size_t)c * a.S + min(jw + 16 * jt + n16, a.S - 1)) * 32 +
-            8 * g);
+            8 * g));
     } else {
       kb[jt][0].u = kb[jt][1].u = make_uint4(0, 0, 0, 0);
     }
@@ -202,9 +202,9 @@ cross_attn_mfma_kernel(AttnMfmaArgs a) {
       if (32 * jb < nw) {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
-          vb[jb][dt].u = *reinterpret_cast<const uint4*>(
+          vb[jb][dt].u = load_kv<ONCE>(reinterpret_cast<const uint4*>(
               vbase + ((size_t)(wave * (kBlockJ / 32) + jb) * kHeadDim +
-                       16 * dt + n16) * 32 + 8 * g);
+                       16 * dt + n16) * 32 + 8 * g));
       } else {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) vb[jb][dt].u = make_uint4(0, 0, 0, 0);
@@ -1129,12 +1129,29 @@ static void launch_cross(const AttnMfmaArgs& a, int B, hipStream_t s) {
                          a);
     return;
   }
-  if (waves <= 4)
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 0>), grid, block, 0, s, a);
-  else if (waves <= 8)
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 8, 0>), grid, block, 0, s, a);
-  else
-    hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 16, 0>), grid, block, 0, s, a);
+  // A launch whose keys and values outgrow what the memory-side cache could
+  // hand back to the next step reads them as streaming data (measured at
+  // 67 MB to 2.1 GB per launch: 2-6 % shorter launches, and the step's other
+  // kernels find more of their rows and code still cached); at 33 MB per
+  // launch (400 MB over the layers of T5.1.1-base) ordinary loads are faster.
+  const bool once =
+      (size_t)B * a.H * a.S * kHeadDim * 4 >= ((size_t)48 << 20);
+  if (waves <= 4) {
+    if (once)
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 0, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 4, 0>), grid, block, 0, s, a);
+  } else if (waves <= 8) {
+    if (once)
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 8, 0, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 8, 0>), grid, block, 0, s, a);
+  } else {
+    if (once)
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 16, 0, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((cross_attn_mfma_kernel<NQP, 16, 0>), grid, block, 0, s, a);
+  }
 }
 
 int launch_cross_attention_bf16(hipStream_t s, const void* q, const void* k,

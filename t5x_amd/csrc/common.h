@@ -51,6 +51,21 @@ __device__ __forceinline__ float round_bf16(float f) {
   return __uint_as_float(((uint32_t)f32_to_bf16(f)) << 16);
 }
 // Two values rounded and packed (lo in bits 0..15) by one instruction.
+// Loads of data that no later launch of the step finds cached anyway (cached
+// keys and values by the hundred megabytes): marked non-temporal so that they
+// do not push what is read again (code, kernel arguments, activation rows,
+// weights shared by the batch lanes) out of the caches.
+typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_once(const uint4* p) {
+  u32x4_v v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_v*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+template <bool ONCE>
+__device__ __forceinline__ uint4 load_kv(const uint4* p) {
+  if constexpr (ONCE) return load_once(p);
+  return *p;
+}
+
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   const f32x2_v v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_v));
