@@ -115,12 +115,18 @@ enc_attn_kernel(EncAttnArgs a) {
       kop.u = ol.to_operand(ka[c].u);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qb[c].v, acc, 0, 0, 0);
     }
+    // validity of the tile's 16 keys: from the prefix length alone, or one
+    // (broadcast) LDS word when the caller gave bits
+    const int left = n - 16 * kt;
+    const uint32_t tile_bits =
+        a.valid ? (s_valid[kt >> 1] >> ((kt & 1) * 16)) & 0xffffu
+                : (left >= 16 ? 0xffffu : (left <= 0 ? 0u : (1u << left) - 1u));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = 16 * kt + 4 * gq + i;
       float x = round_bf16(acc[i]);
       if (key < E) {
-        const bool ok = q_valid && is_valid(key);
+        const bool ok = q_valid && ((tile_bits >> (4 * gq + i)) & 1u) != 0;
         x = ok ? round_bf16(x + bias_row[key]) : kMasked;
       } else {
         x = -INFINITY;
