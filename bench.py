@@ -58,13 +58,18 @@ def parse_args():
   ap.add_argument('--lanes', type=int, default=None,
                   help='batch slices stepped concurrently (default: library)')
   ap.add_argument('--stage', default='decode',
-                  choices=['decode', 'encoder', 'dense'],
+                  choices=['decode', 'encoder', 'dense', 'memory'],
                   help="'encoder': the once-per-batch stage before the decode "
                        'loop (encoder forward + cross K/V projection); a step '
                        "is one batch.  'dense': the decoder's dense layers on "
                        'their own, each kind replayed over the layers (a step '
                        'is one pass over every dense layer of the decoder): '
-                       'weight streaming rate and matrix-core rate per kind')
+                       "weight streaming rate and matrix-core rate per kind.  "
+                       "'memory': what serves a buffer that one kernel wrote "
+                       'and the next reads (an XCD\'s own L2, the memory-side '
+                       'cache, HBM), for plain streaming kernels and for the '
+                       'logits between the vocabulary projection and the '
+                       'selection kernel')
   ap.add_argument('--in-flight', type=int, default=None,
                   help='also measure this many whole decodes of different '
                        'batches running on the device at once (default for '
@@ -826,6 +831,111 @@ def main_dense(args):
   print(json.dumps(out))
 
 
+def main_memory(args):
+  """Who serves data that one kernel wrote and the next kernel reads.  Every
+  case is `reps` rounds of (writer, [evictor,] reader) with HIP events around
+  the reader.
+  Plain kernels of known size (t5d_measure_fill / t5d_measure_read): the
+  reader takes each piece on the XCD that wrote it, on another XCD, or after
+  1.5 GB of other data has gone through the caches.  Then the pair this
+  question is about: the float32 logits written by the vocabulary projection
+  and read back by the selection kernel."""
+  import torch
+  from t5x_amd import _lib, network, ops
+  size, B, K, E, Emin, L, dtype, wdt, loop = CONFIGS[args.config]
+  dev = torch.device('cuda')
+  reps, blocks = 20, 1024
+  sink = torch.zeros(4, dtype=torch.int32, device=dev)
+  big_a = torch.zeros((768 << 20,), dtype=torch.uint8, device=dev)
+  big_b = torch.zeros_like(big_a)
+  evict = lambda: big_b.copy_(big_a)   # 768 MB read + 768 MB written
+
+  def reader_us(write, read, evicted):
+    """Median duration of `read` between two events on its stream.  A busy
+    kernel in front of every round lets the host enqueue the whole round
+    before the device reaches it, so no launch latency falls between the
+    events; what two events cost with nothing between them is taken off."""
+    def rounds(with_read):
+      ts = []
+      for _ in range(reps + 4):
+        torch.cuda._sleep(400000)
+        write()
+        if evicted:
+          evict()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        if with_read:
+          read()
+        e1.record()
+        ts.append((e0, e1))
+      torch.cuda.synchronize()
+      return float(np.median([a.elapsed_time(b) for a, b in ts[4:]])) * 1e3
+    return rounds(True) - rounds(False)
+
+  s = _lib.stream_handle
+  plain = []
+  for mb in (16.45, 65.8):
+    nbytes = int(mb * 1e6) // 16 * 16
+    buf = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    fill = lambda: _lib.call('t5d_measure_fill', s(), buf.data_ptr(), nbytes,
+                             1, blocks)
+    rd = lambda shift, tag: (lambda: _lib.call(
+        't5d_measure_read', s(), buf.data_ptr(), nbytes, shift, blocks,
+        sink.data_ptr(), tag))
+    row = {'bytes': nbytes}
+    for case, (name, shift, evicted) in enumerate((
+        ('same_xcd_us', 0, False), ('other_xcd_us', 3, False),
+        ('evicted_us', 3, True))):
+      # measure_read_kernel<tag> in a kernel trace: tag = 3 * size + case
+      us = reader_us(fill, rd(shift, 3 * len(plain) + case), evicted)
+      row[name] = round(us, 2)
+      row[name.replace('_us', '_gbps')] = round(nbytes / us / 1e3, 1)
+    plain.append(row)
+
+  cfg = network.t5_1_1_config(size, dtype=dtype, weight_dtype=wdt)
+  params = network.init_params(cfg, args.seed, dev, with_encoder=False)
+  module = network.Transformer(cfg, dev)
+  w = module.decoder_weights(params)
+  R, d, V = B * K, cfg.emb_dim, cfg.vocab_size
+  x = torch.randn((R, d), device=dev).to(torch.bfloat16)
+  logits = torch.empty((R, V), dtype=torch.float32, device=dev)
+  live = torch.zeros((B, K), dtype=torch.float32, device=dev)
+  k2 = 2 * K
+  bufs = (torch.empty((B, k2), dtype=torch.float32, device=dev),
+          torch.empty((B, k2), dtype=torch.int32, device=dev),
+          torch.empty((R,), dtype=torch.float32, device=dev),
+          torch.empty((R,), dtype=torch.float32, device=dev),
+          torch.empty((2 * R * k2,), dtype=torch.int32, device=dev))
+  project = lambda: ops.gemm(x, w.logits, norm_scale=w.ln_final,
+                             out_dtype=torch.float32, out=logits)
+  select = lambda: ops.beam_topk(logits, live, k2, bufs)
+  fresh = reader_us(project, select, False)
+  stale = reader_us(project, select, True)
+  out = {
+      'metric': 'read-back of data the previous kernel wrote, by what serves '
+                'it, on 1 GPU',
+      'value': plain[0]['other_xcd_gbps'], 'unit': 'GB/s', 'n_gpus': 1,
+      'steps': reps, 'warmup': 1, 'ms_per_step': plain[0]['other_xcd_us'] / 1e3,
+      'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+      'dtype': 'u8', 'data': 'synthetic',
+      'config': {'workload': 'plain 16-byte streaming reads of a buffer a '
+                             'plain kernel just wrote; logits [%d, %d] float32 '
+                             'between projection and selection' % (R, V),
+                 'stage': 'memory', 'plain': plain,
+                 'logits_bytes': R * V * 4,
+                 'selection_after_projection_us': round(fresh, 2),
+                 'selection_after_eviction_us': round(stale, 2)},
+      'roofline': {'kernel': 'measure_read_kernel (evicted: from HBM)',
+                   'bound': 'hbm', 'achieved': plain[1]['evicted_gbps'],
+                   'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                   'frac': round(plain[1]['evicted_gbps'] / HBM_PEAK_GBPS, 4),
+                   'traffic': None, 'bytes_per_launch': plain[1]['bytes'],
+                   'avg_launch_us': plain[1]['evicted_us']},
+  }
+  print(json.dumps(out))
+
+
 def host_threads():
   try:
     from threadpoolctl import threadpool_info
@@ -884,6 +994,8 @@ def main():
     return main_encoder(args)
   if args.stage == 'dense':
     return main_dense(args)
+  if args.stage == 'memory':
+    return main_memory(args)
   w = Workload(args.config, args.seed, args.lanes)
   if args.roofline_only:
     w.new_decode()  # builds the cross-attention K/V

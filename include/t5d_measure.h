@@ -23,6 +23,25 @@ enum {
  * is what the family costs where it runs, between the step's other kernels. */
 int t5d_measure_leave_out(int mask);
 
+/* Two plain streaming kernels of known size, for what the memory system
+ * gives a kernel that does nothing else (bench.py --stage memory; also the
+ * copy of known size that counter readings are calibrated on).  `bytes` is a
+ * multiple of 16; `blocks` workgroups of 256 threads walk the buffer with
+ * 16-byte accesses, workgroup b taking the pieces b, b + blocks, ...
+ *   t5d_measure_fill: writes the buffer.
+ *   t5d_measure_read: reads it; workgroup b takes the pieces that workgroup
+ *   (b + shift) % blocks of a fill or read with the same `blocks` took
+ *   (workgroups are dealt to the XCDs in turn, so a shift that is not a
+ *   multiple of 8 reads every piece through another XCD's L2 than wrote it).
+ *   `sink` (4 bytes of device memory) keeps the loads alive; `tag` (0..5)
+ *   picks one of six identical kernels, so that a kernel trace keeps the
+ *   launches of different measurements apart.
+ * Both return 0 or a negative T5D_E* code, like the boundary's calls. */
+int t5d_measure_fill(void* stream, void* buffer, long long bytes,
+                     unsigned seed, int blocks);
+int t5d_measure_read(void* stream, const void* buffer, long long bytes,
+                     int shift, int blocks, void* sink, int tag);
+
 #ifdef __cplusplus
 }
 #endif

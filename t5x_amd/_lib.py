@@ -8,7 +8,7 @@ needs a kernel raises.  Pointers are passed as plain integers
 import ctypes
 import os
 from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int32,
-                    c_int64, c_uint8, c_void_p)
+                    c_int64, c_uint, c_uint8, c_void_p)
 
 F32, BF16, I8 = 0, 1, 2
 EPI_NONE, EPI_RESIDUAL, EPI_GEGLU = 0, 1, 2
@@ -89,6 +89,8 @@ _SIGNATURES = {
     't5d_graph_destroy': (c_int, [_P]),
     't5d_version': (c_int, []),
     't5d_measure_leave_out': (c_int, [c_int]),
+    't5d_measure_fill': (c_int, [_P, _P, c_int64, c_uint, c_int]),
+    't5d_measure_read': (c_int, [_P, _P, c_int64, c_int, c_int, _P, c_int]),
     't5d_last_error': (c_char_p, []),
     't5d_packed_weight_bytes': (c_int64, [c_int, c_int, c_int]),
     't5d_pack_weight': (c_int, [_P, c_int, _P, _P, _P, c_int, c_int, c_int]),

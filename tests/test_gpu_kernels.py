@@ -1159,3 +1159,29 @@ def test_sample_tokens_topp_table(ops):
       for r in range(2):
         survived = int(host(tok)[r]) == j
         assert survived == (j in keep[r]), (p, r, j)
+
+
+def test_measurement_aids_fill_and_read(ops):
+  """t5d_measure_fill writes the documented pattern over exactly the buffer;
+  t5d_measure_read reads it (any shift) without touching it or the sink, and
+  both refuse sizes that are not a multiple of 16."""
+  from t5x_amd import _lib
+  n = 16 * 1000 + 16
+  buf = torch.full((n + 64,), 0x5a, dtype=torch.uint8, device='cuda')
+  sink = torch.zeros(4, dtype=torch.int32, device='cuda')
+  s = _lib.stream_handle()
+  _lib.call('t5d_measure_fill', s, buf.data_ptr(), n, 7, 3)
+  words = buf[:n].view(torch.int32).view(-1, 4).cpu().numpy()
+  np.testing.assert_array_equal(words[:, 0], 7 + np.arange(n // 16))
+  np.testing.assert_array_equal(words[:, 1:], np.tile([1, 2, 3], (n // 16, 1)))
+  assert bool((buf[n:] == 0x5a).all())
+  before = buf.clone()
+  for shift, tag in ((0, 0), (2, 5)):
+    _lib.call('t5d_measure_read', s, buf.data_ptr(), n, shift, 3,
+              sink.data_ptr(), tag)
+  torch.cuda.synchronize()
+  assert torch.equal(buf, before) and int(sink.abs().sum()) == 0
+  with pytest.raises(ValueError, match='t5d_measure_fill'):
+    _lib.call('t5d_measure_fill', s, buf.data_ptr(), n + 8, 7, 3)
+  with pytest.raises(ValueError, match='tag=6'):
+    _lib.call('t5d_measure_read', s, buf.data_ptr(), n, 0, 3, sink.data_ptr(), 6)
