@@ -25,7 +25,9 @@
 
 namespace t5d {
 
-template <int MP, int NT, typename WT>
+// NJ > 0: K is NJ * 256, every wavefront owns exactly NJ k-tile pairs and the K
+// loop is straight-line code (see gemm_big_kernel).
+template <int MP, int NT, typename WT, int NJ = 0>
 __global__ void __launch_bounds__(256)
 gemm_mfma_kernel(GemmArgs g) {
   constexpr int ACC = MP * NT;
@@ -74,7 +76,11 @@ gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
       for (int nn = 0; nn < NT; ++nn) {
         const int nt = nt0 + nn;
-        if (nt < n_tiles_total && kt + h < KT)
+        if (NJ > 0)  // every k-tile exists; tiles past the edge are never stored
+          bq[slot_][h][nn] = WeightTile<WT>::load(
+              wbase + ((size_t)min(nt, n_tiles_total - 1) * KT + kt + h) * TB,
+              lane);
+        else if (nt < n_tiles_total && kt + h < KT)
           bq[slot_][h][nn] = WeightTile<WT>::load(
               wbase + ((size_t)nt * KT + kt + h) * TB, lane);
         else
@@ -95,7 +101,10 @@ gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
       for (int mt = 0; mt < MP; ++mt) {
         const int row = m0 + mt * 16 + arow;
-        if (row < g.M && kt + h < KT)
+        if (NJ > 0)  // rows past the edge are never stored
+          aq[slot_][h][mt] = *reinterpret_cast<const uint4*>(
+              g.A + (size_t)min(row, g.M - 1) * g.K + (kt + h) * 32 + akoff);
+        else if (row < g.M && kt + h < KT)
           aq[slot_][h][mt] = *reinterpret_cast<const uint4*>(
               g.A + (size_t)row * g.K + (kt + h) * 32 + akoff);
         else
@@ -104,7 +113,7 @@ gemm_mfma_kernel(GemmArgs g) {
   };
 #pragma unroll
   for (int p = 0; p < PF; ++p)
-    if (p < nj) {
+    if (NJ > 0 ? p < NJ : p < nj) {
       load_b(p, p);
       if (p < APF) load_a(p, p);
     }
@@ -123,28 +132,42 @@ gemm_mfma_kernel(GemmArgs g) {
   }
   T5D_GATE_TEST();
 
-  for (int j0 = 0; j0 < nj; j0 += PF) {
+  auto consume = [&](int pb_, int pa_) {
+    Frag a[2][MP];
 #pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      const int j = j0 + p;
-      if (j < nj) {
-        Frag a[2][MP];
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+      for (int mt = 0; mt < MP; ++mt)
+        a[h][mt].u = ol.to_operand(aq[pa_][h][mt]);
 #pragma unroll
-          for (int mt = 0; mt < MP; ++mt)
-            a[h][mt].u = ol.to_operand(aq[p % APF][h][mt]);
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+      for (int mt = 0; mt < MP; ++mt)
 #pragma unroll
-          for (int mt = 0; mt < MP; ++mt)
+        for (int nn = 0; nn < NT; ++nn)
+          acc[mt * NT + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              a[h][mt].v, WeightTile<WT>::frag(bq[pb_][h][nn]).v,
+              acc[mt * NT + nn], 0, 0, 0);
+  };
+  if constexpr (NJ > 0) {
 #pragma unroll
-            for (int nn = 0; nn < NT; ++nn)
-              acc[mt * NT + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  a[h][mt].v, WeightTile<WT>::frag(bq[p][h][nn]).v,
-                  acc[mt * NT + nn], 0, 0, 0);
-        if (j + PF < nj) load_b(p, j + PF);
-        if (j + APF < nj) load_a(p % APF, j + APF);
+    for (int j = 0; j < NJ; ++j) {
+      __builtin_amdgcn_sched_barrier(0);
+      consume(j % PF, j % APF);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + PF < NJ) load_b(j % PF, j + PF);
+      if (j + APF < NJ) load_a(j % APF, j + APF);
+    }
+  } else {
+    for (int j0 = 0; j0 < nj; j0 += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) {
+        const int j = j0 + p;
+        if (j < nj) {
+          consume(p, p % APF);
+          if (j + PF < nj) load_b(p, j + PF);
+          if (j + APF < nj) load_a(p % APF, j + APF);
+        }
       }
     }
   }
@@ -919,6 +942,18 @@ static void launch_mfma(const GemmPlan& p, GemmArgs g, hipStream_t s) {
   g.m_parts = p.m_parts;
   const int groups8 = (p.n_groups + 7) / 8 * 8;
   dim3 grid(groups8 * p.m_parts), block(256);
+  // K loops of the benchmark models' layers that need refills, unrolled
+  const int nj = g.K % 256 == 0 ? g.K / 256 : 0;
+#define T5D_GEMM_NJ(MT, NT_, NJ_)                                           \
+  if (p.mp == MT && p.nt == NT_ && nj == NJ_) {                             \
+    hipLaunchKernelGGL((gemm_mfma_kernel<MT, NT_, WT, NJ_>), grid, block, 0, \
+                       s, g);                                               \
+    return;                                                                 \
+  }
+  T5D_GEMM_NJ(1, 1, 3) T5D_GEMM_NJ(1, 1, 4)
+  T5D_GEMM_NJ(1, 1, 8) T5D_GEMM_NJ(1, 1, 11) T5D_GEMM_NJ(1, 1, 20)
+  T5D_GEMM_NJ(1, 2, 8) T5D_GEMM_NJ(1, 4, 8)
+#undef T5D_GEMM_NJ
 #define T5D_GEMM_CASE(MT, NT_)                                              \
   if (p.mp == MT && p.nt == NT_) {                                          \
     hipLaunchKernelGGL((gemm_mfma_kernel<MT, NT_, WT>), grid, block, 0, s, g); \

@@ -24,7 +24,7 @@ namespace t5d {
 // epilogue, to partials[z][M][N]; the kernel that consumes the layer's output
 // (splitk_finish_kernel) adds the parts in ascending order.  No fences, no
 // atomics: the hand-over is the kernel boundary.
-template <int MP, int NT, typename WT>
+template <int MP, int NT, typename WT, int NJ = 0>
 __global__ void __launch_bounds__(256, 1)
 gemm_big_kernel(GemmArgs g, int k_parts, float* __restrict__ partials) {
   constexpr int ACC = MP * NT;
@@ -76,7 +76,11 @@ gemm_big_kernel(GemmArgs g, int k_parts, float* __restrict__ partials) {
 #pragma unroll
       for (int nn = 0; nn < NT; ++nn) {
         const int nt = nt0 + nn;
-        if (nt < n_tiles_total && kt + h < kt_hi)
+        if (NJ > 0)  // every k-tile exists; tiles past the edge are never stored
+          bq[slot_][h][nn] = WeightTile<WT>::load(
+              wbase + ((size_t)min(nt, n_tiles_total - 1) * KT + kt + h) * TB,
+              lane);
+        else if (nt < n_tiles_total && kt + h < kt_hi)
           bq[slot_][h][nn] = WeightTile<WT>::load(
               wbase + ((size_t)nt * KT + kt + h) * TB, lane);
         else
@@ -94,13 +98,56 @@ gemm_big_kernel(GemmArgs g, int k_parts, float* __restrict__ partials) {
 #pragma unroll
       for (int mt = 0; mt < MP; ++mt) {
         const int row = m0 + mt * 16 + arow;
-        if (row < g.M && kt + h < kt_hi)
+        if (NJ > 0)  // rows past the edge are never stored
+          aq[slot_][h][mt] = *reinterpret_cast<const uint4*>(
+              g.A + (size_t)min(row, g.M - 1) * g.K + (kt + h) * 32 + akoff);
+        else if (row < g.M && kt + h < kt_hi)
           aq[slot_][h][mt] = *reinterpret_cast<const uint4*>(
               g.A + (size_t)row * g.K + (kt + h) * 32 + akoff);
         else
           aq[slot_][h][mt] = make_uint4(0, 0, 0, 0);
       }
   };
+  auto consume = [&](int pb_, int pa_) {
+    Frag a[2][MP];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int mt = 0; mt < MP; ++mt)
+        a[h][mt].u = ol.to_operand(aq[pa_][h][mt]);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int nn = 0; nn < NT; ++nn) {
+        const Frag b = WeightTile<WT>::frag(bq[pb_][h][nn]);
+#pragma unroll
+        for (int mt = 0; mt < MP; ++mt)
+          acc[mt * NT + nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              a[h][mt].v, b.v, acc[mt * NT + nn], 0, 0, 0);
+      }
+  };
+  if constexpr (NJ > 0) {
+    // Every wavefront has exactly NJ pairs: the whole K loop as straight-line
+    // code, so the compiler counts the loads in flight exactly and waits for
+    // the oldest pair only (a loop drains the queue at its head every round).
+#pragma unroll
+    for (int p = 0; p < PF; ++p)
+      if (p < NJ) {
+        load_b(p, p);
+        if (p < APF) load_a(p, p);
+      }
+    T5D_GATE_TEST();
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      // (the fences keep the scheduler from sinking the refills down to their
+      // use, which would leave one pair in flight)
+      __builtin_amdgcn_sched_barrier(0);
+      consume(j % PF, j % APF);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + PF < NJ) load_b(j % PF, j + PF);
+      if (j + APF < NJ) load_a(j % APF, j + APF);
+    }
+  } else {
 #pragma unroll
   for (int p = 0; p < PF; ++p)
     if (p < nj) {
@@ -134,6 +181,7 @@ gemm_big_kernel(GemmArgs g, int k_parts, float* __restrict__ partials) {
         if (j + APF < nj) load_a(p % APF, j + APF);
       }
     }
+  }
   }
 
   // Cross-wavefront sums, CH tiles per round: (w0 + w2) + (w1 + w3).  Thread
@@ -274,6 +322,29 @@ void launch_gemm_big(int w_dtype, const GemmPlan& p, GemmArgs g,
   const int groups8 = (p.n_groups + 7) / 8 * 8;
   const int kp = partials ? p.k_parts : 1;
   dim3 grid(groups8 * p.m_parts * kp), block(256);
+  // Without a split and with K a multiple of 256 every wavefront has K / 256
+  // k-tile pairs: the K loops of the benchmark models' widths are unrolled.
+  const int nj = (kp == 1 && g.K % 256 == 0) ? g.K / 256 : 0;
+#define T5D_X(MP_, NT_)                                                        \
+  if (p.mp == MP_ && p.nt == NT_) {                                            \
+    if (w_dtype != T5D_I8 && nj == 16) {                                       \
+      hipLaunchKernelGGL((gemm_big_kernel<MP_, NT_, bf16_t, 16>), grid, block, \
+                         0, s, g, kp, partials);                               \
+      return;                                                                  \
+    }                                                                          \
+    if (w_dtype != T5D_I8 && nj == 40) {                                       \
+      hipLaunchKernelGGL((gemm_big_kernel<MP_, NT_, bf16_t, 40>), grid, block, \
+                         0, s, g, kp, partials);                               \
+      return;                                                                  \
+    }                                                                          \
+  }
+  T5D_BIG_TILES(T5D_X)
+#undef T5D_X
+  if (w_dtype == T5D_I8 && nj == 8 && p.mp == 4 && p.nt == 4) {
+    hipLaunchKernelGGL((gemm_big_kernel<4, 4, int8_t, 8>), grid, block, 0, s, g,
+                       kp, partials);
+    return;
+  }
 #define T5D_X(MP_, NT_)                                                        \
   if (p.mp == MP_ && p.nt == NT_) {                                            \
     if (w_dtype == T5D_I8)                                                     \
