@@ -898,12 +898,12 @@ static double big_cost(int M, int K, int N, int w_bytes, int mp, int nt,
 // to M, K, N, bytes per weight); the cost model covers everything else.
 struct TunedTile { int M, K, N, wb, mp, nt; };
 static const TunedTile kTunedTiles[] = {
-    {128, 4096, 4096, 2, 2, 4},    // XXL attention projections: 19 us
-    {128, 4096, 12288, 2, 4, 6},   // XXL q, k, v: 40 us
-    {128, 4096, 20480, 2, 8, 5},   // XXL MLP in: 67 us
-    {128, 10240, 4096, 2, 2, 4},   // XXL MLP out: 40 us
-    {128, 4096, 32128, 2, 8, 8},   // XXL vocabulary projection: 93 us
-    {64, 2048, 32128, 1, 4, 4},    // XL int8 vocabulary projection: 30 us
+    {128, 4096, 4096, 2, 2, 4},    // XXL attention projections: 18 us
+    {128, 4096, 12288, 2, 4, 6},   // XXL q, k, v: 33 us
+    {128, 4096, 20480, 2, 8, 5},   // XXL MLP in: 55 us
+    {128, 10240, 4096, 2, 2, 4},   // XXL MLP out: 36 us
+    {128, 4096, 32128, 2, 8, 8},   // XXL vocabulary projection: 65 us
+    {64, 2048, 32128, 1, 4, 4},    // XL int8 vocabulary projection: 24 us
 };
 
 // The plan never splits K by itself: at these shapes the split was measured
