@@ -93,7 +93,12 @@ gemm_mfma_kernel(GemmArgs g) {
   // the newest loads in flight, and since loads return in order, waiting for
   // them would drain the whole weight queue once per pair.
   // (at most 64 registers of them: fewer pairs ahead for tall tiles)
-  constexpr int APF = PF * MP <= 8 ? PF : (8 / MP > 0 ? 8 / MP : 1);
+  // (a divisor of PF: pair j then sits in slot j % APF in every round)
+  constexpr int APF_CAP = PF * MP <= 8 ? PF : (8 / MP > 0 ? 8 / MP : 1);
+  constexpr int APF = PF % APF_CAP == 0 ? APF_CAP
+                      : (PF % (APF_CAP - 1) == 0 ? APF_CAP - 1
+                         : (APF_CAP > 2 && PF % (APF_CAP - 2) == 0 ? APF_CAP - 2 : 1));
+  static_assert(PF % APF == 0, "activation ring out of phase with the weight ring");
   uint4 aq[APF][2][MP];
   auto load_a = [&](int slot_, int j) {
     const int kt = (wave + 4 * j) * 2;

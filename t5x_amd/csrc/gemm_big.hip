@@ -35,6 +35,7 @@ gemm_big_kernel(GemmArgs g, int k_parts, float* __restrict__ partials) {
   constexpr int PF = PF0 < 1 ? 1 : (PF0 > 4 ? 4 : PF0);
   constexpr int APF0 = 64 / (2 * MP * 4);
   constexpr int APF = APF0 < 1 ? 1 : (APF0 > PF ? PF : APF0);
+  static_assert(PF % APF == 0, "activation ring out of phase with the weight ring");
   __shared__ float red[4][CH * 4][64];
   T5D_GATE_READ(g.gate);
 

@@ -140,6 +140,66 @@ def test_gemm_large_tiles(ops, mp, nt, wdt):
                                rtol=2**-7)
 
 
+UNROLLED = ([(mp, nt, 4096, torch.bfloat16) for mp, nt in BIG_TILES] +
+            [(mp, nt, 10240, torch.bfloat16) for mp, nt in ((2, 4), (4, 6))] +
+            [(4, 4, 2048, torch.int8)])
+
+
+@pytest.mark.parametrize('mp,nt,K,wdt', UNROLLED)
+def test_gemm_large_tiles_with_the_k_loop_unrolled(ops, mp, nt, K, wdt):
+  """The large-tile kernels whose K loop is straight-line code (K = 4096,
+  10240; int8: 2048) with rows and columns that do not fill the last tile
+  (their loads past the matrix edge are clamped, not skipped): bit for bit
+  against t5d_gemm on its small tiles, which loops, and against the oracle."""
+  rs = np.random.RandomState(mp * 10 + nt + K)
+  M, N = 100, 16 * (2 * nt + 1)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+  k0 = ot5.quantize_int8(w0) if wdt == torch.int8 else w0
+  pw = ops.pack_weight(dev(w0), torch.bfloat16, wdt)
+  pg = ops.pack_weight(dev(w0), torch.bfloat16, wdt, gate_kernel=dev(w1))
+  want = ot5.bf16_round(ot5.dense_general(host(a), k0, 'bfloat16') + host(res))
+  got = ops.gemm_tiled(a, pw, mp, nt, residual=res)
+  np.testing.assert_allclose(host(got), want, atol=2e-2, rtol=2**-7)
+  assert torch.equal(got, ops.gemm(a, pw, residual=res))
+  assert torch.equal(ops.gemm_tiled(a, pg, mp, nt), ops.gemm(a, pg))
+  f32 = ops.gemm_tiled(a, pw, mp, nt, out_dtype=torch.float32)
+  assert torch.equal(f32, ops.gemm(a, pw, out_dtype=torch.float32))
+
+
+@pytest.mark.parametrize('M,K,N,wdt', [
+    (20, 768, 784, torch.bfloat16), (100, 1024, 1040, torch.bfloat16),
+    (50, 2048, 784, torch.bfloat16), (33, 2816, 1040, torch.bfloat16),
+    (64, 1024, 12304, torch.bfloat16),  # 4 x 2 tiles, 4 pairs, ring of 3
+    (50, 2048, 2064, torch.int8), (50, 2048, 6160, torch.int8),
+    (64, 2048, 10256, torch.int8), (50, 5120, 2064, torch.int8)])
+def test_gemm_small_tiles_with_the_k_loop_unrolled(ops, M, K, N, wdt):
+  """The small-tile kernels whose K loop is straight-line code (K = 768,
+  1024, 2048, 2816, 5120), with ragged rows and a last column group that is
+  not full, against the oracle and, bit for bit, against the same layer with
+  one more k-tile pair of zeros appended to K (which takes the looping
+  kernel: same products in the same order, plus zeros).  Two of the shapes
+  take tiles whose ring of weight tiles is deeper than their ring of
+  activation rows and have more k-tile pairs than either (bfloat16 4 x 2 at
+  K = 1024, int8 2 x 2 at K = 2048)."""
+  rs = np.random.RandomState(M + K + N)
+  a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+  w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+  res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+  k0 = ot5.quantize_int8(w0) if wdt == torch.int8 else w0
+  pw = ops.pack_weight(dev(w0), torch.bfloat16, wdt)
+  want = ot5.bf16_round(ot5.dense_general(host(a), k0, 'bfloat16') + host(res))
+  got = ops.gemm(a, pw, residual=res)
+  np.testing.assert_allclose(host(got), want, atol=2e-2, rtol=2**-7)
+  if wdt == torch.bfloat16:
+    a_pad = torch.cat([a, torch.zeros((M, 64), dtype=a.dtype, device=a.device)], 1)
+    w_pad = np.concatenate([w0, np.zeros((64, N), np.float32)], 0)
+    pw_pad = ops.pack_weight(dev(w_pad), torch.bfloat16, wdt)
+    assert torch.equal(got, ops.gemm(a_pad.contiguous(), pw_pad, residual=res))
+
+
 def test_gemm_tiled_rejects_what_it_cannot_run(ops):
   a = dev(np.zeros((16, 64), np.float32), torch.bfloat16)
   pw = ops.pack_weight(dev(np.zeros((64, 64), np.float32)), torch.bfloat16)
