@@ -1245,3 +1245,71 @@ def test_measurement_aids_fill_and_read(ops):
     _lib.call('t5d_measure_fill', s, buf.data_ptr(), n + 8, 7, 3)
   with pytest.raises(ValueError, match='tag=6'):
     _lib.call('t5d_measure_read', s, buf.data_ptr(), n, 0, 3, sink.data_ptr(), 6)
+
+
+def test_gemm_random_shapes_every_tile_choice(ops):
+  """t5d_gemm over 80 random shapes (rows 1..128, K a multiple of 32 up to
+  4096, N a multiple of 16 up to 12288, bfloat16 and int8 weights, with and
+  without a residual): whatever tile the planner picks, the result is the
+  dense layer's (float32 products of the same operands on the device as the
+  yardstick, tolerance 2e-2 + 2^-7 relative)."""
+  rs = np.random.RandomState(2024)
+  for case in range(80):
+    M = int(rs.choice([1, 5, 16, 20, 32, 48, 50, 64, 96, 100, 128]))
+    K = 32 * int(rs.randint(1, 129))
+    N = 16 * int(rs.randint(1, 769))
+    if K * N > 20e6:
+      N = max(16, int(20e6 // K) // 16 * 16)
+    int8 = bool(rs.randint(0, 2))
+    with_res = bool(rs.randint(0, 2))
+    a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+    w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16) if with_res else None
+    if int8:
+      q = ot5.quantize_int8(w0)
+      w_ref = dev(q['q'].astype(np.float32)) * dev(q['scale'].astype(np.float32))
+      pw = ops.pack_weight(dev(w0), torch.bfloat16, torch.int8)
+    else:
+      w_ref = dev(w0).to(torch.bfloat16).float()
+      pw = ops.pack_weight(dev(w0), torch.bfloat16)
+    want = (a.float() @ w_ref).to(torch.bfloat16).float()
+    if with_res:
+      want = (want + res.float()).to(torch.bfloat16).float()
+    got = ops.gemm(a, pw, residual=res).float()
+    err = (got - want).abs()
+    ok = err <= 2e-2 + 2.0**-7 * want.abs()
+    assert bool(ok.all()), (case, M, K, N, int8, with_res, float(err.max()),
+                            float((~ok).float().mean()))
+
+
+def test_norm_gemm_random_shapes(ops):
+  """t5d_norm_gemm (layer norm + dense in one kernel) over 60 random shapes
+  (K a multiple of 64 up to 2048, N a multiple of 16, bfloat16 and int8
+  weights, plain and gated-GELU epilogues, bfloat16 and float32 results)
+  against the two-kernel sequence t5d_rmsnorm -> t5d_gemm, whose pieces are
+  tested against the oracle: same roundings, so within one bfloat16 flip of
+  the sums."""
+  rs = np.random.RandomState(77)
+  for case in range(60):
+    M = int(rs.choice([1, 7, 16, 33, 64, 100, 128]))
+    K = 64 * int(rs.randint(1, 33))
+    N = 16 * int(rs.randint(1, 400))
+    int8 = bool(rs.randint(0, 2))
+    geglu = bool(rs.randint(0, 2))
+    f32_out = (not geglu) and bool(rs.randint(0, 2))
+    wdt = torch.int8 if int8 else torch.bfloat16
+    a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+    scale = dev((1.0 + 0.1 * rs.randn(K)).astype(np.float32), torch.bfloat16)
+    w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    gate = dev((rs.randn(K, N) / np.sqrt(K)).astype(np.float32)) if geglu else None
+    pw = ops.pack_weight(dev(w0), torch.bfloat16, wdt, gate_kernel=gate)
+    od = torch.float32 if f32_out else torch.bfloat16
+    got = ops.gemm(a, pw, norm_scale=scale, out_dtype=od).float()
+    want = ops.gemm(ops.rmsnorm(a, scale), pw, out_dtype=od).float()
+    err = (got - want).abs()
+    ok = err <= 2e-2 + 2.0**-6 * want.abs()
+    assert bool(ok.all()), (case, M, K, N, int8, geglu, f32_out,
+                            float(err.max()), float((~ok).float().mean()))
+    # the row statistics are summed in another order than the norm kernel's:
+    # a rare 1-ulp flip of a normalised value, nothing systematic
+    assert float((err > 0).float().mean()) < 0.2, (case, M, K, N)
