@@ -82,6 +82,93 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
 constexpr int kRowsBM = 256, kRowsBN = 128;  // workgroup tile
 constexpr int kRowsMT = 8, kRowsNT = 4;        // MFMA tiles per wavefront
 
+// What a wavefront does with its finished 8 x 4 accumulator tiles (m0: its
+// first row, nt0: its first 16-column tile).
+template <bool SWAP, int NT>
+__device__ __forceinline__ void rows_epilogue(
+    const RowsGemmArgs& g, const f32x4_r (&acc)[kRowsMT][NT], int m0,
+    int nt0, int n_tiles, int l16, int gq) {
+  constexpr int MT = kRowsMT;
+  if (SWAP) {
+    // acc[mt][nt][i]: row m = m0 + 16 mt + l16, column n = 16 (nt0 + nt) + 4 gq + i
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = m0 + 16 * mt + l16;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        if (nt0 + nt >= n_tiles) continue;
+        const int n = 16 * (nt0 + nt) + 4 * gq;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][i];
+        if (g.scales) {
+          const float4 sc = *reinterpret_cast<const float4*>(g.scales + n);
+          v[0] *= sc.x; v[1] *= sc.y; v[2] *= sc.z; v[3] *= sc.w;
+        }
+        if (g.epilogue == T5D_EPI_GEGLU) {
+          // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the
+          // lanes with gq >= 2 hold the gates of the lanes with gq - 2.
+          float gate[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) gate[i] = __shfl_xor(v[i], 32, 64);
+          if (gq < 2 && m < g.M) {
+            float h[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              h[i] = round_bf16(round_bf16(gelu_tanh(round_bf16(v[i]))) *
+                                round_bf16(gate[i]));
+            const int F = g.N >> 1;
+            *reinterpret_cast<uint2*>(g.C + (size_t)m * F + 8 * (nt0 + nt) +
+                                      4 * gq) = pack4(h[0], h[1], h[2], h[3]);
+          }
+          continue;
+        }
+        if (m >= g.M) continue;
+        size_t o;
+        if (g.layout == T5D_OUT_HEADS_KEY) {
+          // [B, H, 2, Ep, 32]: the two 32-wide halves of the head dim as planes
+          const int b = m / g.E, e = m - b * g.E;
+          const int hh = n >> 6, c = (n >> 5) & 1, j = n & 31;
+          o = ((((size_t)b * g.H + hh) * 2 + c) * g.Ep + e) * 32 + j;
+        } else {
+          o = (size_t)m * g.N + n;
+        }
+        if (g.epilogue == T5D_EPI_RESIDUAL) {
+          const uint2 r = *reinterpret_cast<const uint2*>(
+              g.residual + (size_t)m * g.N + n);
+          v[0] = round_bf16(v[0]) + bf16lo_to_f32(r.x);
+          v[1] = round_bf16(v[1]) + bf16hi_to_f32(r.x);
+          v[2] = round_bf16(v[2]) + bf16lo_to_f32(r.y);
+          v[3] = round_bf16(v[3]) + bf16hi_to_f32(r.y);
+        }
+        *reinterpret_cast<uint2*>(g.C + o) = pack4(v[0], v[1], v[2], v[3]);
+      }
+    }
+  } else {
+    // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
+    // (values layout [B, H, Ep / 32, 64, 32]: 4 consecutive positions per store)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = m0 + 16 * mt + 4 * gq;
+      if (m >= g.M) continue;
+      const int b = m / g.E, e = m - b * g.E;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        if (nt0 + nt >= n_tiles) continue;
+        const int n = 16 * (nt0 + nt) + l16;
+        float s = g.scales ? g.scales[n] : 1.f;
+        const int hh = n >> 6, d = n & 63;
+        const size_t o =
+            ((((size_t)b * g.H + hh) * (g.Ep >> 5) + (e >> 5)) * 64 + d) * 32 +
+            (e & 31);
+        *reinterpret_cast<uint2*>(g.C + o) =
+            pack4(acc[mt][nt][0] * s, acc[mt][nt][1] * s, acc[mt][nt][2] * s,
+                  acc[mt][nt][3] * s);
+      }
+    }
+  }
+}
+
 // SWAP: weights are the MFMA A operand (C^T is formed).
 template <typename WT, bool SWAP>
 __global__ void __launch_bounds__(256, 2)
@@ -183,85 +270,151 @@ rows_gemm_kernel(RowsGemmArgs g) {
 #undef T5D_ROWS_FETCH
 #undef T5D_ROWS_PARK
 
-  // ---- epilogue ---------------------------------------------------------------
-  if (SWAP) {
-    // acc[mt][nt][i]: row m = m0 + 16 mt + l16, column n = 16 (nt0 + nt) + 4 gq + i
+  rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+}
+
+// ---- the same tile with operands loaded straight into LDS ---------------------
+// rows_gemm_kernel keeps one k-tile of loads in flight per workgroup (staging
+// registers), which covers a fifth of the memory latency; the matrix cores
+// wait for the rest.  Here the 24 operand tiles of a k-tile go from memory
+// into LDS without passing through registers (global_load_lds, 16 bytes per
+// lane, lane l of an instruction landing at byte 16 l of the destination), in
+// a ring of three stages, so two k-tiles are in flight while one is
+// multiplied.  One barrier per k-tile, placed by hand together with the wait
+// for "all but my newest six loads": the stages are three separate arrays and
+// the K loop handles three k-tiles per round, so that the compiler can tell a
+// read of one stage from a load into another and adds no wait of its own.
+// An activation tile is fetched with lane 4 q + j reading row q, piece
+// (j + q / 4) % 4 — four neighbouring lanes still read 64 contiguous bytes —
+// which puts piece p of row r at slot 4 r + (p - r / 4) % 4: the 16 lanes of
+// a quarter wavefront then read 16 slots that differ mod 16, i.e. without
+// bank conflicts.  bfloat16 weights (int8 tiles must be widened on the way).
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* glb_ptr_t;
+
+// Measured on the gated MLP input projection of the T5.1.1-base encoder
+// (16384 x 768 x 4096): 182 -> 176 us per launch.  NT (16-column tiles per
+// wavefront) = 8, i.e. a 256 x 256 workgroup tile with one workgroup per CU
+// and the accumulators in the accumulation registers, halves the bytes per
+// flop that a CU takes in but lasts 257 us: with one wavefront per SIMD
+// nothing covers the operand reads from LDS.
+template <bool SWAP, int NT>
+__global__ void __launch_bounds__(256, 2)
+rows_gemm_direct_kernel(RowsGemmArgs g) {
+  constexpr int MT = kRowsMT;
+  constexpr int BN = 2 * NT * 16;       // columns of the workgroup tile
+  constexpr int WL = NT / 2;            // weight tiles a wavefront loads per stage
+  constexpr int TILES = 16 + 2 * NT;
+  // all but my newest 4 + WL loads have landed: s_waitcnt vmcnt(4 + WL)
+  constexpr int kWaitStage = 0xF70 | (4 + WL);
+  // [tile][lane]: tiles 0..15 activations (rows 16 t ..), then the weights
+  __shared__ uint4 s_t0[TILES][64];
+  __shared__ uint4 s_t1[TILES][64];
+  __shared__ uint4 s_t2[TILES][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, gq = lane >> 4;
+  const int m_blocks = (g.M + kRowsBM - 1) / kRowsBM;
+  const int m_blk = blockIdx.x % m_blocks, n_blk = blockIdx.x / m_blocks;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = m_blk * kRowsBM + wm * (16 * MT);
+  const int nt0 = n_blk * (BN / 16) + wn * NT;
+  const int KT = g.K >> 5, n_tiles = g.N >> 4;
+
+  const int ld_row = lane >> 2;
+  const int ld_piece = ((lane & 3) + (ld_row >> 2)) & 3;
+  const int read_slot = 4 * l16 + ((gq - (l16 >> 2)) & 3);
+  // this wavefront's tiles of every stage: activation tiles wave + 4 i,
+  // weight tiles wave + 4 i (rows / tiles past the edge clamped: their
+  // products are discarded in the epilogue)
+  const char* arow[4];
+  const char* wtile[WL];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = m0 + 16 * mt + l16;
+  for (int i = 0; i < 4; ++i)
+    arow[i] = reinterpret_cast<const char*>(
+        g.A +
+        (size_t)min(m_blk * kRowsBM + 16 * (wave + 4 * i) + ld_row, g.M - 1) *
+            g.K + 8 * ld_piece);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        if (nt0 + nt >= n_tiles) continue;
-        const int n = 16 * (nt0 + nt) + 4 * gq;
-        float v[4];
+  for (int i = 0; i < WL; ++i)
+    wtile[i] = g.W + (size_t)min(n_blk * (BN / 16) + wave + 4 * i,
+                                 n_tiles - 1) * KT * 1024 + lane * 16;
+
+  f32x4_r acc[MT][NT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][i];
-        if (g.scales) {
-          const float4 sc = *reinterpret_cast<const float4*>(g.scales + n);
-          v[0] *= sc.x; v[1] *= sc.y; v[2] *= sc.z; v[3] *= sc.w;
-        }
-        if (g.epilogue == T5D_EPI_GEGLU) {
-          // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the
-          // lanes with gq >= 2 hold the gates of the lanes with gq - 2.
-          float gate[4];
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) gate[i] = __shfl_xor(v[i], 32, 64);
-          if (gq < 2 && m < g.M) {
-            float h[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              h[i] = round_bf16(round_bf16(gelu_tanh(round_bf16(v[i]))) *
-                                round_bf16(gate[i]));
-            const int F = g.N >> 1;
-            *reinterpret_cast<uint2*>(g.C + (size_t)m * F + 8 * (nt0 + nt) +
-                                      4 * gq) = pack4(h[0], h[1], h[2], h[3]);
-          }
-          continue;
-        }
-        if (m >= g.M) continue;
-        size_t o;
-        if (g.layout == T5D_OUT_HEADS_KEY) {
-          // [B, H, 2, Ep, 32]: the two 32-wide halves of the head dim as planes
-          const int b = m / g.E, e = m - b * g.E;
-          const int hh = n >> 6, c = (n >> 5) & 1, j = n & 31;
-          o = ((((size_t)b * g.H + hh) * 2 + c) * g.Ep + e) * 32 + j;
-        } else {
-          o = (size_t)m * g.N + n;
-        }
-        if (g.epilogue == T5D_EPI_RESIDUAL) {
-          const uint2 r = *reinterpret_cast<const uint2*>(
-              g.residual + (size_t)m * g.N + n);
-          v[0] = round_bf16(v[0]) + bf16lo_to_f32(r.x);
-          v[1] = round_bf16(v[1]) + bf16hi_to_f32(r.x);
-          v[2] = round_bf16(v[2]) + bf16lo_to_f32(r.y);
-          v[3] = round_bf16(v[3]) + bf16hi_to_f32(r.y);
-        }
-        *reinterpret_cast<uint2*>(g.C + o) = pack4(v[0], v[1], v[2], v[3]);
-      }
-    }
-  } else {
-    // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
-    // (values layout [B, H, Ep / 32, 64, 32]: 4 consecutive positions per store)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = m0 + 16 * mt + 4 * gq;
-      if (m >= g.M) continue;
-      const int b = m / g.E, e = m - b * g.E;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        if (nt0 + nt >= n_tiles) continue;
-        const int n = 16 * (nt0 + nt) + l16;
-        float s = g.scales ? g.scales[n] : 1.f;
-        const int hh = n >> 6, d = n & 63;
-        const size_t o =
-            ((((size_t)b * g.H + hh) * (g.Ep >> 5) + (e >> 5)) * 64 + d) * 32 +
-            (e & 31);
-        *reinterpret_cast<uint2*>(g.C + o) =
-            pack4(acc[mt][nt][0] * s, acc[mt][nt][1] * s, acc[mt][nt][2] * s,
-                  acc[mt][nt][3] * s);
-      }
-    }
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = (f32x4_r){0.f, 0.f, 0.f, 0.f};
+
+#define T5D_ROWS_ISSUE(kt_, S_)                                                \
+  do {                                                                         \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                              \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(arow[i] + 64 * (kt_)),      \
+                                       (lds_ptr_t)&S_[wave + 4 * i][0], 16, 0, \
+                                       0);                                     \
+    _Pragma("unroll") for (int i = 0; i < WL; ++i)                             \
+      __builtin_amdgcn_global_load_lds(                                        \
+          (glb_ptr_t)(wtile[i] + (size_t)(kt_) * 1024),                        \
+          (lds_ptr_t)&S_[16 + wave + 4 * i][0], 16, 0, 0);                     \
+  } while (0)
+#define T5D_ROWS_MULTIPLY(S_)                                                  \
+  do {                                                                         \
+    FragR wb[NT];                                                              \
+    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                          \
+      wb[nt].u = S_[16 + wn * NT + nt][lane];                                  \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                        \
+      FragR xa;                                                                \
+      xa.u = S_[wm * MT + mt][read_slot];                                      \
+      _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                      \
+        if (SWAP)                                                              \
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(               \
+              wb[nt].v, xa.v, acc[mt][nt], 0, 0, 0);                           \
+        else                                                                   \
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(               \
+              xa.v, wb[nt].v, acc[mt][nt], 0, 0, 0);                           \
+      }                                                                        \
+    }                                                                          \
+  } while (0)
+  // s_waitcnt vmcnt(4 + WL): all but this wavefront's newest loads have landed,
+  // i.e. its share of the stage about to be multiplied; after the barrier
+  // every wavefront's share has, and every wavefront is done with the stage
+  // that the next loads overwrite.
+#define T5D_ROWS_STEP(kt_, CUR_, NEXT2_)                                       \
+  do {                                                                         \
+    __builtin_amdgcn_s_waitcnt(kWaitStage);                                    \
+    __builtin_amdgcn_s_barrier();                                              \
+    T5D_ROWS_ISSUE((kt_) + 2, NEXT2_);                                         \
+    __builtin_amdgcn_sched_barrier(0);                                         \
+    T5D_ROWS_MULTIPLY(CUR_);                                                   \
+  } while (0)
+#define T5D_ROWS_LAST(kt_, CUR_, NEXT2_)                                       \
+  do {                                                                         \
+    if ((kt_) + 1 < KT) __builtin_amdgcn_s_waitcnt(kWaitStage);                \
+    else __builtin_amdgcn_s_waitcnt(0xF70);                                    \
+    __builtin_amdgcn_s_barrier();                                              \
+    if ((kt_) + 2 < KT) T5D_ROWS_ISSUE((kt_) + 2, NEXT2_);                     \
+    __builtin_amdgcn_sched_barrier(0);                                         \
+    T5D_ROWS_MULTIPLY(CUR_);                                                   \
+  } while (0)
+  T5D_ROWS_ISSUE(0, s_t0);
+  T5D_ROWS_ISSUE(1, s_t1);  // KT >= 2 (checked by the caller)
+  const int n_main = (KT - 2) / 3 * 3;
+  int kt = 0;
+  for (; kt < n_main; kt += 3) {
+    T5D_ROWS_STEP(kt, s_t0, s_t2);
+    T5D_ROWS_STEP(kt + 1, s_t1, s_t0);
+    T5D_ROWS_STEP(kt + 2, s_t2, s_t1);
   }
+  // the last 2 to 4 k-tiles
+  T5D_ROWS_LAST(kt, s_t0, s_t2);
+  T5D_ROWS_LAST(kt + 1, s_t1, s_t0);
+  if (kt + 2 < KT) T5D_ROWS_LAST(kt + 2, s_t2, s_t1);
+  if (kt + 3 < KT) T5D_ROWS_LAST(kt + 3, s_t0, s_t2);
+#undef T5D_ROWS_ISSUE
+#undef T5D_ROWS_MULTIPLY
+#undef T5D_ROWS_STEP
+#undef T5D_ROWS_LAST
+  rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
 }
 
 }  // namespace t5d
@@ -313,7 +466,14 @@ extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
   dim3 grid((unsigned)m_blocks * n_blocks), block(256);
   hipStream_t s = as_stream(stream);
   const bool swap = out_layout != T5D_OUT_HEADS_VALUE;
-  if (w_dtype == T5D_BF16) {
+  if (w_dtype == T5D_BF16 && K >= 64) {
+    if (swap)
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<true, kRowsNT>), grid, block,
+                         0, s, g);
+    else
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<false, kRowsNT>), grid, block,
+                         0, s, g);
+  } else if (w_dtype == T5D_BF16) {
     if (swap)
       hipLaunchKernelGGL((rows_gemm_kernel<bf16_t, true>), grid, block, 0, s, g);
     else
