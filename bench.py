@@ -452,8 +452,10 @@ def roofline_cross_attention(w, reps_per_layer=4, in_loop=True):
   nbytes = w.cross_attention_bytes()
   if fused:
     name = 'cross_attn_mfma_kernel<4,4,%d>' % ((cfg.emb_dim // 64 + 3) // 4)
-  else:
+  elif w.bf16:
     name = 'cross_attn_mfma_kernel (query projected separately)'
+  else:
+    name = 'cross_attn_f32_kernel (float32 on the vector ALUs)'
   out = {'kernel': name, 'bound': 'hbm', 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
          'traffic': measured_traffic(w.name), 'bytes_per_launch': nbytes,
          # moved by the same launch for the dense layers' account (layer norm
