@@ -447,3 +447,34 @@ def test_cross_kv_projection_layouts_match_oracle():
     np.testing.assert_allclose(pv[..., :E].transpose(0, 3, 1, 2), wv,
                                atol=2e-2, rtol=2**-7)
     assert not pk[:, :, E:].any() and not pv[..., E:].any()
+
+
+def test_gemm_rows_random_shapes_and_repeated_launches(ops):
+  """t5d_gemm_rows over 30 random shapes (rows 1..3000, K a multiple of 32
+  from 64 to 4096, i.e. 2 to 128 rounds of its ring of LDS stages, N a
+  multiple of 16 up to 4096, with and without a residual) against float32
+  products of the same operands on the device, and launched three times:
+  the three results are bit-identical (a stage overwritten or read too early
+  would differ from launch to launch)."""
+  rs = np.random.RandomState(31)
+  for case in range(30):
+    M = int(rs.choice([1, 17, 255, 256, 257, 700, 1024, 3000]))
+    K = 32 * int(rs.randint(2, 129))
+    N = 16 * int(rs.randint(1, 257))
+    with_res = bool(rs.randint(0, 2))
+    a = dev(rs.randn(M, K).astype(np.float32), torch.bfloat16)
+    w0 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
+    pw = ops.pack_weight(dev(w0), torch.bfloat16)
+    res = (dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
+           if with_res else None)
+    want = (a.float() @ dev(w0).to(torch.bfloat16).float()).to(
+        torch.bfloat16).float()
+    if with_res:
+      want = (want + res.float()).to(torch.bfloat16).float()
+    outs = [ops.gemm_rows(a, pw, residual=res) for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (
+        case, M, K, N)
+    err = (outs[0].float() - want).abs()
+    ok = err <= 2e-2 + 2.0**-7 * want.abs()
+    assert bool(ok.all()), (case, M, K, N, with_res, float(err.max()))
