@@ -54,6 +54,14 @@ def parse_args():
   ap.add_argument('--warmup', type=int, default=128)
   ap.add_argument('--config', default=DEFAULT_CONFIG, choices=sorted(CONFIGS))
   ap.add_argument('--seed', type=int, default=0)
+  ap.add_argument('--hw-queues', type=int, default=8,
+                  help='hardware queues of this process (GPU_MAX_HW_QUEUES, '
+                       'which the HIP runtime reads when it starts; its own '
+                       'default is 4, of which one serves the default stream). '
+                       'With 8, four decodes run side by side instead of '
+                       'three: what `in_flight` measures; `value`, the single '
+                       'batch on two lanes, is the same either way.  0: leave '
+                       'the environment as it is')
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--lanes', type=int, default=None,
                   help='batch slices stepped concurrently (default: library)')
@@ -988,6 +996,8 @@ def main():
           'exchange: each GPU would run this program on its share of the '
           'batch.', file=sys.stderr)
     sys.exit(2)
+  if args.hw_queues > 0:  # before anything touches the GPU
+    os.environ['GPU_MAX_HW_QUEUES'] = str(args.hw_queues)
   import torch
   if not torch.cuda.is_available():
     print('bench.py: no GPU visible', file=sys.stderr)
@@ -1039,6 +1049,7 @@ def main():
                  # decode streams the device was found (or told) to run side
                  # by side: decides the lanes above and the batches in flight
                  'streams_side_by_side': w.module.streams_side_by_side(),
+                 'gpu_max_hw_queues': os.environ.get('GPU_MAX_HW_QUEUES'),
                  # positions t of the decode the timed iterations covered:
                  # whole decodes, then a window centred on (L-1)/2
                  't_first': windows[-1][0], 't_last': windows[-1][1],
