@@ -744,6 +744,27 @@ _TAIL_CASES = [
 ]
 
 
+def _random_tail_cases(n, seed):
+  """More of the same with random sizes: every workgroup size the launch can
+  pick (4, 2 or 1 units), beam counts that are not powers of two, cache
+  lengths on both sides of the chunk boundary."""
+  rs = np.random.RandomState(seed)
+  out = []
+  for _ in range(n):
+    beams = int(rs.choice([1, 1, 2, 3, 4, 5, 8]))
+    B = int(rs.randint(1, 41 if beams <= 4 else 9))
+    H = int(rs.randint(1, 13))
+    L = int(rs.choice([32, 64, 96, 128, 160, 256]))
+    steps = int(rs.randint(3, 11))
+    t0 = int(rs.randint(0, L - steps + 1))
+    in_place = bool(beams > 1 and L <= 128 and rs.randint(0, 3) == 0)
+    out.append((B, beams, H, L, t0, steps, in_place))
+  return out
+
+
+_TAIL_CASES += _random_tail_cases(12, 7)
+
+
 @pytest.mark.parametrize('B,beams,H,L,t0,steps,in_place', [
     c if len(c) == 7 else c + (False,) for c in _TAIL_CASES])
 def test_self_attention_steps_in_the_decode_loop_layout(ops, B, beams, H, L, t0,
@@ -1313,3 +1334,42 @@ def test_norm_gemm_random_shapes(ops):
     # the row statistics are summed in another order than the norm kernel's:
     # a rare 1-ulp flip of a normalised value, nothing systematic
     assert float((err > 0).float().mean()) < 0.2, (case, M, K, N)
+
+
+def test_cross_attention_random_shapes(ops):
+  """t5d_cross_attention_step (bfloat16) over 40 random shapes — batch 1..48,
+  1 / 2 / 4 / 8 beams, 1..16 heads, encoder length a multiple of 32 up to
+  1024 with ragged valid lengths (1 included), small and large enough for
+  the kernel's streaming-load variant — against float32 softmax attention of
+  the same operands on the device."""
+  rs = np.random.RandomState(99)
+  bf = torch.bfloat16
+  for case in range(40):
+    B = int(rs.randint(1, 49))
+    beams = int(rs.choice([1, 2, 4, 8]))
+    H = int(rs.randint(1, 17))
+    E = 32 * int(rs.randint(1, 33))
+    if case % 8 == 0:   # 48 MB of keys and values and more per launch
+      B, H, E = 48, 16, 32 * int(rs.randint(8, 33))
+    lens = rs.randint(1, E + 1, size=(B,)).astype(np.int32)
+    lens[rs.randint(0, B)] = E
+    lens[rs.randint(0, B)] = 1
+    gen = torch.Generator(device='cuda')
+    gen.manual_seed(case)
+    k = (0.5 * torch.randn((B, H, E, 64), generator=gen, device='cuda')).to(bf)
+    v = torch.randn((B, H, 64, E), generator=gen, device='cuda').to(bf)
+    R = B * beams
+    q = (0.125 * torch.randn((R, H * 64), generator=gen, device='cuda')).to(bf)
+    lens_d = dev(lens)
+    out = ops.cross_attention_step(q, ops.tile_cross_key(k),
+                                   ops.tile_cross_value(v), lens_d, beams)
+    qf = q.float().view(B, beams, H, 64)
+    s = torch.einsum('bkhd,bhed->bkhe', qf, k.float())
+    s = s.to(bf).float()   # the reference rounds the scores to the activation type
+    valid = torch.arange(E, device='cuda')[None, :] < lens_d[:, None]
+    s = s.masked_fill(~valid[:, None, None, :], -1e10)
+    p = torch.softmax(s, dim=-1).to(bf).float()
+    want = torch.einsum('bkhe,bhde->bkhd', p, v.float()).reshape(R, H * 64)
+    err = (out.float() - want).abs()
+    assert float(err.max()) <= 2e-2 + 2.0**-6 * float(want.abs().max()), (
+        case, B, beams, H, E, float(err.max()))
