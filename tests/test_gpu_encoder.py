@@ -478,3 +478,53 @@ def test_gemm_rows_random_shapes_and_repeated_launches(ops):
     err = (outs[0].float() - want).abs()
     ok = err <= 2e-2 + 2.0**-7 * want.abs()
     assert bool(ok.all()), (case, M, K, N, with_res, float(err.max()))
+
+
+def test_encoder_attention_random_shapes(ops):
+  """t5d_encoder_attention (bfloat16) over 24 random shapes — encoder lengths
+  4..512 (also below one key tile and not a multiple of it), 1..12 heads,
+  ragged valid prefixes, with and without padding inside the text — against
+  float32 attention of the same operands on the device (scores and
+  probabilities rounded to bfloat16 where the reference rounds them)."""
+  rs = np.random.RandomState(5)
+  bf = torch.bfloat16
+  for case in range(24):
+    B = int(rs.randint(1, 7))
+    H = int(rs.randint(1, 13))
+    E = 4 * int(rs.randint(1, 129))
+    holes = bool(case % 2)
+    gen = torch.Generator(device='cuda')
+    gen.manual_seed(1000 + case)
+    rnd = lambda *shape: torch.randn(shape, generator=gen, device='cuda')
+    q = (0.125 * rnd(B, E, H, 64)).to(bf)
+    k = rnd(B, E, H, 64).to(bf)
+    v = rnd(B, E, H, 64).to(bf)
+    rel = rnd(H, 2 * E - 1).to(bf)
+    lens = rs.randint(1, E + 1, size=(B,))
+    lens[0] = E
+    valid = np.arange(E)[None, :] < lens[:, None]
+    if holes:
+      valid = valid & (rs.rand(B, E) > 0.2)
+      valid[:, 0] = True
+    last = (valid * np.arange(1, E + 1)[None, :]).max(axis=1).astype(np.int32)
+    vd = dev(valid)
+    bits = ops.pack_valid_bits(vd) if holes else None
+    Ep = (E + 31) // 32 * 32
+    v_t = torch.zeros((B, H, 64, Ep), dtype=bf, device='cuda')
+    v_t[..., :E] = v.permute(0, 2, 3, 1)
+    out = ops.encoder_attention(q.reshape(B * E, H * 64), k.reshape(B * E, H * 64),
+                                ops.tile_cross_value(v_t), rel.contiguous(),
+                                dev(last), valid_bits=bits)
+    idx = (torch.arange(E, device='cuda')[None, :] -
+           torch.arange(E, device='cuda')[:, None] + E - 1)
+    s = torch.einsum('bqhd,bkhd->bhqk', q.float(), k.float()).to(bf).float()
+    s = (s + rel.float()[:, idx][None]).to(bf).float()
+    mask = vd[:, None, :, None] & vd[:, None, None, :]
+    s = torch.where(mask, s, torch.full_like(s, -1e10))
+    p = torch.softmax(s, dim=-1).to(bf).float()
+    want = torch.einsum('bhqk,bkhd->bqhd', p, v.float())
+    got = out.float().reshape(B, E, H, 64)
+    # rows of padding queries attend uniformly over everything: compare too
+    err = (got - want).abs()
+    assert float(err.max()) <= 2e-2 + 2.0**-6 * float(want.abs().max()), (
+        case, B, H, E, holes, float(err.max()))
