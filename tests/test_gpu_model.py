@@ -373,11 +373,19 @@ def _decode_setup(dtype, B, K, E, L, seed, eos_bias=0.0, scan_layers=False):
   return module, fn
 
 
+def _random_loop_shapes(n, seed):
+  rs = np.random.RandomState(seed)
+  return [(int(rs.randint(1, 10)), int(rs.choice([1, 2, 3, 4, 5, 6, 7, 8])),
+           int(rs.choice([5, 31, 33, 64, 97, 129, 257])), int(rs.randint(1, 4)))
+          for _ in range(n)]
+
+
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
 @pytest.mark.parametrize('B,K,L,lanes', [(3, 4, 12, 1), (3, 4, 12, 2),
                                          (2, 2, 140, 2), (5, 1, 9, 3),
                                          (5, 3, 20, 8), (3, 8, 30, 1),
-                                         (2, 8, 200, 1)])
+                                         (2, 8, 200, 1)] +
+                         _random_loop_shapes(6, 3))
 def test_fused_graph_loop_equals_generic_loop(dtype, B, K, L, lanes):
   """The captured whole-iteration graph (in-place state, gated kernels,
   reorder deferred into the next step's attention for bf16) and the
