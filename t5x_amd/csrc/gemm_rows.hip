@@ -286,9 +286,13 @@ rows_gemm_kernel(RowsGemmArgs g) {
 // read of one stage from a load into another and adds no wait of its own.
 // An activation tile is fetched with lane 4 q + j reading row q, piece
 // (j + q / 4) % 4 — four neighbouring lanes still read 64 contiguous bytes —
-// which puts piece p of row r at slot 4 r + (p - r / 4) % 4: the 16 lanes of
-// a quarter wavefront then read 16 slots that differ mod 16, i.e. without
-// bank conflicts.  bfloat16 weights (int8 tiles must be widened on the way).
+// which puts piece p of row r at slot 4 r + (p - r / 4) % 4, so that the 16
+// lanes of a quarter wavefront read 16 slots that differ mod 16.  The LDS
+// still counts bank conflicts for these reads (its rule for 16-byte reads is
+// not the plain one; other rotations measured the same or worse), but the
+// alternative without any — every lane fetching its own operand piece, 16
+// rows per quarter wavefront — loses more in the fetch (185 us against 174).
+// bfloat16 weights (int8 tiles must be widened on the way).
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* glb_ptr_t;
 
