@@ -677,7 +677,7 @@ class EncoderStage:
     return enc + cross
 
   def roofline(self):
-    """The stage's dominant kernel: rows_gemm_kernel on the gated MLP input
+    """The stage's dominant kernel: rows_gemm_direct_kernel on the gated MLP input
     projection ([B*E, d] x [d, 2F], GELU gate in the epilogue), one launch per
     encoder layer; replayed over the layers' kernels and timed with HIP events
     on the launch stream."""
@@ -696,7 +696,7 @@ class EncoderStage:
     sec = time_kernel(torch, launch, 2 * len(layers))
     flops = 2.0 * M * c.emb_dim * 2 * c.mlp_dim
     achieved = flops / sec / 1e12
-    return {'kernel': 'rows_gemm_kernel (gated MLP input projection)',
+    return {'kernel': 'rows_gemm_direct_kernel (gated MLP input projection)',
             'bound': 'mfma', 'achieved': round(achieved, 1),
             'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s',
             'frac': round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),

@@ -105,6 +105,9 @@ _SIGNATURES = {
                                           c_int, c_int]),
     't5d_gemm_rows': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int,
                               c_int, c_int, c_int, c_int, c_int]),
+    't5d_gemm_rows_tiled': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int64,
+                                    c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int]),
     't5d_gemm_tiled': (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P,
                                c_int, c_int, c_int, c_int, _P, c_int, c_int,
                                c_int]),

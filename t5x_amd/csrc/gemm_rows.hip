@@ -169,6 +169,101 @@ __device__ __forceinline__ void rows_epilogue(
   }
 }
 
+// The tanh form of GELU written as x * sigmoid(2 c (x + 0.044715 x^3)): one
+// exponential and one reciprocal instead of the library tanh, whose ~50
+// instructions per element made the gated epilogue a third of the launch.
+// Relative error ~3e-7 before the rounding to bfloat16.
+__device__ __forceinline__ float gelu_sigmoid_form(float x) {
+  const float k = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  const float y = k * (x + 0.044715f * (x * x * x));
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y));
+}
+
+// Epilogue of the C^T form (bfloat16 weights, no scales) with the stores
+// made whole: a lane holds 4 consecutive columns of one row, so storing from
+// the accumulators writes 16 rows x 8..32 bytes per instruction.  Each
+// wavefront instead parks one 16-row slice at a time in a private piece of
+// LDS (rounded to bfloat16, rows padded by 16 bytes) and reads it back with 4
+// or 8 lanes per row, 16 bytes per lane: every store instruction then writes
+// whole 64-byte (gated) or 128-byte rows, and the residual is read the same
+// way.  LDS operations of one wavefront complete in order, so the slices
+// follow one another through the same piece without a wait in between.
+constexpr int kRowsStageBytes = 16 * 144;
+template <int NT>
+__device__ __forceinline__ void rows_epilogue_staged(
+    const RowsGemmArgs& g, const f32x4_r (&acc)[kRowsMT][NT], int m0, int nt0,
+    int n_tiles, int lane, char* stage) {
+  static_assert(NT == 4, "a wavefront's slice is 64 columns wide");
+  constexpr int MT = kRowsMT;
+  const int l16 = lane & 15, gq = lane >> 4;
+  if (g.epilogue == T5D_EPI_GEGLU) {
+    // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the lanes
+    // with gq >= 2 hold the gates of the lanes with gq - 2.  32 output columns.
+    const int F = g.N >> 1;
+    const int row = lane >> 2, piece = lane & 3;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        float h[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = acc[mt][nt][i];
+          const float gate = __shfl_xor(v, 32, 64);
+          h[i] = round_bf16(gelu_sigmoid_form(round_bf16(v))) * round_bf16(gate);
+        }
+        if (gq < 2)
+          *reinterpret_cast<uint2*>(stage + l16 * 80 + (8 * nt + 4 * gq) * 2) =
+              pack4(h[0], h[1], h[2], h[3]);
+      }
+      const uint4 q = *reinterpret_cast<const uint4*>(stage + row * 80 + piece * 16);
+      const int m = m0 + 16 * mt + row;
+      if (m < g.M && nt0 + piece < n_tiles)
+        *reinterpret_cast<uint4*>(g.C + (size_t)m * F + 8 * (nt0 + piece)) = q;
+    }
+    return;
+  }
+  const int piece = lane & 7;
+  const int n = 16 * nt0 + 8 * piece;
+  const bool n_ok = nt0 + (piece >> 1) < n_tiles;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      *reinterpret_cast<uint2*>(stage + l16 * 144 + (16 * nt + 4 * gq) * 2) =
+          pack4(acc[mt][nt][0], acc[mt][nt][1], acc[mt][nt][2], acc[mt][nt][3]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = 8 * j + (lane >> 3);
+      uint4 q = *reinterpret_cast<const uint4*>(stage + row * 144 + piece * 16);
+      const int m = m0 + 16 * mt + row;
+      if (m >= g.M || !n_ok) continue;
+      size_t o;
+      if (g.layout == T5D_OUT_HEADS_KEY) {
+        // [B, H, 2, Ep, 32]: the two 32-wide halves of the head dim as planes
+        const int b = m / g.E, e = m - b * g.E;
+        const int hh = n >> 6, c = (n >> 5) & 1, jj = n & 31;
+        o = ((((size_t)b * g.H + hh) * 2 + c) * g.Ep + e) * 32 + jj;
+      } else {
+        o = (size_t)m * g.N + n;
+      }
+      if (g.epilogue == T5D_EPI_RESIDUAL) {
+        const uint4 r = *reinterpret_cast<const uint4*>(
+            g.residual + (size_t)m * g.N + n);
+        q.x = pack_bf16x2(bf16lo_to_f32(q.x) + bf16lo_to_f32(r.x),
+                          bf16hi_to_f32(q.x) + bf16hi_to_f32(r.x));
+        q.y = pack_bf16x2(bf16lo_to_f32(q.y) + bf16lo_to_f32(r.y),
+                          bf16hi_to_f32(q.y) + bf16hi_to_f32(r.y));
+        q.z = pack_bf16x2(bf16lo_to_f32(q.z) + bf16lo_to_f32(r.z),
+                          bf16hi_to_f32(q.z) + bf16hi_to_f32(r.z));
+        q.w = pack_bf16x2(bf16lo_to_f32(q.w) + bf16lo_to_f32(r.w),
+                          bf16hi_to_f32(q.w) + bf16hi_to_f32(r.w));
+      }
+      *reinterpret_cast<uint4*>(g.C + o) = q;
+    }
+  }
+}
+
 // SWAP: weights are the MFMA A operand (C^T is formed).
 template <typename WT, bool SWAP>
 __global__ void __launch_bounds__(256, 2)
@@ -296,21 +391,26 @@ rows_gemm_kernel(RowsGemmArgs g) {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* glb_ptr_t;
 
+// WN: wavefront columns of the workgroup, 2 (256 x 128 tile, 4 wavefronts, two
+// workgroups per CU) or 4 (256 x 256, 8 wavefronts, one per CU).
 // Measured on the gated MLP input projection of the T5.1.1-base encoder
-// (16384 x 768 x 4096): 182 -> 176 us per launch.  NT (16-column tiles per
-// wavefront) = 8, i.e. a 256 x 256 workgroup tile with one workgroup per CU
-// and the accumulators in the accumulation registers, halves the bytes per
-// flop that a CU takes in but lasts 257 us: with one wavefront per SIMD
-// nothing covers the operand reads from LDS.
-template <bool SWAP, int NT>
-__global__ void __launch_bounds__(256, 2)
+// (16384 x 768 x 4096): 182 -> 176 us per launch with the ring alone, 123 us
+// with the epilogue below (the library tanh and the 8-byte stores were a
+// third of the launch), 118 us with the 256 x 256 tile.  The same tile from 4
+// wavefronts of 128 x 128 (accumulators in the accumulation registers) lasts
+// 257 us: with one wavefront per SIMD nothing covers the operand reads from
+// LDS.
+template <bool SWAP, int NT, int WN>
+__global__ void __launch_bounds__(128 * WN, WN == 2 ? 2 : 1)
 rows_gemm_direct_kernel(RowsGemmArgs g) {
   constexpr int MT = kRowsMT;
-  constexpr int BN = 2 * NT * 16;       // columns of the workgroup tile
-  constexpr int WL = NT / 2;            // weight tiles a wavefront loads per stage
-  constexpr int TILES = 16 + 2 * NT;
-  // all but my newest 4 + WL loads have landed: s_waitcnt vmcnt(4 + WL)
-  constexpr int kWaitStage = 0xF70 | (4 + WL);
+  constexpr int WAVES = 2 * WN;         // 2 rows of WN wavefronts
+  constexpr int BN = WN * NT * 16;      // columns of the workgroup tile
+  constexpr int AL = 16 / WAVES;        // activation tiles a wavefront loads per stage
+  constexpr int WL = WN * NT / WAVES;   // weight tiles a wavefront loads per stage
+  constexpr int TILES = 16 + WN * NT;
+  // all but my newest AL + WL loads have landed: s_waitcnt vmcnt(AL + WL)
+  constexpr int kWaitStage = 0xF70 | (AL + WL);
   // [tile][lane]: tiles 0..15 activations (rows 16 t ..), then the weights
   __shared__ uint4 s_t0[TILES][64];
   __shared__ uint4 s_t1[TILES][64];
@@ -320,7 +420,7 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
   const int l16 = lane & 15, gq = lane >> 4;
   const int m_blocks = (g.M + kRowsBM - 1) / kRowsBM;
   const int m_blk = blockIdx.x % m_blocks, n_blk = blockIdx.x / m_blocks;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int m0 = m_blk * kRowsBM + wm * (16 * MT);
   const int nt0 = n_blk * (BN / 16) + wn * NT;
   const int KT = g.K >> 5, n_tiles = g.N >> 4;
@@ -328,20 +428,21 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
   const int ld_row = lane >> 2;
   const int ld_piece = ((lane & 3) + (ld_row >> 2)) & 3;
   const int read_slot = 4 * l16 + ((gq - (l16 >> 2)) & 3);
-  // this wavefront's tiles of every stage: activation tiles wave + 4 i,
-  // weight tiles wave + 4 i (rows / tiles past the edge clamped: their
+  // this wavefront's tiles of every stage: activation tiles wave + WAVES i,
+  // weight tiles wave + WAVES i (rows / tiles past the edge clamped: their
   // products are discarded in the epilogue)
-  const char* arow[4];
+  const char* arow[AL];
   const char* wtile[WL];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < AL; ++i)
     arow[i] = reinterpret_cast<const char*>(
         g.A +
-        (size_t)min(m_blk * kRowsBM + 16 * (wave + 4 * i) + ld_row, g.M - 1) *
+        (size_t)min(m_blk * kRowsBM + 16 * (wave + WAVES * i) + ld_row,
+                    g.M - 1) *
             g.K + 8 * ld_piece);
 #pragma unroll
   for (int i = 0; i < WL; ++i)
-    wtile[i] = g.W + (size_t)min(n_blk * (BN / 16) + wave + 4 * i,
+    wtile[i] = g.W + (size_t)min(n_blk * (BN / 16) + wave + WAVES * i,
                                  n_tiles - 1) * KT * 1024 + lane * 16;
 
   f32x4_r acc[MT][NT];
@@ -352,14 +453,14 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
 
 #define T5D_ROWS_ISSUE(kt_, S_)                                                \
   do {                                                                         \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                              \
+    _Pragma("unroll") for (int i = 0; i < AL; ++i)                             \
       __builtin_amdgcn_global_load_lds((glb_ptr_t)(arow[i] + 64 * (kt_)),      \
-                                       (lds_ptr_t)&S_[wave + 4 * i][0], 16, 0, \
-                                       0);                                     \
+                                       (lds_ptr_t)&S_[wave + WAVES * i][0],    \
+                                       16, 0, 0);                              \
     _Pragma("unroll") for (int i = 0; i < WL; ++i)                             \
       __builtin_amdgcn_global_load_lds(                                        \
           (glb_ptr_t)(wtile[i] + (size_t)(kt_) * 1024),                        \
-          (lds_ptr_t)&S_[16 + wave + 4 * i][0], 16, 0, 0);                     \
+          (lds_ptr_t)&S_[16 + wave + WAVES * i][0], 16, 0, 0);                 \
   } while (0)
 #define T5D_ROWS_MULTIPLY(S_)                                                  \
   do {                                                                         \
@@ -379,7 +480,7 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
       }                                                                        \
     }                                                                          \
   } while (0)
-  // s_waitcnt vmcnt(4 + WL): all but this wavefront's newest loads have landed,
+  // s_waitcnt vmcnt(AL + WL): all but this wavefront's newest loads have landed,
   // i.e. its share of the stage about to be multiplied; after the barrier
   // every wavefront's share has, and every wavefront is done with the stage
   // that the next loads overwrite.
@@ -418,7 +519,15 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
 #undef T5D_ROWS_MULTIPLY
 #undef T5D_ROWS_STEP
 #undef T5D_ROWS_LAST
-  rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+  if (SWAP) {
+    static_assert(sizeof(s_t0) >= WAVES * kRowsStageBytes, "stage too small");
+    __syncthreads();  // every wavefront is done with the ring
+    rows_epilogue_staged<NT>(
+        g, acc, m0, nt0, n_tiles, lane,
+        reinterpret_cast<char*>(&s_t0[0][0]) + wave * kRowsStageBytes);
+  } else {
+    rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+  }
 }
 
 }  // namespace t5d
@@ -430,7 +539,19 @@ extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
                              const void* residual, void* C, int64_t M, int K,
                              int N, int epilogue, int out_layout, int E,
                              int Ep) {
+  return t5d_gemm_rows_tiled(stream, w_dtype, A, W, scales, residual, C, M, K,
+                             N, epilogue, out_layout, E, Ep, 0);
+}
+
+extern "C" int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
+                                   const void* W, const float* scales,
+                                   const void* residual, void* C, int64_t M,
+                                   int K, int N, int epilogue, int out_layout,
+                                   int E, int Ep, int tile) {
   T5D_REQUIRE(A && W && C, T5D_EINVAL, "t5d_gemm_rows: null pointer");
+  T5D_REQUIRE(tile >= 0 && tile <= 2, T5D_EINVAL,
+              "t5d_gemm_rows_tiled: tile %d (0 chosen here, 1: 256 x 128, "
+              "2: 256 x 256)", tile);
   T5D_REQUIRE(w_dtype == T5D_BF16 || w_dtype == T5D_I8, T5D_EINVAL,
               "t5d_gemm_rows: w_dtype %d (packed bfloat16 or int8)", w_dtype);
   T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
@@ -470,13 +591,29 @@ extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
   dim3 grid((unsigned)m_blocks * n_blocks), block(256);
   hipStream_t s = as_stream(stream);
   const bool swap = out_layout != T5D_OUT_HEADS_VALUE;
-  if (w_dtype == T5D_BF16 && K >= 64) {
+  // 256 x 256 tiles (8 wavefronts, one workgroup per CU) halve the operand
+  // bytes per flop and measure 3-11 % faster than 256 x 128 whenever their
+  // workgroups fill the 256 CUs evenly; with a ragged last round (1.5 or 5.5
+  // rounds) the smaller tile, two workgroups per CU, loses less to the tail.
+  const int n_wide = (N + 2 * kRowsBN - 1) / (2 * kRowsBN);
+  const int wide_wgs = m_blocks * n_wide, tail = wide_wgs % 256;
+  const bool wide =
+      tile ? tile == 2 : (wide_wgs <= 256 || tail == 0 || tail >= 192);
+  if (w_dtype == T5D_BF16 && K >= 64 && wide) {
+    dim3 wgrid((unsigned)wide_wgs), wblock(512);
     if (swap)
-      hipLaunchKernelGGL((rows_gemm_direct_kernel<true, kRowsNT>), grid, block,
-                         0, s, g);
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<true, kRowsNT, 4>), wgrid,
+                         wblock, 0, s, g);
     else
-      hipLaunchKernelGGL((rows_gemm_direct_kernel<false, kRowsNT>), grid, block,
-                         0, s, g);
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<false, kRowsNT, 4>), wgrid,
+                         wblock, 0, s, g);
+  } else if (w_dtype == T5D_BF16 && K >= 64) {
+    if (swap)
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<true, kRowsNT, 2>), grid,
+                         block, 0, s, g);
+    else
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<false, kRowsNT, 2>), grid,
+                         block, 0, s, g);
   } else if (w_dtype == T5D_BF16) {
     if (swap)
       hipLaunchKernelGGL((rows_gemm_kernel<bf16_t, true>), grid, block, 0, s, g);

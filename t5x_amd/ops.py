@@ -455,10 +455,11 @@ def cross_attention_step_norm_q(x, ln_scale, wq: PackedWeight, cross_key,
 
 
 def gemm_rows(a, w: PackedWeight, out=None, residual=None,
-              layout=_lib.OUT_ROWS, E=0, Ep=0):
+              layout=_lib.OUT_ROWS, E=0, Ep=0, tile=0):
   """Dense layer over any number of rows (bfloat16).  layout OUT_HEADS_KEY /
   OUT_HEADS_VALUE writes [B, H, 2, Ep, 32] / [B, H, Ep/32, 64, 32] (rows
-  m = b*E + e; Ep a multiple of 32, positions e >= E stay zero)."""
+  m = b*E + e; Ep a multiple of 32, positions e >= E stay zero).  tile: 0 =
+  chosen from the shape, 1 = 256 x 128, 2 = 256 x 256 (t5d_gemm_rows_tiled)."""
   _chk(a, 'a', torch.bfloat16, 2)
   M, K = a.shape
   if K != w.K or w.w_dtype == F32:
@@ -483,9 +484,10 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
     _chk(residual, 'residual', a.dtype, 2)
     if tuple(residual.shape) != (M, w.N):
       raise ValueError('residual shape mismatch')
-  _lib.call('t5d_gemm_rows', _s(), w.w_dtype, a.data_ptr(), w.data.data_ptr(),
-            _lib.ptr(w.scales), _lib.ptr(residual), out.data_ptr(), M, K, w.N,
-            epi, int(layout), int(E), int(Ep))
+  _lib.call('t5d_gemm_rows_tiled', _s(), w.w_dtype, a.data_ptr(),
+            w.data.data_ptr(), _lib.ptr(w.scales), _lib.ptr(residual),
+            out.data_ptr(), M, K, w.N, epi, int(layout), int(E), int(Ep),
+            int(tile))
   return out
 
 

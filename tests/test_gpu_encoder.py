@@ -43,7 +43,8 @@ def test_gemm_rows(ops, M, K, N, mode):
     w1 = (rs.randn(K, N) / np.sqrt(K)).astype(np.float32)
     q1 = ot5.quantize_int8(w1) if wd == torch.int8 else w1
     pw = ops.pack_weight(dev(w0), torch.bfloat16, wd, gate_kernel=dev(w1))
-    out = ops.gemm_rows(a, pw)
+    out = ops.gemm_rows(a, pw, tile=1)
+    wide = ops.gemm_rows(a, pw, tile=2)
     want = ot5.mlp_block({'wi_0': {'kernel': q0}, 'wi_1': {'kernel': q1},
                           'wo': {'kernel': np.eye(N, dtype=np.float32)}},
                          host(a), ('gelu', 'linear'), 'bfloat16')
@@ -54,9 +55,15 @@ def test_gemm_rows(ops, M, K, N, mode):
     if mode == 'residual':
       res = dev(rs.randn(M, N).astype(np.float32), torch.bfloat16)
       want = ot5.bf16_round(want + host(res))
-    out = ops.gemm_rows(a, pw, residual=res)
+    out = ops.gemm_rows(a, pw, residual=res, tile=1)
+    wide = ops.gemm_rows(a, pw, residual=res, tile=2)
   assert out.shape == want.shape
   np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
+  # both workgroup tiles (256 x 128, 256 x 256) and the one picked from the
+  # shape give the same bits
+  assert torch.equal(out, wide)
+  chosen = ops.gemm_rows(a, pw, residual=None if mode != 'residual' else res)
+  assert torch.equal(out, chosen)
   if M <= 128 and not mode.startswith('int8'):
     # same weights, same rounding points as the decode-step kernel
     small = ops.gemm(a, pw, residual=None if mode != 'residual' else res)
@@ -77,8 +84,31 @@ def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
   from t5x_amd import _lib
   pw = ops.pack_weight(w, torch.bfloat16)
   rows = ops.gemm_rows(x, pw).view(B, E, H, 64)
-  keys = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep)
-  vals = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep)
+  for tile in (1, 2):
+    keys = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep,
+                         tile=tile)
+    vals = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep,
+                         tile=tile)
+    _check_head_layouts(ops, rows, keys, vals, B, E, Ep, H)
+
+
+def test_gemm_rows_plain_entry_point(ops):
+  """t5d_gemm_rows itself (ops.gemm_rows goes through t5d_gemm_rows_tiled)."""
+  from t5x_amd import _lib
+  rs = np.random.RandomState(9)
+  a = dev(rs.randn(300, 96).astype(np.float32), torch.bfloat16)
+  pw = ops.pack_weight(dev((rs.randn(96, 80) / 10).astype(np.float32)),
+                       torch.bfloat16)
+  out = torch.empty((300, 80), dtype=torch.bfloat16, device='cuda')
+  _lib.call('t5d_gemm_rows', _lib.stream_handle(), pw.w_dtype, a.data_ptr(),
+            pw.data.data_ptr(), None, None, out.data_ptr(), 300, 96, 80,
+            _lib.EPI_NONE, _lib.OUT_ROWS, 0, 0)
+  assert torch.equal(out, ops.gemm_rows(a, pw))
+  with pytest.raises(ValueError):
+    ops.gemm_rows(a, pw, tile=3)
+
+
+def _check_head_layouts(ops, rows, keys, vals, B, E, Ep, H):
   plain_k = torch.zeros((B, H, Ep, 64), dtype=rows.dtype, device='cuda')
   plain_k[:, :, :E] = rows.permute(0, 2, 1, 3)
   plain_v = torch.zeros((B, H, 64, Ep), dtype=rows.dtype, device='cuda')
@@ -450,7 +480,7 @@ def test_cross_kv_projection_layouts_match_oracle():
 
 
 def test_gemm_rows_random_shapes_and_repeated_launches(ops):
-  """t5d_gemm_rows over 30 random shapes (rows 1..3000, K a multiple of 32
+  """t5d_gemm_rows (both workgroup tiles) over 30 random shapes (rows 1..3000, K a multiple of 32
   from 64 to 4096, i.e. 2 to 128 rounds of its ring of LDS stages, N a
   multiple of 16 up to 4096, with and without a residual) against float32
   products of the same operands on the device, and launched three times:
@@ -471,10 +501,13 @@ def test_gemm_rows_random_shapes_and_repeated_launches(ops):
         torch.bfloat16).float()
     if with_res:
       want = (want + res.float()).to(torch.bfloat16).float()
-    outs = [ops.gemm_rows(a, pw, residual=res) for _ in range(3)]
+    outs = [ops.gemm_rows(a, pw, residual=res, tile=1 + case % 2)
+            for _ in range(3)]
+    other = ops.gemm_rows(a, pw, residual=res, tile=2 - case % 2)
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (
         case, M, K, N)
+    assert torch.equal(outs[0], other), (case, M, K, N)
     err = (outs[0].float() - want).abs()
     ok = err <= 2e-2 + 2.0**-7 * want.abs()
     assert bool(ok.all()), (case, M, K, N, with_res, float(err.max()))
