@@ -221,6 +221,17 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x * (0.5f * (1.0f + tanhf(c * (x + 0.044715f * (x * x * x)))));
 }
 
+// The tanh form of GELU written as x * sigmoid(2 c (x + 0.044715 x^3)): one
+// exponential and one reciprocal instead of the library tanh, whose ~50
+// instructions per element made the gated epilogue of the many-row dense
+// kernel a third of its launch.
+// Relative error ~3e-7 before the rounding to bfloat16.
+__device__ __forceinline__ float gelu_sigmoid_form(float x) {
+  const float k = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  const float y = k * (x + 0.044715f * (x * x * x));
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y));
+}
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 // Optional device-side gate.  While a fused multi-kernel entry point is

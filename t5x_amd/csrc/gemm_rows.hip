@@ -115,7 +115,7 @@ __device__ __forceinline__ void rows_epilogue(
             float h[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              h[i] = round_bf16(round_bf16(gelu_tanh(round_bf16(v[i]))) *
+              h[i] = round_bf16(round_bf16(gelu_sigmoid_form(round_bf16(v[i]))) *
                                 round_bf16(gate[i]));
             const int F = g.N >> 1;
             *reinterpret_cast<uint2*>(g.C + (size_t)m * F + 8 * (nt0 + nt) +
@@ -167,16 +167,6 @@ __device__ __forceinline__ void rows_epilogue(
       }
     }
   }
-}
-
-// The tanh form of GELU written as x * sigmoid(2 c (x + 0.044715 x^3)): one
-// exponential and one reciprocal instead of the library tanh, whose ~50
-// instructions per element made the gated epilogue a third of the launch.
-// Relative error ~3e-7 before the rounding to bfloat16.
-__device__ __forceinline__ float gelu_sigmoid_form(float x) {
-  const float k = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
-  const float y = k * (x + 0.044715f * (x * x * x));
-  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y));
 }
 
 // Epilogue of the C^T form (bfloat16 weights, no scales) with the stores

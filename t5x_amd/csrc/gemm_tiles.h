@@ -81,7 +81,7 @@ __device__ __forceinline__ void store_result(const GemmArgs& g, int m, int n,
     const int f = (n >> 4) * 8 + (n & 7);
     const int F = g.N >> 1;
     float a0 = round_bf16(v), a1 = round_bf16(v_gate);
-    float h = round_bf16(round_bf16(gelu_tanh(a0)) * a1);
+    float h = round_bf16(round_bf16(gelu_sigmoid_form(a0)) * a1);
     reinterpret_cast<bf16_t*>(g.C)[(size_t)m * F + f] = f32_to_bf16(h);
     return;
   }
