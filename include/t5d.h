@@ -303,6 +303,21 @@ int t5d_encoder_attention(void* stream, const void* q, const void* k,
                           void* out, int B, int H, int E, int Ep, int q_stride,
                           int k_stride);
 
+/* t5d_encoder_attention on the kernel of the caller's choice: variant 1 walks
+ * the keys twice and forms every score twice (any E up to 2048), variant 2
+ * keeps the scores of pass 1 in registers and shares K and V between the
+ * wavefronts of a workgroup through LDS (E <= 512), variant 0 is what
+ * t5d_encoder_attention picks (2 when E <= 512).  Same scores and
+ * probabilities; the two sum a 32-key step's products in different orders, so
+ * outputs agree to the last bfloat16 bit except for rare roundings.  For
+ * testing both kernels on one shape. */
+int t5d_encoder_attention_variant(void* stream, const void* q, const void* k,
+                                  const void* v_t, const void* rel_bias,
+                                  const int32_t* enc_len,
+                                  const uint32_t* valid_bits, void* out, int B,
+                                  int H, int E, int Ep, int q_stride,
+                                  int k_stride, int variant);
+
 /* The same attention in float32 (the dtype of the exactness tests), straight
  * from the fused projection: qkv [B*E, 3*H*64] holds q | k | v per row;
  * rel_bias [H, 2E-1] float32; enc_len / valid_bits as above; out

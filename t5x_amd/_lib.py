@@ -101,6 +101,9 @@ _SIGNATURES = {
                          c_int, c_int, c_int, _P, _P]),
     't5d_encoder_attention': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int,
                                       c_int, c_int, c_int, c_int, c_int]),
+    't5d_encoder_attention_variant': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P,
+                                              c_int, c_int, c_int, c_int,
+                                              c_int, c_int, c_int]),
     't5d_encoder_attention_f32': (c_int, [_P, _P, _P, _P, _P, _P, c_int,
                                           c_int, c_int]),
     't5d_gemm_rows': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int64, c_int,

@@ -71,7 +71,7 @@ enc_attn_kernel(EncAttnArgs a) {
   auto is_valid = [&](int pos) {
     return pos < E && ((s_valid[pos >> 5] >> (pos & 31)) & 1u) != 0;
   };
-  const float kMasked = -9.9857e9f;  // bf16(-1e10), layers.py:309-311
+  const float kMasked = -9999220736.0f;  // bf16(-1e10) exactly, layers.py:309-311
   const size_t row0 = (size_t)b * E;
 
   // B operand of S^T: lane (col = query l16, g) holds Q[q][32c + 8g .. +8]
@@ -115,12 +115,14 @@ enc_attn_kernel(EncAttnArgs a) {
       kop.u = ol.to_operand(ka[c].u);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qb[c].v, acc, 0, 0, 0);
     }
-    // validity of the tile's 16 keys: from the prefix length alone, or one
-    // (broadcast) LDS word when the caller gave bits
-    const int left = n - 16 * kt;
-    const uint32_t tile_bits =
-        a.valid ? (s_valid[kt >> 1] >> ((kt & 1) * 16)) & 0xffffu
-                : (left >= 16 ? 0xffffu : (left <= 0 ? 0u : (1u << left) - 1u));
+    // validity of the tile's 16 keys: one (broadcast) LDS word, which holds
+    // the prefix when the caller gave no bits.  Deliberately without a branch
+    // on a.valid here: with one between the matrix instructions above and the
+    // first read of their result, the compiler's wait-state count followed
+    // the fall-through side only and the taken side read the accumulator 6
+    // issue slots after the v_mfma (9 are needed; at 4 a stale value comes
+    // back).
+    const uint32_t tile_bits = (s_valid[kt >> 1] >> ((kt & 1) * 16)) & 0xffffu;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = 16 * kt + 4 * gq + i;
@@ -230,6 +232,280 @@ enc_attn_kernel(EncAttnArgs a) {
   }
 }
 
+// ---- the same attention for E <= 512, scores kept in registers ---------------
+// enc_attn_kernel walks the keys twice and forms every score twice, each
+// wavefront fetching K and V for itself.  For encoder lengths up to 512 the 16
+// x E scores of a wavefront fit its registers as bfloat16 pairs (they ARE
+// bfloat16 values at that point), so here
+//   pass 1 forms the scores once, keeps them, and tracks max / sum as before;
+//   pass 2 turns the kept scores into P in registers, already in the layout
+//          of the matrix cores' B operand: a lane holds keys 4g .. 4g+3 of two
+//          neighbouring 16-key tiles, and the V^T operand is read from LDS in
+//          that same key order, so P never goes through LDS.
+// K (pass 1) and V^T (pass 2) are fetched once per workgroup, 64 keys = 8 KB
+// at a time, straight from memory into a ring of three LDS stages
+// (global_load_lds: lane l of an instruction lands at byte 16 l, so the
+// address each lane reads from picks the XOR swizzle that makes the operand
+// reads spread over the banks); the four wavefronts read their operand
+// fragments from there.  One barrier per 64 keys, placed by hand with the wait
+// for "all but my newest two loads"; the stages are separate arrays and the
+// loops are unrolled so that every stage is named at compile time.
+// Scores, maxima, sums and probabilities have the bits of enc_attn_kernel's;
+// the products of a 32-key step enter the matrix instruction in another key
+// order, so an output can differ from enc_attn_kernel's in its last bit (1
+// in 4000 measured).
+typedef __attribute__((address_space(3))) void* enc_lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* enc_glb_ptr_t;
+
+template <int MAXB>  // 64-key blocks: E <= 64 MAXB
+__global__ void __launch_bounds__(256)
+enc_attn_ring_kernel(EncAttnArgs a) {
+  __shared__ uint4 s_r0[512];
+  __shared__ uint4 s_r1[512];
+  __shared__ uint4 s_r2[512];
+  __shared__ float s_bias[128 * MAXB + 16];
+  __shared__ uint32_t s_valid[2 * MAXB];
+  // what a score is capped by, per key: [0] for a valid query (+inf for a
+  // valid key, bf16(-1e10) for a masked one, -inf past E), [1] for a padded
+  // query (bf16(-1e10) for every key that exists)
+  __shared__ __attribute__((aligned(16))) float s_lim[2][64 * MAXB + 16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, gq = lane >> 4;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int E = a.E;
+  for (int i = threadIdx.x; i < 2 * E - 1; i += 256)
+    s_bias[i] = bf16_to_f32(a.bias[(size_t)h * (2 * E - 1) + i]);
+  int n = a.len[b];
+  n = n < 0 ? 0 : (n > E ? E : n);
+  const int words = (E + 31) >> 5;
+  for (int i = threadIdx.x; i < words; i += 256) {
+    const int left = n - 32 * i;
+    const uint32_t prefix =
+        left >= 32 ? 0xffffffffu : (left <= 0 ? 0u : ((1u << left) - 1u));
+    s_valid[i] = a.valid ? (a.valid[(size_t)b * words + i] & prefix) : prefix;
+  }
+  __syncthreads();
+  const float kMasked = -9999220736.0f;  // bf16(-1e10) exactly, layers.py:309-311
+  for (int i = threadIdx.x; i < 64 * MAXB + 16; i += 256) {
+    const bool ok = i < E && ((s_valid[i >> 5] >> (i & 31)) & 1u) != 0;
+    s_lim[0][i] = ok ? INFINITY : (i < E ? kMasked : -INFINITY);
+    s_lim[1][i] = i < E ? kMasked : -INFINITY;
+  }
+  __syncthreads();
+  // Key tiles each wavefront walks (as in enc_attn_kernel: the valid prefix
+  // when all of its 16 queries are valid — the keys beyond add exact zeros —
+  // else every key; none when its queries lie beyond E) and what the
+  // workgroup as a whole must fetch, in 64-key blocks.
+  const int all_tiles = (E + 15) >> 4;
+  int my_tiles = 0, wg_tiles = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int qw = blockIdx.x * 64 + w * 16;
+    int t = 0;
+    if (qw < E) {
+      const bool all_valid =
+          qw + 15 < E &&
+          ((s_valid[qw >> 5] >> (qw & 31)) & 0xffffu) == 0xffffu;
+      t = all_valid ? (n + 15) >> 4 : all_tiles;
+    }
+    if (w == wave) my_tiles = t;
+    wg_tiles = max(wg_tiles, t);
+  }
+  my_tiles = __builtin_amdgcn_readfirstlane(my_tiles);
+  const int nb = __builtin_amdgcn_readfirstlane((wg_tiles + 3) >> 2);
+  const int q0 = blockIdx.x * 64 + wave * 16;
+  const size_t row0 = (size_t)b * E;
+
+  const int qi = min(q0 + l16, E - 1);
+  FragE qb[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+    qb[c].u = *reinterpret_cast<const uint4*>(
+        a.q + (row0 + qi) * a.q_stride + h * 64 + 32 * c + 8 * gq);
+  const bool q_valid =
+      q0 + l16 < E &&
+      ((s_valid[(q0 + l16) >> 5] >> ((q0 + l16) & 31)) & 1u) != 0;
+  // this lane's 4 keys of key tile kt: bias and cap at [16 kt .. 16 kt + 3].
+  // Masking is a minimum with the cap: a score never lies below -1e10, so
+  // min(x, bf16(-1e10)) is the reference's masked value, min(x, -inf) removes
+  // a key that does not exist, min(x, +inf) keeps x.
+  const float* bias_g = s_bias + (E - 1) - qi + 4 * gq;
+  const float* lim_g = s_lim[q_valid ? 0 : 1] + 4 * gq;
+
+  // What this lane fetches of a 64-key block of K: chunks (8 keys, 1 KB)
+  // wave and wave + 4; lane s lands at slot s & 7 of key s >> 3 and therefore
+  // reads piece (s & 7) ^ (s >> 3) of that key.
+  const int k_r = lane >> 3, k_piece = (lane & 7) ^ k_r;
+  const char* kbase = reinterpret_cast<const char*>(a.k) +
+                      (size_t)h * 128 + k_piece * 16;
+  // ... and of a 64-key block of V^T (two [64 d][32 keys] blocks, 4 KB each):
+  // chunks (16 rows d, 1 KB) wave and wave + 4; lane s lands at slot s & 3 of
+  // row s >> 2 and reads piece (s & 3) ^ ((row >> 1) & 3).
+  const int v_r = lane >> 2, v_piece = (lane & 3) ^ ((v_r >> 1) & 3);
+  const char* vbase = reinterpret_cast<const char*>(a.vt) +
+                      ((size_t)b * a.H + h) * 128 * (size_t)a.Ep;
+  const int v_blocks = a.Ep >> 5;
+#define T5D_ENC_ISSUE_K(i_, S_)                                                \
+  do {                                                                         \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                            \
+      const int c = wave + 4 * u;                                              \
+      const int key = min(64 * (i_) + 8 * c + k_r, E - 1);                     \
+      __builtin_amdgcn_global_load_lds(                                        \
+          (enc_glb_ptr_t)(kbase + (row0 + key) * (size_t)a.k_stride * 2),      \
+          (enc_lds_ptr_t)&S_[64 * c], 16, 0, 0);                               \
+    }                                                                          \
+  } while (0)
+#define T5D_ENC_ISSUE_V(i_, S_)                                                \
+  do {                                                                         \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                            \
+      const int c = wave + 4 * u;                                              \
+      const int blk = min(2 * (i_) + (c >> 2), v_blocks - 1);                  \
+      __builtin_amdgcn_global_load_lds(                                        \
+          (enc_glb_ptr_t)(vbase + (size_t)blk * 4096 +                         \
+                          (16 * (c & 3) + v_r) * 64 + v_piece * 16),           \
+          (enc_lds_ptr_t)&S_[64 * c], 16, 0, 0);                               \
+    }                                                                          \
+  } while (0)
+  // all but my newest two loads (the next block) have landed and my reads of
+  // LDS have returned (vmcnt(2) lgkmcnt(0): a barrier orders issued
+  // instructions, not completed LDS reads); after the barrier so have
+  // everyone's, and everyone is done with the stage that the loads issued
+  // next overwrite.  Nothing in a step is conditional — the loads past the
+  // last block fetch clamped addresses into a stage nobody reads, every
+  // wavefront forms all four key tiles of a block — and the only branch is
+  // the loop exit in front of a step: where two paths meet between a load
+  // into LDS and a read of LDS the compiler waits for every load in flight.
+#define T5D_ENC_STEP(i_, CUR_, NEXT2_, ISSUE_, BODY_)                          \
+  if ((i_) >= nb) break;                                                       \
+  __builtin_amdgcn_s_waitcnt(0x070 | 2);                                       \
+  __builtin_amdgcn_s_barrier();                                                \
+  ISSUE_((i_) + 2, NEXT2_);                                                    \
+  __builtin_amdgcn_sched_barrier(0);                                           \
+  BODY_(i_, CUR_);
+
+  // scores of key tile kt for this lane: keys 16 kt + 4 g + i of query l16
+  constexpr int ROUNDS = (MAXB + 2) / 3;
+  uint32_t sc[12 * ROUNDS][2];
+#pragma unroll
+  for (int t = 0; t < 12 * ROUNDS; ++t)
+    sc[t][0] = sc[t][1] = 0xFF80FF80u;  // -inf
+  float m = -3.0e38f, l = 0.f;
+  const int swz = l16 & 7;
+#define T5D_ENC_SCORES(i_, S_)                                                 \
+  _Pragma("unroll") for (int t = 0; t < 4; ++t) {                              \
+    const int kt = 4 * (i_) + t;                                               \
+    if (kt < my_tiles) {                                                       \
+      f32x4_e acc = (f32x4_e){0.f, 0.f, 0.f, 0.f};                             \
+      _Pragma("unroll") for (int c = 0; c < 2; ++c) {                          \
+        FragE kop;                                                             \
+        kop.u = S_[(16 * t + l16) * 8 + ((4 * c + gq) ^ swz)];                 \
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qb[c].v, acc, 0,  \
+                                                      0, 0);                   \
+      }                                                                        \
+      const float4 cap = *reinterpret_cast<const float4*>(lim_g + 16 * kt);    \
+      float s[4];                                                              \
+      s[0] = fminf(round_bf16(round_bf16(acc[0]) + bias_g[16 * kt]), cap.x);   \
+      s[1] = fminf(round_bf16(round_bf16(acc[1]) + bias_g[16 * kt + 1]),       \
+                   cap.y);                                                     \
+      s[2] = fminf(round_bf16(round_bf16(acc[2]) + bias_g[16 * kt + 2]),       \
+                   cap.z);                                                     \
+      s[3] = fminf(round_bf16(round_bf16(acc[3]) + bias_g[16 * kt + 3]),       \
+                   cap.w);                                                     \
+      const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));            \
+      const float nm = fmaxf(m, tm);                                           \
+      float add = 0.f;                                                         \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) add += __expf(s[i] - nm);  \
+      l = l * __expf(m - nm) + add;                                            \
+      m = nm;                                                                  \
+      sc[kt][0] = pack_bf16x2(s[0], s[1]);                                     \
+      sc[kt][1] = pack_bf16x2(s[2], s[3]);                                     \
+    }                                                                          \
+  }
+
+  T5D_ENC_ISSUE_K(0, s_r0);
+  T5D_ENC_ISSUE_K(1, s_r1);
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    T5D_ENC_STEP(3 * r, s_r0, s_r2, T5D_ENC_ISSUE_K, T5D_ENC_SCORES)
+    T5D_ENC_STEP(3 * r + 1, s_r1, s_r0, T5D_ENC_ISSUE_K, T5D_ENC_SCORES)
+    T5D_ENC_STEP(3 * r + 2, s_r2, s_r1, T5D_ENC_ISSUE_K, T5D_ENC_SCORES)
+  }
+  // combine the 4 lanes (g) that share a query
+#pragma unroll
+  for (int o = 16; o <= 32; o <<= 1) {
+    const float om = __shfl_xor(m, o, 64), ol = __shfl_xor(l, o, 64);
+    const float nm = fmaxf(m, om);
+    l = l * __expf(m - nm) + ol * __expf(om - nm);
+    m = nm;
+  }
+  const float inv = 1.0f / l;
+
+  f32x4_e oc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_e){0.f, 0.f, 0.f, 0.f};
+  // V^T operand of a 32-key step: row d = 16 dt + l16, the 8 bytes of keys
+  // 4g .. 4g+3 and of keys 16+4g .. 16+4g+3 (pieces g / 2 and 2 + g / 2)
+  const int v_swz = (l16 >> 1) & 3;
+  const int v_off0 = l16 * 64 + (((gq >> 1) ^ v_swz) * 16) + (gq & 1) * 8;
+  const int v_off1 = l16 * 64 + (((2 + (gq >> 1)) ^ v_swz) * 16) + (gq & 1) * 8;
+  auto prob2 = [&](uint32_t packed) {
+    return pack_bf16x2(__expf(bf16lo_to_f32(packed) - m) * inv,
+                       __expf(bf16hi_to_f32(packed) - m) * inv);
+  };
+#define T5D_ENC_VALUES(i_, S_)                                                 \
+  _Pragma("unroll") for (int hb = 0; hb < 2; ++hb) {                           \
+    const int kt = 4 * (i_) + 2 * hb;                                          \
+    if (kt < my_tiles) {                                                       \
+      FragE pb;                                                                \
+      pb.u.x = prob2(sc[kt][0]);                                               \
+      pb.u.y = prob2(sc[kt][1]);                                               \
+      pb.u.z = prob2(sc[kt + 1][0]);                                           \
+      pb.u.w = prob2(sc[kt + 1][1]);                                           \
+      const char* blk = reinterpret_cast<const char*>(&S_[0]) + hb * 4096;     \
+      _Pragma("unroll") for (int dt = 0; dt < 4; ++dt) {                       \
+        const uint2 lo =                                                       \
+            *reinterpret_cast<const uint2*>(blk + dt * 1024 + v_off0);         \
+        const uint2 hi =                                                       \
+            *reinterpret_cast<const uint2*>(blk + dt * 1024 + v_off1);         \
+        FragE va;                                                              \
+        va.u = make_uint4(lo.x, lo.y, hi.x, hi.y);                             \
+        oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, oc[dt],   \
+                                                         0, 0, 0);             \
+      }                                                                        \
+    }                                                                          \
+  }
+  __builtin_amdgcn_s_waitcnt(0x070);
+  __builtin_amdgcn_s_barrier();  // every wavefront is done with the K stages
+  T5D_ENC_ISSUE_V(0, s_r0);
+  T5D_ENC_ISSUE_V(1, s_r1);
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    T5D_ENC_STEP(3 * r, s_r0, s_r2, T5D_ENC_ISSUE_V, T5D_ENC_VALUES)
+    T5D_ENC_STEP(3 * r + 1, s_r1, s_r0, T5D_ENC_ISSUE_V, T5D_ENC_VALUES)
+    T5D_ENC_STEP(3 * r + 2, s_r2, s_r1, T5D_ENC_ISSUE_V, T5D_ENC_VALUES)
+  }
+  // the loads issued past the last block must land before this workgroup's
+  // LDS can go to another
+  __builtin_amdgcn_s_waitcnt(0x070);
+#undef T5D_ENC_ISSUE_K
+#undef T5D_ENC_ISSUE_V
+#undef T5D_ENC_STEP
+#undef T5D_ENC_SCORES
+#undef T5D_ENC_VALUES
+  // oc[dt][i]: out[q = l16][d = 16 dt + 4 g + i]
+  if (q0 + l16 < E) {
+    bf16_t* o = a.out + (row0 + q0 + l16) * (size_t)(a.H * 64) + h * 64 + 4 * gq;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      uint2 pk;
+      pk.x = pack_bf16x2(oc[dt][0], oc[dt][1]);
+      pk.y = pack_bf16x2(oc[dt][2], oc[dt][3]);
+      *reinterpret_cast<uint2*>(o + 16 * dt) = pk;
+    }
+  }
+}
+
 // ---- float32 -------------------------------------------------------------------
 // The exactness-test dtype: plain vector arithmetic, one wavefront per query
 // row.  Scores (lane = key, ascending head dim), bias and mask summed first and
@@ -316,6 +592,21 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
                                      const uint32_t* valid_bits, void* out,
                                      int B, int H, int E, int Ep, int q_stride,
                                      int k_stride) {
+  return t5d_encoder_attention_variant(stream, q, k, v_t, rel_bias, enc_len,
+                                       valid_bits, out, B, H, E, Ep, q_stride,
+                                       k_stride, 0);
+}
+
+extern "C" int t5d_encoder_attention_variant(
+    void* stream, const void* q, const void* k, const void* v_t,
+    const void* rel_bias, const int32_t* enc_len, const uint32_t* valid_bits,
+    void* out, int B, int H, int E, int Ep, int q_stride, int k_stride,
+    int variant) {
+  T5D_REQUIRE(variant >= 0 && variant <= 2 && (variant != 2 || E <= 512),
+              T5D_EINVAL,
+              "t5d_encoder_attention_variant: variant %d (0 chosen here, 1 "
+              "scores formed twice, 2 scores kept in registers: E <= 512)",
+              variant);
   T5D_REQUIRE(q && k && v_t && rel_bias && enc_len && out, T5D_EINVAL,
               "t5d_encoder_attention: null pointer");
   T5D_REQUIRE(B > 0 && H > 0 && E > 0 && Ep >= E && Ep % 32 == 0,
@@ -338,7 +629,19 @@ extern "C" int t5d_encoder_attention(void* stream, const void* q, const void* k,
   a.valid = valid_bits;
   a.H = H; a.E = E; a.Ep = Ep; a.q_stride = q_stride; a.k_stride = k_stride;
   dim3 grid((E + 63) / 64, H, B), block(256);
-  hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
+  if (variant == 1)
+    hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
+  else if (E <= 128)
+    hipLaunchKernelGGL(enc_attn_ring_kernel<2>, grid, block, 0,
+                       as_stream(stream), a);
+  else if (E <= 256)
+    hipLaunchKernelGGL(enc_attn_ring_kernel<4>, grid, block, 0,
+                       as_stream(stream), a);
+  else if (E <= 512)
+    hipLaunchKernelGGL(enc_attn_ring_kernel<8>, grid, block, 0,
+                       as_stream(stream), a);
+  else
+    hipLaunchKernelGGL(enc_attn_kernel, grid, block, 0, as_stream(stream), a);
   T5D_CHECK_LAUNCH("t5d_encoder_attention");
   return T5D_OK;
 }

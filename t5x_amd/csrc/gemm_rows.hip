@@ -399,8 +399,16 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
   constexpr int AL = 16 / WAVES;        // activation tiles a wavefront loads per stage
   constexpr int WL = WN * NT / WAVES;   // weight tiles a wavefront loads per stage
   constexpr int TILES = 16 + WN * NT;
-  // all but my newest AL + WL loads have landed: s_waitcnt vmcnt(AL + WL)
-  constexpr int kWaitStage = 0xF70 | (AL + WL);
+  // Before every barrier: all but my newest AL + WL loads have landed AND all
+  // my reads of LDS have returned, s_waitcnt vmcnt(AL + WL) lgkmcnt(0).  The
+  // second half matters: the barrier orders instructions that have been
+  // issued, not LDS reads that have completed, and the compiler is free to
+  // sink the last operand reads and matrix instructions of a k-tile below the
+  // next barrier.  Without the wait a workgroup's fastest wavefront could
+  // refill the stage while the slowest still had reads of it queued (seen as
+  // one wrong 16-row slice in about one launch in ten at 16384 x 768).
+  constexpr int kWaitStage = 0x070 | (AL + WL);
+  constexpr int kWaitAll = 0x070;
   // [tile][lane]: tiles 0..15 activations (rows 16 t ..), then the weights
   __shared__ uint4 s_t0[TILES][64];
   __shared__ uint4 s_t1[TILES][64];
@@ -470,10 +478,11 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
       }                                                                        \
     }                                                                          \
   } while (0)
-  // s_waitcnt vmcnt(AL + WL): all but this wavefront's newest loads have landed,
-  // i.e. its share of the stage about to be multiplied; after the barrier
-  // every wavefront's share has, and every wavefront is done with the stage
-  // that the next loads overwrite.
+  // kWaitStage: all but this wavefront's newest loads have landed, i.e. its
+  // share of the stage about to be multiplied, and its reads of the previous
+  // stage have returned; after the barrier every wavefront's share has
+  // landed, and every wavefront is done with the stage that the next loads
+  // overwrite.
 #define T5D_ROWS_STEP(kt_, CUR_, NEXT2_)                                       \
   do {                                                                         \
     __builtin_amdgcn_s_waitcnt(kWaitStage);                                    \
@@ -485,7 +494,7 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
 #define T5D_ROWS_LAST(kt_, CUR_, NEXT2_)                                       \
   do {                                                                         \
     if ((kt_) + 1 < KT) __builtin_amdgcn_s_waitcnt(kWaitStage);                \
-    else __builtin_amdgcn_s_waitcnt(0xF70);                                    \
+    else __builtin_amdgcn_s_waitcnt(kWaitAll);                                 \
     __builtin_amdgcn_s_barrier();                                              \
     if ((kt_) + 2 < KT) T5D_ROWS_ISSUE((kt_) + 2, NEXT2_);                     \
     __builtin_amdgcn_sched_barrier(0);                                         \

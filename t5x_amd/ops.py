@@ -514,11 +514,14 @@ def pack_valid_bits(valid):
   return packed.to(torch.int32).contiguous()
 
 
-def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None, valid_bits=None):
+def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None, valid_bits=None,
+                      variant=0):
   """q, k: [B*E, >= H*64] row-major views (row stride = stride(0)); v_t
   [B, H, Ep/32, 64, 32] (tile_cross_value of [B, H, 64, Ep]); rel_bias
   [H, 2E-1]; enc_len [B]; valid_bits: None or pack_valid_bits of the
-  per-position mask -> out [B*E, H*64]."""
+  per-position mask -> out [B*E, H*64].  variant: 0 = chosen from E, 1 / 2 =
+  the kernel that forms the scores twice / keeps them in registers
+  (t5d_encoder_attention_variant)."""
   _chk(v_t, 'v_t', torch.bfloat16, 5)
   _chk(rel_bias, 'rel_bias', torch.bfloat16, 2)
   _chk(enc_len, 'enc_len', torch.int32, 1)
@@ -538,10 +541,10 @@ def encoder_attention(q, k, v_t, rel_bias, enc_len, out=None, valid_bits=None):
   if out is None:
     out = torch.empty((B * E, H * 64), dtype=torch.bfloat16, device=v_t.device)
   _chk(out, 'out', torch.bfloat16, 2)
-  _lib.call('t5d_encoder_attention', _s(), q.data_ptr(), k.data_ptr(),
+  _lib.call('t5d_encoder_attention_variant', _s(), q.data_ptr(), k.data_ptr(),
             v_t.data_ptr(), rel_bias.data_ptr(), enc_len.data_ptr(),
             _valid_bits(valid_bits, B, E), out.data_ptr(), B, H, E, Ep,
-            q.stride(0), k.stride(0))
+            q.stride(0), k.stride(0), int(variant))
   return out
 
 

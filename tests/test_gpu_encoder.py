@@ -92,6 +92,32 @@ def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
     _check_head_layouts(ops, rows, keys, vals, B, E, Ep, H)
 
 
+def test_gemm_rows_repeated_launches_at_full_size(ops):
+  """40 launches of each workgroup tile at the encoder's own size (16384 rows,
+  two workgroups per CU for tile 1) give one result.  A wavefront used to be
+  able to refill an LDS stage while another still had operand reads of it
+  queued: one 16-row slice of one launch in ten came out wrong."""
+  g = torch.Generator(device='cuda')
+  g.manual_seed(3)
+  a = torch.randn(16384, 768, device='cuda', generator=g).to(torch.bfloat16)
+  w0 = torch.randn(768, 768, device='cuda', generator=g) / 768**0.5
+  w1 = torch.randn(768, 768, device='cuda', generator=g) / 768**0.5
+  res = torch.randn(16384, 768, device='cuda', generator=g).to(torch.bfloat16)
+  gated = ops.pack_weight(w0, torch.bfloat16, gate_kernel=w1)
+  plain = ops.pack_weight(w0, torch.bfloat16)
+  want = (a.float() @ w0.to(torch.bfloat16).float()).to(torch.bfloat16).float()
+  want = (want + res.float()).to(torch.bfloat16).float()
+  for tile in (1, 2):
+    first = ops.gemm_rows(a, gated, tile=tile)
+    first_res = ops.gemm_rows(a, plain, residual=res, tile=tile)
+    err = (first_res.float() - want).abs()
+    assert bool((err <= 2e-2 + 2.0**-7 * want.abs()).all())
+    for _ in range(40):
+      assert torch.equal(ops.gemm_rows(a, gated, tile=tile), first)
+      assert torch.equal(ops.gemm_rows(a, plain, residual=res, tile=tile),
+                         first_res)
+
+
 def test_gemm_rows_plain_entry_point(ops):
   """t5d_gemm_rows itself (ops.gemm_rows goes through t5d_gemm_rows_tiled)."""
   from t5x_amd import _lib
@@ -117,6 +143,32 @@ def _check_head_layouts(ops, rows, keys, vals, B, E, Ep, H):
   assert tuple(vals.shape) == (B, H, Ep // 32, 64, 32)
   assert torch.equal(keys, ops.tile_cross_key(plain_k))
   assert torch.equal(vals, ops.tile_cross_value(plain_v))
+
+
+def _same_bits_from_both_kernels(ops, out, q, k, v_t, rel_bias, lens, bits):
+  """The kernel that forms the scores twice (any length) and the one that
+  keeps them in registers (lengths up to 512) form the same scores and
+  probabilities; only the order in which a 32-key step's products are summed
+  on the matrix cores differs, so outputs agree except for a rare last-bit
+  rounding (measured: 1 element in 4000)."""
+  E = (rel_bias.shape[1] + 1) // 2
+  twice = ops.encoder_attention(q, k, v_t, rel_bias, lens, valid_bits=bits,
+                                variant=1)
+  if E > 512:
+    assert torch.equal(out, twice)
+    with pytest.raises(ValueError):
+      ops.encoder_attention(q, k, v_t, rel_bias, lens, valid_bits=bits,
+                            variant=2)
+    return
+  kept = ops.encoder_attention(q, k, v_t, rel_bias, lens, valid_bits=bits,
+                               variant=2)
+  assert torch.equal(out, kept)
+  a, b = twice.float(), kept.float()
+  # one bfloat16 step of the value, or the float32 noise of a sum of
+  # magnitude ~1 where the value itself is nearly zero
+  one_ulp = 2.0**-7 * torch.maximum(a.abs(), b.abs()) + 1e-6
+  assert bool(((a - b).abs() <= one_ulp).all())
+  assert float((a != b).float().mean()) < 2e-3
 
 
 def _enc_attn_oracle(q, k, v, rel_emb, lens, valid=None):
@@ -161,6 +213,8 @@ def test_encoder_attention(ops, B, E, H):
   qk = qk.reshape(B * E, 2 * H * 64)                      # strided q | k views
   out = ops.encoder_attention(qk[:, :H * 64], qk[:, H * 64:], v_t, rel_bias,
                               dev(lens))
+  _same_bits_from_both_kernels(ops, out, qk[:, :H * 64], qk[:, H * 64:], v_t,
+                               rel_bias, dev(lens), None)
   got = host(out).reshape(B, E, H, 64)
   # rows of valid queries: to the attention tolerance; padded queries attend
   # uniformly in both (their values are never used downstream)
@@ -206,6 +260,7 @@ def test_encoder_attention_with_padding_inside_the_text(ops, B, E, H):
   kh = dev(k, torch.bfloat16).reshape(B * E, H * 64)
   out = ops.encoder_attention(qh, kh, v_t, rel_bias, dev(last),
                               valid_bits=bits)
+  _same_bits_from_both_kernels(ops, out, qh, kh, v_t, rel_bias, dev(last), bits)
   got = host(out).reshape(B, E, H, 64)
   np.testing.assert_allclose(got, want, atol=2e-2, rtol=2**-6)
   # float32 kernel, closed form
@@ -548,6 +603,9 @@ def test_encoder_attention_random_shapes(ops):
     out = ops.encoder_attention(q.reshape(B * E, H * 64), k.reshape(B * E, H * 64),
                                 ops.tile_cross_value(v_t), rel.contiguous(),
                                 dev(last), valid_bits=bits)
+    _same_bits_from_both_kernels(
+        ops, out, q.reshape(B * E, H * 64), k.reshape(B * E, H * 64),
+        ops.tile_cross_value(v_t), rel.contiguous(), dev(last), bits)
     idx = (torch.arange(E, device='cuda')[None, :] -
            torch.arange(E, device='cuda')[:, None] + E - 1)
     s = torch.einsum('bqhd,bkhd->bhqk', q.float(), k.float()).to(bf).float()
