@@ -476,7 +476,9 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
     want = ((B, H, 2, Ep, 32) if layout == _lib.OUT_HEADS_KEY else
             (B, H, Ep // 32, 64, 32))
     if out is None:
-      out = torch.zeros(want, dtype=a.dtype, device=a.device)
+      # positions e >= E are not written: they start at zero (none if Ep == E)
+      make = torch.empty if Ep == E else torch.zeros
+      out = make(want, dtype=a.dtype, device=a.device)
     if tuple(out.shape) != want:
       raise ValueError(f'out shape {tuple(out.shape)} != {want}')
   _chk(out, 'out', a.dtype)
