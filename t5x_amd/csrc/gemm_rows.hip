@@ -177,7 +177,9 @@ __device__ __forceinline__ void rows_epilogue(
 // or 8 lanes per row, 16 bytes per lane: every store instruction then writes
 // whole 64-byte (gated) or 128-byte rows, and the residual is read the same
 // way.  LDS operations of one wavefront complete in order, so the slices
-// follow one another through the same piece without a wait in between.
+// follow one another through the same piece without a wait in between; the
+// empty asm statements keep the compiler from moving one lane's read above
+// another lane's write (to it they are accesses of unrelated addresses).
 constexpr int kRowsStageBytes = 16 * 144;
 template <int NT>
 __device__ __forceinline__ void rows_epilogue_staged(
@@ -206,7 +208,9 @@ __device__ __forceinline__ void rows_epilogue_staged(
           *reinterpret_cast<uint2*>(stage + l16 * 80 + (8 * nt + 4 * gq) * 2) =
               pack4(h[0], h[1], h[2], h[3]);
       }
+      asm volatile("" ::: "memory");
       const uint4 q = *reinterpret_cast<const uint4*>(stage + row * 80 + piece * 16);
+      asm volatile("" ::: "memory");
       const int m = m0 + 16 * mt + row;
       if (m < g.M && nt0 + piece < n_tiles)
         *reinterpret_cast<uint4*>(g.C + (size_t)m * F + 8 * (nt0 + piece)) = q;
@@ -222,10 +226,17 @@ __device__ __forceinline__ void rows_epilogue_staged(
     for (int nt = 0; nt < NT; ++nt)
       *reinterpret_cast<uint2*>(stage + l16 * 144 + (16 * nt + 4 * gq) * 2) =
           pack4(acc[mt][nt][0], acc[mt][nt][1], acc[mt][nt][2], acc[mt][nt][3]);
+    asm volatile("" ::: "memory");
+    uint4 back[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      back[j] = *reinterpret_cast<const uint4*>(
+          stage + (8 * j + (lane >> 3)) * 144 + piece * 16);
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int row = 8 * j + (lane >> 3);
-      uint4 q = *reinterpret_cast<const uint4*>(stage + row * 144 + piece * 16);
+      uint4 q = back[j];
       const int m = m0 + 16 * mt + row;
       if (m >= g.M || !n_ok) continue;
       size_t o;
