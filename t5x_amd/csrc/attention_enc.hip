@@ -341,8 +341,10 @@ enc_attn_ring_kernel(EncAttnArgs a) {
                       (size_t)h * 128 + k_piece * 16;
   // ... and of a 64-key block of V^T (two [64 d][32 keys] blocks, 4 KB each):
   // chunks (16 rows d, 1 KB) wave and wave + 4; lane s lands at slot s & 3 of
-  // row s >> 2 and reads piece (s & 3) ^ ((row >> 1) & 3).
-  const int v_r = lane >> 2, v_piece = (lane & 3) ^ ((v_r >> 1) & 3);
+  // row s >> 2 and reads piece (s & 3) ^ ((row >> 1) & 1): one swizzle bit, so
+  // that the two pieces a lane needs in pass 2 (p and p + 2) stay 32 bytes
+  // apart and come with one two-address read, already in operand order.
+  const int v_r = lane >> 2, v_piece = (lane & 3) ^ ((v_r >> 1) & 1);
   const char* vbase = reinterpret_cast<const char*>(a.vt) +
                       ((size_t)b * a.H + h) * 128 * (size_t)a.Ep;
   const int v_blocks = a.Ep >> 5;
@@ -395,7 +397,9 @@ enc_attn_ring_kernel(EncAttnArgs a) {
 #define T5D_ENC_SCORES(i_, S_)                                                 \
   _Pragma("unroll") for (int t = 0; t < 4; ++t) {                              \
     const int kt = 4 * (i_) + t;                                               \
-    if (kt < my_tiles) {                                                       \
+    /* two key tiles per test: their chains of dependent instructions (LDS   \
+       read, matrix instruction, rounding, exp) interleave */                 \
+    if ((kt & ~1) < my_tiles) {                                                \
       f32x4_e acc = (f32x4_e){0.f, 0.f, 0.f, 0.f};                             \
       _Pragma("unroll") for (int c = 0; c < 2; ++c) {                          \
         FragE kop;                                                             \
@@ -404,14 +408,21 @@ enc_attn_ring_kernel(EncAttnArgs a) {
                                                       0, 0);                   \
       }                                                                        \
       const float4 cap = *reinterpret_cast<const float4*>(lim_g + 16 * kt);    \
+      /* two values per rounding instruction; the cap as a median with -inf   \
+         (one instruction: fminf would first make both operands canonical) */ \
+      const uint32_t r01 = pack_bf16x2(acc[0], acc[1]);                        \
+      const uint32_t r23 = pack_bf16x2(acc[2], acc[3]);                        \
+      const uint32_t x01 =                                                     \
+          pack_bf16x2(bf16lo_to_f32(r01) + bias_g[16 * kt],                    \
+                      bf16hi_to_f32(r01) + bias_g[16 * kt + 1]);               \
+      const uint32_t x23 =                                                     \
+          pack_bf16x2(bf16lo_to_f32(r23) + bias_g[16 * kt + 2],                \
+                      bf16hi_to_f32(r23) + bias_g[16 * kt + 3]);               \
       float s[4];                                                              \
-      s[0] = fminf(round_bf16(round_bf16(acc[0]) + bias_g[16 * kt]), cap.x);   \
-      s[1] = fminf(round_bf16(round_bf16(acc[1]) + bias_g[16 * kt + 1]),       \
-                   cap.y);                                                     \
-      s[2] = fminf(round_bf16(round_bf16(acc[2]) + bias_g[16 * kt + 2]),       \
-                   cap.z);                                                     \
-      s[3] = fminf(round_bf16(round_bf16(acc[3]) + bias_g[16 * kt + 3]),       \
-                   cap.w);                                                     \
+      s[0] = __builtin_amdgcn_fmed3f(bf16lo_to_f32(x01), cap.x, -INFINITY);    \
+      s[1] = __builtin_amdgcn_fmed3f(bf16hi_to_f32(x01), cap.y, -INFINITY);    \
+      s[2] = __builtin_amdgcn_fmed3f(bf16lo_to_f32(x23), cap.z, -INFINITY);    \
+      s[3] = __builtin_amdgcn_fmed3f(bf16hi_to_f32(x23), cap.w, -INFINITY);    \
       const float tm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));            \
       const float nm = fmaxf(m, tm);                                           \
       float add = 0.f;                                                         \
@@ -446,9 +457,8 @@ enc_attn_ring_kernel(EncAttnArgs a) {
   for (int dt = 0; dt < 4; ++dt) oc[dt] = (f32x4_e){0.f, 0.f, 0.f, 0.f};
   // V^T operand of a 32-key step: row d = 16 dt + l16, the 8 bytes of keys
   // 4g .. 4g+3 and of keys 16+4g .. 16+4g+3 (pieces g / 2 and 2 + g / 2)
-  const int v_swz = (l16 >> 1) & 3;
+  const int v_swz = (l16 >> 1) & 1;
   const int v_off0 = l16 * 64 + (((gq >> 1) ^ v_swz) * 16) + (gq & 1) * 8;
-  const int v_off1 = l16 * 64 + (((2 + (gq >> 1)) ^ v_swz) * 16) + (gq & 1) * 8;
   auto prob2 = [&](uint32_t packed) {
     return pack_bf16x2(__expf(bf16lo_to_f32(packed) - m) * inv,
                        __expf(bf16hi_to_f32(packed) - m) * inv);
@@ -456,7 +466,7 @@ enc_attn_ring_kernel(EncAttnArgs a) {
 #define T5D_ENC_VALUES(i_, S_)                                                 \
   _Pragma("unroll") for (int hb = 0; hb < 2; ++hb) {                           \
     const int kt = 4 * (i_) + 2 * hb;                                          \
-    if (kt < my_tiles) {                                                       \
+    {                                                                          \
       FragE pb;                                                                \
       pb.u.x = prob2(sc[kt][0]);                                               \
       pb.u.y = prob2(sc[kt][1]);                                               \
@@ -464,10 +474,9 @@ enc_attn_ring_kernel(EncAttnArgs a) {
       pb.u.w = prob2(sc[kt + 1][1]);                                           \
       const char* blk = reinterpret_cast<const char*>(&S_[0]) + hb * 4096;     \
       _Pragma("unroll") for (int dt = 0; dt < 4; ++dt) {                       \
-        const uint2 lo =                                                       \
-            *reinterpret_cast<const uint2*>(blk + dt * 1024 + v_off0);         \
-        const uint2 hi =                                                       \
-            *reinterpret_cast<const uint2*>(blk + dt * 1024 + v_off1);         \
+        const uint2* vp =                                                      \
+            reinterpret_cast<const uint2*>(blk + dt * 1024 + v_off0);          \
+        const uint2 lo = vp[0], hi = vp[4];                                    \
         FragE va;                                                              \
         va.u = make_uint4(lo.x, lo.y, hi.x, hi.y);                             \
         oc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, oc[dt],   \
