@@ -168,7 +168,7 @@ def _same_bits_from_both_kernels(ops, out, q, k, v_t, rel_bias, lens, bits):
   # magnitude ~1 where the value itself is nearly zero
   one_ulp = 2.0**-7 * torch.maximum(a.abs(), b.abs()) + 1e-6
   assert bool(((a - b).abs() <= one_ulp).all())
-  assert float((a != b).float().mean()) < 2e-3
+  assert int((a != b).sum()) <= max(2, 2e-3 * a.numel())
 
 
 def _enc_attn_oracle(q, k, v, rel_emb, lens, valid=None):
