@@ -191,22 +191,33 @@ __device__ __forceinline__ void rows_epilogue_staged(
   if (g.epilogue == T5D_EPI_GEGLU) {
     // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the lanes
     // with gq >= 2 hold the gates of the lanes with gq - 2.  32 output columns.
+    // Two v_permlane32_swap hand every lane two (value, gate) pairs — the
+    // lower half of the wavefront keeps its values 2, 3 and receives their
+    // gates, the upper half keeps its gates 0, 1 and receives their values —
+    // so all 64 lanes evaluate GELU on values that are used.
     const int F = g.N >> 1;
     const int row = lane >> 2, piece = lane & 3;
+    const bool lower = gq < 2;
+    const int col0 = 4 * (gq & 1) + (lower ? 2 : 0);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        float h[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = acc[mt][nt][i];
-          const float gate = __shfl_xor(v, 32, 64);
-          h[i] = round_bf16(gelu_sigmoid_form(round_bf16(v))) * round_bf16(gate);
-        }
-        if (gq < 2)
-          *reinterpret_cast<uint2*>(stage + l16 * 80 + (8 * nt + 4 * gq) * 2) =
-              pack4(h[0], h[1], h[2], h[3]);
+        const auto a = __builtin_amdgcn_permlane32_swap(
+            __float_as_uint(acc[mt][nt][2]), __float_as_uint(acc[mt][nt][0]),
+            false, false);
+        const auto b = __builtin_amdgcn_permlane32_swap(
+            __float_as_uint(acc[mt][nt][3]), __float_as_uint(acc[mt][nt][1]),
+            false, false);
+        // [0]: the value (own in the lower half), [1]: its gate
+        const float h0 =
+            round_bf16(gelu_sigmoid_form(round_bf16(__uint_as_float(a[0])))) *
+            round_bf16(__uint_as_float(a[1]));
+        const float h1 =
+            round_bf16(gelu_sigmoid_form(round_bf16(__uint_as_float(b[0])))) *
+            round_bf16(__uint_as_float(b[1]));
+        *reinterpret_cast<uint32_t*>(stage + l16 * 80 + (8 * nt + col0) * 2) =
+            pack_bf16x2(h0, h1);
       }
       asm volatile("" ::: "memory");
       const uint4 q = *reinterpret_cast<const uint4*>(stage + row * 80 + piece * 16);
