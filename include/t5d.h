@@ -163,10 +163,10 @@ int t5d_gemm_rows(void* stream, int w_dtype, const void* A, const void* W,
 
 /* t5d_gemm_rows with the workgroup tile of the caller's choice: tile 1 =
  * 256 rows x 128 columns (4 wavefronts, two workgroups per CU), tile 2 =
- * 256 x 256 (8 wavefronts; bfloat16 weights and K >= 64, otherwise tile 1 is
- * used), tile 0 = what t5d_gemm_rows picks from the shape.  Results have the
- * same bits for every tile.  For tuning and for testing both kernels at any
- * size. */
+ * 256 x 256 and tile 3 = 256 x 192 (8 wavefronts, one workgroup per CU;
+ * bfloat16 weights and K >= 64, otherwise tile 1 is used), tile 0 = what
+ * t5d_gemm_rows picks from the shape.  Results have the same bits for every
+ * tile.  For tuning and for testing every kernel at any size. */
 int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
                         const void* W, const float* scales,
                         const void* residual, void* C, int64_t M, int K, int N,

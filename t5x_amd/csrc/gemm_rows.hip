@@ -185,7 +185,7 @@ template <int NT>
 __device__ __forceinline__ void rows_epilogue_staged(
     const RowsGemmArgs& g, const f32x4_r (&acc)[kRowsMT][NT], int m0, int nt0,
     int n_tiles, int lane, char* stage) {
-  static_assert(NT == 4, "a wavefront's slice is 64 columns wide");
+  static_assert(NT == 3 || NT == 4, "a wavefront's slice: 48 or 64 columns");
   constexpr int MT = kRowsMT;
   const int l16 = lane & 15, gq = lane >> 4;
   if (g.epilogue == T5D_EPI_GEGLU) {
@@ -196,7 +196,7 @@ __device__ __forceinline__ void rows_epilogue_staged(
     // gates, the upper half keeps its gates 0, 1 and receives their values —
     // so all 64 lanes evaluate GELU on values that are used.
     const int F = g.N >> 1;
-    const int row = lane >> 2, piece = lane & 3;
+    const int row = lane / NT, piece = lane % NT;  // NT 16-byte pieces per row
     const bool lower = gq < 2;
     const int col0 = 4 * (gq & 1) + (lower ? 2 : 0);
 #pragma unroll
@@ -220,15 +220,18 @@ __device__ __forceinline__ void rows_epilogue_staged(
             pack_bf16x2(h0, h1);
       }
       asm volatile("" ::: "memory");
-      const uint4 q = *reinterpret_cast<const uint4*>(stage + row * 80 + piece * 16);
+      const uint4 q = *reinterpret_cast<const uint4*>(
+          stage + min(row, 15) * 80 + piece * 16);
       asm volatile("" ::: "memory");
       const int m = m0 + 16 * mt + row;
-      if (m < g.M && nt0 + piece < n_tiles)
+      if (row < 16 && m < g.M && nt0 + piece < n_tiles)
         *reinterpret_cast<uint4*>(g.C + (size_t)m * F + 8 * (nt0 + piece)) = q;
     }
     return;
   }
-  const int piece = lane & 7;
+  constexpr int PP = 2 * NT;    // 16-byte pieces per row of the slice
+  constexpr int RPI = 64 / PP;  // rows per instruction (8, or 10 with 4 lanes idle)
+  const int piece = lane % PP, prow = lane / PP;
   const int n = 16 * nt0 + 8 * piece;
   const bool n_ok = nt0 + (piece >> 1) < n_tiles;
 #pragma unroll
@@ -242,11 +245,12 @@ __device__ __forceinline__ void rows_epilogue_staged(
 #pragma unroll
     for (int j = 0; j < 2; ++j)
       back[j] = *reinterpret_cast<const uint4*>(
-          stage + (8 * j + (lane >> 3)) * 144 + piece * 16);
+          stage + min(RPI * j + prow, 15) * 144 + piece * 16);
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int row = 8 * j + (lane >> 3);
+      const int row = RPI * j + prow;
+      if (prow >= RPI || row >= 16) continue;
       uint4 q = back[j];
       const int m = m0 + 16 * mt + row;
       if (m >= g.M || !n_ok) continue;
@@ -419,7 +423,10 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
   constexpr int WAVES = 2 * WN;         // 2 rows of WN wavefronts
   constexpr int BN = WN * NT * 16;      // columns of the workgroup tile
   constexpr int AL = 16 / WAVES;        // activation tiles a wavefront loads per stage
-  constexpr int WL = WN * NT / WAVES;   // weight tiles a wavefront loads per stage
+  constexpr int WTILES = WN * NT;       // weight tiles of a stage
+  // weight tiles a wavefront loads per stage; when they do not divide evenly
+  // some wavefronts load a tile a second time (same bytes to the same place)
+  constexpr int WL = (WTILES + WAVES - 1) / WAVES;
   constexpr int TILES = 16 + WN * NT;
   // Before every barrier: all but my newest AL + WL loads have landed AND all
   // my reads of LDS have returned, s_waitcnt vmcnt(AL + WL) lgkmcnt(0).  The
@@ -462,7 +469,8 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
             g.K + 8 * ld_piece);
 #pragma unroll
   for (int i = 0; i < WL; ++i)
-    wtile[i] = g.W + (size_t)min(n_blk * (BN / 16) + wave + WAVES * i,
+    wtile[i] = g.W + (size_t)min(n_blk * (BN / 16) +
+                                     (wave + WAVES * i) % WTILES,
                                  n_tiles - 1) * KT * 1024 + lane * 16;
 
   f32x4_r acc[MT][NT];
@@ -480,7 +488,7 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
     _Pragma("unroll") for (int i = 0; i < WL; ++i)                             \
       __builtin_amdgcn_global_load_lds(                                        \
           (glb_ptr_t)(wtile[i] + (size_t)(kt_) * 1024),                        \
-          (lds_ptr_t)&S_[16 + wave + WAVES * i][0], 16, 0, 0);                 \
+          (lds_ptr_t)&S_[16 + (wave + WAVES * i) % WTILES][0], 16, 0, 0);      \
   } while (0)
 #define T5D_ROWS_MULTIPLY(S_)                                                  \
   do {                                                                         \
@@ -570,9 +578,9 @@ extern "C" int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
                                    int K, int N, int epilogue, int out_layout,
                                    int E, int Ep, int tile) {
   T5D_REQUIRE(A && W && C, T5D_EINVAL, "t5d_gemm_rows: null pointer");
-  T5D_REQUIRE(tile >= 0 && tile <= 2, T5D_EINVAL,
+  T5D_REQUIRE(tile >= 0 && tile <= 3, T5D_EINVAL,
               "t5d_gemm_rows_tiled: tile %d (0 chosen here, 1: 256 x 128, "
-              "2: 256 x 256)", tile);
+              "2: 256 x 256, 3: 256 x 192)", tile);
   T5D_REQUIRE(w_dtype == T5D_BF16 || w_dtype == T5D_I8, T5D_EINVAL,
               "t5d_gemm_rows: w_dtype %d (packed bfloat16 or int8)", w_dtype);
   T5D_REQUIRE(w_dtype != T5D_I8 || scales, T5D_EINVAL,
@@ -612,16 +620,41 @@ extern "C" int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
   dim3 grid((unsigned)m_blocks * n_blocks), block(256);
   hipStream_t s = as_stream(stream);
   const bool swap = out_layout != T5D_OUT_HEADS_VALUE;
-  // 256 x 256 tiles (8 wavefronts, one workgroup per CU) halve the operand
-  // bytes per flop and measure 3-11 % faster than 256 x 128 whenever their
-  // workgroups fill the 256 CUs evenly; with a ragged last round (1.5 or 5.5
-  // rounds) the smaller tile, two workgroups per CU, loses less to the tail.
-  const int n_wide = (N + 2 * kRowsBN - 1) / (2 * kRowsBN);
-  const int wide_wgs = m_blocks * n_wide, tail = wide_wgs % 256;
-  const bool wide =
-      tile ? tile == 2 : (wide_wgs <= 256 || tail == 0 || tail >= 192);
-  if (w_dtype == T5D_BF16 && K >= 64 && wide) {
-    dim3 wgrid((unsigned)wide_wgs), wblock(512);
+  // Three workgroup tiles.  256 x 256 (8 wavefronts, one workgroup per CU)
+  // halves the operand bytes per flop of 256 x 128 (4 wavefronts, two per CU)
+  // and measures 3-11 % faster whenever its workgroups fill the 256 CUs
+  // evenly; 256 x 192 (8 wavefronts of 128 x 48) is for the shapes where
+  // neither does: N = 768 over 16384 rows is 192 tiles of 256 x 256 (a quarter
+  // of the chip idle) but exactly 256 of 256 x 192.  Picked by the cost of the
+  // rounds each tile needs, a last round that fills at most half of the CUs'
+  // two slots counting 0.6 for the 256 x 128 tile.
+  const auto rounds = [](int wgs, int slots) {
+    return (wgs + slots - 1) / slots;
+  };
+  const int n192 = (N + 191) / 192, n256 = (N + 255) / 256;
+  const int wgs128 = m_blocks * n_blocks, wgs192 = m_blocks * n192,
+            wgs256 = m_blocks * n256;
+  double c128 = rounds(wgs128, 512) * 2.0 * 128;
+  if ((wgs128 - 1) % 512 < 256) c128 -= 0.4 * 2.0 * 128;
+  const double c192 = rounds(wgs192, 256) * 192.0,
+               c256 = rounds(wgs256, 256) * 256.0;
+  int pick = tile;
+  if (pick == 0) {
+    pick = 2;
+    double best = c256;
+    if (c192 < best) { best = c192; pick = 3; }
+    if (c128 < 0.97 * best) pick = 1;
+  }
+  if (w_dtype == T5D_BF16 && K >= 64 && pick == 3) {
+    dim3 wgrid((unsigned)wgs192), wblock(512);
+    if (swap)
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<true, 3, 4>), wgrid, wblock,
+                         0, s, g);
+    else
+      hipLaunchKernelGGL((rows_gemm_direct_kernel<false, 3, 4>), wgrid, wblock,
+                         0, s, g);
+  } else if (w_dtype == T5D_BF16 && K >= 64 && pick == 2) {
+    dim3 wgrid((unsigned)wgs256), wblock(512);
     if (swap)
       hipLaunchKernelGGL((rows_gemm_direct_kernel<true, kRowsNT, 4>), wgrid,
                          wblock, 0, s, g);

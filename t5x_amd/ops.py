@@ -459,7 +459,8 @@ def gemm_rows(a, w: PackedWeight, out=None, residual=None,
   """Dense layer over any number of rows (bfloat16).  layout OUT_HEADS_KEY /
   OUT_HEADS_VALUE writes [B, H, 2, Ep, 32] / [B, H, Ep/32, 64, 32] (rows
   m = b*E + e; Ep a multiple of 32, positions e >= E stay zero).  tile: 0 =
-  chosen from the shape, 1 = 256 x 128, 2 = 256 x 256 (t5d_gemm_rows_tiled)."""
+  chosen from the shape, 1 = 256 x 128, 2 = 256 x 256, 3 = 256 x 192
+  (t5d_gemm_rows_tiled)."""
   _chk(a, 'a', torch.bfloat16, 2)
   M, K = a.shape
   if K != w.K or w.w_dtype == F32:

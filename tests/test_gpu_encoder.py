@@ -45,6 +45,7 @@ def test_gemm_rows(ops, M, K, N, mode):
     pw = ops.pack_weight(dev(w0), torch.bfloat16, wd, gate_kernel=dev(w1))
     out = ops.gemm_rows(a, pw, tile=1)
     wide = ops.gemm_rows(a, pw, tile=2)
+    mid = ops.gemm_rows(a, pw, tile=3)
     want = ot5.mlp_block({'wi_0': {'kernel': q0}, 'wi_1': {'kernel': q1},
                           'wo': {'kernel': np.eye(N, dtype=np.float32)}},
                          host(a), ('gelu', 'linear'), 'bfloat16')
@@ -57,11 +58,13 @@ def test_gemm_rows(ops, M, K, N, mode):
       want = ot5.bf16_round(want + host(res))
     out = ops.gemm_rows(a, pw, residual=res, tile=1)
     wide = ops.gemm_rows(a, pw, residual=res, tile=2)
+    mid = ops.gemm_rows(a, pw, residual=res, tile=3)
   assert out.shape == want.shape
   np.testing.assert_allclose(host(out), want, atol=2e-2, rtol=2**-7)
-  # both workgroup tiles (256 x 128, 256 x 256) and the one picked from the
-  # shape give the same bits
+  # every workgroup tile (256 x 128, 256 x 256, 256 x 192) and the one picked
+  # from the shape give the same bits
   assert torch.equal(out, wide)
+  assert torch.equal(out, mid)
   chosen = ops.gemm_rows(a, pw, residual=None if mode != 'residual' else res)
   assert torch.equal(out, chosen)
   if M <= 128 and not mode.startswith('int8'):
@@ -84,7 +87,7 @@ def test_gemm_rows_head_layouts(ops, B, E, Ep, H, d):
   from t5x_amd import _lib
   pw = ops.pack_weight(w, torch.bfloat16)
   rows = ops.gemm_rows(x, pw).view(B, E, H, 64)
-  for tile in (1, 2):
+  for tile in (1, 2, 3):
     keys = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_KEY, E=E, Ep=Ep,
                          tile=tile)
     vals = ops.gemm_rows(x, pw, layout=_lib.OUT_HEADS_VALUE, E=E, Ep=Ep,
@@ -107,7 +110,7 @@ def test_gemm_rows_repeated_launches_at_full_size(ops):
   plain = ops.pack_weight(w0, torch.bfloat16)
   want = (a.float() @ w0.to(torch.bfloat16).float()).to(torch.bfloat16).float()
   want = (want + res.float()).to(torch.bfloat16).float()
-  for tile in (1, 2):
+  for tile in (1, 2, 3):
     first = ops.gemm_rows(a, gated, tile=tile)
     first_res = ops.gemm_rows(a, plain, residual=res, tile=tile)
     err = (first_res.float() - want).abs()
@@ -131,7 +134,7 @@ def test_gemm_rows_plain_entry_point(ops):
             _lib.EPI_NONE, _lib.OUT_ROWS, 0, 0)
   assert torch.equal(out, ops.gemm_rows(a, pw))
   with pytest.raises(ValueError):
-    ops.gemm_rows(a, pw, tile=3)
+    ops.gemm_rows(a, pw, tile=4)
 
 
 def _check_head_layouts(ops, rows, keys, vals, B, E, Ep, H):
@@ -535,7 +538,7 @@ def test_cross_kv_projection_layouts_match_oracle():
 
 
 def test_gemm_rows_random_shapes_and_repeated_launches(ops):
-  """t5d_gemm_rows (both workgroup tiles) over 30 random shapes (rows 1..3000, K a multiple of 32
+  """t5d_gemm_rows (every workgroup tile) over 30 random shapes (rows 1..3000, K a multiple of 32
   from 64 to 4096, i.e. 2 to 128 rounds of its ring of LDS stages, N a
   multiple of 16 up to 4096, with and without a residual) against float32
   products of the same operands on the device, and launched three times:
@@ -556,13 +559,15 @@ def test_gemm_rows_random_shapes_and_repeated_launches(ops):
         torch.bfloat16).float()
     if with_res:
       want = (want + res.float()).to(torch.bfloat16).float()
-    outs = [ops.gemm_rows(a, pw, residual=res, tile=1 + case % 2)
+    outs = [ops.gemm_rows(a, pw, residual=res, tile=1 + case % 3)
             for _ in range(3)]
-    other = ops.gemm_rows(a, pw, residual=res, tile=2 - case % 2)
+    others = [ops.gemm_rows(a, pw, residual=res, tile=1 + (case + d) % 3)
+              for d in (1, 2)]
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), (
         case, M, K, N)
-    assert torch.equal(outs[0], other), (case, M, K, N)
+    assert torch.equal(outs[0], others[0]), (case, M, K, N)
+    assert torch.equal(outs[0], others[1]), (case, M, K, N)
     err = (outs[0].float() - want).abs()
     ok = err <= 2e-2 + 2.0**-7 * want.abs()
     assert bool(ok.all()), (case, M, K, N, with_res, float(err.max()))
