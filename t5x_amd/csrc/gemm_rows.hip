@@ -82,96 +82,40 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
 constexpr int kRowsBM = 256, kRowsBN = 128;  // workgroup tile
 constexpr int kRowsMT = 8, kRowsNT = 4;        // MFMA tiles per wavefront
 
-// What a wavefront does with its finished 8 x 4 accumulator tiles (m0: its
-// first row, nt0: its first 16-column tile).
-template <bool SWAP, int NT>
-__device__ __forceinline__ void rows_epilogue(
+// What a wavefront does with its finished accumulator tiles (m0: its first
+// row, nt0: its first 16-column tile) when the product was formed as C, for
+// the value layout:
+template <int NT>
+__device__ __forceinline__ void rows_epilogue_values(
     const RowsGemmArgs& g, const f32x4_r (&acc)[kRowsMT][NT], int m0,
     int nt0, int n_tiles, int l16, int gq) {
   constexpr int MT = kRowsMT;
-  if (SWAP) {
-    // acc[mt][nt][i]: row m = m0 + 16 mt + l16, column n = 16 (nt0 + nt) + 4 gq + i
+  // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
+  // (values layout [B, H, Ep / 32, 64, 32]: 4 consecutive positions per store)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = m0 + 16 * mt + l16;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + 16 * mt + 4 * gq;
+    if (m >= g.M) continue;
+    const int b = m / g.E, e = m - b * g.E;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        if (nt0 + nt >= n_tiles) continue;
-        const int n = 16 * (nt0 + nt) + 4 * gq;
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][i];
-        if (g.scales) {
-          const float4 sc = *reinterpret_cast<const float4*>(g.scales + n);
-          v[0] *= sc.x; v[1] *= sc.y; v[2] *= sc.z; v[3] *= sc.w;
-        }
-        if (g.epilogue == T5D_EPI_GEGLU) {
-          // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the
-          // lanes with gq >= 2 hold the gates of the lanes with gq - 2.
-          float gate[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) gate[i] = __shfl_xor(v[i], 32, 64);
-          if (gq < 2 && m < g.M) {
-            float h[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              h[i] = round_bf16(round_bf16(gelu_sigmoid_form(round_bf16(v[i]))) *
-                                round_bf16(gate[i]));
-            const int F = g.N >> 1;
-            *reinterpret_cast<uint2*>(g.C + (size_t)m * F + 8 * (nt0 + nt) +
-                                      4 * gq) = pack4(h[0], h[1], h[2], h[3]);
-          }
-          continue;
-        }
-        if (m >= g.M) continue;
-        size_t o;
-        if (g.layout == T5D_OUT_HEADS_KEY) {
-          // [B, H, 2, Ep, 32]: the two 32-wide halves of the head dim as planes
-          const int b = m / g.E, e = m - b * g.E;
-          const int hh = n >> 6, c = (n >> 5) & 1, j = n & 31;
-          o = ((((size_t)b * g.H + hh) * 2 + c) * g.Ep + e) * 32 + j;
-        } else {
-          o = (size_t)m * g.N + n;
-        }
-        if (g.epilogue == T5D_EPI_RESIDUAL) {
-          const uint2 r = *reinterpret_cast<const uint2*>(
-              g.residual + (size_t)m * g.N + n);
-          v[0] = round_bf16(v[0]) + bf16lo_to_f32(r.x);
-          v[1] = round_bf16(v[1]) + bf16hi_to_f32(r.x);
-          v[2] = round_bf16(v[2]) + bf16lo_to_f32(r.y);
-          v[3] = round_bf16(v[3]) + bf16hi_to_f32(r.y);
-        }
-        *reinterpret_cast<uint2*>(g.C + o) = pack4(v[0], v[1], v[2], v[3]);
-      }
-    }
-  } else {
-    // acc[mt][nt][i]: row m = m0 + 16 mt + 4 gq + i, column n = 16 (nt0 + nt) + l16
-    // (values layout [B, H, Ep / 32, 64, 32]: 4 consecutive positions per store)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = m0 + 16 * mt + 4 * gq;
-      if (m >= g.M) continue;
-      const int b = m / g.E, e = m - b * g.E;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        if (nt0 + nt >= n_tiles) continue;
-        const int n = 16 * (nt0 + nt) + l16;
-        float s = g.scales ? g.scales[n] : 1.f;
-        const int hh = n >> 6, d = n & 63;
-        const size_t o =
-            ((((size_t)b * g.H + hh) * (g.Ep >> 5) + (e >> 5)) * 64 + d) * 32 +
-            (e & 31);
-        *reinterpret_cast<uint2*>(g.C + o) =
-            pack4(acc[mt][nt][0] * s, acc[mt][nt][1] * s, acc[mt][nt][2] * s,
-                  acc[mt][nt][3] * s);
-      }
+    for (int nt = 0; nt < NT; ++nt) {
+      if (nt0 + nt >= n_tiles) continue;
+      const int n = 16 * (nt0 + nt) + l16;
+      float s = g.scales ? g.scales[n] : 1.f;
+      const int hh = n >> 6, d = n & 63;
+      const size_t o =
+          ((((size_t)b * g.H + hh) * (g.Ep >> 5) + (e >> 5)) * 64 + d) * 32 +
+          (e & 31);
+      *reinterpret_cast<uint2*>(g.C + o) =
+          pack4(acc[mt][nt][0] * s, acc[mt][nt][1] * s, acc[mt][nt][2] * s,
+                acc[mt][nt][3] * s);
     }
   }
 }
 
-// Epilogue of the C^T form (bfloat16 weights, no scales) with the stores
-// made whole: a lane holds 4 consecutive columns of one row, so storing from
-// the accumulators writes 16 rows x 8..32 bytes per instruction.  Each
+// ... and when it was formed as C^T, with the stores made whole: a lane holds
+// 4 consecutive columns of one row, so storing from the accumulators would
+// write 16 rows x 8..32 bytes per instruction.  Each
 // wavefront instead parks one 16-row slice at a time in a private piece of
 // LDS (rounded to bfloat16, rows padded by 16 bytes) and reads it back with 4
 // or 8 lanes per row, 16 bytes per lane: every store instruction then writes
@@ -188,6 +132,14 @@ __device__ __forceinline__ void rows_epilogue_staged(
   static_assert(NT == 3 || NT == 4, "a wavefront's slice: 48 or 64 columns");
   constexpr int MT = kRowsMT;
   const int l16 = lane & 15, gq = lane >> 4;
+  // int8 weights: the scale of each of this lane's 4 columns (1 otherwise)
+  float4 sc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+    sc[nt] = (g.scales && nt0 + nt < n_tiles)
+                 ? *reinterpret_cast<const float4*>(g.scales +
+                                                    16 * (nt0 + nt) + 4 * gq)
+                 : make_float4(1.f, 1.f, 1.f, 1.f);
   if (g.epilogue == T5D_EPI_GEGLU) {
     // tile columns 0..7 are wi_0, 8..15 the matching wi_1 columns: the lanes
     // with gq >= 2 hold the gates of the lanes with gq - 2.  32 output columns.
@@ -204,11 +156,11 @@ __device__ __forceinline__ void rows_epilogue_staged(
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const auto a = __builtin_amdgcn_permlane32_swap(
-            __float_as_uint(acc[mt][nt][2]), __float_as_uint(acc[mt][nt][0]),
-            false, false);
+            __float_as_uint(acc[mt][nt][2] * sc[nt].z),
+            __float_as_uint(acc[mt][nt][0] * sc[nt].x), false, false);
         const auto b = __builtin_amdgcn_permlane32_swap(
-            __float_as_uint(acc[mt][nt][3]), __float_as_uint(acc[mt][nt][1]),
-            false, false);
+            __float_as_uint(acc[mt][nt][3] * sc[nt].w),
+            __float_as_uint(acc[mt][nt][1] * sc[nt].y), false, false);
         // [0]: the value (own in the lower half), [1]: its gate
         const float h0 =
             round_bf16(gelu_sigmoid_form(round_bf16(__uint_as_float(a[0])))) *
@@ -239,7 +191,8 @@ __device__ __forceinline__ void rows_epilogue_staged(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       *reinterpret_cast<uint2*>(stage + l16 * 144 + (16 * nt + 4 * gq) * 2) =
-          pack4(acc[mt][nt][0], acc[mt][nt][1], acc[mt][nt][2], acc[mt][nt][3]);
+          pack4(acc[mt][nt][0] * sc[nt].x, acc[mt][nt][1] * sc[nt].y,
+                acc[mt][nt][2] * sc[nt].z, acc[mt][nt][3] * sc[nt].w);
     asm volatile("" ::: "memory");
     uint4 back[2];
 #pragma unroll
@@ -381,7 +334,15 @@ rows_gemm_kernel(RowsGemmArgs g) {
 #undef T5D_ROWS_FETCH
 #undef T5D_ROWS_PARK
 
-  rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+  if (SWAP) {
+    // (the loop ends with a barrier: every wavefront is done with the tiles)
+    static_assert(sizeof(s_t[0]) >= 4 * kRowsStageBytes, "stage too small");
+    rows_epilogue_staged<NT>(
+        g, acc, m0, nt0, n_tiles, lane,
+        reinterpret_cast<char*>(&s_t[0][0][0]) + wave * kRowsStageBytes);
+  } else {
+    rows_epilogue_values<NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+  }
 }
 
 // ---- the same tile with operands loaded straight into LDS ---------------------
@@ -555,7 +516,7 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
         g, acc, m0, nt0, n_tiles, lane,
         reinterpret_cast<char*>(&s_t0[0][0]) + wave * kRowsStageBytes);
   } else {
-    rows_epilogue<SWAP, NT>(g, acc, m0, nt0, n_tiles, l16, gq);
+    rows_epilogue_values<NT>(g, acc, m0, nt0, n_tiles, l16, gq);
   }
 }
 
