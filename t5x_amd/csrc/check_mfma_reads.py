@@ -14,6 +14,16 @@ and fails when any path from a v_mfma / v_smfmac to a reader of its
 destination is shorter than NEED slots (9: what the compiler itself pads
 straight-line code to for the 16x16x32 instructions used here).
 
+A second check, for the kernels that fill LDS with global_load_lds behind
+hand-placed barriers: a barrier orders instructions that have been issued,
+not LDS reads that have completed, and the compiler may sink a k-tile's last
+operand reads below the next barrier; a faster wavefront could then refill
+the stage while those reads were still queued (seen as a wrong 16-row slice
+in one launch in ten of the many-row dense kernel).  So in such a kernel
+every s_barrier must come after an s_waitcnt that includes
+lgkmcnt(0) — checked as: walking backwards from a barrier, over branches too,
+no LDS instruction is met before such a wait.
+
 usage: check_mfma_reads.py file.s [...]
 """
 import collections
@@ -107,12 +117,60 @@ def short_reads(text, need=NEED):
   return found, hist
 
 
+def unguarded_barriers(text, depth=96):
+  """-> [(kernel, index of the barrier among the kernel's barriers)] for
+  kernels that use global_load_lds: barriers that an LDS read can reach
+  without a wait for lgkmcnt(0) in between, on any path (walking backwards
+  from the barrier, over branches too, until such a wait ends the path)."""
+  ins, labels = parse(text)
+  uses_dma = {k for k, t in ins if t.startswith('global_load_lds')}
+  if not uses_dma:
+    return []
+  preds = collections.defaultdict(list)
+  for i, (kernel, t) in enumerate(ins):
+    m = re.match(r's_(c?)branch\w*\s+(\.LBB\w+)', t)
+    if m:
+      target = labels.get((kernel, m.group(2)))
+      if target is not None:
+        preds[target].append(i)
+    falls_through = not (m and not m.group(1)) and not t.startswith('s_endpgm')
+    if falls_through and i + 1 < len(ins) and ins[i + 1][0] == kernel:
+      preds[i + 1].append(i)
+  found, count = [], collections.Counter()
+  for i, (kernel, t) in enumerate(ins):
+    if kernel not in uses_dma or not t.startswith('s_barrier'):
+      continue
+    count[kernel] += 1
+    seen, stack, bad = set(), [(p, 0) for p in preds[i]], False
+    while stack and not bad:
+      j, d = stack.pop()
+      if j in seen or d > depth:
+        continue
+      seen.add(j)
+      tj = ins[j][1]
+      if tj.startswith('s_waitcnt') and 'lgkmcnt(0)' in tj:
+        continue                   # this path is guarded
+      if tj.startswith('ds_'):
+        bad = True
+        break
+      stack.extend((p, d + 1) for p in preds[j])
+    if bad:
+      found.append((kernel, count[kernel]))
+  return found
+
+
 def main(paths):
-  bad = 0
+  bad = barriers = 0
   total = collections.Counter()
   for path in paths:
     with open(path) as f:
-      found, hist = short_reads(f.read())
+      text = f.read()
+    found, hist = short_reads(text)
+    for kernel, nth in unguarded_barriers(text):
+      barriers += 1
+      print(f'{path}: {kernel}: barrier {nth} of a kernel that loads into LDS '
+            'is reached by an LDS instruction with no wait for lgkmcnt(0) '
+            'in between')
     total.update(hist)
     for kernel, t, n, t2 in found:
       bad += 1
@@ -120,8 +178,8 @@ def main(paths):
             f'(need {NEED})')
   print(f'check_mfma_reads: {sum(total.values())} reads of matrix results in '
         f'{len(paths)} files, shortest {min(total) if total else "-"} slots, '
-        f'{bad} too early')
-  return 1 if bad else 0
+        f'{bad} too early; {barriers} unguarded barriers')
+  return 1 if bad or barriers else 0
 
 
 if __name__ == '__main__':

@@ -91,6 +91,52 @@ def test_overwritten_result_is_not_a_read():
   assert found == [] and not hist
 
 
+_RING_GUARDED = """
+_Z6kernelv:
+	global_load_lds_dwordx4 v[4:5], off
+.LBB0_1:
+	ds_read_b128 v[0:3], v8
+	s_cbranch_scc1 .LBB0_3
+	s_waitcnt vmcnt(2) lgkmcnt(0)
+	s_branch .LBB0_4
+.LBB0_3:
+	s_waitcnt vmcnt(0) lgkmcnt(0)
+.LBB0_4:
+	s_add_i32 s6, s33, 4
+	s_barrier
+	global_load_lds_dwordx4 v[4:5], off
+	s_cbranch_scc0 .LBB0_1
+	s_endpgm
+"""
+
+# the operand read after the last full wait reaches the barrier unwaited
+_RING_SUNK_READ = """
+_Z6kernelv:
+	global_load_lds_dwordx4 v[4:5], off
+	s_waitcnt vmcnt(0) lgkmcnt(0)
+	ds_read_b128 v[0:3], v8
+	s_waitcnt vmcnt(2)
+	s_barrier
+	global_load_lds_dwordx4 v[4:5], off
+	s_waitcnt lgkmcnt(0)
+	s_endpgm
+"""
+
+_NO_DMA = """
+_Z6kernelv:
+	ds_read_b128 v[0:3], v8
+	s_barrier
+	s_endpgm
+"""
+
+
+def test_barriers_of_kernels_that_load_into_lds_need_a_wait_for_lds_reads():
+  mod = _checker()
+  assert mod.unguarded_barriers(_RING_GUARDED) == []
+  assert mod.unguarded_barriers(_RING_SUNK_READ) == [('_Z6kernelv', 1)]
+  assert mod.unguarded_barriers(_NO_DMA) == []   # other kernels: not checked
+
+
 def test_built_kernels_have_no_early_read():
   files = sorted(glob.glob(os.path.join(CSRC, 'isa', '*.s')))
   if not files:
@@ -100,3 +146,4 @@ def test_built_kernels_have_no_early_read():
     with open(path) as f:
       found, _ = mod.short_reads(f.read())
     assert found == [], (path, found[:3])
+    assert mod.unguarded_barriers(open(path).read()) == [], path
