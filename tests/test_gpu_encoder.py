@@ -224,6 +224,29 @@ def test_encoder_attention(ops, B, E, H):
   np.testing.assert_allclose(got, want, atol=2e-2, rtol=2**-6)
 
 
+def test_encoder_attention_repeated_launches(ops):
+  """30 launches of the attention kernel for lengths up to 512 (K and V go
+  through a ring of LDS stages behind hand-placed barriers) at 8 x 12 heads x
+  512 positions give one result, and so does the kernel for longer texts."""
+  g = torch.Generator(device='cuda')
+  g.manual_seed(11)
+  bf = torch.bfloat16
+  for E, variants in ((512, (1, 2)), (640, (1,))):
+    B, H = 8, 12
+    q = (torch.randn(B * E, H * 64, device='cuda', generator=g) * 0.125).to(bf)
+    k = torch.randn(B * E, H * 64, device='cuda', generator=g).to(bf)
+    v = torch.randn(B, H, 64, E, device='cuda', generator=g).to(bf)
+    rel = torch.randn(H, 2 * E - 1, device='cuda', generator=g).to(bf)
+    lens = torch.tensor([E, 1, 17, 300, E - 1, 64, 65, 480][:B],
+                        dtype=torch.int32, device='cuda')
+    v_t = ops.tile_cross_value(v.contiguous())
+    for variant in variants:
+      first = ops.encoder_attention(q, k, v_t, rel, lens, variant=variant)
+      for _ in range(30):
+        again = ops.encoder_attention(q, k, v_t, rel, lens, variant=variant)
+        assert torch.equal(first, again), (E, variant)
+
+
 def _holes(rs, B, E):
   """A validity mask with padding inside the text: row 0 all valid, the others
   with a valid prefix that has holes, and padding at the end."""
