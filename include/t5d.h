@@ -172,6 +172,11 @@ int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
                         const void* residual, void* C, int64_t M, int K, int N,
                         int epilogue, int out_layout, int E, int Ep, int tile);
 
+/* The workgroup tile (1, 2 or 3, as in t5d_gemm_rows_tiled) that t5d_gemm_rows
+ * uses for a shape: the cheapest by the rounds of workgroups each tile needs
+ * on 256 CUs.  No device work; for tests and for reading a profile. */
+int t5d_gemm_rows_tile(int w_dtype, int64_t M, int K, int N);
+
 /* One step of cached decoder self-attention
  * (MultiHeadDotProductAttention decode branch,
  * t5x/examples/t5/layers.py:223-346, and dot_product_attention :52-129).

@@ -111,6 +111,7 @@ _SIGNATURES = {
     't5d_gemm_rows_tiled': (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int64,
                                     c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int]),
+    't5d_gemm_rows_tile': (c_int, [c_int, c_int64, c_int, c_int]),
     't5d_gemm_tiled': (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P,
                                c_int, c_int, c_int, c_int, _P, c_int, c_int,
                                c_int]),

@@ -524,6 +524,34 @@ rows_gemm_direct_kernel(RowsGemmArgs g) {
 
 using namespace t5d;
 
+// Three workgroup tiles.  256 x 256 (8 wavefronts, one workgroup per CU)
+// halves the operand bytes per flop of 256 x 128 (4 wavefronts, two per CU)
+// and measures 3-11 % faster whenever its workgroups fill the 256 CUs
+// evenly; 256 x 192 (8 wavefronts of 128 x 48) is for the shapes where
+// neither does: N = 768 over 16384 rows is 192 tiles of 256 x 256 (a quarter
+// of the chip idle) but exactly 256 of 256 x 192.  Picked by the cost of the
+// rounds each tile needs, a last round that fills at most half of the CUs'
+// two slots counting 0.6 for the 256 x 128 tile.
+extern "C" int t5d_gemm_rows_tile(int w_dtype, int64_t M, int K, int N) {
+  if (w_dtype != T5D_BF16 || K < 64 || M <= 0 || N <= 0) return 1;
+  const auto rounds = [](int64_t wgs, int slots) {
+    return (double)((wgs + slots - 1) / slots);
+  };
+  const int64_t m_blocks = (M + kRowsBM - 1) / kRowsBM;
+  const int64_t wgs128 = m_blocks * ((N + 127) / 128),
+                wgs192 = m_blocks * ((N + 191) / 192),
+                wgs256 = m_blocks * ((N + 255) / 256);
+  double c128 = rounds(wgs128, 512) * 2.0 * 128;
+  if ((wgs128 - 1) % 512 < 256) c128 -= 0.4 * 2.0 * 128;
+  const double c192 = rounds(wgs192, 256) * 192.0,
+               c256 = rounds(wgs256, 256) * 256.0;
+  int pick = 2;
+  double best = c256;
+  if (c192 < best) { best = c192; pick = 3; }
+  if (c128 < 0.97 * best) pick = 1;
+  return pick;
+}
+
 extern "C" int t5d_gemm_rows(void* stream, int w_dtype, const void* A,
                              const void* W, const float* scales,
                              const void* residual, void* C, int64_t M, int K,
@@ -581,31 +609,9 @@ extern "C" int t5d_gemm_rows_tiled(void* stream, int w_dtype, const void* A,
   dim3 grid((unsigned)m_blocks * n_blocks), block(256);
   hipStream_t s = as_stream(stream);
   const bool swap = out_layout != T5D_OUT_HEADS_VALUE;
-  // Three workgroup tiles.  256 x 256 (8 wavefronts, one workgroup per CU)
-  // halves the operand bytes per flop of 256 x 128 (4 wavefronts, two per CU)
-  // and measures 3-11 % faster whenever its workgroups fill the 256 CUs
-  // evenly; 256 x 192 (8 wavefronts of 128 x 48) is for the shapes where
-  // neither does: N = 768 over 16384 rows is 192 tiles of 256 x 256 (a quarter
-  // of the chip idle) but exactly 256 of 256 x 192.  Picked by the cost of the
-  // rounds each tile needs, a last round that fills at most half of the CUs'
-  // two slots counting 0.6 for the 256 x 128 tile.
-  const auto rounds = [](int wgs, int slots) {
-    return (wgs + slots - 1) / slots;
-  };
-  const int n192 = (N + 191) / 192, n256 = (N + 255) / 256;
-  const int wgs128 = m_blocks * n_blocks, wgs192 = m_blocks * n192,
-            wgs256 = m_blocks * n256;
-  double c128 = rounds(wgs128, 512) * 2.0 * 128;
-  if ((wgs128 - 1) % 512 < 256) c128 -= 0.4 * 2.0 * 128;
-  const double c192 = rounds(wgs192, 256) * 192.0,
-               c256 = rounds(wgs256, 256) * 256.0;
-  int pick = tile;
-  if (pick == 0) {
-    pick = 2;
-    double best = c256;
-    if (c192 < best) { best = c192; pick = 3; }
-    if (c128 < 0.97 * best) pick = 1;
-  }
+  const int pick = tile ? tile : t5d_gemm_rows_tile(w_dtype, M, K, N);
+  const int wgs192 = m_blocks * ((N + 191) / 192),
+            wgs256 = m_blocks * ((N + 255) / 256);
   if (w_dtype == T5D_BF16 && K >= 64 && pick == 3) {
     dim3 wgrid((unsigned)wgs192), wblock(512);
     if (swap)

@@ -81,6 +81,23 @@ def test_version_and_error_string_without_gpu():
   assert b'dtype' in lib.t5d_last_error()
 
 
+def test_many_row_tile_choice_without_gpu():
+  """t5d_gemm_rows_tile: which workgroup tile the many-row dense kernel runs a
+  shape on (1: 256 x 128, 2: 256 x 256, 3: 256 x 192), by the rounds of
+  workgroups on 256 CUs.  The T5.1.1-base encoder over 32 x 512 positions:"""
+  lib = _lib.load()
+  pick = lambda M, K, N, w=_lib.BF16: lib.t5d_gemm_rows_tile(w, M, K, N)
+  assert pick(16384, 768, 768) == 3     # 192 tiles of 256 x 256, 256 of 256 x 192
+  assert pick(16384, 2048, 768) == 3
+  assert pick(16384, 768, 4096) == 2    # 4 full rounds of 256 x 256
+  assert pick(16384, 768, 1536) == 3    # 2 rounds of 512 tiles of 256 x 192
+  assert pick(16384, 4096, 4096) == 2
+  assert pick(300, 96, 80) == 1         # one small workgroup
+  # int8 weights and K < 64 run on the staging-register kernel: 256 x 128
+  assert pick(16384, 768, 768, _lib.I8) == 1
+  assert pick(16384, 32, 768) == 1
+
+
 def test_product_path_has_no_cpu_fallback():
   import torch
   if torch.cuda.is_available():
